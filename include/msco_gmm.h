@@ -1,0 +1,141 @@
+/*
+ * msco_gmm.h -- C ABI of the MI355X (gfx950) backend for the grouped quantized matmul path.
+ *
+ * This is the boundary the C++ operator-registration layer calls instead of the reference's
+ * closed kernel objects:
+ *
+ *   reference kernel-object life cycle (what the op glue calls)          this ABI
+ *   ------------------------------------------------------------------  ---------------------------
+ *   internal_v2::CreateGroupedMatmulOp(inputs, outputs, MatmulParam)     msco_gmm_create
+ *     ops/c_api/grouped_matmul/grouped_matmul.cc:216-232,266-276
+ *   InternalOp::Init / UpdateShape / GetTilingSize / Tiling /            msco_gmm_plan
+ *   GetWorkspaceSize
+ *     ops/framework/ms_kernels_internal/pyboost/internal_pyboost_runner.cc:34-58,99-113
+ *   InternalOp::Launch(in_addrs, out_addrs, ws_addrs, stream, name)      msco_gmm_launch
+ *     ops/framework/ms_kernels_internal/pyboost/internal_pyboost_runner.cc:210-231
+ *   aclnnGroupedMatmulV4 GetWorkspaceSize + execute                      msco_gmm_plan + msco_gmm_launch
+ *     ops/c_api/grouped_matmul_v4_cops/grouped_matmul_v4_cops.cc:94-97,359-363
+ *   aclnnQuantMatmulV4  GetWorkspaceSize + execute                       msco_gmm_plan + msco_gmm_launch
+ *     ops/c_api/quant_batch_matmul/quant_batch_matmul.cc:78-80,144-145
+ *   INTERNAL_PRINT_TILING (tests/st/test_grouped_matmul.py:86)           msco_gmm_plan_info
+ *
+ * Conventions
+ *   - every entry point returns an int status, 0 (MSCO_OK) on success; the C++ layer above turns a
+ *     non-zero status into an exception exactly where the reference does
+ *     (internal_pyboost_runner.cc:227-229);
+ *   - all tensor arguments are raw device pointers to contiguous row-major buffers that the caller
+ *     owns; an absent optional input is a NULL pointer (internal_pyboost_runner.h:69-78);
+ *   - group_list stays on the device: nothing in plan or launch reads tensor values on the host;
+ *   - launch enqueues on the given stream, never synchronises and never allocates.  A plan that
+ *     needs cross-workgroup reduction state keeps a few KiB of device memory inside the handle
+ *     (allocated by msco_gmm_plan, released by msco_gmm_destroy); because that state is per handle,
+ *     one handle must not be launched concurrently on two streams.
+ */
+#ifndef MSCO_GMM_H_
+#define MSCO_GMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MSCO_GMM_ABI_VERSION 1
+
+#if defined(MSCO_BUILDING_LIB)
+#define MSCO_API __attribute__((visibility("default")))
+#else
+#define MSCO_API
+#endif
+
+typedef enum msco_status {
+  MSCO_OK = 0,
+  MSCO_ERR_INVALID_ARG = 1,   /* NULL where a pointer is required, bad enum value */
+  MSCO_ERR_UNSUPPORTED = 2,   /* dtype / layout combination the backend does not implement */
+  MSCO_ERR_SHAPE = 3,         /* shape rule violated (K, N, E alignment or mismatch) */
+  MSCO_ERR_NOT_PLANNED = 4,   /* launch before plan */
+  MSCO_ERR_WORKSPACE = 5,     /* workspace too small or NULL when the plan needs one */
+  MSCO_ERR_DEVICE = 6         /* HIP runtime error (no device, launch failure) */
+} msco_status;
+
+typedef enum msco_dtype {
+  MSCO_DT_NONE = 0,  /* input absent */
+  MSCO_DT_I8 = 1,
+  MSCO_DT_I32 = 2,
+  MSCO_DT_I64 = 3,
+  MSCO_DT_U64 = 4,
+  MSCO_DT_F16 = 5,
+  MSCO_DT_BF16 = 6,
+  MSCO_DT_F32 = 7
+} msco_dtype;
+
+/* Positional inputs of msco_gmm_launch.  Slots 0..6 follow the order the reference passes to its
+ * kernel object (grouped_matmul.cc:201-207,301-307); slot 7 is the V4 antiquant offset
+ * (grouped_matmul_v4_cops.cc:94-97). */
+enum {
+  MSCO_IN_X = 0,               /* [M,K] int8 (W8A8) or bf16/f16 (W8A16) */
+  MSCO_IN_WEIGHT = 1,          /* [E,K,N] int8, or [E,N,K] when transpose_b */
+  MSCO_IN_BIAS = 2,            /* [E,N] int32, optional */
+  MSCO_IN_SCALE = 3,           /* [E,N] f32 / bf16 / int64|uint64 carrying f32 bits in the low word; optional */
+  MSCO_IN_GROUP_LIST = 4,      /* [E] int32 / int64; NULL = E equal groups of M/E rows (dense / batched) */
+  MSCO_IN_PER_TOKEN_SCALE = 5, /* [M] f32, optional */
+  MSCO_IN_ANTIQUANT_SCALE = 6, /* [E,N] in x's dtype, W8A16 only */
+  MSCO_IN_ANTIQUANT_OFFSET = 7,/* [E,N] in x's dtype, W8A16 only, optional */
+  MSCO_IN_COUNT = 8
+};
+
+/* Immutable description of one operator instance (dtypes, layouts, flags) -- the part the
+ * reference hashes into its op key (internal_pyboost_runner.h:43-48). */
+typedef struct msco_gmm_desc {
+  int32_t abi_version;       /* MSCO_GMM_ABI_VERSION */
+  int32_t x_dtype;           /* I8 | BF16 | F16 */
+  int32_t weight_dtype;      /* I8 */
+  int32_t out_dtype;         /* BF16 | F16 | I32 (raw accumulator + bias; scales are not applied) */
+  int32_t group_list_dtype;  /* I32 | I64 | NONE */
+  int32_t group_list_type;   /* 0 cumulative row ends, 1 per-group row counts */
+  int32_t bias_dtype;        /* NONE | I32 */
+  int32_t scale_dtype;       /* NONE | F32 | BF16 | I64 | U64 */
+  int32_t per_token_dtype;   /* NONE | F32 */
+  int32_t antiquant_dtype;   /* NONE | BF16 | F16 (scale and offset share it) */
+  int32_t has_antiquant_offset;
+  int32_t transpose_b;       /* 0: weight [E,K,N]; 1: weight [E,N,K] */
+  int32_t scale_per_group;   /* 1: scale/bias are [E,N]; 0: one [N] (or [1]) row shared by all groups */
+  int32_t scale_is_scalar;   /* 1: scale holds a single element broadcast over N */
+  int32_t kernel_override;   /* 0 auto; else force a kernel family (see msco_gmm_plan_info), for tests */
+  int32_t reserved[5];
+} msco_gmm_desc;
+
+typedef struct msco_gmm_op *msco_gmm_handle;
+
+/* Create an operator instance.  Replaces CreateGroupedMatmulOp + Init. */
+MSCO_API int msco_gmm_create(const msco_gmm_desc *desc, msco_gmm_handle *out_handle);
+
+/* Fix the shapes (shape-dependent work of Resize: kernel choice, grid, workspace size).
+ * m = rows of x, k = reduction length, n = output columns, e = number of groups.
+ * Replaces UpdateShape + Tiling + GetWorkspaceSize.  May be called again with new shapes. */
+MSCO_API int msco_gmm_plan(msco_gmm_handle h, int64_t m, int64_t k, int64_t n, int64_t e, size_t *workspace_bytes);
+
+/* Enqueue the computation.  inputs[MSCO_IN_COUNT] are device pointers (NULL = absent);
+ * out is [M,N] in out_dtype; stream is a hipStream_t (NULL = default stream). */
+MSCO_API int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, void *workspace,
+                    size_t workspace_bytes, void *stream);
+
+/* Human-readable description of the current plan (kernel family, tile, grid, split) -- the
+ * counterpart of the reference's INTERNAL_PRINT_TILING switch.  Returns the number of characters
+ * that the full text needs (excluding the terminating NUL). */
+MSCO_API int msco_gmm_plan_info(msco_gmm_handle h, char *buf, size_t buf_len);
+
+/* Release the instance and any device state it holds. */
+MSCO_API int msco_gmm_destroy(msco_gmm_handle h);
+
+/* Static text for a status code. */
+MSCO_API const char *msco_status_string(int status);
+
+/* ABI version the library was built with. */
+MSCO_API int msco_gmm_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* MSCO_GMM_H_ */

@@ -1,0 +1,101 @@
+"""In-tree build of the native parts: the HIP backend behind the C ABI (libmsco_gmm.so) and the
+pybind11 operator-registration module (ms_custom_ops.*.so).  hipcc cross-compiles gfx950 code
+objects without a GPU, so this runs anywhere the ROCm toolchain is installed."""
+from __future__ import annotations
+
+import concurrent.futures as cf
+import os
+import shutil
+import subprocess
+import sys
+import sysconfig
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_DIR = os.path.dirname(PKG_DIR)
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+OBJ_DIR = os.path.join(PKG_DIR, "lib", "obj")
+INCLUDE = os.path.join(REPO_DIR, "include")
+
+BACKEND_LIB = os.path.join(LIB_DIR, "libmsco_gmm.so")
+HIP_SOURCES = ["gmm_tile_w8a8.hip", "gmm_skinny_w8a8.hip", "gmm_skinny_a16w8.hip", "gmm_generic.hip", "msco_gmm.hip"]
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the HIP backend cannot be built")
+    return exe
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+    return proc.stdout
+
+
+def build_backend(verbose: bool = False) -> str:
+    """Compile every HIP source for gfx950 and link libmsco_gmm.so."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    hipcc = _hipcc()
+    hip_dir = os.path.join(CSRC, "hip")
+
+    def compile_one(src):
+        obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+        cmd = [hipcc] + HIP_FLAGS + ["-DMSCO_BUILDING_LIB", "-I", INCLUDE, "-I", hip_dir, "-c",
+                                     os.path.join(hip_dir, src), "-o", obj]
+        out = _run(cmd)
+        if verbose and out.strip():
+            print(out)
+        return obj
+
+    with cf.ThreadPoolExecutor(max_workers=min(8, len(HIP_SOURCES))) as pool:
+        objs = list(pool.map(compile_one, HIP_SOURCES))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", BACKEND_LIB] + objs)
+    return BACKEND_LIB
+
+
+def pybind_module_path() -> str:
+    suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
+    return os.path.join(PKG_DIR, "ms_custom_ops" + suffix)
+
+
+def build_pybind(verbose: bool = False) -> str:
+    """Compile the C++ operator layer (framework + one translation unit per op) into a pybind11
+    module that links against libmsco_gmm.so."""
+    import pybind11
+
+    cxx = shutil.which("g++") or "g++"
+    srcs = []
+    for root, _, files in os.walk(os.path.join(CSRC, "ops")):
+        for f in sorted(files):
+            if f.endswith(".cc"):
+                srcs.append(os.path.join(root, f))
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    flags = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-DMS_EXTENSION_NAME=ms_custom_ops",
+             "-I", INCLUDE, "-I", CSRC, "-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"]]
+
+    def compile_one(src):
+        obj = os.path.join(OBJ_DIR, os.path.relpath(src, CSRC).replace(os.sep, "_").replace(".cc", ".o"))
+        out = _run([cxx] + flags + ["-c", src, "-o", obj])
+        if verbose and out.strip():
+            print(out)
+        return obj
+
+    with cf.ThreadPoolExecutor(max_workers=8) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    target = pybind_module_path()
+    _run([cxx, "-shared", "-o", target] + objs + ["-L", LIB_DIR, "-lmsco_gmm", "-Wl,-rpath,$ORIGIN/lib"])
+    return target
+
+
+def build_all(verbose: bool = False):
+    return build_backend(verbose), build_pybind(verbose)
+
+
+if __name__ == "__main__":
+    for path in build_all(verbose="-v" in sys.argv):
+        print("built", path)

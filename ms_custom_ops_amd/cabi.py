@@ -1,0 +1,134 @@
+"""ctypes binding of the backend's C ABI (include/msco_gmm.h).
+
+This is the thinnest possible host: it loads libmsco_gmm.so, mirrors ``msco_gmm_desc`` and hands
+raw device pointers to the library.  Tests and the benchmark use it to call the backend exactly the
+way a foreign-language binding would; the operator layer proper is the pybind11 module.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmsco_gmm.so")
+
+ABI_VERSION = 1
+
+# msco_dtype
+DT_NONE, DT_I8, DT_I32, DT_I64, DT_U64, DT_F16, DT_BF16, DT_F32 = range(8)
+
+# positional launch inputs
+IN_X, IN_WEIGHT, IN_BIAS, IN_SCALE, IN_GROUP_LIST, IN_PER_TOKEN_SCALE, IN_ANTIQUANT_SCALE, IN_ANTIQUANT_OFFSET = range(8)
+IN_COUNT = 8
+
+# msco_gmm_desc.kernel_override
+OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC = range(6)
+
+EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco_gmm_plan_info", "msco_gmm_destroy",
+                    "msco_status_string", "msco_gmm_abi_version")
+
+
+class GmmDesc(ctypes.Structure):
+    _fields_ = [(name, ctypes.c_int32) for name in (
+        "abi_version", "x_dtype", "weight_dtype", "out_dtype", "group_list_dtype", "group_list_type", "bias_dtype",
+        "scale_dtype", "per_token_dtype", "antiquant_dtype", "has_antiquant_offset", "transpose_b", "scale_per_group",
+        "scale_is_scalar", "kernel_override")] + [("reserved", ctypes.c_int32 * 5)]
+
+
+class BackendError(RuntimeError):
+    def __init__(self, where: str, status: int, text: str):
+        super().__init__(f"{where} failed: status {status} ({text})")
+        self.status = status
+
+
+_lib = None
+
+
+def load():
+    """Load the backend library; raises if it has not been built (there is no fallback path)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"HIP backend library missing: {LIB_PATH}; build it with "
+                              "`python -m ms_custom_ops_amd.build`")
+        lib = ctypes.CDLL(LIB_PATH)
+        lib.msco_gmm_create.restype = ctypes.c_int
+        lib.msco_gmm_create.argtypes = [ctypes.POINTER(GmmDesc), ctypes.POINTER(ctypes.c_void_p)]
+        lib.msco_gmm_plan.restype = ctypes.c_int
+        lib.msco_gmm_plan.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                      ctypes.POINTER(ctypes.c_size_t)]
+        lib.msco_gmm_launch.restype = ctypes.c_int
+        lib.msco_gmm_launch.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p,
+                                        ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        lib.msco_gmm_plan_info.restype = ctypes.c_int
+        lib.msco_gmm_plan_info.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]
+        lib.msco_gmm_destroy.restype = ctypes.c_int
+        lib.msco_gmm_destroy.argtypes = [ctypes.c_void_p]
+        lib.msco_status_string.restype = ctypes.c_char_p
+        lib.msco_status_string.argtypes = [ctypes.c_int]
+        lib.msco_gmm_abi_version.restype = ctypes.c_int
+        lib.msco_gmm_abi_version.argtypes = []
+        _lib = lib
+    return _lib
+
+
+def status_string(status: int) -> str:
+    return load().msco_status_string(int(status)).decode()
+
+
+def _check(where: str, status: int):
+    if status != 0:
+        raise BackendError(where, status, status_string(status))
+
+
+class GmmOp:
+    """One backend operator instance: create -> plan -> launch* -> destroy."""
+
+    def __init__(self, **fields):
+        lib = load()
+        desc = GmmDesc()
+        desc.abi_version = ABI_VERSION
+        desc.weight_dtype = DT_I8
+        desc.scale_per_group = 1
+        for key, value in fields.items():
+            if not hasattr(desc, key):
+                raise AttributeError(key)
+            setattr(desc, key, int(value))
+        self.desc = desc
+        self._h = ctypes.c_void_p()
+        _check("msco_gmm_create", lib.msco_gmm_create(ctypes.byref(desc), ctypes.byref(self._h)))
+        self.workspace_bytes = 0
+
+    def plan(self, m: int, k: int, n: int, e: int) -> int:
+        ws = ctypes.c_size_t(0)
+        _check("msco_gmm_plan", load().msco_gmm_plan(self._h, m, k, n, e, ctypes.byref(ws)))
+        self.workspace_bytes = int(ws.value)
+        return self.workspace_bytes
+
+    def plan_info(self) -> str:
+        buf = ctypes.create_string_buffer(512)
+        load().msco_gmm_plan_info(self._h, buf, 512)
+        return buf.value.decode()
+
+    def launch(self, inputs: Sequence[Optional[int]], out: int, workspace: Optional[int] = None,
+               workspace_bytes: int = 0, stream: Optional[int] = None):
+        """inputs: IN_COUNT device addresses (None/0 = absent)."""
+        arr = (ctypes.c_void_p * IN_COUNT)()
+        for i in range(IN_COUNT):
+            v = inputs[i] if i < len(inputs) else None
+            arr[i] = ctypes.c_void_p(v if v else None)
+        _check("msco_gmm_launch", load().msco_gmm_launch(self._h, arr, ctypes.c_void_p(out),
+                                                         ctypes.c_void_p(workspace if workspace else None),
+                                                         workspace_bytes, ctypes.c_void_p(stream if stream else None)))
+
+    def close(self):
+        if self._h:
+            load().msco_gmm_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # interpreter shutdown
+            pass

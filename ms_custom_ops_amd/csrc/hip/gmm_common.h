@@ -1,0 +1,150 @@
+// Shared device-side definitions for the gfx950 grouped quantized matmul kernels.
+#ifndef MSCO_GMM_COMMON_H_
+#define MSCO_GMM_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace msco {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+// dtype codes shared with include/msco_gmm.h (msco_dtype)
+enum : int { DT_NONE = 0, DT_I8 = 1, DT_I32 = 2, DT_I64 = 3, DT_U64 = 4, DT_F16 = 5, DT_BF16 = 6, DT_F32 = 7 };
+
+constexpr int kNumXcd = 8;        // MI355X: 8 accelerator complex dies, workgroups are dealt round-robin
+constexpr int kSkinnyRows = 16;   // rows one MFMA covers in the skinny kernels
+constexpr int kSkinnyCols = 128;  // output columns one skinny workgroup owns
+
+// Kernel argument block.  Plain pointers and sizes only.
+struct GmmParams {
+  const void *x;            // [M,K] int8 or bf16/f16
+  const int8_t *w;          // [E,K,N] or [E,N,K]
+  const int32_t *bias;      // [E,N] or [N] or null
+  const void *scale;        // [E,N] / [N] / [1] in scale_dtype, or null
+  const void *group_list;   // [E] int32/int64 or null
+  const float *per_token;   // [M] or null
+  const void *aq_scale;     // [E,N] bf16/f16 (W8A16)
+  const void *aq_offset;    // [E,N] bf16/f16 or null
+  void *out;                // [M,N]
+  int32_t *partial;         // split-K partial tiles (workspace)
+  unsigned *counters;       // split-K arrival counters (handle-owned, self-resetting)
+  int m, k, n, e;
+  int gl_dtype;             // DT_NONE / DT_I32 / DT_I64
+  int gl_type;              // 0 cumulative ends, 1 counts
+  int scale_dtype;          // DT_NONE / DT_F32 / DT_BF16 / DT_I64 / DT_U64
+  int scale_per_group;      // scale & bias carry a row per group
+  int scale_is_scalar;      // scale has a single element
+  int out_dtype;            // DT_BF16 / DT_F16 / DT_I32
+  int x_dtype;              // DT_I8 / DT_BF16 / DT_F16
+  int split_k;              // number of K splits across workgroups (skinny kernels)
+  int n_strips;             // ceil(N / kSkinnyCols)
+};
+
+// ---- group_list --------------------------------------------------------------------------------
+// Row end of group g given the previous end; the result is clamped into [prev, M] so a malformed
+// list can never produce an out-of-range row.
+__device__ __forceinline__ int group_end(const GmmParams &p, int g, int prev) {
+  long long v;
+  if (p.gl_dtype == DT_I64) {
+    v = reinterpret_cast<const long long *>(p.group_list)[g];
+  } else if (p.gl_dtype == DT_I32) {
+    v = reinterpret_cast<const int *>(p.group_list)[g];
+  } else {
+    v = (long long)(p.m / p.e) * (g + 1);  // dense / batched: equal groups
+  }
+  long long end = (p.gl_type == 1 && p.gl_dtype != DT_NONE) ? (long long)prev + v : v;
+  if (end < prev) end = prev;
+  if (end > p.m) end = p.m;
+  return (int)end;
+}
+
+// ---- number formats ----------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_bits_to_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
+
+// float32 -> bfloat16, round to nearest even (NaN stays quiet NaN).
+__device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) return (unsigned short)((u >> 16) | 0x40u);
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (unsigned short)(u >> 16);
+}
+
+__device__ __forceinline__ unsigned short f32_to_f16_rne(float f) {
+  _Float16 h = (_Float16)f;  // v_cvt_f16_f32, IEEE round to nearest even
+  return __builtin_bit_cast(unsigned short, h);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(unsigned short b) {
+  return (float)__builtin_bit_cast(_Float16, b);
+}
+
+// Dequant scale of column n for group g.  int64/uint64 scales carry float32 bits in the low word.
+__device__ __forceinline__ float load_scale(const GmmParams &p, int g, int n) {
+  if (p.scale_dtype == DT_NONE) return 1.0f;
+  long long idx = p.scale_is_scalar ? 0 : ((p.scale_per_group ? (long long)g * p.n : 0) + n);
+  if (p.scale_dtype == DT_F32) return reinterpret_cast<const float *>(p.scale)[idx];
+  if (p.scale_dtype == DT_BF16) return bf16_bits_to_f32(reinterpret_cast<const unsigned short *>(p.scale)[idx]);
+  return __uint_as_float(reinterpret_cast<const unsigned *>(p.scale)[2 * idx]);
+}
+
+__device__ __forceinline__ int load_bias(const GmmParams &p, int g, int n) {
+  if (p.bias == nullptr) return 0;
+  return p.bias[(p.scale_per_group ? (long long)g * p.n : 0) + n];
+}
+
+// Epilogue of one element in the reference golden's operation order:
+// float32(acc + bias) * scale[n] * per_token[m], each product rounded to float32.
+__device__ __forceinline__ float dequant(int acc_plus_bias, float scale, float per_token) {
+  float f = (float)acc_plus_bias;
+  f = f * scale;
+  f = f * per_token;
+  return f;
+}
+
+__device__ __forceinline__ void store_out(const GmmParams &p, long long idx, int acc_plus_bias, float f) {
+  if (p.out_dtype == DT_BF16) {
+    reinterpret_cast<unsigned short *>(p.out)[idx] = f32_to_bf16_rne(f);
+  } else if (p.out_dtype == DT_F16) {
+    reinterpret_cast<unsigned short *>(p.out)[idx] = f32_to_f16_rne(f);
+  } else {
+    reinterpret_cast<int *>(p.out)[idx] = acc_plus_bias;
+  }
+}
+
+// ---- byte shuffles -----------------------------------------------------------------------------
+// v_perm_b32: result byte i = byte sel[i] of the 8-byte value {hi:lo} (0..3 -> lo, 4..7 -> hi).
+__device__ __forceinline__ unsigned perm(unsigned hi, unsigned lo, unsigned sel) {
+  return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+// 4x4 byte transpose: r[i] holds 4 column bytes of row i; c[j] receives the 4 row bytes of column j.
+__device__ __forceinline__ void transpose4x4(unsigned r0, unsigned r1, unsigned r2, unsigned r3, unsigned &c0,
+                                             unsigned &c1, unsigned &c2, unsigned &c3) {
+  const unsigned lo01 = perm(r1, r0, 0x05010400u);  // r0.b0 r1.b0 r0.b1 r1.b1
+  const unsigned hi01 = perm(r1, r0, 0x07030602u);  // r0.b2 r1.b2 r0.b3 r1.b3
+  const unsigned lo23 = perm(r3, r2, 0x05010400u);
+  const unsigned hi23 = perm(r3, r2, 0x07030602u);
+  c0 = perm(lo23, lo01, 0x05040100u);
+  c1 = perm(lo23, lo01, 0x07060302u);
+  c2 = perm(hi23, hi01, 0x05040100u);
+  c3 = perm(hi23, hi01, 0x07060302u);
+}
+
+// Transpose a 16 (rows, k) x 8 (cols, n) byte block held as 16 uint2 row pieces into 8 column
+// fragments of 16 k-bytes each (v4i = k 0..3, 4..7, 8..11, 12..15).
+__device__ __forceinline__ void transpose16x8(const uint2 (&r)[16], v4i (&frag)[8]) {
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    unsigned c0, c1, c2, c3;
+    transpose4x4(r[4 * q].x, r[4 * q + 1].x, r[4 * q + 2].x, r[4 * q + 3].x, c0, c1, c2, c3);
+    frag[0][q] = (int)c0; frag[1][q] = (int)c1; frag[2][q] = (int)c2; frag[3][q] = (int)c3;
+    transpose4x4(r[4 * q].y, r[4 * q + 1].y, r[4 * q + 2].y, r[4 * q + 3].y, c0, c1, c2, c3);
+    frag[4][q] = (int)c0; frag[5][q] = (int)c1; frag[6][q] = (int)c2; frag[7][q] = (int)c3;
+  }
+}
+
+}  // namespace msco
+#endif  // MSCO_GMM_COMMON_H_

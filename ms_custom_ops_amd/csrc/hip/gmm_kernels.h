@@ -1,0 +1,29 @@
+// Host-side declarations of the kernel launchers (one translation unit per kernel family).
+#ifndef MSCO_GMM_KERNELS_H_
+#define MSCO_GMM_KERNELS_H_
+
+#include <hip/hip_runtime.h>
+#include "gmm_common.h"
+
+namespace msco {
+
+enum TileCfg : int { TILE_256x256 = 0, TILE_128x128 = 1, TILE_64x128 = 2, TILE_CFG_COUNT = 3 };
+
+// MFMA tile kernel for W8A8 (prefill shapes).  nk: weights stored [E,N,K].
+hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream_t stream);
+const char *tile_cfg_name(int tile_cfg);
+void tile_cfg_dims(int tile_cfg, int *bm, int *bn);
+
+// Skinny (decode) kernels: one workgroup streams a 128-column weight strip of one group over a K
+// range; waves split K and reduce through LDS, workgroups split K and reduce through the workspace.
+hipError_t launch_skinny_w8a8(const GmmParams &p, bool nk, hipStream_t stream);
+hipError_t launch_skinny_a16w8(const GmmParams &p, hipStream_t stream);
+size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t e, int split_k, bool fp32_partials);
+size_t skinny_counter_count(int64_t n, int64_t e);
+
+// Shape-agnostic fallback kernels (one output element per thread), any K / N.
+hipError_t launch_generic_w8a8(const GmmParams &p, bool nk, hipStream_t stream);
+hipError_t launch_generic_a16w8(const GmmParams &p, hipStream_t stream);
+
+}  // namespace msco
+#endif  // MSCO_GMM_KERNELS_H_

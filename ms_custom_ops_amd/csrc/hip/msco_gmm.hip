@@ -1,0 +1,297 @@
+// C ABI of the gfx950 grouped quantized matmul backend (see include/msco_gmm.h).
+// Host side only: argument checking, kernel-family choice from shapes (never from tensor values),
+// workspace sizing and the launches.
+#include "msco_gmm.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+
+#include "gmm_kernels.h"
+
+namespace {
+
+using namespace msco;
+
+enum Family : int { FAM_NONE = 0, FAM_TILE = 1, FAM_SKINNY = 2, FAM_GENERIC = 3 };
+
+// values of msco_gmm_desc::kernel_override
+enum Override : int { OV_AUTO = 0, OV_TILE_256 = 1, OV_TILE_128 = 2, OV_TILE_64 = 3, OV_SKINNY = 4, OV_GENERIC = 5 };
+
+constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned
+constexpr int kTargetWorkgroups = 1024;  // skinny kernels: aim for this many workgroups (4 per CU)
+
+int env_int(const char *name, int fallback) {
+  const char *v = std::getenv(name);
+  return (v && *v) ? std::atoi(v) : fallback;
+}
+
+}  // namespace
+
+struct msco_gmm_op {
+  msco_gmm_desc desc{};
+  bool planned = false;
+  int64_t m = 0, k = 0, n = 0, e = 0;
+  int family = FAM_NONE;
+  int tile_cfg = 0;
+  int split_k = 1;
+  int n_strips = 0;
+  size_t workspace_bytes = 0;
+  unsigned *counters = nullptr;
+  size_t counters_cap = 0;
+  std::string info;
+  std::mutex mu;
+};
+
+namespace {
+
+bool is_w8a8(const msco_gmm_desc &d) { return d.x_dtype == MSCO_DT_I8; }
+bool is_a16w8(const msco_gmm_desc &d) { return d.x_dtype == MSCO_DT_BF16 || d.x_dtype == MSCO_DT_F16; }
+
+int check_desc(const msco_gmm_desc &d) {
+  if (d.abi_version != MSCO_GMM_ABI_VERSION) return MSCO_ERR_INVALID_ARG;
+  if (d.weight_dtype != MSCO_DT_I8) return MSCO_ERR_UNSUPPORTED;
+  if (d.group_list_dtype != MSCO_DT_NONE && d.group_list_dtype != MSCO_DT_I32 && d.group_list_dtype != MSCO_DT_I64)
+    return MSCO_ERR_UNSUPPORTED;
+  if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
+  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_GENERIC) return MSCO_ERR_INVALID_ARG;
+  if (is_w8a8(d)) {
+    if (d.out_dtype != MSCO_DT_BF16 && d.out_dtype != MSCO_DT_F16 && d.out_dtype != MSCO_DT_I32)
+      return MSCO_ERR_UNSUPPORTED;
+    if (d.bias_dtype != MSCO_DT_NONE && d.bias_dtype != MSCO_DT_I32) return MSCO_ERR_UNSUPPORTED;
+    if (d.scale_dtype != MSCO_DT_NONE && d.scale_dtype != MSCO_DT_F32 && d.scale_dtype != MSCO_DT_BF16 &&
+        d.scale_dtype != MSCO_DT_I64 && d.scale_dtype != MSCO_DT_U64)
+      return MSCO_ERR_UNSUPPORTED;
+    if (d.per_token_dtype != MSCO_DT_NONE && d.per_token_dtype != MSCO_DT_F32) return MSCO_ERR_UNSUPPORTED;
+    if (d.antiquant_dtype != MSCO_DT_NONE) return MSCO_ERR_UNSUPPORTED;
+    return MSCO_OK;
+  }
+  if (is_a16w8(d)) {
+    if (d.out_dtype != d.x_dtype) return MSCO_ERR_UNSUPPORTED;       // weight-only output keeps x's dtype
+    if (d.antiquant_dtype != d.x_dtype) return MSCO_ERR_UNSUPPORTED; // scale / offset share x's dtype
+    if (d.transpose_b) return MSCO_ERR_UNSUPPORTED;
+    if (d.bias_dtype != MSCO_DT_NONE || d.scale_dtype != MSCO_DT_NONE || d.per_token_dtype != MSCO_DT_NONE)
+      return MSCO_ERR_UNSUPPORTED;
+    return MSCO_OK;
+  }
+  return MSCO_ERR_UNSUPPORTED;
+}
+
+int pow2_at_least(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+void choose_plan(msco_gmm_op *op) {
+  const msco_gmm_desc &d = op->desc;
+  const int64_t m = op->m, k = op->k, n = op->n, e = op->e;
+  const bool aligned = (k % 16 == 0) && (n % 16 == 0) && k >= 16 && n >= 16;
+  op->split_k = 1;
+  op->n_strips = (int)((n + kSkinnyCols - 1) / kSkinnyCols);
+  op->workspace_bytes = 0;
+  op->tile_cfg = TILE_256x256;
+
+  int family;
+  if (!aligned) {
+    family = FAM_GENERIC;
+  } else if (is_a16w8(d)) {
+    family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
+  } else if (m <= kSkinnyMaxRows) {
+    family = FAM_SKINNY;
+  } else {
+    family = FAM_TILE;
+    // tile shape from shapes only: average rows per group and how many tiles fill 256 CUs
+    const int64_t rows_per_group = m / (e > 0 ? e : 1);
+    auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    if (rows_per_group >= 192 && tiles(256, 256) >= 256) {
+      op->tile_cfg = TILE_256x256;
+    } else if (rows_per_group >= 96 && tiles(128, 128) >= 256) {
+      op->tile_cfg = TILE_128x128;
+    } else if (tiles(128, 128) >= 512) {
+      op->tile_cfg = TILE_128x128;
+    } else {
+      op->tile_cfg = TILE_64x128;
+    }
+  }
+  switch (d.kernel_override) {
+    case OV_TILE_256: family = FAM_TILE; op->tile_cfg = TILE_256x256; break;
+    case OV_TILE_128: family = FAM_TILE; op->tile_cfg = TILE_128x128; break;
+    case OV_TILE_64: family = FAM_TILE; op->tile_cfg = TILE_64x128; break;
+    case OV_SKINNY: family = FAM_SKINNY; break;
+    case OV_GENERIC: family = FAM_GENERIC; break;
+    default: break;
+  }
+  if ((family == FAM_TILE || family == FAM_SKINNY) && !aligned) family = FAM_GENERIC;
+  if (family == FAM_TILE && !is_w8a8(d)) family = FAM_SKINNY;
+  if (family == FAM_TILE) {
+    const int forced = env_int("MSCO_TILE_CFG", -1);
+    if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO) op->tile_cfg = forced;
+  }
+  if (family == FAM_SKINNY) {
+    // Cross-workgroup K split only when every group is guaranteed to fit one 16-row chunk.
+    if (m <= kSkinnyRows) {
+      const int64_t base = (int64_t)op->n_strips * e;
+      const int k_blocks = (int)((k + 63) / 64);
+      int want = pow2_at_least((int)((kTargetWorkgroups + base - 1) / base));
+      int cap = k_blocks / 4;  // every wave of a workgroup keeps at least one 64-row block
+      if (cap < 1) cap = 1;
+      while (want > cap) want >>= 1;
+      if (want < 1) want = 1;
+      const int forced = env_int("MSCO_SKINNY_SPLIT_K", 0);
+      if (forced > 0) want = forced;
+      op->split_k = want;
+    }
+    op->workspace_bytes = skinny_workspace_bytes(m, n, e, op->split_k, is_a16w8(d));
+  }
+  op->family = family;
+
+  char buf[320];
+  const char *fam = family == FAM_TILE ? "tile" : family == FAM_SKINNY ? "skinny" : "generic";
+  std::snprintf(buf, sizeof(buf),
+                "msco_gmm plan: kernel=%s%s%s layout=%s m=%lld k=%lld n=%lld e=%lld split_k=%d strips=%d "
+                "workspace=%zu",
+                is_w8a8(d) ? "w8a8_" : "a16w8_", fam,
+                family == FAM_TILE ? (std::string("_") + tile_cfg_name(op->tile_cfg)).c_str() : "",
+                d.transpose_b ? "[E,N,K]" : "[E,K,N]", (long long)m, (long long)k, (long long)n, (long long)e,
+                op->split_k, op->n_strips, op->workspace_bytes);
+  op->info = buf;
+}
+
+}  // namespace
+
+extern "C" {
+
+int msco_gmm_abi_version(void) { return MSCO_GMM_ABI_VERSION; }
+
+const char *msco_status_string(int status) {
+  switch (status) {
+    case MSCO_OK: return "ok";
+    case MSCO_ERR_INVALID_ARG: return "invalid argument";
+    case MSCO_ERR_UNSUPPORTED: return "unsupported dtype or layout";
+    case MSCO_ERR_SHAPE: return "shape rule violated";
+    case MSCO_ERR_NOT_PLANNED: return "launch before plan";
+    case MSCO_ERR_WORKSPACE: return "workspace missing or too small";
+    case MSCO_ERR_DEVICE: return "HIP runtime error";
+    default: return "unknown status";
+  }
+}
+
+int msco_gmm_create(const msco_gmm_desc *desc, msco_gmm_handle *out_handle) {
+  if (desc == nullptr || out_handle == nullptr) return MSCO_ERR_INVALID_ARG;
+  const int rc = check_desc(*desc);
+  if (rc != MSCO_OK) return rc;
+  msco_gmm_op *op = new (std::nothrow) msco_gmm_op();
+  if (op == nullptr) return MSCO_ERR_DEVICE;
+  op->desc = *desc;
+  *out_handle = op;
+  return MSCO_OK;
+}
+
+int msco_gmm_plan(msco_gmm_handle h, int64_t m, int64_t k, int64_t n, int64_t e, size_t *workspace_bytes) {
+  if (h == nullptr) return MSCO_ERR_INVALID_ARG;
+  if (m < 0 || k <= 0 || n <= 0 || e <= 0) return MSCO_ERR_SHAPE;
+  if (m > INT32_MAX || k > INT32_MAX || n > INT32_MAX || e > 65535 || m * n > ((int64_t)1 << 40)) return MSCO_ERR_SHAPE;
+  if (h->desc.group_list_dtype == MSCO_DT_NONE && m % e != 0) return MSCO_ERR_SHAPE;
+  std::lock_guard<std::mutex> lock(h->mu);
+  h->m = m; h->k = k; h->n = n; h->e = e;
+  choose_plan(h);
+  if (h->family == FAM_SKINNY && h->split_k > 1) {
+    const size_t need = skinny_counter_count(n, e);
+    if (need > h->counters_cap) {
+      if (h->counters) (void)hipFree(h->counters);
+      h->counters = nullptr;
+      h->counters_cap = 0;
+      if (hipMalloc(reinterpret_cast<void **>(&h->counters), need * sizeof(unsigned)) != hipSuccess) {
+        (void)hipGetLastError();
+        return MSCO_ERR_DEVICE;
+      }
+      if (hipMemset(h->counters, 0, need * sizeof(unsigned)) != hipSuccess) {
+        (void)hipGetLastError();
+        return MSCO_ERR_DEVICE;
+      }
+      h->counters_cap = need;
+    }
+  }
+  h->planned = true;
+  if (workspace_bytes) *workspace_bytes = h->workspace_bytes;
+  if (env_int("MSCO_PRINT_PLAN", 0)) std::fprintf(stderr, "%s\n", h->info.c_str());
+  return MSCO_OK;
+}
+
+int msco_gmm_plan_info(msco_gmm_handle h, char *buf, size_t buf_len) {
+  if (h == nullptr) return -1;
+  std::lock_guard<std::mutex> lock(h->mu);
+  if (buf && buf_len) {
+    std::strncpy(buf, h->info.c_str(), buf_len - 1);
+    buf[buf_len - 1] = '\0';
+  }
+  return (int)h->info.size();
+}
+
+int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, void *workspace, size_t workspace_bytes,
+                    void *stream) {
+  if (h == nullptr || inputs == nullptr) return MSCO_ERR_INVALID_ARG;
+  if (!h->planned) return MSCO_ERR_NOT_PLANNED;
+  const msco_gmm_desc &d = h->desc;
+  if (h->m == 0) return MSCO_OK;
+  if (out == nullptr || inputs[MSCO_IN_X] == nullptr || inputs[MSCO_IN_WEIGHT] == nullptr) return MSCO_ERR_INVALID_ARG;
+  // a present dtype needs a pointer, an absent one must not get one
+  auto need = [&](int slot, int dtype) { return (dtype != MSCO_DT_NONE) == (inputs[slot] != nullptr); };
+  if (!need(MSCO_IN_BIAS, d.bias_dtype) || !need(MSCO_IN_SCALE, d.scale_dtype) ||
+      !need(MSCO_IN_GROUP_LIST, d.group_list_dtype) || !need(MSCO_IN_PER_TOKEN_SCALE, d.per_token_dtype) ||
+      !need(MSCO_IN_ANTIQUANT_SCALE, d.antiquant_dtype))
+    return MSCO_ERR_INVALID_ARG;
+  if ((d.has_antiquant_offset != 0) != (inputs[MSCO_IN_ANTIQUANT_OFFSET] != nullptr)) return MSCO_ERR_INVALID_ARG;
+  if (h->workspace_bytes > 0 && (workspace == nullptr || workspace_bytes < h->workspace_bytes))
+    return MSCO_ERR_WORKSPACE;
+
+  GmmParams p{};
+  p.x = inputs[MSCO_IN_X];
+  p.w = static_cast<const int8_t *>(inputs[MSCO_IN_WEIGHT]);
+  p.bias = static_cast<const int32_t *>(inputs[MSCO_IN_BIAS]);
+  p.scale = inputs[MSCO_IN_SCALE];
+  p.group_list = inputs[MSCO_IN_GROUP_LIST];
+  p.per_token = static_cast<const float *>(inputs[MSCO_IN_PER_TOKEN_SCALE]);
+  p.aq_scale = inputs[MSCO_IN_ANTIQUANT_SCALE];
+  p.aq_offset = inputs[MSCO_IN_ANTIQUANT_OFFSET];
+  p.out = out;
+  p.partial = static_cast<int32_t *>(workspace);
+  p.counters = h->counters;
+  p.m = (int)h->m; p.k = (int)h->k; p.n = (int)h->n; p.e = (int)h->e;
+  p.gl_dtype = d.group_list_dtype;
+  p.gl_type = d.group_list_type;
+  p.scale_dtype = d.scale_dtype;
+  p.scale_per_group = d.scale_per_group;
+  p.scale_is_scalar = d.scale_is_scalar;
+  p.out_dtype = d.out_dtype;
+  p.x_dtype = d.x_dtype;
+  p.split_k = h->split_k;
+  p.n_strips = h->n_strips;
+
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipError_t err = hipSuccess;
+  const bool nk = d.transpose_b != 0;
+  if (is_w8a8(d)) {
+    if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, s);
+    else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, s);
+    else err = launch_generic_w8a8(p, nk, s);
+  } else {
+    if (h->family == FAM_SKINNY) err = launch_skinny_a16w8(p, s);
+    else err = launch_generic_a16w8(p, s);
+  }
+  return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
+}
+
+int msco_gmm_destroy(msco_gmm_handle h) {
+  if (h == nullptr) return MSCO_ERR_INVALID_ARG;
+  if (h->counters) (void)hipFree(h->counters);
+  delete h;
+  return MSCO_OK;
+}
+
+}  // extern "C"
