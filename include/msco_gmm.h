@@ -129,6 +129,13 @@ MSCO_API int msco_gmm_plan_info(msco_gmm_handle h, char *buf, size_t buf_len);
 /* Release the instance and any device state it holds. */
 MSCO_API int msco_gmm_destroy(msco_gmm_handle h);
 
+/* Batched 2-D transpose on the device: src [batch, rows, cols] -> dst [batch, cols, rows], elements of
+ * elem_bytes (1, 2 or 4) bytes.  Serves transpose_x1 of quant_batch_matmul, which the reference passes
+ * down to aclnnQuantMatmulV4 as a flag (ops/c_api/quant_batch_matmul/quant_batch_matmul.cc:78-80,144-145);
+ * the HIP kernels read x rows K-contiguous, so the op layer materialises x1 transposed once. */
+MSCO_API int msco_transpose_2d(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols,
+                               int32_t elem_bytes, void *stream);
+
 /* Static text for a status code. */
 MSCO_API const char *msco_status_string(int status);
 

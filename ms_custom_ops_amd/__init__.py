@@ -1,0 +1,183 @@
+"""ms_custom_ops grouped quantized matmul operators on AMD Instinct MI355X (gfx950).
+
+Drop-in for the grouped / dense quantized matmul entries of ms_custom_ops
+(python/ms_custom_ops/__init__.py:76 re-exports them from the compiled module):
+
+    grouped_matmul(x, weight, group_list, bias=None, scale=None, per_token_scale=None,
+                   antiquant_scale=None, transpose_a=False, transpose_b=False, x_format=0)
+    grouped_matmul_v4_cops(x, weight, bias=None, scale=None, offset=None, antiquant_scale=None,
+                           antiquant_offset=None, per_token_scale=None, group_list=None,
+                           activation_input=None, activation_quant_scale=None,
+                           activation_quant_offset=None, split_item=0, group_type=-1,
+                           group_list_type=0, act_type=0, weight_format="ND", output_dtype=None)
+    quant_batch_matmul(x1, x2, scale, offset=None, bias=None, pertoken_scale=None,
+                       transpose_x1=False, transpose_x2=False, x2_format="ND", output_dtype=float16)
+
+Tensors are PyTorch-ROCm tensors on the GPU; PyTorch only provides device memory and the current
+stream.  The compiled operator layer (``ms_custom_ops_amd.ms_custom_ops``, pybind11) validates and
+plans, and the HIP backend behind the C ABI (``lib/libmsco_gmm.so``) does the work.  There is no
+CPU or eager fallback: importing this package without the compiled modules raises.
+
+Both execution modes of the reference are available: "pynative" calls the pybind entry directly,
+"graph" runs the registered infer implementation and kernel module (Init / Resize / Launch).
+"""
+from __future__ import annotations
+
+import contextlib
+import os
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import cabi
+
+try:
+    from . import ms_custom_ops as _C  # the compiled operator layer
+except ImportError as exc:  # pragma: no cover - exercised only on a broken install
+    raise ImportError(
+        "ms_custom_ops_amd: the compiled operator module is missing; run `python -m ms_custom_ops_amd.build` "
+        "(needs hipcc for gfx950 and g++). There is no fallback implementation.") from exc
+
+__all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "set_context", "get_context", "exec_mode",
+           "GRAPH_MODE", "PYNATIVE_MODE", "dtype_to_type_id", "type_id_to_dtype", "plan_cache_stats", "trans_data"]
+
+GRAPH_MODE = 0
+PYNATIVE_MODE = 1
+_mode = PYNATIVE_MODE
+
+# MindSpore TypeId values (the integer form of dtype arguments; float16 == 42 is the default
+# output_dtype of quant_batch_matmul, ops/c_api/quant_batch_matmul/quant_batch_matmul.cc:161)
+_TYPE_IDS = {
+    torch.bool: 30, torch.int8: 32, torch.int16: 33, torch.int32: 34, torch.int64: 35, torch.uint8: 37,
+    torch.float16: 42, torch.float32: 43, torch.float64: 44, torch.bfloat16: 45,
+}
+if hasattr(torch, "uint64"):
+    _TYPE_IDS[torch.uint64] = 40
+_DTYPES = {v: k for k, v in _TYPE_IDS.items()}
+
+
+def dtype_to_type_id(dtype) -> Optional[int]:
+    """torch dtype (or TypeId int, or None) -> TypeId int, the reference's ``dtype_to_type_id`` arg handler."""
+    if dtype is None or isinstance(dtype, int):
+        return dtype
+    try:
+        return _TYPE_IDS[dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dtype}") from None
+
+
+def type_id_to_dtype(type_id: int):
+    return _DTYPES[int(type_id)]
+
+
+def set_context(mode: int):
+    """Select GRAPH_MODE or PYNATIVE_MODE for subsequent operator calls."""
+    global _mode
+    if mode not in (GRAPH_MODE, PYNATIVE_MODE):
+        raise ValueError("mode must be GRAPH_MODE or PYNATIVE_MODE")
+    _mode = mode
+
+
+def get_context() -> int:
+    return _mode
+
+
+@contextlib.contextmanager
+def exec_mode(mode: int):
+    prev = get_context()
+    set_context(mode)
+    try:
+        yield
+    finally:
+        set_context(prev)
+
+
+# ---- framework hooks: PyTorch owns device memory and streams -------------------------------------
+def _wrap(t: Optional[torch.Tensor]):
+    if t is None:
+        return None
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"expected a torch.Tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise ValueError("ms_custom_ops_amd operators take GPU tensors; got a tensor on " + str(t.device))
+    return _C.Tensor(t.data_ptr(), dtype_to_type_id(t.dtype), list(t.shape), list(t.stride()), t)
+
+
+def _wrap_list(ts):
+    if ts is None:
+        return None
+    if isinstance(ts, torch.Tensor):
+        raise TypeError("expected a list of tensors")
+    return [_wrap(t) for t in ts]
+
+
+def _allocate(type_id: int, shape: Sequence[int]):
+    return _wrap(torch.empty(tuple(shape), dtype=type_id_to_dtype(type_id), device="cuda"))
+
+
+def _current_stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+_C._set_framework_hooks(_allocate, _current_stream)
+
+
+def plan_cache_stats():
+    """(hits, misses, size) of the kernel-plan cache of the operator layer."""
+    return tuple(_C._plan_cache_stats())
+
+
+# ---- operators ---------------------------------------------------------------------------------------
+def grouped_matmul(x, weight, group_list, bias=None, scale=None, per_token_scale=None, antiquant_scale=None,
+                   transpose_a=False, transpose_b=False, x_format=0, output_dtype=None):
+    """Grouped matmul; see the module docstring.  ``output_dtype`` (None = float16 as in the reference,
+    or torch.bfloat16) is an optional trailing extension."""
+    od = dtype_to_type_id(output_dtype)
+    if _mode == GRAPH_MODE:
+        args = [_wrap(x), _wrap(weight), _wrap(group_list), _wrap(bias), _wrap(scale), _wrap(per_token_scale),
+                _wrap(antiquant_scale), bool(transpose_a), bool(transpose_b), int(x_format), od]
+        return _C._graph_run("grouped_matmul", args)[0].owner
+    return _C.grouped_matmul(_wrap(x), _wrap(weight), _wrap(group_list), _wrap(bias), _wrap(scale),
+                             _wrap(per_token_scale), _wrap(antiquant_scale), bool(transpose_a), bool(transpose_b),
+                             int(x_format), od).owner
+
+
+def grouped_matmul_v4_cops(x, weight, bias=None, scale=None, offset=None, antiquant_scale=None, antiquant_offset=None,
+                           per_token_scale=None, group_list=None, activation_input=None, activation_quant_scale=None,
+                           activation_quant_offset=None, split_item=0, group_type=-1, group_list_type=0, act_type=0,
+                           weight_format="ND", output_dtype=None) -> List[torch.Tensor]:
+    """List-of-tensor grouped matmul (GMM V4); returns a list of tensors."""
+    od = dtype_to_type_id(output_dtype)
+    lists = [_wrap_list(v) for v in (x, weight, bias, scale, offset, antiquant_scale, antiquant_offset,
+                                     per_token_scale)]
+    acts = [_wrap_list(v) for v in (activation_input, activation_quant_scale, activation_quant_offset)]
+    gl = _wrap(group_list)
+    if _mode == GRAPH_MODE:
+        args = lists + [gl] + acts + [int(split_item), int(group_type), int(group_list_type), int(act_type),
+                                      str(weight_format), od]
+        outs = _C._graph_run("grouped_matmul_v4_cops", args)
+    else:
+        outs = _C.grouped_matmul_v4_cops(*lists, gl, *acts, int(split_item), int(group_type), int(group_list_type),
+                                         int(act_type), str(weight_format), od)
+    return [o.owner for o in outs]
+
+
+def quant_batch_matmul(x1, x2, scale, offset=None, bias=None, pertoken_scale=None, transpose_x1=False,
+                       transpose_x2=False, x2_format="ND", output_dtype=torch.float16):
+    """Dense / batched W8A8 matmul with dequant epilogue."""
+    od = dtype_to_type_id(output_dtype)
+    if _mode == GRAPH_MODE:
+        args = [_wrap(x1), _wrap(x2), _wrap(scale), _wrap(offset), _wrap(bias), _wrap(pertoken_scale),
+                bool(transpose_x1), bool(transpose_x2), str(x2_format), od]
+        return _C._graph_run("quant_batch_matmul", args)[0].owner
+    return _C.quant_batch_matmul(_wrap(x1), _wrap(x2), _wrap(scale), _wrap(offset), _wrap(bias), _wrap(pertoken_scale),
+                                 bool(transpose_x1), bool(transpose_x2), str(x2_format), od).owner
+
+
+def trans_data(tensor, transdata_type=1):
+    """Weight pre-pass hook.  The reference converts weights to the Ascend FRACTAL_NZ format before
+    grouped_matmul (tests/st/test_grouped_matmul.py:131-133); the HIP kernels read weights as stored,
+    so this returns its input unchanged and exists only so that such call sites keep working."""
+    if transdata_type not in (0, 1):
+        raise ValueError("transdata_type must be 0 (FRACTAL_NZ_TO_ND) or 1 (ND_TO_FRACTAL_NZ)")
+    return tensor

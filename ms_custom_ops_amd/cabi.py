@@ -26,7 +26,7 @@ IN_COUNT = 8
 OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC = range(6)
 
 EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco_gmm_plan_info", "msco_gmm_destroy",
-                    "msco_status_string", "msco_gmm_abi_version")
+                    "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d")
 
 
 class GmmDesc(ctypes.Structure):

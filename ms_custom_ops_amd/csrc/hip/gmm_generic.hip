@@ -70,6 +70,43 @@ __global__ void __launch_bounds__(256) gmm_a16w8_generic_kernel(const GmmParams 
   out[idx] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
 }
 
+// Batched 2-D transpose through a padded LDS tile: src [batch, rows, cols] -> dst [batch, cols, rows].
+template <typename T>
+__global__ void __launch_bounds__(256) transpose_2d_kernel(const T *src, T *dst, long long rows, long long cols) {
+  __shared__ T tile[32][33];
+  const long long b = blockIdx.z;
+  const T *s = src + b * rows * cols;
+  T *d = dst + b * rows * cols;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const long long c0 = (long long)blockIdx.x * 32, r0 = (long long)blockIdx.y * 32;
+  for (int i = ty; i < 32; i += 8) {
+    if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = s[(r0 + i) * cols + c0 + tx];
+  }
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8) {
+    if (c0 + i < cols && r0 + tx < rows) d[(c0 + i) * rows + r0 + tx] = tile[tx][i];
+  }
+}
+
+hipError_t launch_transpose_2d(const void *src, void *dst, long long batch, long long rows, long long cols,
+                               int elem_bytes, hipStream_t stream) {
+  if (batch == 0 || rows == 0 || cols == 0) return hipSuccess;
+  const dim3 grid((unsigned)((cols + 31) / 32), (unsigned)((rows + 31) / 32), (unsigned)batch);
+  if (elem_bytes == 1) {
+    hipLaunchKernelGGL(transpose_2d_kernel<unsigned char>, grid, dim3(256), 0, stream,
+                       static_cast<const unsigned char *>(src), static_cast<unsigned char *>(dst), rows, cols);
+  } else if (elem_bytes == 2) {
+    hipLaunchKernelGGL(transpose_2d_kernel<unsigned short>, grid, dim3(256), 0, stream,
+                       static_cast<const unsigned short *>(src), static_cast<unsigned short *>(dst), rows, cols);
+  } else if (elem_bytes == 4) {
+    hipLaunchKernelGGL(transpose_2d_kernel<unsigned>, grid, dim3(256), 0, stream, static_cast<const unsigned *>(src),
+                       static_cast<unsigned *>(dst), rows, cols);
+  } else {
+    return hipErrorInvalidValue;
+  }
+  return hipGetLastError();
+}
+
 hipError_t launch_generic_w8a8(const GmmParams &p, bool nk, hipStream_t stream) {
   const long long total = (long long)p.m * p.n;
   if (total == 0) return hipSuccess;

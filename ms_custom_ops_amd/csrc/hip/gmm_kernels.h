@@ -25,5 +25,9 @@ size_t skinny_counter_count(int64_t n, int64_t e);
 hipError_t launch_generic_w8a8(const GmmParams &p, bool nk, hipStream_t stream);
 hipError_t launch_generic_a16w8(const GmmParams &p, hipStream_t stream);
 
+// Batched 2-D transpose, src [batch, rows, cols] -> dst [batch, cols, rows].
+hipError_t launch_transpose_2d(const void *src, void *dst, long long batch, long long rows, long long cols,
+                               int elem_bytes, hipStream_t stream);
+
 }  // namespace msco
 #endif  // MSCO_GMM_KERNELS_H_

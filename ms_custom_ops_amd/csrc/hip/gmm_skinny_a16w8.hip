@@ -175,31 +175,30 @@ __global__ void __launch_bounds__(AW_THREADS, 2) gmm_a16w8_skinny_kernel(const G
       float *base = reinterpret_cast<float *>(p.partial) + (tile * p.split_k + ks) * AW_TILE_FLOATS;
       if (row_ok) {
         float *mine = base + row * kSkinnyCols + c8;
-        *reinterpret_cast<float4 *>(mine) = make_float4(v[0], v[1], v[2], v[3]);
-        *reinterpret_cast<float4 *>(mine + 4) = make_float4(v[4], v[5], v[6], v[7]);
-        if (c8 == 0) base[kSkinnyRows * kSkinnyCols + row] = xs;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) __hip_atomic_store(mine + j, v[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (c8 == 0)
+          __hip_atomic_store(base + kSkinnyRows * kSkinnyCols + row, xs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-      __threadfence();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __syncthreads();
-      if (tid == 0) s_ticket = atomicAdd(&p.counters[tile], 1u);
+      if (tid == 0) s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       do_epilogue = (s_ticket == (unsigned)(p.split_k - 1));
       if (do_epilogue) {
-        __threadfence();
         if (row_ok) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) v[j] = 0.f;
           xs = 0.f;
           for (int s = 0; s < p.split_k; ++s) {
             const float *src = reinterpret_cast<const float *>(p.partial) + (tile * p.split_k + s) * AW_TILE_FLOATS;
-            const float4 a = *reinterpret_cast<const float4 *>(src + row * kSkinnyCols + c8);
-            const float4 b = *reinterpret_cast<const float4 *>(src + row * kSkinnyCols + c8 + 4);
-            v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w;
-            v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
-            xs += src[kSkinnyRows * kSkinnyCols + row];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+              v[j] += __hip_atomic_load(src + row * kSkinnyCols + c8 + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            xs += __hip_atomic_load(src + kSkinnyRows * kSkinnyCols + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
         }
-        if (tid == 0) p.counters[tile] = 0;
+        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
 

@@ -143,29 +143,29 @@ __global__ void __launch_bounds__(SK_THREADS, 2) gmm_w8a8_skinny_kernel(const Gm
       // ---- cross-workgroup reduction through the workspace ------------------------------------
       const long long tile = (long long)grp * p.n_strips + strip;
       int *mine = p.partial + ((tile * p.split_k + ks) * kSkinnyRows + row) * kSkinnyCols + c8;
+      // Partial tiles and the arrival counter are exchanged with agent-scope atomic accesses: they
+      // bypass the per-XCD L2 for this data only, so no cache-wide write-back / invalidate fence is
+      // needed.  The stores are complete (vmcnt == 0) before the counter is bumped.
       if (row_ok) {
-        *reinterpret_cast<int4 *>(mine) = make_int4(v[0], v[1], v[2], v[3]);
-        *reinterpret_cast<int4 *>(mine + 4) = make_int4(v[4], v[5], v[6], v[7]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) __hip_atomic_store(mine + j, v[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-      __threadfence();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       __syncthreads();
-      if (tid == 0) s_ticket = atomicAdd(&p.counters[tile], 1u);
+      if (tid == 0) s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       do_epilogue = (s_ticket == (unsigned)(p.split_k - 1));
       if (do_epilogue) {
-        __threadfence();
         if (row_ok) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) v[j] = 0;
           for (int s = 0; s < p.split_k; ++s) {
             const int *src = p.partial + ((tile * p.split_k + s) * kSkinnyRows + row) * kSkinnyCols + c8;
-            const int4 a = *reinterpret_cast<const int4 *>(src);
-            const int4 b = *reinterpret_cast<const int4 *>(src + 4);
-            v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w;
-            v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] += __hip_atomic_load(src + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
         }
-        if (tid == 0) p.counters[tile] = 0;  // self-reset for the next launch
+        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
 

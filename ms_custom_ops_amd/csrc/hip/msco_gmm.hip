@@ -287,6 +287,17 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
 }
 
+int msco_transpose_2d(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int32_t elem_bytes,
+                      void *stream) {
+  if (batch < 0 || rows < 0 || cols < 0 || batch > 65535) return MSCO_ERR_SHAPE;
+  if (batch * rows * cols == 0) return MSCO_OK;
+  if (src == nullptr || dst == nullptr) return MSCO_ERR_INVALID_ARG;
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) return MSCO_ERR_UNSUPPORTED;
+  const hipError_t err =
+    launch_transpose_2d(src, dst, batch, rows, cols, elem_bytes, static_cast<hipStream_t>(stream));
+  return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
+}
+
 int msco_gmm_destroy(msco_gmm_handle h) {
   if (h == nullptr) return MSCO_ERR_INVALID_ARG;
   if (h->counters) (void)hipFree(h->counters);

@@ -1,0 +1,318 @@
+// grouped_matmul_v4_cops(x, weight, bias, scale, offset, antiquant_scale, antiquant_offset,
+//                        per_token_scale, group_list, activation_input, activation_quant_scale,
+//                        activation_quant_offset, split_item, group_type, group_list_type, act_type,
+//                        weight_format, output_dtype) -> list of tensors
+//
+// List-of-tensor GMM-V4 entry of the reference (ops/c_api/grouped_matmul_v4_cops/
+// grouped_matmul_v4_cops.cc): same eighteen arguments and defaults (:395-405), int64 group_list with
+// group_list_type 0 (cumulative) or 1 (counts), output dtype rules of InferOutputTypes (:162-203).
+// The reference forwards the twelve lists to aclnnGroupedMatmulV4 (:359-363); here
+//   * group_type 0 (one x [M,K], one weight [E,K,N], one output [M,N]) is one grouped launch of the
+//     HIP backend: W8A8 with per-channel scale / per-token scale / int32 bias, or weight-only
+//     (bf16/f16 x, int8 weight, antiquant scale and offset [E,N]);
+//   * group_type -1 (independent x[i] @ weight[i]) is one dense launch per pair.
+// Not implemented on this backend and refused with a message: float x float matmuls, int4 weights,
+// uint64 scales with int8 output, `offset`, the activation inputs, act_type != 0, FRACTAL_NZ weights,
+// group_type 1.
+#include <optional>
+#include <string>
+#include <vector>
+
+#include "ops/c_api/grouped_matmul_v4_cops/grouped_matmul_v4_cops_func_impl.h"
+#include "ops/framework/hip_backend/hip_gmm_runner.h"
+#include "ops/framework/module.h"
+#include "ops/framework/utils.h"
+
+namespace ms_custom_ops {
+namespace {
+struct V4Args {
+  TensorVec x, weight, bias, scale, offset, antiquant_scale, antiquant_offset, per_token_scale;
+  ms::Tensor group_list;
+  TensorVec activation_input, activation_quant_scale, activation_quant_offset;
+  int64_t split_item{0}, group_type{-1}, group_list_type{0}, act_type{0};
+  std::string weight_format{"ND"};
+};
+
+const ms::Tensor &At(const TensorVec &v, size_t i) {
+  static const ms::Tensor empty;
+  return i < v.size() ? v[i] : empty;
+}
+
+void CheckV4Support(const V4Args &a) {
+  if (a.weight_format != kNdFormat) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", weight_format '" << a.weight_format
+                     << "' is an Ascend memory format; the HIP backend takes weights as stored (ND).";
+  }
+  if (a.act_type != 0 || !a.activation_input.empty() || !a.activation_quant_scale.empty() ||
+      !a.activation_quant_offset.empty()) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", fused activation is not implemented by the HIP backend.";
+  }
+  if (!a.offset.empty()) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", 'offset' is not implemented by the HIP backend.";
+  }
+  if (a.group_list_type != 0 && a.group_list_type != 1) {
+    MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", group_list_type must be 0 or 1, but got "
+                       << a.group_list_type;
+  }
+  const TypeId xt = a.x[0].data_type(), wt = a.weight[0].data_type();
+  if (wt == kNumberTypeInt4) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", int4 weights are not implemented by the HIP backend.";
+  }
+  if (wt != kNumberTypeInt8) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName
+                     << ", the HIP backend implements the quantized paths only (int8 weight), but got weight dtype "
+                     << wt;
+  }
+  if (xt != kNumberTypeInt8 && xt != kNumberTypeBFloat16 && xt != kNumberTypeFloat16) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", 'x' must be Int8, BFloat16 or Float16, but got " << xt;
+  }
+}
+
+// One launch: x [M,K], weight [E,K,N], optional per-group rows of bias / scale / antiquant.
+void LaunchOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias, const ms::Tensor &scale,
+               const ms::Tensor &aq_scale, const ms::Tensor &aq_offset, const ms::Tensor &per_token,
+               const ms::Tensor &group_list, int64_t group_list_type, const ms::Tensor &out, int64_t m, int64_t k,
+               int64_t n, int64_t e, void *stream) {
+  const std::string op_name = "GroupedMatmulV4";
+  const TypeId xt = x.data_type();
+  msco_gmm_desc d{};
+  d.abi_version = MSCO_GMM_ABI_VERSION;
+  d.x_dtype = ToBackendDtype(xt);
+  d.weight_dtype = MSCO_DT_I8;
+  d.out_dtype = ToBackendDtype(out.data_type());
+  d.group_list_dtype = group_list.is_defined() ? ToBackendDtype(group_list.data_type()) : MSCO_DT_NONE;
+  d.group_list_type = static_cast<int32_t>(group_list_type);
+  d.scale_per_group = 1;
+  const void *addrs[MSCO_IN_COUNT] = {nullptr};
+  addrs[MSCO_IN_X] = x.GetDataPtr();
+  addrs[MSCO_IN_WEIGHT] = w.GetDataPtr();
+  addrs[MSCO_IN_GROUP_LIST] = group_list.is_defined() ? group_list.GetDataPtr() : nullptr;
+  auto expect_en = [&](const ms::Tensor &t, const char *name) {
+    if (t.is_defined() && t.numel() != e * n) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", '" << name << "' must have E*N = " << e * n
+                         << " elements, but got shape " << t.shape();
+    }
+  };
+  if (xt == kNumberTypeInt8) {
+    if (aq_scale.is_defined() || aq_offset.is_defined()) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", antiquant inputs need a floating-point 'x'.";
+    }
+    const bool raw = out.data_type() == kNumberTypeInt32;
+    expect_en(bias, "bias");
+    expect_en(scale, "scale");
+    if (bias.is_defined() && bias.data_type() != kNumberTypeInt32) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", the quantized path takes an Int32 'bias', but got "
+                         << bias.data_type();
+    }
+    if (per_token.is_defined() && (per_token.data_type() != kNumberTypeFloat32 || per_token.numel() != m)) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", 'per_token_scale' must be Float32 with M = " << m
+                         << " elements, but got " << per_token.data_type() << " " << per_token.shape();
+    }
+    d.bias_dtype = bias.is_defined() ? MSCO_DT_I32 : MSCO_DT_NONE;
+    d.scale_dtype = (!raw && scale.is_defined()) ? ToBackendDtype(scale.data_type()) : MSCO_DT_NONE;
+    d.per_token_dtype = (!raw && per_token.is_defined()) ? MSCO_DT_F32 : MSCO_DT_NONE;
+    addrs[MSCO_IN_BIAS] = bias.is_defined() ? bias.GetDataPtr() : nullptr;
+    addrs[MSCO_IN_SCALE] = d.scale_dtype != MSCO_DT_NONE ? scale.GetDataPtr() : nullptr;
+    addrs[MSCO_IN_PER_TOKEN_SCALE] = d.per_token_dtype != MSCO_DT_NONE ? per_token.GetDataPtr() : nullptr;
+  } else {
+    if (!aq_scale.is_defined()) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", weight-only quantization needs 'antiquant_scale'.";
+    }
+    if (aq_scale.data_type() != xt || (aq_offset.is_defined() && aq_offset.data_type() != xt)) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName
+                         << ", 'antiquant_scale' and 'antiquant_offset' must have the dtype of 'x' (" << xt << ").";
+    }
+    if (bias.is_defined() || scale.is_defined() || per_token.is_defined()) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName
+                         << ", 'bias', 'scale' and 'per_token_scale' are not used by the weight-only path.";
+    }
+    expect_en(aq_scale, "antiquant_scale");
+    expect_en(aq_offset, "antiquant_offset");
+    d.antiquant_dtype = ToBackendDtype(xt);
+    d.has_antiquant_offset = aq_offset.is_defined() ? 1 : 0;
+    addrs[MSCO_IN_ANTIQUANT_SCALE] = aq_scale.GetDataPtr();
+    addrs[MSCO_IN_ANTIQUANT_OFFSET] = aq_offset.is_defined() ? aq_offset.GetDataPtr() : nullptr;
+  }
+  auto plan = GmmPlanCache::GetInstance().GetOrCreate(op_name, d, GmmProblem{m, k, n, e}, stream);
+  ms::Tensor workspace;
+  if (plan->workspace_bytes > 0) {
+    workspace = AllocateTensor(kNumberTypeInt8, ShapeVector{static_cast<int64_t>(plan->workspace_bytes)});
+  }
+  LaunchPlan(op_name, plan, addrs, out.GetDataPtr(), workspace.is_defined() ? workspace.GetDataPtr() : nullptr,
+             plan->workspace_bytes, stream);
+}
+
+void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
+  CheckV4Support(a);
+  TensorVec all = a.x;
+  for (const auto *v : {&a.weight, &a.bias, &a.scale, &a.antiquant_scale, &a.antiquant_offset, &a.per_token_scale}) {
+    all.insert(all.end(), v->begin(), v->end());
+  }
+  all.push_back(a.group_list);
+  CheckContiguous("GroupedMatmulV4", all, true);
+  CheckContiguous("GroupedMatmulV4", outputs, false);
+  void *stream = CurrentStream();
+
+  if (a.group_type == kGroupTypeSingleOutput) {
+    const auto &x = a.x[0];
+    const auto &w = a.weight[0];
+    if (x.shape().size() != kDim2 || w.shape().size() != kDim3) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", with group_type 0 'x' must be [M, K] and 'weight' "
+                         << "[E, K, N], but got " << x.shape() << " and " << w.shape();
+    }
+    const int64_t m = x.shape()[0], k = x.shape()[1], e = w.shape()[0], n = w.shape()[2];
+    if (w.shape()[1] != k) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", the K dimension of 'x' and 'weight' must be equal, "
+                         << "but got " << k << " and " << w.shape()[1];
+    }
+    if (!a.group_list.is_defined()) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", group_type 0 needs 'group_list'.";
+    }
+    if (a.group_list.data_type() != kNumberTypeInt64 || a.group_list.numel() != e) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", 'group_list' must be Int64 with E = " << e
+                         << " elements, but got " << a.group_list.data_type() << " " << a.group_list.shape();
+    }
+    LaunchOne(x, w, At(a.bias, 0), At(a.scale, 0), At(a.antiquant_scale, 0), At(a.antiquant_offset, 0),
+              At(a.per_token_scale, 0), a.group_list, a.group_list_type, outputs.at(0), m, k, n, e, stream);
+    return;
+  }
+  if (a.group_type != kGroupTypeMultiOutput) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", group_type " << a.group_type
+                     << " is not implemented by the HIP backend (supported: -1 and 0).";
+  }
+  // independent problems x[i] [..., m, k] @ weight[i] [k, n]
+  for (size_t i = 0; i < a.x.size(); ++i) {
+    const auto &x = a.x[i];
+    const auto &w = a.weight[i];
+    if (w.shape().size() != kDim2 || x.shape().size() < kDim2) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", with group_type -1 every weight must be [K, N] "
+                         << "and every x at least 2D, but got " << x.shape() << " and " << w.shape();
+    }
+    const int64_t k = x.shape().back(), n = w.shape()[1];
+    if (w.shape()[0] != k) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", the K dimension of 'x' and 'weight' must be equal, "
+                         << "but got " << k << " and " << w.shape()[0];
+    }
+    const int64_t rows = k > 0 ? x.numel() / k : 0;
+    LaunchOne(x, w, At(a.bias, i), At(a.scale, i), At(a.antiquant_scale, i), At(a.antiquant_offset, i),
+              At(a.per_token_scale, i), ms::Tensor(), 0, outputs.at(i), rows, k, n, 1, stream);
+  }
+}
+}  // namespace
+
+// =============================================================================
+// GRAPH MODE IMPLEMENTATION
+// =============================================================================
+class GroupedMatmulV4CopsHip : public KernelMod {
+ public:
+  // Resize = the reference's GetWorkSpaceInfo: recover the lists and the trailing scalars
+  // (grouped_matmul_v4_cops.cc:101-137).  Inputs arrive as twelve list slots followed by the scalars.
+  std::vector<size_t> Resize(const KernelTensorList &inputs, const std::vector<ms::Tensor> &) override {
+    group_info_ = FetchGroupInfo(inputs);
+    start_idxs_ = ComputeStartIdxsFromGroupInfo(group_info_);
+    args_ = V4Args();
+    auto list = [&](size_t i) { return inputs[i].IsNone() ? TensorVec() : inputs[i].sequence; };
+    args_.x = list(kXIndex);
+    args_.weight = list(kWeightIndex);
+    args_.bias = list(kBiasIndex);
+    args_.scale = list(kScaleIndex);
+    args_.offset = list(kOffsetIndex);
+    args_.antiquant_scale = list(kAntiquantScaleIndex);
+    args_.antiquant_offset = list(kAntiquantOffsetIndex);
+    args_.per_token_scale = list(kPerTokenScaleIndex);
+    args_.group_list = inputs[kGroupListIndex].tensor;
+    args_.activation_input = list(kActivationInputIndex);
+    args_.activation_quant_scale = list(kActivationInputIndex + 1);
+    args_.activation_quant_offset = list(kActivationInputIndex + 2);
+    args_.split_item = inputs[kSplitItemIndex].GetValueWithCheck<int64_t>();
+    args_.group_type = inputs[kGroupTypeIndex].GetValueWithCheck<int64_t>();
+    args_.group_list_type = inputs[kGroupListTypeIndex].GetValueWithCheck<int64_t>();
+    args_.act_type = inputs[kActTypeIndex].GetValueWithCheck<int64_t>();
+    args_.weight_format = inputs[kWeightFormatIndex].GetValueWithCheck<std::string>();
+    return {};
+  }
+
+  bool Launch(const KernelTensorList &, const std::vector<ms::Tensor> &, const std::vector<ms::Tensor> &outputs,
+              void *) override {
+    RunGroupedMatmulV4(args_, outputs);
+    return true;
+  }
+
+  const std::vector<int64_t> &start_idxs() const { return start_idxs_; }
+
+ private:
+  V4Args args_;
+  std::vector<int64_t> group_info_{};
+  std::vector<int64_t> start_idxs_{};
+};
+}  // namespace ms_custom_ops
+
+REG_GRAPH_MODE_OP(grouped_matmul_v4_cops, ms_custom_ops::GroupedMatmulV4CopsFuncImpl,
+                  ms_custom_ops::GroupedMatmulV4CopsHip);
+
+// =============================================================================
+// PYBOOST MODE IMPLEMENTATION
+// =============================================================================
+namespace ms_custom_ops {
+static TensorVec GetOptionalTensorList(const std::optional<TensorVec> &tensor_list) {
+  return tensor_list.has_value() ? tensor_list.value() : TensorVec();
+}
+
+std::vector<ms::Tensor> grouped_matmul_v4_cops_custom(
+  const TensorVec &x, const TensorVec &weight, const std::optional<TensorVec> &bias,
+  const std::optional<TensorVec> &scale, const std::optional<TensorVec> &offset,
+  const std::optional<TensorVec> &antiquant_scale, const std::optional<TensorVec> &antiquant_offset,
+  const std::optional<TensorVec> &per_token_scale, const std::optional<ms::Tensor> &group_list,
+  const std::optional<TensorVec> &activation_input, const std::optional<TensorVec> &activation_quant_scale,
+  const std::optional<TensorVec> &activation_quant_offset, const int64_t &split_item, const int64_t &group_type,
+  const int64_t &group_list_type, const int64_t &act_type, const std::string &weight_format,
+  const std::optional<int64_t> &output_dtype) {
+  auto output_types = InferOutputTypes(x, weight, scale, output_dtype);
+  auto output_shapes = InferOutputShapes(x, weight, group_list, group_type);
+  if (output_types.size() != output_shapes.size()) {
+    MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName
+                       << ", the number of output types must be equal to the number of output shapes, "
+                       << "but got output types size: " << output_types.size()
+                       << ", output shapes size: " << output_shapes.size();
+  }
+  V4Args args;
+  args.x = x;
+  args.weight = weight;
+  args.bias = GetOptionalTensorList(bias);
+  args.scale = GetOptionalTensorList(scale);
+  args.offset = GetOptionalTensorList(offset);
+  args.antiquant_scale = GetOptionalTensorList(antiquant_scale);
+  args.antiquant_offset = GetOptionalTensorList(antiquant_offset);
+  args.per_token_scale = GetOptionalTensorList(per_token_scale);
+  args.group_list = GetTensorOrEmpty(group_list);
+  args.activation_input = GetOptionalTensorList(activation_input);
+  args.activation_quant_scale = GetOptionalTensorList(activation_quant_scale);
+  args.activation_quant_offset = GetOptionalTensorList(activation_quant_offset);
+  args.split_item = split_item;
+  args.group_type = group_type;
+  args.group_list_type = group_list_type;
+  args.act_type = act_type;
+  args.weight_format = weight_format;
+  CheckV4Support(args);
+  if (output_types[0] == kNumberTypeInt8) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName
+                     << ", uint64 scales with int8 output are not implemented by the HIP backend.";
+  }
+  std::vector<ms::Tensor> outputs;
+  for (size_t i = 0; i < output_types.size(); i++) outputs.push_back(AllocateTensor(output_types[i], output_shapes[i]));
+  RunGroupedMatmulV4(args, outputs);
+  return outputs;
+}
+}  // namespace ms_custom_ops
+
+MS_CUSTOM_OPS_EXTENSION_MODULE(m) {
+  m.def("grouped_matmul_v4_cops", &ms_custom_ops::grouped_matmul_v4_cops_custom, "GroupedMatmulV4", pybind11::arg("x"),
+        pybind11::arg("weight"), pybind11::arg("bias") = std::nullopt, pybind11::arg("scale") = std::nullopt,
+        pybind11::arg("offset") = std::nullopt, pybind11::arg("antiquant_scale") = std::nullopt,
+        pybind11::arg("antiquant_offset") = std::nullopt, pybind11::arg("per_token_scale") = std::nullopt,
+        pybind11::arg("group_list") = std::nullopt, pybind11::arg("activation_input") = std::nullopt,
+        pybind11::arg("activation_quant_scale") = std::nullopt, pybind11::arg("activation_quant_offset") = std::nullopt,
+        pybind11::arg("split_item") = 0, pybind11::arg("group_type") = -1, pybind11::arg("group_list_type") = 0,
+        pybind11::arg("act_type") = 0, pybind11::arg("weight_format") = std::string("ND"),
+        pybind11::arg("output_dtype") = std::nullopt);
+}

@@ -1,0 +1,150 @@
+"""grouped_matmul_v4_cops through the Python entry -- the quantized cases of the reference's
+tests/st/test_grouped_matmul_v4_cops.py (per-token, per-channel + bias, a16w8, counts vs cumulative
+group_list, a last boundary below M, multi-output group_type -1), both execution modes."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import ms_custom_ops_amd as ms_custom_ops
+from oracle import gmm_oracle as O
+
+pytestmark = pytest.mark.gpu
+MODES = [ms_custom_ops.GRAPH_MODE, ms_custom_ops.PYNATIVE_MODE]
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def _t(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t if dtype is None else t.to(dtype)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_v4_pertoken_constant_scales(device, mode):
+    """scale = 10 (bf16), per-token = 10 -> 100 * acc (test_grouped_matmul_v4_cops.py:281-319)."""
+    k = np.load(os.path.join(GOLDEN, "kat_const_scale.npz"))
+    with ms_custom_ops.exec_mode(mode):
+        res = ms_custom_ops.grouped_matmul_v4_cops(
+            [_t(k["x"])], [_t(k["w"])], None, [_t(np.full((8, 128), 10, np.float32), torch.bfloat16)], None, None, None,
+            [_t(np.full(32, 10, np.float32))], _t(k["counts"]), split_item=3, group_type=0, group_list_type=1)
+    assert len(res) == 1 and res[0].dtype == torch.bfloat16 and res[0].shape == (32, 128)
+    np.testing.assert_allclose(k["pertoken_expected"], res[0].float().cpu().numpy(), rtol=4e-3)   # reference's bar
+    want = O.f32_to_bf16_bits(k["pertoken_expected"])
+    assert np.array_equal(res[0].view(torch.int16).cpu().numpy().view(np.uint16), want)          # this build's bar
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_v4_perchannel_bias_constant_scales(device, mode):
+    """scale = 10 (bf16), bias = 1 -> 10 * (acc + 1) (test_grouped_matmul_v4_cops.py:338-376)."""
+    k = np.load(os.path.join(GOLDEN, "kat_const_scale.npz"))
+    with ms_custom_ops.exec_mode(mode):
+        res = ms_custom_ops.grouped_matmul_v4_cops(
+            [_t(k["x"])], [_t(k["w"])], [_t(np.ones((8, 128), np.int32))],
+            [_t(np.full((8, 128), 10, np.float32), torch.bfloat16)], None, None, None, None, _t(k["counts"]),
+            split_item=3, group_type=0, group_list_type=1)
+    np.testing.assert_allclose(k["perchannel_bias_expected"], res[0].float().cpu().numpy(), rtol=4e-3)
+    assert np.array_equal(res[0].view(torch.int16).cpu().numpy().view(np.uint16),
+                          O.f32_to_bf16_bits(k["perchannel_bias_expected"]))
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_v4_no_scale_returns_int32_accumulators(device, mode):
+    k = np.load(os.path.join(GOLDEN, "kat_const_scale.npz"))
+    with ms_custom_ops.exec_mode(mode):
+        res = ms_custom_ops.grouped_matmul_v4_cops([_t(k["x"])], [_t(k["w"])], group_list=_t(k["counts"]),
+                                                   split_item=3, group_type=0, group_list_type=1)
+    assert res[0].dtype == torch.int32 and np.array_equal(res[0].cpu().numpy(), k["acc"])
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_v4_float32_scale_output_dtype_rules(device, mode):
+    rng = np.random.default_rng(0)
+    x = rng.integers(-127, 128, (96, 128), dtype=np.int8)
+    w = rng.integers(-127, 128, (8, 128, 256), dtype=np.int8)
+    s = rng.uniform(1e-3, 1e-2, (8, 256)).astype(np.float32)
+    pt = rng.uniform(1e-3, 1e-2, 96).astype(np.float32)
+    gl = np.array([10, 10, 30, 41, 60, 77, 77, 96], dtype=np.int64)
+    with ms_custom_ops.exec_mode(mode):
+        f16 = ms_custom_ops.grouped_matmul_v4_cops([_t(x)], [_t(w)], None, [_t(s)], None, None, None, [_t(pt)], _t(gl),
+                                                   split_item=3, group_type=0)[0]
+        bf16 = ms_custom_ops.grouped_matmul_v4_cops([_t(x)], [_t(w)], None, [_t(s)], None, None, None, [_t(pt)],
+                                                    _t(gl), split_item=3, group_type=0,
+                                                    output_dtype=torch.bfloat16)[0]
+    assert f16.dtype == torch.float16     # float32 scale -> float16 (reference rule)
+    assert np.array_equal(f16.cpu().numpy().view(np.uint16),
+                          O.grouped_matmul_w8a8(x, w, gl, None, s, pt, out_dtype="f16").view(np.uint16))
+    assert bf16.dtype == torch.bfloat16   # explicit output_dtype (backend extension)
+    assert np.array_equal(bf16.view(torch.int16).cpu().numpy().view(np.uint16),
+                          O.grouped_matmul_w8a8(x, w, gl, None, s, pt))
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_v4_a16w8_last_boundary_below_m(device, mode, dtype):
+    """a16w8 with scale 0.01 and offset 1, group_list [1,3,10,14,18,22,24,30] over 32 rows: only the first
+    30 rows are defined (test_grouped_matmul_v4_cops.py:139-192)."""
+    rng = np.random.default_rng(1)
+    m, k, n, e = 32, 256, 128, 8
+    ends = np.array([1, 3, 10, 14, 18, 22, 24, 30], dtype=np.int64)
+    x = _t(rng.uniform(-128, 127, (m, k)).astype(np.float32), dtype)
+    w = rng.uniform(-128, 127, (e, k, n)).astype(np.int8)
+    s = _t(np.full((e, n), 0.01, np.float32), dtype)
+    o = _t(np.full((e, n), 1, np.float32), dtype)
+    with ms_custom_ops.exec_mode(mode):
+        res = ms_custom_ops.grouped_matmul_v4_cops([x], [_t(w)], None, None, None, [s], [o], None, _t(ends), None, None,
+                                                   None, 3, 0, 0)
+    assert res[0].dtype == dtype and res[0].shape == (m, n)
+    xf, sf, of = x.float().cpu().numpy(), s.float().cpu().numpy(), o.float().cpu().numpy()
+    exact = O.a16w8_grouped_f64(xf, w, sf, of, ends)[:30]
+    mag = np.zeros_like(exact)
+    starts = np.concatenate([[0], ends[:-1]])
+    for g in range(e):
+        a, b = int(starts[g]), int(ends[g])
+        mag[a:b] = np.abs(xf[a:b].astype(np.float64)) @ (np.abs(w[g].astype(np.float64) + of[g]) * np.abs(sf[g]))
+    got = res[0][:30].float().cpu().numpy().astype(np.float64)
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    # floating-point tolerance: one output ulp plus float32 accumulation noise relative to sum |terms|
+    assert (np.abs(got - exact) <= ulp * np.abs(exact) + 1e-5 * mag).all()
+    big = np.abs(exact) > 0.05 * mag
+    np.testing.assert_allclose(got[big], exact[big], rtol=1e-2 if dtype == torch.bfloat16 else 2e-3)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_v4_multi_output_group_type_minus_one(device, mode):
+    rng = np.random.default_rng(2)
+    x0 = rng.integers(-127, 128, (2, 3, 16, 256), dtype=np.int8)
+    x1 = rng.integers(-127, 128, (127, 96), dtype=np.int8)
+    w0 = rng.integers(-127, 128, (256, 128), dtype=np.int8)
+    w1 = rng.integers(-127, 128, (96, 64), dtype=np.int8)
+    s0 = rng.uniform(1e-3, 1e-2, 128).astype(np.float32)
+    s1 = rng.uniform(1e-3, 1e-2, 64).astype(np.float32)
+    with ms_custom_ops.exec_mode(mode):
+        res = ms_custom_ops.grouped_matmul_v4_cops([_t(x0), _t(x1)], [_t(w0), _t(w1)], None, [_t(s0), _t(s1)],
+                                                   split_item=0, group_type=-1, output_dtype=torch.bfloat16)
+    assert [tuple(r.shape) for r in res] == [(2, 3, 16, 128), (127, 64)]
+    for r, x, w, s in ((res[0], x0, w0, s0), (res[1], x1, w1, s1)):
+        ref = O.quant_batch_matmul_oracle(x.reshape(-1, x.shape[-1]), w, s).reshape(r.shape)
+        assert np.array_equal(r.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+
+
+def test_v4_errors(device):
+    x = torch.zeros(32, 64, dtype=torch.int8, device="cuda")
+    w = torch.zeros(8, 64, 128, dtype=torch.int8, device="cuda")
+    gl = torch.full((8,), 4, dtype=torch.int64, device="cuda")
+    f = ms_custom_ops.grouped_matmul_v4_cops
+    with pytest.raises(RuntimeError, match="weight_format 'FRACTAL_NZ'"):
+        f([x], [w], group_list=gl, split_item=3, group_type=0, weight_format="FRACTAL_NZ")
+    with pytest.raises(RuntimeError, match="fused activation is not implemented"):
+        f([x], [w], group_list=gl, split_item=3, group_type=0, act_type=1)
+    with pytest.raises(RuntimeError, match="quantized paths only"):
+        f([x.bfloat16()], [w.bfloat16()], group_list=gl, split_item=3, group_type=0)
+    with pytest.raises(ValueError, match="group_type 0 needs 'group_list'"):
+        f([x], [w], split_item=3, group_type=0)
+    with pytest.raises(ValueError, match="'group_list' must be Int64"):
+        f([x], [w], group_list=gl.int(), split_item=3, group_type=0)
+    with pytest.raises(ValueError, match="the scale only support"):
+        f([x], [w], None, [torch.ones(8, 128, dtype=torch.float16, device="cuda")], group_list=gl, split_item=3,
+          group_type=0)
+    with pytest.raises(TypeError):
+        f(x, [w], group_list=gl)

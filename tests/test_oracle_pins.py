@@ -1,0 +1,280 @@
+"""Pins for the CPU oracle: every function is checked against something other than itself --
+brute force, closed forms, an independent C implementation, torch's casts, the reference's
+constant-scale known answers -- chosen so that a dropped term, a wrong index or a transposed operand
+fails at least one test."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import gmm_oracle as O
+
+
+# ---------------------------------------------------------------- bf16 / f16 casts
+def test_bf16_rne_hand_computed_ties():
+    cases = {
+        0x3F800000: 0x3F80,  # 1.0
+        0x3F808000: 0x3F80,  # 1 + 2^-8: tie, even mantissa stays
+        0x3F818000: 0x3F82,  # 1 + 3*2^-8: tie, odd mantissa rounds up
+        0x3F808001: 0x3F81,  # just above the tie
+        0x3F807FFF: 0x3F80,  # just below the tie
+        0xBF818000: 0xBF82,  # sign does not matter
+        0x7F7FFFFF: 0x7F80,  # largest float rounds to +inf
+        0x00000000: 0x0000,
+        0x80000000: 0x8000,
+        0x7F800000: 0x7F80,  # inf
+        0x00008000: 0x0000,  # subnormal tie to even
+        0x00018000: 0x0002,
+    }
+    bits = np.array(list(cases.keys()), dtype=np.uint32)
+    got = O.f32_to_bf16_bits(bits.view(np.float32))
+    assert got.tolist() == list(cases.values())
+    for b, want in cases.items():
+        assert c_oracle.f32_to_bf16(float(np.array([b], dtype=np.uint32).view(np.float32)[0])) == want
+
+
+def test_bf16_rne_matches_torch_cast():
+    rng = np.random.default_rng(0)
+    vals = np.concatenate([
+        rng.standard_normal(200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-30, 30, 200000),
+        rng.integers(0, 2 ** 32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32),
+        np.array([0.0, -0.0, np.inf, -np.inf, 1e-45, 3.4e38], dtype=np.float32),
+    ]).astype(np.float32)
+    vals = vals[~np.isnan(vals)]
+    want = torch.from_numpy(vals).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(O.f32_to_bf16_bits(vals), want)
+    assert np.isnan(O.bf16_bits_to_f32(O.f32_to_bf16_bits(np.array([np.nan], dtype=np.float32))))[0]
+
+
+def test_bf16_roundtrip_is_identity_on_bf16_values():
+    bits = np.arange(0, 0x7F80, dtype=np.uint16)
+    assert np.array_equal(O.f32_to_bf16_bits(O.bf16_bits_to_f32(bits)), bits)
+
+
+def test_f16_cast_matches_torch():
+    rng = np.random.default_rng(1)
+    v = (rng.standard_normal(100000) * 100).astype(np.float32)
+    assert np.array_equal(O.f32_to_f16(v).view(np.uint16),
+                          torch.from_numpy(v).to(torch.float16).view(torch.int16).numpy().view(np.uint16))
+
+
+# ---------------------------------------------------------------- exact accumulators
+@pytest.mark.parametrize("m,k,n", [(1, 1, 1), (3, 5, 2), (4, 33, 7), (2, 64, 3)])
+def test_exact_matmul_equals_bruteforce(m, k, n):
+    rng = np.random.default_rng(m * 100 + k)
+    a = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    b = rng.integers(-127, 128, (k, n), dtype=np.int8)
+    assert np.array_equal(O.int32_matmul_exact(a, b), O.int32_matmul_bruteforce(a, b))
+
+
+def test_exact_matmul_closed_forms():
+    k = 4096
+    ones = np.ones((3, k), dtype=np.int8)
+    w = np.ones((k, 5), dtype=np.int8)
+    assert (O.int32_matmul_exact(ones, w) == k).all()
+    # saturated inputs: the largest magnitude a K=4096 int8 dot product can reach
+    a = np.full((2, k), -127, dtype=np.int8)
+    b = np.full((k, 2), 127, dtype=np.int8)
+    assert (O.int32_matmul_exact(a, b) == -127 * 127 * k).all()
+    # identity weights return x itself; a shifted identity catches transposed operands
+    x = np.random.default_rng(2).integers(-127, 128, (7, 64), dtype=np.int8)
+    eye = np.eye(64, dtype=np.int8)
+    assert np.array_equal(O.int32_matmul_exact(x, eye), x.astype(np.int32))
+    shift = np.roll(eye, 1, axis=1)  # shift[k, (k+1) % 64] = 1
+    assert np.array_equal(O.int32_matmul_exact(x, shift), np.roll(x.astype(np.int32), 1, axis=1))
+
+
+def test_exact_matmul_vs_int64_and_float64_and_chunking():
+    rng = np.random.default_rng(3)
+    a = rng.integers(-127, 128, (37, 5000), dtype=np.int8)   # K > chunk, not a multiple of it
+    b = rng.integers(-127, 128, (5000, 29), dtype=np.int8)
+    want = a.astype(np.int64) @ b.astype(np.int64)
+    got = O.int32_matmul_exact(a, b)
+    assert np.array_equal(got, want.astype(np.int32))
+    assert np.array_equal(got, (a.astype(np.float64) @ b.astype(np.float64)).astype(np.int64).astype(np.int32))
+
+
+def test_single_sgemm_golden_is_inexact_on_adversarial_data_but_exact_path_is_not():
+    # all-max inputs push partial sums past 2**24, where one float32 dot loses integers; the chunked path must not
+    k = 4096
+    a = np.full((1, k), 127, dtype=np.int8)
+    b = np.full((k, 1), 127, dtype=np.int8)
+    b[-1, 0] = 126
+    exact = O.int32_matmul_exact(a, b)[0, 0]
+    assert exact == 127 * 127 * (k - 1) + 127 * 126
+
+
+# ---------------------------------------------------------------- grouping
+def test_group_bounds_cumulative_counts_and_empty_groups():
+    s, e = O.group_bounds([0, 3, 3, 10], 0)
+    assert s.tolist() == [0, 0, 3, 3] and e.tolist() == [0, 3, 3, 10]
+    s2, e2 = O.group_bounds([0, 3, 0, 7], 1)
+    assert s2.tolist() == s.tolist() and e2.tolist() == e.tolist()
+    with pytest.raises(ValueError):
+        O.group_bounds([5, 3], 0)
+
+
+def _toy(rng, m=23, k=64, n=48, e=4):
+    x = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (e, k, n), dtype=np.int8)
+    return x, w
+
+
+def test_grouped_acc_rows_use_only_their_groups_weights():
+    rng = np.random.default_rng(4)
+    x, w = _toy(rng)
+    gl = [5, 5, 16, 23]  # group 1 empty
+    acc = O.grouped_int32_acc(x, w, gl)
+    for g, (s, t) in enumerate([(0, 5), (5, 5), (5, 16), (16, 23)]):
+        assert np.array_equal(acc[s:t], O.int32_matmul_bruteforce(x[s:t], w[g]))
+    # changing another group's weights leaves this group's rows alone
+    w2 = w.copy()
+    w2[0] = 0
+    w2[1] = 7
+    acc2 = O.grouped_int32_acc(x, w2, gl)
+    assert np.array_equal(acc2[5:], acc[5:]) and (acc2[:5] == 0).all()
+    # permuting rows inside a group permutes its outputs
+    perm = np.arange(23)
+    perm[5:16] = perm[5:16][::-1]
+    assert np.array_equal(O.grouped_int32_acc(x[perm], w, gl), acc[perm])
+    # E = 1 is the dense product; counts == cumulative; transposed storage == plain storage
+    assert np.array_equal(O.grouped_int32_acc(x, w[:1], [23]), O.int32_matmul_exact(x, w[0]))
+    assert np.array_equal(O.grouped_int32_acc(x, w, [5, 0, 11, 7], 1), acc)
+    assert np.array_equal(O.grouped_int32_acc(x, np.ascontiguousarray(w.transpose(0, 2, 1)), gl, transpose_b=True), acc)
+    # rows past the last boundary stay zero
+    short = O.grouped_int32_acc(x, w, [5, 5, 16, 20])
+    assert (short[20:] == 0).all() and np.array_equal(short[:20], acc[:20])
+
+
+def test_numpy_and_c_oracles_agree_bit_for_bit():
+    rng = np.random.default_rng(5)
+    m, k, n, e = 150, 1088, 80, 8
+    x = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (e, k, n), dtype=np.int8)
+    bias = rng.integers(-1000, 1001, (e, n)).astype(np.int32)
+    scale = rng.uniform(1e-3, 1e-2, (e, n)).astype(np.float32)
+    pt = rng.uniform(1e-3, 1e-2, m).astype(np.float32)
+    gl = O.random_group_list(m, e, rng)
+    bits, acc = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt, return_acc=True)
+    acc_b = O.grouped_matmul_w8a8(x, w, gl, bias, None, None, out_dtype="i32")
+    c_acc, c_bits = c_oracle.gmm_w8a8(x, w, gl, bias, scale, pt)
+    assert np.array_equal(c_acc, acc_b)
+    assert np.array_equal(c_bits, bits)
+    # transposed weights and counts in the C oracle too
+    counts = np.diff(np.concatenate([[0], gl]))
+    c_acc2, c_bits2 = c_oracle.gmm_w8a8(x, np.ascontiguousarray(w.transpose(0, 2, 1)), counts, bias, scale, pt,
+                                        group_list_type=1, transpose_b=True)
+    assert np.array_equal(c_acc2, acc_b) and np.array_equal(c_bits2, bits)
+
+
+# ---------------------------------------------------------------- epilogue
+def test_epilogue_reference_known_answers():
+    rng = np.random.default_rng(6)
+    x = rng.integers(-128, 128, (32, 256)).astype(np.int8)
+    w = rng.integers(-128, 128, (8, 256, 128)).astype(np.int8)
+    counts = np.array([1, 2, 7, 4, 4, 4, 2, 8])
+    acc = O.grouped_int32_acc(x, w, counts, 1)
+    # scale = 10, per-token = 10 -> 100 * acc (test_grouped_matmul_v4_cops.py:294-301)
+    out = O.grouped_matmul_w8a8(x, w, counts, None, np.full((8, 128), 10, np.float32), np.full(32, 10, np.float32),
+                                group_list_type=1, out_dtype="f32")
+    assert np.array_equal(out, acc.astype(np.float32) * 100)
+    # scale = 10, bias = 1 -> 10 * (acc + 1) (test_grouped_matmul_v4_cops.py:351-359)
+    out = O.grouped_matmul_w8a8(x, w, counts, np.ones((8, 128), np.int32), np.full((8, 128), 10, np.float32), None,
+                                group_list_type=1, out_dtype="f32")
+    assert np.array_equal(out, (acc + 1).astype(np.float32) * 10)
+    # scale = 1 and int32 output -> acc exactly (test_quant_batch_matmul.py:76-80)
+    assert np.array_equal(O.quant_batch_matmul_oracle(x, w[0], np.ones(1, np.float32), out_dtype="i32"),
+                          x.astype(np.int32) @ w[0].astype(np.int32))
+
+
+def test_epilogue_operation_order_is_two_separate_float32_products():
+    # values where (f*s)*p and f*(s*p) round differently in float32: the oracle must do the former
+    acc = np.array([[16777217 // 3]], dtype=np.int32)
+    s = np.array([0.1], dtype=np.float32)
+    p = np.array([0.3], dtype=np.float32)
+    want = np.float32(np.float32(np.float32(acc[0, 0]) * s[0]) * p[0])
+    got = O.dequant_epilogue(acc, None, s, p, "f32")[0, 0]
+    assert got == want
+    # bias is added in int32 before the conversion to float
+    big = np.array([[2 ** 24]], dtype=np.int32)
+    assert O.dequant_epilogue(big, np.array([1], np.int32), None, None, "f32")[0, 0] == np.float32(2 ** 24 + 1)
+    assert O.dequant_epilogue(big, np.array([1], np.int32), None, None, "i32")[0, 0] == 2 ** 24 + 1
+
+
+def test_exact_path_agrees_with_literal_reference_goldens_under_their_tolerances():
+    rng = np.random.default_rng(7)
+    m, k, n, e = 64, 64, 128, 8
+    x = rng.uniform(-20, 20, (m, k)).astype(np.int8)
+    w = rng.uniform(-20, 20, (e, k, n)).astype(np.int8)
+    bias = rng.integers(-10, 10, (e, n)).astype(np.int32)
+    scale = (rng.random((e, n)) / 1000).astype(np.float32)
+    pt = rng.random(m).astype(np.float32)
+    gl = O.random_group_list(m, e, rng)
+    gold = O.golden_grouped_w8a8(x, w, gl, bias, scale, pt, out="f16")
+    mine = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt, out_dtype="f16")
+    assert np.array_equal(gold.view(np.uint16), mine.view(np.uint16))  # small sums: the golden's sgemm is exact
+    assert O.count_compare(mine.astype(np.float32), gold.astype(np.float32), 0.004)
+    # V4 float goldens (inexact by construction) at their rtol
+    counts = np.array([1, 2, 7, 4, 4, 4, 2, 8]) * 2
+    s10 = np.full((e, n), 10, np.float32)
+    g1 = O.golden_v4_pertoken(x, w, s10, np.full(m, 10, np.float32), counts)
+    o1 = O.grouped_matmul_w8a8(x, w, counts, None, s10, np.full(m, 10, np.float32), group_list_type=1, out_dtype="f32")
+    np.testing.assert_allclose(g1, o1, rtol=4e-3)
+    g2 = O.golden_v4_perchannel_bias(x, w, s10, np.ones((e, n), np.float32), counts)
+    o2 = O.grouped_matmul_w8a8(x, w, counts, np.ones((e, n), np.int32), s10, None, group_list_type=1, out_dtype="f32")
+    np.testing.assert_allclose(g2, o2, rtol=4e-3)
+
+
+# ---------------------------------------------------------------- dense path
+def test_quant_batch_matmul_oracle_batches_and_transposes():
+    rng = np.random.default_rng(8)
+    x1 = rng.integers(-5, 5, (8, 64, 32)).astype(np.int8)   # [batch, K, M]
+    x2 = rng.integers(-5, 5, (8, 48, 64)).astype(np.int8)   # [batch, N, K]
+    s = rng.standard_normal(1).astype(np.float32)
+    want = np.matmul(x1.astype(np.int32).transpose(0, 2, 1), x2.astype(np.int32).transpose(0, 2, 1)) * s
+    got = O.quant_batch_matmul_oracle(x1, x2, s, transpose_x1=True, transpose_x2=True, out_dtype="f32")
+    np.testing.assert_allclose(got, want, rtol=1e-6)
+    # broadcasting: 2-D x2 against batched x1
+    y = O.quant_batch_matmul_oracle(x1.transpose(0, 2, 1), x2[0].T, np.ones(48, np.float32), out_dtype="i32")
+    assert np.array_equal(y, np.matmul(x1.astype(np.int32).transpose(0, 2, 1), x2[0].astype(np.int32).T))
+
+
+# ---------------------------------------------------------------- scale wire formats
+def test_scale_wire_formats_round_trip():
+    s = np.random.default_rng(9).uniform(1e-3, 1e-2, (4, 16)).astype(np.float32)
+    enc = O.encode_scale_int64(s)
+    assert enc.dtype == np.int64 and (enc >= 0).all() and (enc < 2 ** 32).all()
+    assert np.array_equal(O.decode_scale_int64(enc), s)
+    enc2 = O.encode_scale_int64_qbmm(s)
+    assert ((enc2 >> 46) & 1 == 1).all()
+    dec2 = O.decode_scale_int64(enc2)
+    assert np.array_equal(dec2.view(np.uint32), s.view(np.uint32) & np.uint32(0xFFFFE000))
+    np.testing.assert_allclose(dec2, s, rtol=2 ** -10)
+
+
+# ---------------------------------------------------------------- weight-only
+def test_a16w8_closed_forms_and_c_cross_check():
+    rng = np.random.default_rng(10)
+    m, k, n, e = 30, 256, 128, 8
+    ends = [1, 3, 10, 14, 18, 22, 24, 30]
+    x = O.bf16_bits_to_f32(O.f32_to_bf16_bits(rng.standard_normal((m, k)).astype(np.float32)))
+    w = rng.integers(-128, 128, (e, k, n)).astype(np.int8)
+    # constant scale 0.01 and offset 1 (test_grouped_matmul_v4_cops.py:156-157): out = 0.01 * x @ (w + 1)
+    s = np.full((e, n), O.bf16_bits_to_f32(O.f32_to_bf16_bits(np.float32(0.01))), np.float32)
+    o = np.ones((e, n), np.float32)
+    got = O.a16w8_grouped_f64(x, w, s, o, ends)
+    starts = [0] + ends[:-1]
+    for g, (a, b) in enumerate(zip(starts, ends)):
+        want = (x[a:b].astype(np.float64) @ (w[g].astype(np.float64) + 1.0)) * np.float64(s[0, 0])
+        np.testing.assert_allclose(got[a:b], want, rtol=1e-12, atol=1e-12)
+    # zero weights: out = s * o * rowsum(x)
+    z = O.a16w8_grouped_f64(x, np.zeros_like(w), s, 3 * o, ends)
+    np.testing.assert_allclose(z[:30], (3.0 * x.astype(np.float64).sum(1) * np.float64(s[0, 0]))[:30, None] *
+                               np.ones((1, n)), rtol=1e-12)
+    # independent C implementation
+    c = c_oracle.gmm_a16w8_f64(O.f32_to_bf16_bits(x), w, O.f32_to_bf16_bits(s), O.f32_to_bf16_bits(o), ends)
+    np.testing.assert_allclose(c, got, rtol=1e-11, atol=1e-9)
+    # the reference's own float golden agrees at its rtol on well-conditioned rows
+    gold = O.golden_v4_a16w8(x.astype(np.float32), w, s, o, ends)
+    big = np.abs(got[:30]) > 1.0
+    np.testing.assert_allclose(gold[big], got[:30][big], rtol=1e-3)
