@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the grouped W8A8 matmul path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout kn|nk] [--no-sweep] [--no-cpu]
+
+A step is one pass of the hot path over one batch of synthetic input (inputs resident in HBM before
+the timed region).  The headline workload is the Mixtral-shaped MoE configuration (E=8, top-2 over
+4096 tokens = 8192 rows, K=4096, N=14336, weights stored [E,K,N]); `value` is its int8 throughput.
+Prints ONE JSON line.  Besides the contract keys it carries
+  roofline      the dominant kernel's achieved algorithmic rate against the MI355X peak,
+  cpu_baseline  the numpy restatement of the reference golden timed on this box's host cores,
+  sweep         the other configurations (dense decode / prefill sweep, skewed MoE, weight-only
+                decode) as TOPS and GB/s with their roofline fractions.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, REPO)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+ROTATE_BYTES = 768e6      # HBM-bound cases rotate over weight copies totalling more than the 256 MB Infinity Cache
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c3")
+    ap.add_argument("--layout", default="kn", choices=["kn", "nk"], help="weight storage: kn=[E,K,N], nk=[E,N,K]")
+    ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    return ap.parse_args()
+
+
+class DeviceProblem:
+    """One workload resident on the GPU plus a planned backend operator."""
+
+    def __init__(self, wl, layout="kn", copies=1):
+        import torch
+        from ms_custom_ops_amd import cabi
+        self.torch, self.cabi, self.wl = torch, cabi, wl
+        dev = torch.device("cuda:0")
+        nk = layout == "nk"
+        self.a16 = wl.kind == "a16w8"
+        t = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+        self.x = t(wl.x.view(np.int16)) if self.a16 else t(wl.x)
+        w0 = t(wl.w)
+        if nk:
+            w0 = w0.transpose(1, 2).contiguous()
+        # extra weight copies (random bytes; only the timing uses them) defeat the Infinity Cache
+        self.w = [w0] + [torch.randint(-127, 128, w0.shape, dtype=torch.int8, device=dev) for _ in range(copies - 1)]
+        self.gl = t(wl.group_list)
+        self.out = torch.empty((wl.m, wl.n), dtype=torch.int16, device=dev)
+        if self.a16:
+            self.scale, self.offset = t(wl.scale.view(np.int16)), t(wl.offset.view(np.int16))
+            self.op = cabi.GmmOp(x_dtype=cabi.DT_BF16, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,
+                                 antiquant_dtype=cabi.DT_BF16, has_antiquant_offset=1)
+        else:
+            self.scale, self.pt, self.bias = t(wl.scale), t(wl.per_token), t(wl.bias)
+            self.op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,
+                                 scale_dtype=cabi.DT_F32, per_token_dtype=cabi.DT_F32,
+                                 bias_dtype=cabi.DT_I32 if self.bias is not None else cabi.DT_NONE,
+                                 transpose_b=int(nk))
+        self.ws_bytes = self.op.plan(wl.m, wl.k, wl.n, wl.e)
+        self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
+        self.stream = torch.cuda.current_stream().cuda_stream
+        self.i = 0
+
+    def step(self):
+        w = self.w[self.i % len(self.w)]
+        self.i += 1
+        p = lambda v: None if v is None else v.data_ptr()
+        if self.a16:
+            ins = [p(self.x), p(w), None, None, p(self.gl), None, p(self.scale), p(self.offset)]
+        else:
+            ins = [p(self.x), p(w), p(self.bias), p(self.scale), p(self.gl), p(self.pt), None, None]
+        self.op.launch(ins, self.out.data_ptr(), self.ws.data_ptr(), self.ws_bytes, self.stream)
+
+    def time(self, steps, warmup):
+        """Returns (wall seconds of `steps` steps, mean per-launch seconds from HIP events on the launch stream)."""
+        torch = self.torch
+        for _ in range(warmup):
+            self.step()
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        t0 = time.perf_counter()
+        for a, b in ev:
+            a.record()
+            self.step()
+            b.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        per_launch = sum(a.elapsed_time(b) for a, b in ev) / steps * 1e-3
+        return wall, per_launch
+
+
+def rates(wl, seconds):
+    from ms_custom_ops_amd import workloads
+    work = workloads.algorithmic_work(wl)
+    tops = work["ops"] / seconds / 1e12
+    gbs = work["bytes"] / seconds / 1e9
+    return work, tops, gbs
+
+
+def cpu_baseline(wl, budget_s=15.0):
+    """The reference golden restated in numpy (one float32 dot per group, then the dequant epilogue,
+    bf16 cast), timed group by group on the host until the budget is used up."""
+    from oracle import gmm_oracle as O
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    starts, ends = O.group_bounds(wl.group_list)
+    done_ops, spent, groups = 0.0, 0.0, 0
+    for g in range(wl.e):
+        a, b = int(starts[g]), int(ends[g])
+        if b <= a:
+            continue
+        t0 = time.perf_counter()
+        O.golden_np_qbmm(wl.x[a:b], wl.w[g], wl.scale[g], None if wl.bias is None else wl.bias[g], wl.per_token[a:b],
+                         out="bf16")
+        dt = time.perf_counter() - t0
+        spent += dt
+        done_ops += 2.0 * (b - a) * wl.k * wl.n
+        groups += 1
+        if spent > budget_s:
+            break
+    return {"value": done_ops / spent / 1e12, "unit": "TOPS", "cores": int(threads), "kind": "port",
+            "sample": f"{groups} of {wl.e} expert groups of the {wl.name} workload ({done_ops:.3g} ops in {spent:.2f} s), "
+                      "numpy float32 dot per group + dequant epilogue + bf16 cast"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this build has no multi-GPU path)",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from ms_custom_ops_amd import workloads
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the operators have no CPU path)", file=sys.stderr)
+        sys.exit(1)
+
+    wl = workloads.make(args.workload)
+    prob = DeviceProblem(wl, args.layout)
+    wall, per_launch = prob.time(args.steps, args.warmup)
+    work, _, _ = rates(wl, per_launch)
+    step_s = wall / args.steps
+    tops_wall = work["ops"] / step_s / 1e12
+    tops_kernel = work["ops"] / per_launch / 1e12
+    plan = prob.op.plan_info()
+    mfma_bound = (work["ops"] / work["bytes"]) > (PEAK_INT8_TOPS * 1e12) / (PEAK_HBM_GBS * 1e9)
+    if mfma_bound:
+        roof = {"bound": "mfma", "achieved": tops_kernel, "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
+                "frac": tops_kernel / PEAK_INT8_TOPS, "traffic": None}
+    else:
+        gbs = work["bytes"] / per_launch / 1e9
+        roof = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                "traffic": None}
+    roof["kernel"] = plan.split("kernel=")[1].split(" ")[0]
+    roof["launch_us"] = per_launch * 1e6
+    roof["ops_per_launch"] = work["ops"]
+    roof["bytes_per_launch"] = work["bytes"]
+
+    result = {
+        "metric": "int8 TOPS and HBM GB/s (% roofline) for grouped W8A8 GEMM, 1 MI355X",
+        "value": tops_wall, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": step_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 (int32 accumulate, bf16 out)", "data": "synthetic",
+        "config": {"workload": f"{wl.name}: grouped W8A8, E={wl.e}, rows={work['rows']}, K={wl.k}, N={wl.n}, "
+                               f"weights {'[E,N,K]' if args.layout == 'nk' else '[E,K,N]'}, routing top-2 of softmax(N(0,1))",
+                   "plan": plan},
+        "hbm_gbs": work["bytes"] / step_s / 1e9, "hbm_frac": work["bytes"] / step_s / 1e9 / PEAK_HBM_GBS,
+        "int8_frac": tops_wall / PEAK_INT8_TOPS,
+        "roofline": roof,
+    }
+    del prob
+    torch.cuda.empty_cache()
+
+    if not args.no_sweep:
+        sweep = []
+        for name, layout in [("c3", "nk"), ("c2_m2048", "kn"), ("c4", "kn"), ("c1", "kn"), ("c2_m256", "kn"),
+                             ("c2_m16", "kn"), ("c2_m1", "kn"), ("c5", "kn")]:
+            w2 = workloads.make(name)
+            w_bytes = w2.w.nbytes
+            hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5")
+            copies = max(1, int(np.ceil(ROTATE_BYTES / w_bytes))) if hbm_bound_guess else 1
+            p2 = DeviceProblem(w2, layout, copies)
+            _, sec = p2.time(max(20, min(200, args.steps * 2)), args.warmup)
+            wk, tops, gbs = rates(w2, sec)
+            sweep.append({"workload": name, "layout": layout, "launch_us": sec * 1e6, "tops": tops,
+                          "int8_frac": tops / PEAK_INT8_TOPS, "gbs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS,
+                          "weight_copies_rotated": copies, "kernel": p2.op.plan_info().split("kernel=")[1].split(" m=")[0]})
+            del p2
+            torch.cuda.empty_cache()
+        result["sweep"] = sweep
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(wl)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
