@@ -35,7 +35,7 @@ try:
     from . import ms_custom_ops as _C  # the compiled operator layer
 except ImportError as exc:  # pragma: no cover - exercised only on a broken install
     raise ImportError(
-        "ms_custom_ops_amd: the compiled operator module is missing; run `python -m ms_custom_ops_amd.build` "
+        "ms_custom_ops_amd: the compiled operator module is missing; run `python ms_custom_ops_amd/build.py` "
         "(needs hipcc for gfx950 and g++). There is no fallback implementation.") from exc
 
 __all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "set_context", "get_context", "exec_mode",

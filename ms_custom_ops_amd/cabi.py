@@ -51,7 +51,7 @@ def load():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise ImportError(f"HIP backend library missing: {LIB_PATH}; build it with "
-                              "`python -m ms_custom_ops_amd.build`")
+                              "`python ms_custom_ops_amd/build.py`")
         lib = ctypes.CDLL(LIB_PATH)
         lib.msco_gmm_create.restype = ctypes.c_int
         lib.msco_gmm_create.argtypes = [ctypes.POINTER(GmmDesc), ctypes.POINTER(ctypes.c_void_p)]

@@ -8,6 +8,7 @@
 namespace msco {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
@@ -70,6 +71,15 @@ __device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
   if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) return (unsigned short)((u >> 16) | 0x40u);
   u += 0x7FFFu + ((u >> 16) & 1u);
   return (unsigned short)(u >> 16);
+}
+
+// Two float32 -> packed bfloat16 (lo in bits 0..15) with the hardware's round-to-nearest-even
+// conversion (v_cvt_pk_bf16_f32).
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned pack_bf16x2(float lo, float hi) {
+  const v2f v = {lo, hi};
+  return __builtin_bit_cast(unsigned, __builtin_convertvector(v, v2bf));
 }
 
 __device__ __forceinline__ unsigned short f32_to_f16_rne(float f) {

@@ -1,9 +1,10 @@
 // Grouped W8A8 GEMM, MFMA tile kernel (prefill shapes) for gfx950.
 //
-// One workgroup computes one BM x BN output tile of one group with v_mfma_i32_16x16x64_i8.  The
-// large configuration uses 8 wavefronts (2 x 4, two per SIMD, a 128 x 64 sub-tile of accumulators
-// each), so that one wave's LDS reads, LDS writes and barrier waits are covered by the other wave's
-// MFMAs; the small configurations use 4 wavefronts (2 x 2).
+// One workgroup computes one BM x BN output tile of one group with v_mfma_i32_32x32x32_i8 (the int8
+// MFMA that issues at full rate on this part; measured: the 16x16x64 form sustains about half of it).
+// The large configuration uses 8 wavefronts (2 x 4, two per SIMD, a 128 x 64 sub-tile of accumulators
+// each), so that one wave's LDS reads and barrier waits are covered by the other wave's MFMAs; the
+// small configurations use 4 wavefronts (2 x 2).
 //
 //   * Tile scheduling on the device.  The tile -> (group, m-tile, n-tile) mapping is computed by
 //     walking group_list, so the host never reads it; the grid is sized from an upper bound and
@@ -11,62 +12,99 @@
 //     panel) are dealt to the same XCD so that the x rows of a group and the streamed weight panel
 //     stay in that XCD's L2.
 //   * Memory.  Operands are read through buffer descriptors (scalar base, one per-lane offset,
-//     out-of-range rows read as zero, so no clamping or branching in the loop) in 128-byte K slabs.
-//     Slab t+1 is in flight in registers while slab t is multiplied out of LDS; it is written to the
-//     other LDS stage at the end of the iteration, behind an LDS-only barrier.
-//   * Weights stored [K,N] are transposed into K-contiguous MFMA fragments with v_perm_b32 on the
-//     way into LDS; weights stored [N,K] are copied as they are.
-//   * The dequant epilogue (int32 bias, per-channel scale, per-token scale, bf16/f16 cast) is fused;
-//     every lane owns FN consecutive output columns of a row and stores them with one vector store.
+//     out-of-range rows read as zero, so no clamping or branching in the loop) in 64-byte K slabs,
+//     three slabs ahead of the one being multiplied.  x rows and [N,K] weights go straight from
+//     memory into a 4-stage LDS ring (buffer_load ... lds), so slabs in flight cost no registers.
+//   * Weights stored [K,N] are held in a 3-deep register ring, transposed into K-contiguous MFMA
+//     fragments with v_perm_b32 and written to a 2-stage LDS buffer.
+//   * One LDS-only barrier per slab (it does not wait for the global loads in flight).
+//   * Operand roles.  The weights are the MFMA's first operand and x the second, so a lane owns one
+//     output row m and, after permuting which weight column feeds which MFMA row, two runs of 8
+//     consecutive output columns per 32-column block: the fused dequant epilogue (int32 bias,
+//     per-channel scale, per-token scale, bf16/f16 cast) stores 16 bytes per lane and instruction.
 //
-// LDS layouts (every fragment read is 16 lanes x 16 B over consecutive rows -> conflict free):
-//   x rows and [N,K] weights: row-major, 128 B per row, 16-byte chunk c of row r stored at chunk
-//     position c ^ swz(r);
+// LDS layouts (a fragment read is 16 B per lane over 32 consecutive rows, conflict free per 16 lanes):
+//   x rows and [N,K] weights: row-major, 64 B per row, 16-byte chunk c of row r stored at chunk
+//     position c ^ ((r >> 2) & 3);
 //   [K,N] weights: chunk-major, address = (c * BN + slot) * 16.
 #include "gmm_common.h"
 #include "gmm_kernels.h"
 
+#include <type_traits>
+
 namespace msco {
 
-constexpr int BK = 128;           // bytes of K per LDS slab
+constexpr int BK = 64;        // bytes of K per slab = one MFMA K step
+constexpr int NSTAGE = 4;     // LDS ring depth of operands that are loaded straight into LDS
+constexpr int KN_STAGES = 2;  // LDS stages of the transposed [K,N] weight slab
+constexpr int KN_RING = 3;    // [K,N] weight slabs in flight in registers
 
-typedef unsigned v4u __attribute__((ext_vector_type(4)));
-typedef unsigned v2u __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ int swz64(int r) { return (r >> 2) & 3; }
 
-__device__ __forceinline__ int swz_a(int r) { return (r >> 1) & 7; }
-__device__ __forceinline__ int swz_b(int r) { return ((r >> 1) ^ (r >> 4)) & 7; }
+// MFMA output row q (0..31) of a 32 x 32 block <-> weight column inside the block.  Lane half hh holds
+// rows q = 8 g + 4 hh + t (g = 0..3, t = 0..3); mapping them to columns 16 (g/2) + 8 hh + 4 (g%2) + t
+// gives every lane two runs of 8 consecutive output columns.
+__device__ __forceinline__ int col_of_q(int q) {
+  const int g = q >> 3, hh = (q >> 2) & 1, t = q & 3;
+  return 16 * (g >> 1) + 8 * hh + 4 * (g & 1) + t;
+}
+__device__ __forceinline__ int q_of_col(int c) {
+  const int a = c >> 4, hh = (c >> 3) & 1, b = (c >> 2) & 1, t = c & 3;
+  return 8 * (2 * a + b) + 4 * hh + t;
+}
+
+// 16 bytes per lane from a buffer straight into LDS: lane L of the wave writes lds_base + 16 L.
+// (The address-space cast only exists in the device pass.)
+__device__ __forceinline__ void buffer_load_lds_b128(__amdgpu_buffer_rsrc_t rsrc, void *lds_base, unsigned voffset,
+                                                     unsigned soffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (void __attribute__((address_space(3))) *)(lds_base), 16, voffset,
+                                           soffset, 0, 0);
+#else
+  (void)rsrc; (void)lds_base; (void)voffset; (void)soffset;
+#endif
+}
 
 // LDS-only barrier: waits for this wave's LDS traffic, not for global loads still in flight.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, long long bytes) {
-  const unsigned n = bytes > 0xFFFFFFFFll ? 0xFFFFFFFFu : (unsigned)bytes;
+  const unsigned n = bytes > 0xFFFFFFFFll ? 0xFFFFFFFFu : (unsigned)(bytes < 0 ? 0 : bytes);
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(const GmmParams p) {
-  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int NW = WAVES_M * WAVES_N;
+  constexpr int NT = NW * 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
-  constexpr int FM = WTM / 16, FN = WTN / 16;
-  constexpr int ROWS_IT = NT / 8;                   // rows covered by one pass of 16-byte chunk loads
-  constexpr int A_IT = BM * 8 / NT;                 // 16-byte chunks of the x slab per thread
-  constexpr int B_IT = BN * 8 / NT;                 // same for an [N,K] weight slab
+  constexpr int FM = WTM / 32, FN = WTN / 32;     // 32 x 32 MFMA blocks per wave
+  constexpr int A_LD = BM / 16 / NW;                // 16-row blocks (1 KiB of LDS) of the x slab per wave
+  constexpr int B_LD = BN / 16 / NW;                // same for an [N,K] weight slab
+  constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK;
   constexpr int PANEL = 8;                          // m-tiles that share a streamed weight panel
   constexpr unsigned OOB = 0x80000000u;             // buffer offset that always reads zero
-  // [K,N] weight slab: 8 K-chunks x BN/4 column groups of 16(k) x 4(n)-byte blocks, one per thread
+  constexpr int VM_PER_SLAB = A_LD + (NK ? B_LD : 8);   // vector-memory loads a wave issues per slab
+  // [K,N] weight slab: 8 K-chunks of 8 rows x BN/4 column groups -> one 8(k) x 4(n)-byte block per thread
   static_assert(NT == 2 * BN, "one [K,N] block per thread");
-  static_assert(FM >= 1 && FN >= 1 && A_IT >= 1 && B_IT >= 1 && ROWS_IT % 16 == 0, "tile shape");
+  static_assert(FM >= 1 && FN >= 1 && A_LD >= 1 && B_LD >= 1, "tile shape");
+  static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "row blocks per wave");
 
   extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char *lds_a = smem;                      // [2][BM * BK]
-  unsigned char *lds_b = smem + 2 * BM * BK;        // [2][BN * BK]
+  unsigned char *lds_a = smem;                      // [NSTAGE][BM * BK], rows of 64 B, chunk c at c ^ swz64(row)
+  unsigned char *lds_b = smem + NSTAGE * A_STAGE;   // [N,K]: [NSTAGE][BN * BK] like x; [K,N]: [KN_STAGES][4][BN][16]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
-  const int lane16 = lane & 15, h = lane >> 4;
+  const int l32 = lane & 31, hh = lane >> 5;
 
   // ---- tile lookup: walk group_list twice (count, then locate) -------------------------------
   const int n_tiles = (p.n + BN - 1) / BN;
@@ -122,194 +160,248 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   const __amdgpu_buffer_rsrc_t rw = NK ? make_rsrc(wg + (long long)n0 * p.k, (long long)(p.n - n0) * p.k)
                                        : make_rsrc(wg + n0, w_elems - n0);
 
-  // ---- per-thread load / store coordinates ----------------------------------------------------
-  const int a_row = tid >> 3, a_c = tid & 7;        // + ROWS_IT rows per iteration
-  const unsigned a_voff = (unsigned)a_row * (unsigned)p.k + a_c * 16;
-  const unsigned a_lds = a_row * BK + ((a_c ^ swz_a(a_row)) << 4);   // + it * ROWS_IT * BK (swz_a has period 16 rows)
-  const unsigned bnk_voff = a_voff;
-  const int kn_i = tid % (BN / 4), kn_kc = tid / (BN / 4);
-  const unsigned bkn_voff = (unsigned)(16 * kn_kc) * (unsigned)p.n + 4 * kn_i;
-
-  v4u ra[A_IT];
-  v4u rb[NK ? B_IT : 1];
-  unsigned rkn[NK ? 1 : 16];
-
-  auto load_slab = [&](int kt) {
-    const unsigned kbase = kt * BK;
-    unsigned av = a_voff, bv = bnk_voff;
-    if (k_tail && kbase + a_c * 16 >= (unsigned)p.k) { av = OOB; }
+  // ---- operands loaded straight into LDS (x rows, [N,K] weights) -----------------------------
+  // One wave instruction fills 1 KiB of LDS = 16 rows x 64 B, lane L writing bytes [16 L, 16 L + 16).
+  // With the swizzle, LDS position (row L/4, chunk position L%4) holds logical chunk (L%4) ^ (L/16).
+  // Only the per-lane offset is range-checked by the buffer unit, so everything that can run past
+  // the tensor (rows, columns, the K tail) lives in the per-lane offset; the scalar offset carries
+  // just the slab position inside a row.
+  const int d_row = lane >> 2;
+  const int d_c = (lane & 3) ^ (lane >> 4);
+  unsigned a_voff[A_LD];
 #pragma unroll
-    for (int it = 0; it < A_IT; ++it)
-      ra[it] = __builtin_amdgcn_raw_buffer_load_b128(rx, av, kbase + it * ROWS_IT * p.k, 0);
+  for (int u = 0; u < A_LD; ++u) a_voff[u] = (unsigned)((wave * A_LD + u) * 16 + d_row) * (unsigned)p.k + d_c * 16;
+  // [N,K] weights: LDS row rho = 32 * block + q feeds MFMA row q of that block and holds weight
+  // column 32 * block + col_of_q(q) of the tile.
+  unsigned b_voff[NK ? B_LD : 1];
+  if constexpr (NK) {
+#pragma unroll
+    for (int u = 0; u < B_LD; ++u) {
+      const int blk = wave * B_LD + u;
+      const int rho = blk * 16 + d_row;
+      b_voff[u] = (unsigned)((rho & ~31) + col_of_q(rho & 31)) * (unsigned)p.k + d_c * 16;
+    }
+  }
+  auto issue_direct = [&](int kt) {
+    const int stage = kt & (NSTAGE - 1);
+    const unsigned kbase = kt * BK;
+    const unsigned kill = (k_tail && kbase + d_c * 16 >= (unsigned)p.k) ? OOB : 0u;
+#pragma unroll
+    for (int u = 0; u < A_LD; ++u) {
+      const int blk = wave * A_LD + u;
+      buffer_load_lds_b128(rx, lds_a + stage * A_STAGE + blk * 1024, a_voff[u] | kill, kbase);
+    }
     if constexpr (NK) {
 #pragma unroll
-      for (int it = 0; it < B_IT; ++it)
-        rb[it] = __builtin_amdgcn_raw_buffer_load_b128(rw, bv, kbase + it * ROWS_IT * p.k, 0);
-    } else {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) rkn[r] = __builtin_amdgcn_raw_buffer_load_b32(rw, bkn_voff, (kbase + r) * p.n, 0);
+      for (int u = 0; u < B_LD; ++u) {
+        const int blk = wave * B_LD + u;
+        buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill, kbase);
+      }
     }
   };
 
-  auto store_slab = [&](int buf) {
-    unsigned char *a = lds_a + buf * (BM * BK);
-    unsigned char *b = lds_b + buf * (BN * BK);
+  // ---- [K,N] weights: registers -> v_perm transpose -> LDS -----------------------------------
+  const int kn_i = tid % (BN / 4), kn_k8 = tid / (BN / 4);   // column group of 4, K block of 8 rows
+  // columns past N and K rows past K are turned into out-of-range offsets (they read as zero)
+  const unsigned bkn_voff = (n0 + 4 * kn_i < p.n) ? (unsigned)(8 * kn_k8) * (unsigned)p.n + 4 * kn_i : OOB;
+  unsigned rkn[NK ? 1 : KN_RING][8];
+  auto load_kn = [&](int kt, int slot) {
+    if constexpr (!NK) {
+      const unsigned voff = (k_tail && kt * BK + 8 * kn_k8 >= p.k) ? OOB : bkn_voff;
 #pragma unroll
-    for (int it = 0; it < A_IT; ++it) *reinterpret_cast<v4u *>(a + a_lds + it * ROWS_IT * BK) = ra[it];
-    if constexpr (NK) {
-#pragma unroll
-      for (int it = 0; it < B_IT; ++it) {
-        const int row = a_row + ROWS_IT * it;
-        const int wn = row / WTN, nn = row % WTN;
-        const int l16 = nn / FN, j = nn % FN;
-        const int rho = wn * WTN + j * 16 + (l16 ^ (j & 1));
-        *reinterpret_cast<v4u *>(b + rho * BK + ((a_c ^ swz_b(rho)) << 4)) = rb[it];
-      }
-    } else {
-      // 16(k) x 4(n) byte block -> 4 column fragments of 16 K bytes
-      v4i frag[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        unsigned c0, c1, c2, c3;
-        transpose4x4(rkn[4 * q], rkn[4 * q + 1], rkn[4 * q + 2], rkn[4 * q + 3], c0, c1, c2, c3);
-        frag[0][q] = (int)c0; frag[1][q] = (int)c1; frag[2][q] = (int)c2; frag[3][q] = (int)c3;
-      }
+      for (int r = 0; r < 8; ++r)
+        rkn[slot][r] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff, (kt * BK + r) * p.n, 0);
+    }
+  };
+  auto store_kn = [&](int kt, int slot) {
+    if constexpr (!NK) {
+      unsigned char *b = lds_b + (kt & (KN_STAGES - 1)) * B_STAGE;
+      unsigned lo[4], hi[4];
+      transpose4x4(rkn[slot][0], rkn[slot][1], rkn[slot][2], rkn[slot][3], lo[0], lo[1], lo[2], lo[3]);
+      transpose4x4(rkn[slot][4], rkn[slot][5], rkn[slot][6], rkn[slot][7], hi[0], hi[1], hi[2], hi[3]);
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         const int nl = 4 * kn_i + jj;
-        const int wn = nl / WTN, nn = nl % WTN;
-        const int slot = wn * WTN + (nn % FN) * 16 + nn / FN;
-        *reinterpret_cast<v4i *>(b + ((kn_kc * BN + slot) << 4)) = frag[jj];
+        const int slot_n = (nl & ~31) + q_of_col(nl & 31);
+        // chunk c = kn_k8 / 2 (16 K rows), half kn_k8 % 2 (8 K rows = 8 bytes)
+        *reinterpret_cast<uint2 *>(b + ((((kn_k8 >> 1) * BN + slot_n) << 4) | ((kn_k8 & 1) << 3))) =
+          make_uint2(lo[jj], hi[jj]);
       }
     }
   };
 
   // ---- fragment reads (one 16-byte LDS read per lane and fragment) ----------------------------
-  auto read_a = [&](int buf, int s, int i) -> v4i {
-    const unsigned char *a = lds_a + buf * (BM * BK);
-    const int row = wave_m * WTM + 16 * i + lane16;
-    return *reinterpret_cast<const v4i *>(a + row * BK + (((4 * s + h) ^ swz_a(row)) << 4));
+  // lane (l32, hh) of k-half kk reads row l32 of its 32-row block, 16-byte chunk c = 2 kk + hh
+  auto read_x = [&](int kt, int i, int kk) -> v4i {
+    const unsigned char *a = lds_a + (kt & (NSTAGE - 1)) * A_STAGE;
+    const int row = wave_m * WTM + 32 * i + l32;
+    return *reinterpret_cast<const v4i *>(a + row * BK + (((2 * kk + hh) ^ swz64(row)) << 4));
   };
-  auto read_b = [&](int buf, int s, int j) -> v4i {
-    const unsigned char *b = lds_b + buf * (BN * BK);
-    const int c = 4 * s + h;
+  auto read_w = [&](int kt, int f, int kk) -> v4i {
+    const int rho = wave_n * WTN + 32 * f + l32;
     if constexpr (NK) {
-      const int rho = wave_n * WTN + 16 * j + (lane16 ^ (j & 1));
-      return *reinterpret_cast<const v4i *>(b + rho * BK + ((c ^ swz_b(rho)) << 4));
+      const unsigned char *b = lds_b + (kt & (NSTAGE - 1)) * B_STAGE;
+      return *reinterpret_cast<const v4i *>(b + rho * BK + (((2 * kk + hh) ^ swz64(rho)) << 4));
     } else {
-      const int slot = wave_n * WTN + 16 * j + lane16;
-      return *reinterpret_cast<const v4i *>(b + ((c * BN + slot) << 4));
+      const unsigned char *b = lds_b + (kt & (KN_STAGES - 1)) * B_STAGE;
+      return *reinterpret_cast<const v4i *>(b + (((2 * kk + hh) * BN + rho) << 4));
     }
   };
 
-  v4i acc[FM][FN];
+  v16i acc[FN][FM];
 #pragma unroll
-  for (int i = 0; i < FM; ++i)
+  for (int f = 0; f < FN; ++f)
 #pragma unroll
-    for (int j = 0; j < FN; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[f][i][r] = 0;
 
   // ---- main loop ---------------------------------------------------------------------------------
-  // registers: slab t+1 in flight | LDS stage t&1: slab t being multiplied | stage (t+1)&1: written at the end
-  load_slab(0);
-  store_slab(0);
-  lds_barrier();
-  for (int kt = 0; kt < k_slabs; ++kt) {
-    const int buf = kt & 1;
-    const bool has_next = kt + 1 < k_slabs;
-    if (has_next) load_slab(kt + 1);
+  // Slabs t+1 .. t+3 are in flight (LDS ring for the directly loaded operands, register ring for
+  // [K,N] weights) while slab t is multiplied.  One LDS-only barrier per slab publishes slab t+1 and
+  // retires the stage that slab t+3's loads are about to overwrite.
+  auto step = [&](int kt, auto ring_slot) {
+    constexpr int SLOT = decltype(ring_slot)::value;          // == kt % KN_RING, compile-time for register indexing
+    if (kt + 3 < k_slabs) {
+      issue_direct(kt + 3);
+      load_kn(kt + 3, SLOT);                                  // (kt + 3) % 3 == kt % 3: that slot was emptied last step
+    }
+    v4i xf[2][FM], wf[2][FN];
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      v4i af[FM], bf[FN];
+    for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-      for (int i = 0; i < FM; ++i) af[i] = read_a(buf, s, i);
+      for (int i = 0; i < FM; ++i) xf[kk][i] = read_x(kt, i, kk);
 #pragma unroll
-      for (int j = 0; j < FN; ++j) bf[j] = read_b(buf, s, j);
+      for (int f = 0; f < FN; ++f) wf[kk][f] = read_w(kt, f, kk);
+    }
 #pragma unroll
-      for (int j = 0; j < FN; ++j)
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int f = 0; f < FN; ++f)
 #pragma unroll
         for (int i = 0; i < FM; ++i)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
-    }
-    if (has_next) {
-      // every wave has finished reading stage buf^1 (it was the multiplied stage of iteration t-1,
-      // and the barrier below closed that iteration), so it can be overwritten now
-      store_slab(buf ^ 1);
+          acc[f][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[kk][f], xf[kk][i], acc[f][i], 0, 0, 0);
+    if (kt + 1 < k_slabs) {
+      store_kn(kt + 1, (SLOT + 1) % KN_RING);                 // its LDS stage held slab t-1, read before the last barrier
+      // this wave's loads of slab t+1 have landed once at most the loads of slabs t+2, t+3 are outstanding
+      if (kt + 3 < k_slabs) wait_vmcnt<2 * VM_PER_SLAB>();
+      else if (kt + 2 < k_slabs) wait_vmcnt<VM_PER_SLAB>();
+      else wait_vmcnt<0>();
     }
     lds_barrier();
+  };
+
+  // prologue: slabs 0, 1, 2 requested; slab 0 published
+  issue_direct(0);
+  load_kn(0, 0);
+  if (k_slabs > 1) { issue_direct(1); load_kn(1, 1); }
+  if (k_slabs > 2) { issue_direct(2); load_kn(2, 2); }
+  store_kn(0, 0);
+  if (k_slabs > 2) wait_vmcnt<2 * VM_PER_SLAB>();
+  else if (k_slabs > 1) wait_vmcnt<VM_PER_SLAB>();
+  else wait_vmcnt<0>();
+  lds_barrier();
+
+  for (int kt = 0; kt < k_slabs; kt += KN_RING) {
+    step(kt, std::integral_constant<int, 0>{});
+    if (kt + 1 < k_slabs) step(kt + 1, std::integral_constant<int, 1>{});
+    if (kt + 2 < k_slabs) step(kt + 2, std::integral_constant<int, 2>{});
   }
 
   // ---- fused dequant epilogue --------------------------------------------------------------------
-  const int nb = n0 + wave_n * WTN + FN * lane16;   // first of this lane's FN consecutive columns
-  if (nb >= p.n) return;
-  float sc[FN];
-  int bi[FN];
-#pragma unroll
-  for (int j = 0; j < FN; ++j) {
-    const int n = min(nb + j, p.n - 1);
-    sc[j] = load_scale(p, grp, n);
-    bi[j] = load_bias(p, grp, n);
-  }
-  const bool full = (nb + FN <= p.n);
+  // acc[f][i][r] is output row 32 i + l32 and column 32 f + 16 (r / 8) + 8 hh + (r % 8) of the wave tile:
+  // lanes run along rows.  Each wave dequantises its values, parks them in a private LDS region
+  // (rows of 128 payload bytes at a 144-byte pitch, conflict free both ways) and reads them back with
+  // lanes running along columns, so every global store instruction writes 8 full 128-byte row segments.
+  static_assert(WTN == 64, "epilogue staging assumes 64-column wave tiles");
+  constexpr int EP_PITCH = 144;
+  unsigned char *stage = smem + wave * (WTM * EP_PITCH);
+  float pt[FM];
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
+    const int m = m0 + wave_m * WTM + 32 * i + l32;
+    pt[i] = (p.per_token && m < g_end) ? p.per_token[m] : 1.0f;
+  }
+  // int32 rows are 256 bytes: one 32-column block per pass; 16-bit outputs take a single pass
+  auto run_pass = [&](auto raw_c, auto pass_c) {
+    constexpr bool raw = decltype(raw_c)::value;
+    constexpr int pass = decltype(pass_c)::value;
+    constexpr int esize = raw ? 4 : 2;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int m = m0 + wave_m * WTM + 16 * i + 4 * h + r;
-      if (m >= g_end) continue;
-      const float pt = p.per_token ? p.per_token[m] : 1.0f;
-      const long long base = (long long)m * p.n + nb;
-      if (p.out_dtype == DT_I32) {
-        int *o = reinterpret_cast<int *>(p.out) + base;
-        if (full && (FN % 4 == 0)) {
+    for (int f = 0; f < FN; ++f) {
+      if (raw && f != pass) continue;
 #pragma unroll
-          for (int j = 0; j < FN; j += 4)
-            *reinterpret_cast<int4 *>(o + j) = make_int4(acc[i][j][r] + bi[j], acc[i][j + 1][r] + bi[j + 1],
-                                                         acc[i][j + 2][r] + bi[j + 2], acc[i][j + 3][r] + bi[j + 3]);
-        } else {
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const int cw = 32 * f + 16 * s2 + 8 * hh;            // column inside the wave tile
+        const int nb = n0 + wave_n * WTN + cw;
+        float sc[8];
+        int bi[8];
 #pragma unroll
-          for (int j = 0; j < FN; ++j)
-            if (nb + j < p.n) o[j] = acc[i][j][r] + bi[j];
+        for (int j = 0; j < 8; ++j) {
+          const int n = min(nb + j, p.n - 1);
+          sc[j] = load_scale(p, grp, n);
+          bi[j] = load_bias(p, grp, n);
         }
-      } else {
-        unsigned short hv[FN];
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-          const float f = dequant(acc[i][j][r] + bi[j], sc[j], pt);
-          hv[j] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
-        }
-        unsigned short *o = reinterpret_cast<unsigned short *>(p.out) + base;
-        if (full && (FN % 8 == 0)) {
+        for (int i = 0; i < FM; ++i) {
+          unsigned char *dst = stage + (32 * i + l32) * EP_PITCH;
+          if (raw) {
+            int *d = reinterpret_cast<int *>(dst + (16 * s2 + 8 * hh) * 4);
+            *reinterpret_cast<int4 *>(d) = make_int4(acc[f][i][8 * s2] + bi[0], acc[f][i][8 * s2 + 1] + bi[1],
+                                                     acc[f][i][8 * s2 + 2] + bi[2], acc[f][i][8 * s2 + 3] + bi[3]);
+            *reinterpret_cast<int4 *>(d + 4) = make_int4(acc[f][i][8 * s2 + 4] + bi[4], acc[f][i][8 * s2 + 5] + bi[5],
+                                                         acc[f][i][8 * s2 + 6] + bi[6], acc[f][i][8 * s2 + 7] + bi[7]);
+          } else {
+            float v[8];
 #pragma unroll
-          for (int j = 0; j < FN; j += 8) {
-            uint4 v;
-            v.x = hv[j] | ((unsigned)hv[j + 1] << 16);
-            v.y = hv[j + 2] | ((unsigned)hv[j + 3] << 16);
-            v.z = hv[j + 4] | ((unsigned)hv[j + 5] << 16);
-            v.w = hv[j + 6] | ((unsigned)hv[j + 7] << 16);
-            *reinterpret_cast<uint4 *>(o + j) = v;
+            for (int j = 0; j < 8; ++j) v[j] = dequant(acc[f][i][8 * s2 + j] + bi[j], sc[j], pt[i]);
+            uint4 q;
+            if (p.out_dtype == DT_BF16) {
+              q.x = pack_bf16x2(v[0], v[1]); q.y = pack_bf16x2(v[2], v[3]);
+              q.z = pack_bf16x2(v[4], v[5]); q.w = pack_bf16x2(v[6], v[7]);
+            } else {
+              q.x = f32_to_f16_rne(v[0]) | ((unsigned)f32_to_f16_rne(v[1]) << 16);
+              q.y = f32_to_f16_rne(v[2]) | ((unsigned)f32_to_f16_rne(v[3]) << 16);
+              q.z = f32_to_f16_rne(v[4]) | ((unsigned)f32_to_f16_rne(v[5]) << 16);
+              q.w = f32_to_f16_rne(v[6]) | ((unsigned)f32_to_f16_rne(v[7]) << 16);
+            }
+            *reinterpret_cast<uint4 *>(dst + cw * 2) = q;
           }
-        } else if (full && (FN % 4 == 0)) {
-#pragma unroll
-          for (int j = 0; j < FN; j += 4) {
-            uint2 v;
-            v.x = hv[j] | ((unsigned)hv[j + 1] << 16);
-            v.y = hv[j + 2] | ((unsigned)hv[j + 3] << 16);
-            *reinterpret_cast<uint2 *>(o + j) = v;
-          }
-        } else {
-#pragma unroll
-          for (int j = 0; j < FN; ++j)
-            if (nb + j < p.n) o[j] = hv[j];
         }
       }
     }
+    // read back row-major: lane -> (row = 8 t + lane / 8, 16-byte column piece lane % 8)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    const int piece = lane & 7;
+    const int col = raw ? (32 * pass + 4 * piece) : 8 * piece;   // first column of the piece inside the wave tile
+    const int n_first = n0 + wave_n * WTN + col;
+#pragma unroll
+    for (int t = 0; t < WTM / 8; ++t) {
+      const int row = 8 * t + (lane >> 3);
+      const int m = m0 + wave_m * WTM + row;
+      const uint4 q = *reinterpret_cast<const uint4 *>(stage + row * EP_PITCH + piece * 16);
+      if (m < g_end && n_first < p.n) {
+        unsigned char *o = reinterpret_cast<unsigned char *>(p.out) + ((long long)m * p.n + n_first) * esize;
+        *reinterpret_cast<uint4 *>(o) = q;
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
+  if (p.out_dtype == DT_I32) {
+    run_pass(std::true_type{}, std::integral_constant<int, 0>{});
+    if constexpr (FN > 1) run_pass(std::true_type{}, std::integral_constant<int, 1>{});
+    static_assert(FN <= 2, "int32 epilogue passes");
+  } else {
+    run_pass(std::false_type{}, std::integral_constant<int, 0>{});
   }
 }
 
 // ---- host launcher ---------------------------------------------------------------------------------
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK>
 static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
-  const size_t lds = 2 * (size_t)(BM + BN) * BK;
+  const size_t loop_lds = (size_t)NSTAGE * BM * BK + (size_t)(NK ? NSTAGE : KN_STAGES) * BN * BK;
+  const size_t epi_lds = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * 144;   // epilogue staging, 144-byte row pitch
+  const size_t lds = loop_lds > epi_lds ? loop_lds : epi_lds;
   auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK>;
   static bool attr_set = false;
   if (!attr_set) {
@@ -342,9 +434,9 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream
 
 const char *tile_cfg_name(int tile_cfg) {
   switch (tile_cfg) {
-    case TILE_256x256: return "256x256x128";
-    case TILE_128x128: return "128x128x128";
-    case TILE_64x128: return "64x128x128";
+    case TILE_256x256: return "256x256x64";
+    case TILE_128x128: return "128x128x64";
+    case TILE_64x128: return "64x128x64";
     default: return "?";
   }
 }
