@@ -11,7 +11,8 @@ import os
 from typing import Optional, Sequence
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libmsco_gmm.so")
+# MSCO_GMM_LIB selects another build of the backend library (used to compare kernel versions side by side)
+LIB_PATH = os.environ.get("MSCO_GMM_LIB") or os.path.join(_HERE, "lib", "libmsco_gmm.so")
 
 ABI_VERSION = 1
 

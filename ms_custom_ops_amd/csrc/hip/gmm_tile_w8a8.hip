@@ -26,7 +26,7 @@
 // LDS layouts (a fragment read is 16 B per lane over 32 consecutive rows, conflict free per 16 lanes):
 //   x rows and [N,K] weights: row-major, 64 B per row, 16-byte chunk c of row r stored at chunk
 //     position c ^ ((r >> 2) & 3);
-//   [K,N] weights: chunk-major, address = (c * BN + slot) * 16.
+//   [K,N] weights: 8 planes (one per 8 K rows) of BN slots x 8 bytes.
 #include "gmm_common.h"
 #include "gmm_kernels.h"
 
@@ -201,9 +201,16 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   };
 
   // ---- [K,N] weights: registers -> v_perm transpose -> LDS -----------------------------------
-  const int kn_i = tid % (BN / 4), kn_k8 = tid / (BN / 4);   // column group of 4, K block of 8 rows
+  // Thread (plane k8 = tid / (BN/4), i = tid % (BN/4)) loads 8 K rows x 4 columns (one dword per row),
+  // transposes them to 4 columns x 8 K bytes and writes 32 contiguous bytes into plane k8 of the LDS
+  // stage: plane k8 is an array of BN slots x 8 bytes, slot s = MFMA row feed position.  Its 4 columns
+  // are chosen so that they land in slots 4 i .. 4 i + 3: within a 32-column block, lane i % 8 takes the
+  // dword at column {0, 8, 4, 12, 16, 24, 20, 28}[i % 8] (all 8 dwords of the 32 bytes are covered, so
+  // the global loads stay fully coalesced).
+  const int kn_i = tid % (BN / 4), kn_k8 = tid / (BN / 4);
+  const int kn_col = 32 * (kn_i >> 3) + col_of_q(4 * (kn_i & 7));
   // columns past N and K rows past K are turned into out-of-range offsets (they read as zero)
-  const unsigned bkn_voff = (n0 + 4 * kn_i < p.n) ? (unsigned)(8 * kn_k8) * (unsigned)p.n + 4 * kn_i : OOB;
+  const unsigned bkn_voff = (n0 + kn_col < p.n) ? (unsigned)(8 * kn_k8) * (unsigned)p.n + kn_col : OOB;
   unsigned rkn[NK ? 1 : KN_RING][8];
   auto load_kn = [&](int kt, int slot) {
     if constexpr (!NK) {
@@ -215,18 +222,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   };
   auto store_kn = [&](int kt, int slot) {
     if constexpr (!NK) {
-      unsigned char *b = lds_b + (kt & (KN_STAGES - 1)) * B_STAGE;
+      unsigned char *b = lds_b + (kt & (KN_STAGES - 1)) * B_STAGE + kn_k8 * (BN * 8) + kn_i * 32;
       unsigned lo[4], hi[4];
       transpose4x4(rkn[slot][0], rkn[slot][1], rkn[slot][2], rkn[slot][3], lo[0], lo[1], lo[2], lo[3]);
       transpose4x4(rkn[slot][4], rkn[slot][5], rkn[slot][6], rkn[slot][7], hi[0], hi[1], hi[2], hi[3]);
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) {
-        const int nl = 4 * kn_i + jj;
-        const int slot_n = (nl & ~31) + q_of_col(nl & 31);
-        // chunk c = kn_k8 / 2 (16 K rows), half kn_k8 % 2 (8 K rows = 8 bytes)
-        *reinterpret_cast<uint2 *>(b + ((((kn_k8 >> 1) * BN + slot_n) << 4) | ((kn_k8 & 1) << 3))) =
-          make_uint2(lo[jj], hi[jj]);
-      }
+      *reinterpret_cast<uint4 *>(b) = make_uint4(lo[0], hi[0], lo[1], hi[1]);
+      *reinterpret_cast<uint4 *>(b + 16) = make_uint4(lo[2], hi[2], lo[3], hi[3]);
     }
   };
 
@@ -243,8 +244,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
       const unsigned char *b = lds_b + (kt & (NSTAGE - 1)) * B_STAGE;
       return *reinterpret_cast<const v4i *>(b + rho * BK + (((2 * kk + hh) ^ swz64(rho)) << 4));
     } else {
-      const unsigned char *b = lds_b + (kt & (KN_STAGES - 1)) * B_STAGE;
-      return *reinterpret_cast<const v4i *>(b + (((2 * kk + hh) * BN + rho) << 4));
+      // 16 K bytes of chunk c = 2 kk + hh: planes 2 c and 2 c + 1, 8 bytes each
+      const unsigned char *b = lds_b + (kt & (KN_STAGES - 1)) * B_STAGE + (2 * (2 * kk + hh)) * (BN * 8) + rho * 8;
+      const uint2 lo = *reinterpret_cast<const uint2 *>(b);
+      const uint2 hi = *reinterpret_cast<const uint2 *>(b + BN * 8);
+      return v4i{(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
     }
   };
 
