@@ -17,7 +17,7 @@ enum : int { DT_NONE = 0, DT_I8 = 1, DT_I32 = 2, DT_I64 = 3, DT_U64 = 4, DT_F16 
 
 constexpr int kNumXcd = 8;        // MI355X: 8 accelerator complex dies, workgroups are dealt round-robin
 constexpr int kSkinnyRows = 16;   // rows one MFMA covers in the skinny kernels
-constexpr int kSkinnyCols = 128;  // output columns one skinny workgroup owns
+constexpr int kSkinnyCols = 256;  // output columns one skinny workgroup owns
 
 // Kernel argument block.  Plain pointers and sizes only.
 struct GmmParams {
@@ -42,6 +42,7 @@ struct GmmParams {
   int x_dtype;              // DT_I8 / DT_BF16 / DT_F16
   int split_k;              // number of K splits across workgroups (skinny kernels)
   int n_strips;             // ceil(N / kSkinnyCols)
+  int max_chunks;           // ceil(M / kSkinnyRows): 16-row chunks a group can have (skinny W8A8 kernel)
 };
 
 // ---- group_list --------------------------------------------------------------------------------
@@ -122,6 +123,15 @@ __device__ __forceinline__ void store_out(const GmmParams &p, long long idx, int
   } else {
     reinterpret_cast<int *>(p.out)[idx] = acc_plus_bias;
   }
+}
+
+// ---- buffer descriptors ---------------------------------------------------------------------------
+// Raw buffer over [base, base + bytes): loads whose *vector* offset is at or beyond `bytes` return 0
+// (the scalar offset is not range-checked), so tails are masked by setting bit 31 of the vector offset.
+constexpr unsigned kBufferOob = 0x80000000u;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_over(const void *base, long long bytes) {
+  const unsigned n = bytes > 0x7FFFFFFFll ? 0x7FFFFFFFu : (unsigned)(bytes < 0 ? 0 : bytes);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
 }
 
 // ---- byte shuffles -----------------------------------------------------------------------------

@@ -16,10 +16,12 @@ void tile_cfg_dims(int tile_cfg, int *bm, int *bn);
 
 // Skinny (decode) kernels: one workgroup streams a 128-column weight strip of one group over a K
 // range; waves split K and reduce through LDS, workgroups split K and reduce through the workspace.
-hipError_t launch_skinny_w8a8(const GmmParams &p, bool nk, hipStream_t stream);
+// wide16: the 16-wave / 128-column-strip variant for small weight sets, else 4 waves / 256-column strips
+hipError_t launch_skinny_w8a8(const GmmParams &p, bool nk, bool wide16, hipStream_t stream);
 hipError_t launch_skinny_a16w8(const GmmParams &p, hipStream_t stream);
-size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t e, int split_k, bool fp32_partials);
-size_t skinny_counter_count(int64_t n, int64_t e);
+size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t e, int split_k, int cols);
+size_t skinny_counter_count(int64_t m, int64_t n, int64_t e, int cols);
+size_t a16w8_workspace_bytes(int64_t m, int64_t n, int64_t e, int split_k);
 
 // Shape-agnostic fallback kernels (one output element per thread), any K / N.
 hipError_t launch_generic_w8a8(const GmmParams &p, bool nk, hipStream_t stream);

@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -23,7 +24,9 @@ enum Family : int { FAM_NONE = 0, FAM_TILE = 1, FAM_SKINNY = 2, FAM_GENERIC = 3 
 enum Override : int { OV_AUTO = 0, OV_TILE_256 = 1, OV_TILE_128 = 2, OV_TILE_64 = 3, OV_SKINNY = 4, OV_GENERIC = 5 };
 
 constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned
-constexpr int kTargetWorkgroups = 1024;  // skinny kernels: aim for this many workgroups (4 per CU)
+constexpr int kTargetWorkgroups = 512;  // skinny kernels with a K split: aim for this many workgroups (2 per CU)
+constexpr int kMaxSplitK = 8;             // keeps the last arriver's reduction to two rounds of loads
+constexpr int kNumCUs = 256;
 
 int env_int(const char *name, int fallback) {
   const char *v = std::getenv(name);
@@ -39,6 +42,9 @@ struct msco_gmm_op {
   int family = FAM_NONE;
   int tile_cfg = 0;
   int split_k = 1;
+  int max_chunks = 1;
+  int skinny_wide16 = 0;
+  int skinny_cols = kSkinnyCols;
   int n_strips = 0;
   size_t workspace_bytes = 0;
   unsigned *counters = nullptr;
@@ -92,6 +98,9 @@ void choose_plan(msco_gmm_op *op) {
   const int64_t m = op->m, k = op->k, n = op->n, e = op->e;
   const bool aligned = (k % 16 == 0) && (n % 16 == 0) && k >= 16 && n >= 16;
   op->split_k = 1;
+  op->max_chunks = 1;
+  op->skinny_wide16 = 0;
+  op->skinny_cols = kSkinnyCols;
   op->n_strips = (int)((n + kSkinnyCols - 1) / kSkinnyCols);
   op->workspace_bytes = 0;
   op->tile_cfg = TILE_256x256;
@@ -126,37 +135,61 @@ void choose_plan(msco_gmm_op *op) {
     case OV_GENERIC: family = FAM_GENERIC; break;
     default: break;
   }
-  if ((family == FAM_TILE || family == FAM_SKINNY) && !aligned) family = FAM_GENERIC;
+  // the MFMA kernels address x and one group's weights through 32-bit buffer offsets
+  const bool fits32 = k * n < ((int64_t)1 << 31) && m * k < ((int64_t)1 << 31);
+  if ((family == FAM_TILE || family == FAM_SKINNY) && !(aligned && fits32)) family = FAM_GENERIC;
   if (family == FAM_TILE && !is_w8a8(d)) family = FAM_SKINNY;
   if (family == FAM_TILE) {
     const int forced = env_int("MSCO_TILE_CFG", -1);
     if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO) op->tile_cfg = forced;
   }
   if (family == FAM_SKINNY) {
-    // Cross-workgroup K split only when every group is guaranteed to fit one 16-row chunk.
-    if (m <= kSkinnyRows) {
-      const int64_t base = (int64_t)op->n_strips * e;
-      const int k_blocks = (int)((k + 63) / 64);
-      int want = pow2_at_least((int)((kTargetWorkgroups + base - 1) / base));
-      int cap = k_blocks / 4;  // every wave of a workgroup keeps at least one 64-row block
-      if (cap < 1) cap = 1;
-      while (want > cap) want >>= 1;
-      if (want < 1) want = 1;
-      const int forced = env_int("MSCO_SKINNY_SPLIT_K", 0);
-      if (forced > 0) want = forced;
-      op->split_k = want;
+    // grid.y enumerates (group, 16-row chunk)
+    op->max_chunks = (int)((m + kSkinnyRows - 1) / kSkinnyRows);
+    if (op->max_chunks < 1) op->max_chunks = 1;
+    if (e * op->max_chunks > 65535) family = FAM_GENERIC;
+  }
+  if (family == FAM_SKINNY) {
+    // Only shapes enter: the number of (group, chunk) pairs that can hold rows is estimated from M and E.
+    const int64_t active = std::max<int64_t>(
+      1, std::min<int64_t>(e * op->max_chunks, std::min<int64_t>(m, e) + m / kSkinnyRows));
+    const int64_t tiles128 = ((n + 127) / 128) * active;
+    int wide16 = is_w8a8(d) && tiles128 <= kNumCUs;
+    const int forced_variant = env_int("MSCO_SKINNY_WIDE16", -1);
+    if (forced_variant >= 0 && is_w8a8(d)) wide16 = forced_variant != 0;
+    op->skinny_wide16 = wide16;
+    int want, cap;
+    if (wide16) {
+      // at most one 16-wave workgroup per CU, every wave keeps at least one block
+      want = (int)(kNumCUs / std::max<int64_t>(tiles128, 1));
+      cap = std::max<int>(1, (int)(d.transpose_b ? (k + 63) / 64 : (k + 31) / 32) / 16);
+      want = std::min(want, 8);
+    } else {
+      // K is split across workgroups until about kTargetWorkgroups of them stream weights
+      const int64_t base = (int64_t)op->n_strips * active;
+      const int target = env_int("MSCO_SKINNY_TARGET_WGS", kTargetWorkgroups);
+      want = (int)((target + base / 2) / base);
+      cap = std::max<int>(1, (int)(d.transpose_b ? (k + 63) / 64 : (k + 31) / 32) / 4);
+      want = std::min(want, kMaxSplitK);
     }
-    op->workspace_bytes = skinny_workspace_bytes(m, n, e, op->split_k, is_a16w8(d));
+    want = std::max(1, std::min(want, cap));
+    const int forced = env_int("MSCO_SKINNY_SPLIT_K", 0);
+    if (forced > 0) want = std::min(forced, cap);
+    op->split_k = want;
+    op->skinny_cols = wide16 ? 128 : kSkinnyCols;
+    op->workspace_bytes = is_w8a8(d) ? skinny_workspace_bytes(m, n, e, op->split_k, op->skinny_cols)
+                                     : a16w8_workspace_bytes(m, n, e, op->split_k);
   }
   op->family = family;
 
   char buf[320];
   const char *fam = family == FAM_TILE ? "tile" : family == FAM_SKINNY ? "skinny" : "generic";
   std::snprintf(buf, sizeof(buf),
-                "msco_gmm plan: kernel=%s%s%s layout=%s m=%lld k=%lld n=%lld e=%lld split_k=%d strips=%d "
+                "msco_gmm plan: kernel=%s%s%s%s layout=%s m=%lld k=%lld n=%lld e=%lld split_k=%d strips=%d "
                 "workspace=%zu",
                 is_w8a8(d) ? "w8a8_" : "a16w8_", fam,
                 family == FAM_TILE ? (std::string("_") + tile_cfg_name(op->tile_cfg)).c_str() : "",
+                (family == FAM_SKINNY && op->skinny_wide16) ? "_16w" : "",
                 d.transpose_b ? "[E,N,K]" : "[E,K,N]", (long long)m, (long long)k, (long long)n, (long long)e,
                 op->split_k, op->n_strips, op->workspace_bytes);
   op->info = buf;
@@ -201,7 +234,7 @@ int msco_gmm_plan(msco_gmm_handle h, int64_t m, int64_t k, int64_t n, int64_t e,
   h->m = m; h->k = k; h->n = n; h->e = e;
   choose_plan(h);
   if (h->family == FAM_SKINNY && h->split_k > 1) {
-    const size_t need = skinny_counter_count(n, e);
+    const size_t need = skinny_counter_count(m, n, e, h->skinny_cols);
     if (need > h->counters_cap) {
       if (h->counters) (void)hipFree(h->counters);
       h->counters = nullptr;
@@ -272,13 +305,14 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   p.x_dtype = d.x_dtype;
   p.split_k = h->split_k;
   p.n_strips = h->n_strips;
+  p.max_chunks = h->max_chunks;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t err = hipSuccess;
   const bool nk = d.transpose_b != 0;
   if (is_w8a8(d)) {
     if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, s);
-    else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, s);
+    else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
     else err = launch_generic_w8a8(p, nk, s);
   } else {
     if (h->family == FAM_SKINNY) err = launch_skinny_a16w8(p, s);

@@ -73,7 +73,9 @@ def test_unaligned_shapes_take_the_generic_kernel(device, transpose_b):
 def test_decode_shapes_use_split_k_and_stay_exact(device, m, e, gl, transpose_b):
     rng, x, w, bias, scale, pt = _inputs(4, m, 4096, 1024, e)
     info = _check(x, w, gl, bias, scale, pt, transpose_b=transpose_b, override=cabi.OV_AUTO)
-    assert "skinny" in info and "split_k=1 " not in info
+    # either the K reduction is split across workgroups, or there are enough strips x groups for the
+    # 16-wave workgroups that keep it inside one workgroup
+    assert "skinny" in info and ("split_k=1 " not in info or "16w64c" in info)
 
 
 def test_counts_and_last_boundary_below_m(device):
