@@ -65,6 +65,31 @@ __device__ __forceinline__ void buffer_load_lds_b128(__amdgpu_buffer_rsrc_t rsrc
 #endif
 }
 
+// Two 8-byte LDS reads `stride` bytes apart, invisible to the compiler's wait-count bookkeeping.
+// They must be issued before any compiler-visible LDS read whose result is consumed later (LDS
+// operations complete in order), and lds_reads_done() must precede the first use of the results.
+__device__ __forceinline__ void lds_read_b64_pair(const unsigned char *p, int stride, uint2 &lo, uint2 &hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const unsigned a = (unsigned)(unsigned long)(const __attribute__((address_space(3))) unsigned char *)p;
+  asm volatile("ds_read_b64 %0, %1" : "=v"(lo) : "v"(a));
+  asm volatile("ds_read_b64 %0, %1" : "=v"(hi) : "v"(a + (unsigned)stride));
+#else
+  (void)p; (void)stride; lo = hi = uint2{0, 0};
+#endif
+}
+__device__ __forceinline__ void lds_write_b128(unsigned char *p, msco::v4i v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const unsigned a = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char *)p;
+  asm volatile("ds_write_b128 %0, %1" ::"v"(a), "v"(v) : "memory");
+#else
+  (void)p; (void)v;
+#endif
+}
+template <typename T>
+__device__ __forceinline__ void lds_reads_done(T &frags) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(frags));
+}
+
 // LDS-only barrier: waits for this wave's LDS traffic, not for global loads still in flight.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -149,7 +174,6 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   const int m0 = g_start + mt * BM;
   const int n0 = nt * BN;
   const int k_slabs = (p.k + BK - 1) / BK;
-  const bool k_tail = (p.k % BK) != 0;
 
   // Buffer descriptors start at this tile's first x row / weight column, so per-lane offsets stay
   // small; anything past the end of the tensor reads as zero (no clamping, no branches in the loop).
@@ -185,7 +209,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   auto issue_direct = [&](int kt) {
     const int stage = kt & (NSTAGE - 1);
     const unsigned kbase = kt * BK;
-    const unsigned kill = (k_tail && kbase + d_c * 16 >= (unsigned)p.k) ? OOB : 0u;
+    // K tail, and whole slabs past K (requested by the last steps of the branch-free loop): read as zero
+    const unsigned kill = (kbase + d_c * 16 >= (unsigned)p.k) ? OOB : 0u;
 #pragma unroll
     for (int u = 0; u < A_LD; ++u) {
       const int blk = wave * A_LD + u;
@@ -214,7 +239,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   unsigned rkn[NK ? 1 : KN_RING][8];
   auto load_kn = [&](int kt, int slot) {
     if constexpr (!NK) {
-      const unsigned voff = (k_tail && kt * BK + 8 * kn_k8 >= p.k) ? OOB : bkn_voff;
+      const unsigned voff = (kt * BK + 8 * kn_k8 >= p.k) ? OOB : bkn_voff;
 #pragma unroll
       for (int r = 0; r < 8; ++r)
         rkn[slot][r] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff, (kt * BK + r) * p.n, 0);
@@ -222,12 +247,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   };
   auto store_kn = [&](int kt, int slot) {
     if constexpr (!NK) {
-      unsigned char *b = lds_b + (kt & (KN_STAGES - 1)) * B_STAGE + kn_k8 * (BN * 8) + kn_i * 32;
+      unsigned char *b = lds_b + (kt % KN_STAGES) * B_STAGE + kn_k8 * (BN * 8) + kn_i * 32;
       unsigned lo[4], hi[4];
       transpose4x4(rkn[slot][0], rkn[slot][1], rkn[slot][2], rkn[slot][3], lo[0], lo[1], lo[2], lo[3]);
       transpose4x4(rkn[slot][4], rkn[slot][5], rkn[slot][6], rkn[slot][7], hi[0], hi[1], hi[2], hi[3]);
-      *reinterpret_cast<uint4 *>(b) = make_uint4(lo[0], hi[0], lo[1], hi[1]);
-      *reinterpret_cast<uint4 *>(b + 16) = make_uint4(lo[2], hi[2], lo[3], hi[3]);
+      // hand-written stores for the same reason as the reads of this region (see read_w); the
+      // LDS-only barrier that follows waits for them
+      lds_write_b128(b, v4i{(int)lo[0], (int)hi[0], (int)lo[1], (int)hi[1]});
+      lds_write_b128(b + 16, v4i{(int)lo[2], (int)hi[2], (int)lo[3], (int)hi[3]});
     }
   };
 
@@ -244,10 +271,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
       const unsigned char *b = lds_b + (kt & (NSTAGE - 1)) * B_STAGE;
       return *reinterpret_cast<const v4i *>(b + rho * BK + (((2 * kk + hh) ^ swz64(rho)) << 4));
     } else {
-      // 16 K bytes of chunk c = 2 kk + hh: planes 2 c and 2 c + 1, 8 bytes each
-      const unsigned char *b = lds_b + (kt & (KN_STAGES - 1)) * B_STAGE + (2 * (2 * kk + hh)) * (BN * 8) + rho * 8;
-      const uint2 lo = *reinterpret_cast<const uint2 *>(b);
-      const uint2 hi = *reinterpret_cast<const uint2 *>(b + BN * 8);
+      // 16 K bytes of chunk c = 2 kk + hh: planes 2 c and 2 c + 1, 8 bytes each.  Read with
+      // hand-written ds_read_b64: the compiler makes every LDS read it knows about wait for all
+      // LDS-direct loads in flight unless it can tell them apart, and it cannot for this region
+      // (which those loads never write) -- that wait would serialise the whole operand pipeline.
+      // The caller orders these reads before its own and waits for them (read_w_done).
+      const unsigned char *b = lds_b + (kt % KN_STAGES) * B_STAGE + (2 * (2 * kk + hh)) * (BN * 8) + rho * 8;
+      uint2 lo, hi;
+      lds_read_b64_pair(b, BN * 8, lo, hi);
       return v4i{(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
     }
   };
@@ -262,21 +293,55 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
 
   // ---- main loop ---------------------------------------------------------------------------------
   // Slabs t+1 .. t+3 are in flight (LDS ring for the directly loaded operands, register ring for
-  // [K,N] weights) while slab t is multiplied.  One LDS-only barrier per slab publishes slab t+1 and
-  // retires the stage that slab t+3's loads are about to overwrite.
+  // [K,N] weights) while slab t is multiplied.
+  //
+  // [N,K] weights with 8 waves: every SIMD hosts two waves, one from each half of the workgroup, and
+  // the halves run half a step apart.  While one half issues its 16 MFMAs for slab t, the other half
+  // does the memory side of its own step (requests slab t+3, reads its 12 operand fragments from
+  // LDS).  Two workgroup barriers per step keep the halves in opposite phases, so the matrix pipe and
+  // the LDS / memory pipes are busy at the same time instead of taking turns.  The half that runs
+  // behind enters the loop through one extra barrier and the half that runs ahead leaves it through
+  // one, so all waves execute the same number.  [K,N] weights keep all waves in one phase with one
+  // barrier per slab: their register-staged weight loads stall now and then, and in the two-phase
+  // scheme such a stall stops both halves (measured slower).
+  constexpr bool PINGPONG = (NW == 8) && NK;
+  const bool behind = PINGPONG && wave >= NW / 2;
+  auto phase_barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // The loop body is branch free: the last steps still request "slabs" t+3 past K, whose offsets are
+  // all out of range, so nothing is read and zeros land in a stage nobody reads.  Every path through
+  // the loop then issues the same number of loads, which keeps the vmcnt waits exact -- with
+  // conditional requests the compiler has to assume the shortest path and waits for the loads it has
+  // just issued.
   auto step = [&](int kt, auto ring_slot) {
     constexpr int SLOT = decltype(ring_slot)::value;          // == kt % KN_RING, compile-time for register indexing
-    if (kt + 3 < k_slabs) {
-      issue_direct(kt + 3);
-      load_kn(kt + 3, SLOT);                                  // (kt + 3) % 3 == kt % 3: that slot was emptied last step
-    }
+    issue_direct(kt + 3);
+    load_kn(kt + 3, SLOT);                                    // (kt + 3) % 3 == kt % 3: that slot was emptied last step
     v4i xf[2][FM], wf[2][FN];
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-#pragma unroll
-      for (int i = 0; i < FM; ++i) xf[kk][i] = read_x(kt, i, kk);
+    for (int kk = 0; kk < 2; ++kk)
 #pragma unroll
       for (int f = 0; f < FN; ++f) wf[kk][f] = read_w(kt, f, kk);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+      for (int i = 0; i < FM; ++i) xf[kk][i] = read_x(kt, i, kk);
+    if constexpr (!NK) {
+      // hand-issued weight reads: older than every x read, so one wait covers them
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int f = 0; f < FN; ++f) lds_reads_done(wf[kk][f]);
+    }
+    if constexpr (PINGPONG) {
+      wait_vmcnt<2 * VM_PER_SLAB>();                          // this wave's part of slab t+1 has landed
+      __builtin_amdgcn_sched_barrier(0);
+      lds_barrier();                                          // fragments are in registers, slab t+1 is published
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_setprio(2);
     }
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk)
@@ -285,32 +350,42 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
 #pragma unroll
         for (int i = 0; i < FM; ++i)
           acc[f][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[kk][f], xf[kk][i], acc[f][i], 0, 0, 0);
-    if (kt + 1 < k_slabs) {
+    if constexpr (PINGPONG) {
+      __builtin_amdgcn_s_setprio(0);
+      phase_barrier();
+    } else {
       store_kn(kt + 1, (SLOT + 1) % KN_RING);                 // its LDS stage held slab t-1, read before the last barrier
-      // this wave's loads of slab t+1 have landed once at most the loads of slabs t+2, t+3 are outstanding
-      if (kt + 3 < k_slabs) wait_vmcnt<2 * VM_PER_SLAB>();
-      else if (kt + 2 < k_slabs) wait_vmcnt<VM_PER_SLAB>();
-      else wait_vmcnt<0>();
+      wait_vmcnt<2 * VM_PER_SLAB>();                          // only the loads of slabs t+2, t+3 may be outstanding
+      lds_barrier();
     }
-    lds_barrier();
   };
 
   // prologue: slabs 0, 1, 2 requested; slab 0 published
-  issue_direct(0);
-  load_kn(0, 0);
-  if (k_slabs > 1) { issue_direct(1); load_kn(1, 1); }
-  if (k_slabs > 2) { issue_direct(2); load_kn(2, 2); }
+  issue_direct(0); load_kn(0, 0);
+  issue_direct(1); load_kn(1, 1);
+  issue_direct(2); load_kn(2, 2);
   store_kn(0, 0);
-  if (k_slabs > 2) wait_vmcnt<2 * VM_PER_SLAB>();
-  else if (k_slabs > 1) wait_vmcnt<VM_PER_SLAB>();
-  else wait_vmcnt<0>();
+  wait_vmcnt<2 * VM_PER_SLAB>();
   lds_barrier();
+  if (behind) phase_barrier();
 
-  for (int kt = 0; kt < k_slabs; kt += KN_RING) {
-    step(kt, std::integral_constant<int, 0>{});
+  if constexpr (NK) {
+    for (int kt = 0; kt < k_slabs; ++kt) step(kt, std::integral_constant<int, 0>{});
+  } else {
+    // unrolled by the register ring so that ring slots are compile-time register names
+    int kt = 0;
+    for (; kt + KN_RING <= k_slabs; kt += KN_RING) {
+      step(kt, std::integral_constant<int, 0>{});
+      step(kt + 1, std::integral_constant<int, 1>{});
+      step(kt + 2, std::integral_constant<int, 2>{});
+    }
+    if (kt < k_slabs) step(kt, std::integral_constant<int, 0>{});
     if (kt + 1 < k_slabs) step(kt + 1, std::integral_constant<int, 1>{});
-    if (kt + 2 < k_slabs) step(kt + 2, std::integral_constant<int, 2>{});
   }
+  if (PINGPONG && !behind) phase_barrier();
+  // the epilogue reuses the operand ring: every wave is done reading it and the late zero fills have landed
+  wait_vmcnt<0>();
+  lds_barrier();
 
   // ---- fused dequant epilogue --------------------------------------------------------------------
   // acc[f][i][r] is output row 32 i + l32 and column 32 f + 16 (r / 8) + 8 hh + (r % 8) of the wave tile:
