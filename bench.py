@@ -2,6 +2,7 @@
 """Benchmark of the grouped W8A8 matmul path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout kn|nk] [--no-sweep] [--no-cpu]
+    python bench.py --probe c3|c2_m16|...|copy [--layout kn|nk] [--steps K]     (for rocprofv3 counter runs)
 
 A step is one pass of the hot path over one batch of synthetic input (inputs resident in HBM before
 the timed region).  The headline workload is the Mixtral-shaped MoE configuration (E=8, top-2 over
@@ -11,6 +12,8 @@ Prints ONE JSON line.  Besides the contract keys it carries
   cpu_baseline  the numpy restatement of the reference golden timed on this box's host cores,
   sweep         the other configurations (dense decode / prefill sweep, skewed MoE, weight-only
                 decode) as TOPS and GB/s with their roofline fractions.
+--probe runs a few untimed launches of one workload (or, for `copy`, of a plain device-to-device copy
+of COPY_BYTES bytes, the reference a counter reading is scaled by) so that a profiler sees nothing else.
 """
 import argparse
 import json
@@ -26,17 +29,21 @@ sys.path.insert(0, REPO)
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 ROTATE_BYTES = 768e6      # HBM-bound cases rotate over weight copies totalling more than the 256 MB Infinity Cache
+COPY_BYTES = 1 << 29      # --probe copy: one launch reads and writes this many bytes
+TRAFFIC_FILE = os.path.join(REPO, "ms_custom_ops_amd", "measured_traffic.json")
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=40,
+                    help="untimed steps; the GPU clock needs a few tens of launches to settle")
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--layout", default="kn", choices=["kn", "nk"], help="weight storage: kn=[E,K,N], nk=[E,N,K]")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--probe", default=None, help="workload name or `copy`: untimed launches only, for counter collection")
     return ap.parse_args()
 
 
@@ -139,6 +146,38 @@ def cpu_baseline(wl, budget_s=15.0):
                       "numpy float32 dot per group + dequant epilogue + bf16 cast"}
 
 
+def measured_traffic(workload, layout, kernel):
+    """HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs (scaled by
+    the same counters' reading for a copy of known size); None when no measurement of this kernel is on file."""
+    try:
+        table = json.load(open(TRAFFIC_FILE))
+    except OSError:
+        return None
+    entry = table.get(f"{workload}/{layout}")
+    if not entry or entry.get("kernel") != kernel:
+        return None
+    return entry["hbm_bytes_per_launch"]
+
+
+def probe(args):
+    import torch
+    from ms_custom_ops_amd import workloads
+    if args.probe == "copy":
+        src = torch.randint(-127, 128, (COPY_BYTES,), dtype=torch.int8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "copy", "bytes_read": COPY_BYTES, "bytes_written": COPY_BYTES, "launches": args.steps}))
+        return
+    wl = workloads.make(args.probe)
+    prob = DeviceProblem(wl, args.layout)
+    for _ in range(args.steps):
+        prob.step()
+    torch.cuda.synchronize()
+    print(json.dumps({"probe": args.probe, "plan": prob.op.plan_info(), "launches": args.steps}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -152,6 +191,9 @@ def main():
         print("bench.py needs a GPU (the operators have no CPU path)", file=sys.stderr)
         sys.exit(1)
 
+    if args.probe:
+        probe(args)
+        return
     wl = workloads.make(args.workload)
     prob = DeviceProblem(wl, args.layout)
     wall, per_launch = prob.time(args.steps, args.warmup)
@@ -169,6 +211,7 @@ def main():
         roof = {"bound": "hbm", "achieved": gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                 "traffic": None}
     roof["kernel"] = plan.split("kernel=")[1].split(" ")[0]
+    roof["traffic"] = measured_traffic(wl.name, args.layout, roof["kernel"])
     roof["launch_us"] = per_launch * 1e6
     roof["ops_per_launch"] = work["ops"]
     roof["bytes_per_launch"] = work["bytes"]
@@ -197,7 +240,7 @@ def main():
             hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5")
             copies = max(1, int(np.ceil(ROTATE_BYTES / w_bytes))) if hbm_bound_guess else 1
             p2 = DeviceProblem(w2, layout, copies)
-            _, sec = p2.time(max(20, min(200, args.steps * 2)), args.warmup)
+            _, sec = p2.time(max(20, min(200, args.steps)), args.warmup)
             wk, tops, gbs = rates(w2, sec)
             sweep.append({"workload": name, "layout": layout, "launch_us": sec * 1e6, "tops": tops,
                           "int8_frac": tops / PEAK_INT8_TOPS, "gbs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS,
