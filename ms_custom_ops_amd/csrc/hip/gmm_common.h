@@ -63,6 +63,60 @@ __device__ __forceinline__ int group_end(const GmmParams &p, int g, int prev) {
   return (int)end;
 }
 
+// ---- wave-parallel walk of group_list (tile scheduler) --------------------------------------------
+// Row ends of up to 64 groups at once: lane l handles group g0 + l.  The sequential rule of
+// group_end() has closed forms, so a wave computes it with prefix scans instead of E dependent loads:
+//   cumulative ends: end_g = min(max(carry, v_0..v_g), M)            (prefix maximum)
+//   counts:          end_g = min(carry + max(v_0,0) + .. + max(v_g,0), M)   (saturating prefix sum)
+__device__ __forceinline__ int wave_scan_max(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int t = __shfl_up(v, d);
+    if (lane >= d) v = max(v, t);
+  }
+  return v;
+}
+__device__ __forceinline__ int wave_scan_add_sat(int v, int lane, int cap) {   // operands in [0, cap], cap < 2^30
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int t = __shfl_up(v, d);
+    if (lane >= d) v = min(v + t, cap);
+  }
+  return v;
+}
+__device__ __forceinline__ int wave_scan_add(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int t = __shfl_up(v, d);
+    if (lane >= d) v += t;
+  }
+  return v;
+}
+__device__ __forceinline__ int wave_bcast(int v, int src_lane) {
+  return __builtin_amdgcn_readfirstlane(__shfl(v, src_lane));
+}
+
+// Lane l receives [start, end) of group g0 + l (empty for lanes past E); `carry` is the row end of
+// group g0 - 1 on entry and of the chunk's last group on exit.  Requires M < 2^30 for counts.
+__device__ __forceinline__ void group_rows_chunk(const GmmParams &p, int g0, int lane, int &carry, int &start, int &end) {
+  const int g = g0 + lane;
+  const bool valid = g < p.e;
+  long long v = 0;
+  if (valid) {
+    if (p.gl_dtype == DT_I64) v = reinterpret_cast<const long long *>(p.group_list)[g];
+    else if (p.gl_dtype == DT_I32) v = reinterpret_cast<const int *>(p.group_list)[g];
+    else v = (long long)(p.m / p.e) * (g + 1);
+  }
+  const int c = (int)(v < 0 ? 0 : (v > p.m ? p.m : v));   // clamping the operands first changes neither closed form
+  int e_l;
+  if (p.gl_type == 1 && p.gl_dtype != DT_NONE) e_l = min(carry + wave_scan_add_sat(valid ? c : 0, lane, p.m), p.m);
+  else e_l = max(carry, wave_scan_max(valid ? c : 0, lane));
+  const int prev = __shfl_up(e_l, 1);
+  start = lane == 0 ? carry : prev;
+  end = e_l;
+  carry = wave_bcast(e_l, 63);
+}
+
 // ---- number formats ----------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
 

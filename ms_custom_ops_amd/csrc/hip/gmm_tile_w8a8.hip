@@ -131,16 +131,16 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int l32 = lane & 31, hh = lane >> 5;
 
-  // ---- tile lookup: walk group_list twice (count, then locate) -------------------------------
+  // ---- tile lookup: two wave-parallel passes over group_list (count, then locate) -------------
+  // 64 groups per step with prefix scans, so the cost does not grow with the number of experts;
+  // every wave does the same work, no LDS or barrier is involved.
   const int n_tiles = (p.n + BN - 1) / BN;
   int total = 0;
-  {
-    int prev = 0;
-    for (int g = 0; g < p.e; ++g) {
-      const int end = group_end(p, g, prev);
-      total += ((end - prev + BM - 1) / BM) * n_tiles;
-      prev = end;
-    }
+  for (int g0 = 0, carry = 0; g0 < p.e; g0 += 64) {
+    int s0, e0;
+    group_rows_chunk(p, g0, lane, carry, s0, e0);
+    const int t = wave_scan_add(((e0 - s0 + BM - 1) / BM) * n_tiles, lane);
+    total += wave_bcast(t, 63);
   }
   const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
   const int local = blockIdx.x / kNumXcd;
@@ -149,18 +149,20 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   if (lid >= total) return;
 
   int grp = 0, g_start = 0, g_end = 0, t_in_group = 0;
-  {
-    int prev = 0, acc = 0;
-    for (int g = 0; g < p.e; ++g) {
-      const int end = group_end(p, g, prev);
-      const int tiles = ((end - prev + BM - 1) / BM) * n_tiles;
-      if (lid < acc + tiles) {
-        grp = g; g_start = prev; g_end = end; t_in_group = lid - acc;
-        break;
-      }
-      acc += tiles;
-      prev = end;
+  for (int g0 = 0, carry = 0, tiles_before = 0; g0 < p.e; g0 += 64) {
+    int s0, e0;
+    group_rows_chunk(p, g0, lane, carry, s0, e0);
+    const int tiles = ((e0 - s0 + BM - 1) / BM) * n_tiles;
+    const int upto = tiles_before + wave_scan_add(tiles, lane);      // tiles of groups 0 .. g0 + lane
+    const int first = __popcll(__ballot(upto <= lid));              // `upto` is non-decreasing: first lane beyond lid
+    if (first < 64) {
+      grp = g0 + first;
+      g_start = wave_bcast(s0, first);
+      g_end = wave_bcast(e0, first);
+      t_in_group = lid - (wave_bcast(upto, first) - wave_bcast(tiles, first));
+      break;
     }
+    tiles_before = wave_bcast(upto, 63);
   }
   // order inside a group: panel of PANEL m-tiles, then n-tile, then m-tile inside the panel
   const int m_tiles = (g_end - g_start + BM - 1) / BM;
