@@ -7,7 +7,7 @@
 
 namespace msco {
 
-enum TileCfg : int { TILE_256x256 = 0, TILE_128x128 = 1, TILE_64x128 = 2, TILE_CFG_COUNT = 3 };
+enum TileCfg : int { TILE_256x256 = 0, TILE_128x128 = 1, TILE_64x128 = 2, TILE_128x256 = 3, TILE_CFG_COUNT = 4 };
 
 // MFMA tile kernel for W8A8 (prefill shapes).  nk: weights stored [E,N,K].
 hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream_t stream);

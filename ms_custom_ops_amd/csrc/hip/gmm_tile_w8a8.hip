@@ -35,7 +35,6 @@
 namespace msco {
 
 constexpr int BK = 64;        // bytes of K per slab = one MFMA K step
-constexpr int NSTAGE = 4;     // LDS ring depth of operands that are loaded straight into LDS
 constexpr int KN_STAGES = 2;  // LDS stages of the transposed [K,N] weight slab
 constexpr int KN_RING = 3;    // [K,N] weight slabs in flight in registers
 
@@ -104,8 +103,12 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK>
-__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(const GmmParams p) {
+// STAGES = depth of the LDS ring of the operands that are loaded straight into LDS (STAGES - 1 slabs in flight)
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES>
+__global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel(const GmmParams p) {
+  constexpr int NSTAGE = STAGES;
+  constexpr int AHEAD = STAGES - 1;                 // slabs requested ahead of the one being multiplied
+  static_assert(NK || STAGES == 4, "the [K,N] register ring is three slabs deep");
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int NT = NW * 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -117,10 +120,15 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   constexpr unsigned OOB = 0x80000000u;             // buffer offset that always reads zero
   constexpr int VM_PER_SLAB = A_LD + (NK ? B_LD : 8);   // vector-memory loads a wave issues per slab
   // [K,N] weight slab: 8 K-chunks of 8 rows x BN/4 column groups -> one 8(k) x 4(n)-byte block per thread
-  static_assert(NT == 2 * BN, "one [K,N] block per thread");
+  static_assert(NK || NT == 2 * BN, "one [K,N] block per thread");
   static_assert(FM >= 1 && FN >= 1 && A_LD >= 1 && B_LD >= 1, "tile shape");
   static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "row blocks per wave");
 
+  // LDS: operand ring, reused by the epilogue staging; behind both, the tile's epilogue operands
+  constexpr int LOOP_LDS = NSTAGE * A_STAGE + (NK ? NSTAGE : KN_STAGES) * B_STAGE;
+  constexpr int EPI_LDS = NW * WTM * 144;
+  constexpr int PARAM_OFF = LOOP_LDS > EPI_LDS ? LOOP_LDS : EPI_LDS;
+  static_assert(BM <= 256 && BN <= 256, "epilogue operand table holds 256 entries");
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char *lds_a = smem;                      // [NSTAGE][BM * BK], rows of 64 B, chunk c at c ^ swz64(row)
   unsigned char *lds_b = smem + NSTAGE * A_STAGE;   // [N,K]: [NSTAGE][BN * BK] like x; [K,N]: [KN_STAGES][4][BN][16]
@@ -177,6 +185,19 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   const int n0 = nt * BN;
   const int k_slabs = (p.k + BK - 1) / BK;
 
+  // Epilogue operands of this tile (scale and bias of its columns, per-token scale of its rows) are
+  // requested now, parked in registers during the main loop and handed over through LDS, so that
+  // the epilogue does not start with a chain of global-memory round trips.
+  float pre_scale = 1.0f, pre_pt = 1.0f;
+  int pre_bias = 0;
+  if (tid < 256) {
+    if (tid < BN && n0 + tid < p.n) {
+      pre_scale = load_scale(p, grp, n0 + tid);
+      pre_bias = load_bias(p, grp, n0 + tid);
+    }
+    if (tid < BM && p.per_token && m0 + tid < g_end) pre_pt = p.per_token[m0 + tid];
+  }
+
   // Buffer descriptors start at this tile's first x row / weight column, so per-lane offsets stay
   // small; anything past the end of the tensor reads as zero (no clamping, no branches in the loop).
   const long long w_elems = (long long)p.k * p.n;
@@ -209,7 +230,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
     }
   }
   auto issue_direct = [&](int kt) {
-    const int stage = kt & (NSTAGE - 1);
+    const int stage = kt % NSTAGE;
     const unsigned kbase = kt * BK;
     // K tail, and whole slabs past K (requested by the last steps of the branch-free loop): read as zero
     const unsigned kill = (kbase + d_c * 16 >= (unsigned)p.k) ? OOB : 0u;
@@ -263,14 +284,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   // ---- fragment reads (one 16-byte LDS read per lane and fragment) ----------------------------
   // lane (l32, hh) of k-half kk reads row l32 of its 32-row block, 16-byte chunk c = 2 kk + hh
   auto read_x = [&](int kt, int i, int kk) -> v4i {
-    const unsigned char *a = lds_a + (kt & (NSTAGE - 1)) * A_STAGE;
+    const unsigned char *a = lds_a + (kt % NSTAGE) * A_STAGE;
     const int row = wave_m * WTM + 32 * i + l32;
     return *reinterpret_cast<const v4i *>(a + row * BK + (((2 * kk + hh) ^ swz64(row)) << 4));
   };
   auto read_w = [&](int kt, int f, int kk) -> v4i {
     const int rho = wave_n * WTN + 32 * f + l32;
     if constexpr (NK) {
-      const unsigned char *b = lds_b + (kt & (NSTAGE - 1)) * B_STAGE;
+      const unsigned char *b = lds_b + (kt % NSTAGE) * B_STAGE;
       return *reinterpret_cast<const v4i *>(b + rho * BK + (((2 * kk + hh) ^ swz64(rho)) << 4));
     } else {
       // 16 K bytes of chunk c = 2 kk + hh: planes 2 c and 2 c + 1, 8 bytes each.  Read with
@@ -320,7 +341,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   // just issued.
   auto step = [&](int kt, auto ring_slot) {
     constexpr int SLOT = decltype(ring_slot)::value;          // == kt % KN_RING, compile-time for register indexing
-    issue_direct(kt + 3);
+    issue_direct(kt + AHEAD);
     load_kn(kt + 3, SLOT);                                    // (kt + 3) % 3 == kt % 3: that slot was emptied last step
     v4i xf[2][FM], wf[2][FN];
 #pragma unroll
@@ -339,7 +360,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
         for (int f = 0; f < FN; ++f) lds_reads_done(wf[kk][f]);
     }
     if constexpr (PINGPONG) {
-      wait_vmcnt<2 * VM_PER_SLAB>();                          // this wave's part of slab t+1 has landed
+      wait_vmcnt<(AHEAD - 1) * VM_PER_SLAB>();                // this wave's part of slab t+1 has landed
       __builtin_amdgcn_sched_barrier(0);
       lds_barrier();                                          // fragments are in registers, slab t+1 is published
       __builtin_amdgcn_sched_barrier(0);
@@ -357,7 +378,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
       phase_barrier();
     } else {
       store_kn(kt + 1, (SLOT + 1) % KN_RING);                 // its LDS stage held slab t-1, read before the last barrier
-      wait_vmcnt<2 * VM_PER_SLAB>();                          // only the loads of slabs t+2, t+3 may be outstanding
+      wait_vmcnt<(AHEAD - 1) * VM_PER_SLAB>();                // only the loads of younger slabs may be outstanding
       lds_barrier();
     }
   };
@@ -365,9 +386,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   // prologue: slabs 0, 1, 2 requested; slab 0 published
   issue_direct(0); load_kn(0, 0);
   issue_direct(1); load_kn(1, 1);
-  issue_direct(2); load_kn(2, 2);
+  if constexpr (AHEAD > 2) { issue_direct(2); load_kn(2, 2); }
   store_kn(0, 0);
-  wait_vmcnt<2 * VM_PER_SLAB>();
+  wait_vmcnt<(AHEAD - 1) * VM_PER_SLAB>();
   lds_barrier();
   if (behind) phase_barrier();
 
@@ -385,6 +406,14 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
     if (kt + 1 < k_slabs) step(kt + 1, std::integral_constant<int, 1>{});
   }
   if (PINGPONG && !behind) phase_barrier();
+  float *ep_scale = reinterpret_cast<float *>(smem + PARAM_OFF);
+  int *ep_bias = reinterpret_cast<int *>(smem + PARAM_OFF + 1024);
+  float *ep_pt = reinterpret_cast<float *>(smem + PARAM_OFF + 2048);
+  if (tid < 256) {
+    ep_scale[tid] = pre_scale;
+    ep_bias[tid] = pre_bias;
+    ep_pt[tid] = pre_pt;
+  }
   // the epilogue reuses the operand ring: every wave is done reading it and the late zero fills have landed
   wait_vmcnt<0>();
   lds_barrier();
@@ -400,8 +429,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
   float pt[FM];
 #pragma unroll
   for (int i = 0; i < FM; ++i) {
-    const int m = m0 + wave_m * WTM + 32 * i + l32;
-    pt[i] = (p.per_token && m < g_end) ? p.per_token[m] : 1.0f;
+    pt[i] = ep_pt[wave_m * WTM + 32 * i + l32];
   }
   // int32 rows are 256 bytes: one 32-column block per pass; 16-bit outputs take a single pass
   auto run_pass = [&](auto raw_c, auto pass_c) {
@@ -419,9 +447,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
         int bi[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const int n = min(nb + j, p.n - 1);
-          sc[j] = load_scale(p, grp, n);
-          bi[j] = load_bias(p, grp, n);
+          sc[j] = ep_scale[wave_n * WTN + cw + j];
+          bi[j] = ep_bias[wave_n * WTN + cw + j];
         }
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
@@ -478,12 +505,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64) gmm_w8a8_tile_kernel(co
 }
 
 // ---- host launcher ---------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4>
 static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
-  const size_t loop_lds = (size_t)NSTAGE * BM * BK + (size_t)(NK ? NSTAGE : KN_STAGES) * BN * BK;
+  const size_t loop_lds = (size_t)STAGES * BM * BK + (size_t)(NK ? STAGES : KN_STAGES) * BN * BK;
   const size_t epi_lds = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * 144;   // epilogue staging, 144-byte row pitch
-  const size_t lds = loop_lds > epi_lds ? loop_lds : epi_lds;
-  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK>;
+  const size_t lds = (loop_lds > epi_lds ? loop_lds : epi_lds) + 3 * 1024;   // + epilogue operand table
+  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -508,6 +535,8 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream
       return nk ? launch_cfg<128, 128, 2, 2, true>(p, stream) : launch_cfg<128, 128, 2, 2, false>(p, stream);
     case TILE_64x128:
       return nk ? launch_cfg<64, 128, 2, 2, true>(p, stream) : launch_cfg<64, 128, 2, 2, false>(p, stream);
+    case TILE_128x256:   // two 4-wave workgroups per CU; [N,K] weights only
+      return nk ? launch_cfg<128, 256, 1, 4, true, 3>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     default:
       return hipErrorInvalidValue;
   }
@@ -518,6 +547,7 @@ const char *tile_cfg_name(int tile_cfg) {
     case TILE_256x256: return "256x256x64";
     case TILE_128x128: return "128x128x64";
     case TILE_64x128: return "64x128x64";
+    case TILE_128x256: return "128x256x64";
     default: return "?";
   }
 }
@@ -526,6 +556,7 @@ void tile_cfg_dims(int tile_cfg, int *bm, int *bn) {
   switch (tile_cfg) {
     case TILE_256x256: *bm = 256; *bn = 256; break;
     case TILE_128x128: *bm = 128; *bn = 128; break;
+    case TILE_128x256: *bm = 128; *bn = 256; break;
     default: *bm = 64; *bn = 128; break;
   }
 }
