@@ -24,7 +24,7 @@ IN_X, IN_WEIGHT, IN_BIAS, IN_SCALE, IN_GROUP_LIST, IN_PER_TOKEN_SCALE, IN_ANTIQU
 IN_COUNT = 8
 
 # msco_gmm_desc.kernel_override
-OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC = range(6)
+OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC, OV_TILE_256_W4 = range(7)
 
 EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco_gmm_plan_info", "msco_gmm_destroy",
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d")

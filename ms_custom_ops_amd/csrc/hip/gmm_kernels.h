@@ -7,11 +7,16 @@
 
 namespace msco {
 
-enum TileCfg : int { TILE_256x256 = 0, TILE_128x128 = 1, TILE_64x128 = 2, TILE_128x256 = 3, TILE_CFG_COUNT = 4 };
+enum TileCfg : int {
+  TILE_256x256 = 0, TILE_128x128 = 1, TILE_64x128 = 2, TILE_128x256 = 3,
+  TILE_256x256_W4 = 4,   // four wavefronts with 128 x 128 accumulators each (gmm_tile4_w8a8.hip)
+  TILE_CFG_COUNT = 5
+};
 
 // MFMA tile kernel for W8A8 (prefill shapes).  nk: weights stored [E,N,K].
 hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream_t stream);
 const char *tile_cfg_name(int tile_cfg);
+hipError_t launch_tile4_w8a8_nk(const GmmParams &p, hipStream_t stream);
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn);
 
 // Skinny (decode) kernels: one workgroup streams a 128-column weight strip of one group over a K

@@ -1,0 +1,534 @@
+// Grouped W8A8 GEMM, persistent register-heavy MFMA tile kernel for gfx950: 256 x 256 output tiles,
+// four wavefronts (one per SIMD), 128 x 128 accumulators per wavefront, weights stored [E,N,K].
+//
+// Why this shape.  A wavefront that owns 128 x 128 outputs reads 8 operand fragments from LDS for every
+// 16 MFMAs (a 128 x 64 wave tile reads 12), so LDS traffic per multiply-add drops by a third.  The
+// 256 int32 accumulators of a lane fill the accumulation register file; operand fragments (two sets)
+// and the operand staging registers live in the architectural file.  With one wavefront per SIMD
+// nothing else covers a stall, hence:
+//
+//   * K slab = 128 bytes per row.  Every x row / weight column is requested one full 128-byte line
+//     at a time (measured: 64-byte requests cap the operand stream at ~20 B/clk/CU whatever the
+//     depth, full lines reach 28 B/clk/CU with two slabs in flight).
+//   * Two slabs in flight.  Operands are loaded into staging registers two slabs ahead of their
+//     multiply, written to the LDS stage that the last barrier retired, and the registers are refilled
+//     right behind the write.  One load, one LDS write and two fragment reads are issued per four
+//     MFMAs: a burst of either would stall the in-order issue of the only wave on the SIMD.
+//   * One workgroup barrier per slab (2048 MFMA cycles).  Two LDS stages of 64 KiB.
+//   * LDS rows are 128 B; 16-byte chunk c of row r sits at chunk position c ^ ((r >> 1) & 7), which
+//     makes both the staging writes and the 16-lane fragment reads bank-conflict free.
+//   * Persistent workgroups.  A workgroup walks its share of the tiles and the operand stream never
+//     drains: the first slabs of the next tile are requested during the last slabs of the current
+//     one, so a tile costs its MFMAs plus the epilogue, not a pipeline refill.
+//   * Weights are the MFMA's first operand and x the second, so a lane owns output row m and runs of 8
+//     consecutive columns; the fused dequant epilogue is staged through a small LDS region next to the
+//     ring (32 rows at a time) and stores full 128-byte row segments.
+//   * Partial m-tiles (the last tile of a group) skip the 32-row MFMA blocks that hold no rows.
+#include "gmm_common.h"
+#include "gmm_kernels.h"
+
+#include <type_traits>
+
+namespace msco {
+namespace {
+
+constexpr int T4_BM = 256, T4_BN = 256;
+constexpr int T4_BK = 128;                       // bytes of K per slab and LDS row
+constexpr int T4_NW = 4;                         // wavefronts: 2 (m) x 2 (n)
+constexpr int T4_WT = 128;                       // wave tile edge
+constexpr int T4_F = 4;                          // 32 x 32 MFMA blocks per wave tile edge
+constexpr int T4_OP_STAGE = T4_BM * T4_BK;       // one operand's share of a stage (32 KiB)
+constexpr int T4_STAGE = 2 * T4_OP_STAGE;        // x rows, then weight rows
+constexpr int T4_RING = 2 * T4_STAGE;            // 128 KiB
+constexpr int T4_LD = T4_BM / 8 / T4_NW;         // staging quads (8 rows x 128 B per wave) per operand and slab
+constexpr int T4_EP_PITCH = 144;                 // epilogue staging: 128 payload bytes per row
+constexpr int T4_PARAM_OFF = T4_RING;            // epilogue operand tables (scale, bias, per-token; two tiles) behind the ring
+constexpr int T4_PARAM_BYTES = 3 * 1024;
+constexpr int T4_EP_OFF = T4_PARAM_OFF + 2 * T4_PARAM_BYTES;
+constexpr int T4_EP_WAVE = 32 * T4_EP_PITCH;     // one wave stages 32 rows at a time
+constexpr int T4_META_OFF = T4_EP_OFF + T4_NW * T4_EP_WAVE;   // per group: row end, tiles up to and including it
+constexpr int T4_MAX_E = 1024;
+constexpr int T4_LDS_BYTES = T4_META_OFF + 2 * T4_MAX_E * 4;
+static_assert(T4_LDS_BYTES <= 160 * 1024, "LDS of one CU");
+constexpr int T4_MAX_WGS = 256;                  // one persistent workgroup per CU
+constexpr unsigned T4_OOB = 0x80000000u;
+
+__device__ __forceinline__ int t4_col_of_q(int q) {
+  const int g = q >> 3, hh = (q >> 2) & 1, t = q & 3;
+  return 16 * (g >> 1) + 8 * hh + 4 * (g & 1) + t;
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t t4_rsrc(const void *base, long long bytes) {
+  const unsigned n = bytes > 0x7FFFFFFFll ? 0x7FFFFFFFu : (unsigned)(bytes < 0 ? 0 : bytes);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
+}
+
+// Publishes LDS data and retires a stage: the caller has waited for its own LDS traffic.
+__device__ __forceinline__ void t4_barrier() {
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_barrier" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// Raw buffer descriptor as four scalars (for hand-written buffer instructions).
+__device__ __forceinline__ v4i t4_raw_rsrc(const void *base, long long bytes) {
+  const unsigned long long a = (unsigned long long)base;
+  const unsigned n = bytes > 0x7FFFFFFFll ? 0x7FFFFFFFu : (unsigned)(bytes < 0 ? 0 : bytes);
+  v4i r;
+  r.x = __builtin_amdgcn_readfirstlane((int)(unsigned)a);
+  r.y = __builtin_amdgcn_readfirstlane((int)((unsigned)(a >> 32) & 0xFFFFu));
+  r.z = __builtin_amdgcn_readfirstlane((int)n);
+  r.w = 0x00020000;
+  return r;
+}
+
+// One dword (or zero-extended 16 bits) per lane from a buffer straight into LDS: lane L writes
+// lds_addr + 4 L.  Hand-written so that the compiler's wait-count bookkeeping never sees an LDS
+// write in flight (it would make every later LDS read wait for all outstanding loads); the
+// counter it does not know about can only make its own waits longer, never shorter, because
+// vector memory operations complete in order.
+__device__ __forceinline__ void t4_dma_b32(v4i rsrc, unsigned lds_addr, unsigned voffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory");
+}
+__device__ __forceinline__ void t4_dma_b16(v4i rsrc, unsigned lds_addr, unsigned voffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ushort %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory");
+}
+
+// A tile as the whole workgroup sees it (all fields wave-uniform).
+struct T4Tile {
+  int valid;
+  int grp, m0, n0, g_end;
+};
+
+// Tile lid -> (group, m-tile, n-tile).  The group walk was done once at kernel start and left in LDS
+// (row end and inclusive tile count per group): reading group_list from memory again for every tile
+// would put loads into the middle of the operand stream, and vector loads complete in order.
+// Order inside a group: panels of 8 m-tiles; inside a panel n-tile major, m-tile minor, so that
+// workgroups that run side by side share one streamed weight panel.
+__device__ __forceinline__ T4Tile t4_locate(const int *meta_end, const int *meta_upto, int e, int lid, int total,
+                                            int n_tiles, int lane) {
+  T4Tile t{0, 0, 0, 0, 0};
+  if (lid < 0 || lid >= total) return t;
+  int g_start = 0, t_in_group = 0;
+  for (int g0 = 0; g0 < e; g0 += 64) {
+    const int g = g0 + lane;
+    const int upto = g < e ? meta_upto[g] : 0x7FFFFFFF;
+    const int first = __popcll(__ballot(upto <= lid));              // `upto` is non-decreasing: first group beyond lid
+    if (first < 64) {
+      const int grp = g0 + first;
+      t.grp = grp;
+      t.g_end = __builtin_amdgcn_readfirstlane(meta_end[grp]);
+      g_start = grp > 0 ? __builtin_amdgcn_readfirstlane(meta_end[grp - 1]) : 0;
+      t_in_group = lid - (grp > 0 ? __builtin_amdgcn_readfirstlane(meta_upto[grp - 1]) : 0);
+      t.valid = 1;
+      break;
+    }
+  }
+  constexpr int PANEL = 8;
+  const int m_tiles = (t.g_end - g_start + T4_BM - 1) / T4_BM;
+  const int panel_tiles = PANEL * n_tiles;
+  const int panel = t_in_group / panel_tiles;
+  const int in_panel = t_in_group - panel * panel_tiles;
+  const int panel_m = max(1, min(PANEL, m_tiles - panel * PANEL));
+  const int nt = in_panel / panel_m;
+  const int mt = panel * PANEL + in_panel % panel_m;
+  t.m0 = g_start + mt * T4_BM;
+  t.n0 = nt * T4_BN;
+  return t;
+}
+
+}  // namespace
+
+// MODE: output type, 0 bf16, 1 f16, 2 int32 (raw accumulators plus bias)
+template <int MODE>
+__global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const GmmParams p) {
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_m = wave >> 1, wave_n = wave & 1;
+  const int l32 = lane & 31, hh = lane >> 5;
+
+  // ---- this workgroup's share of the tiles -----------------------------------------------------------
+  // Tiles are numbered so that neighbours share operands; every XCD takes a contiguous range and its
+  // workgroups walk it with a stride, so the workgroups of an XCD work side by side on neighbours.
+  const int n_tiles = (p.n + T4_BN - 1) / T4_BN;
+  int *meta_end = reinterpret_cast<int *>(smem + T4_META_OFF);
+  int *meta_upto = meta_end + T4_MAX_E;
+  int total = 0;
+  for (int g0 = 0, carry = 0; g0 < p.e; g0 += 64) {
+    int s0, e0;
+    group_rows_chunk(p, g0, lane, carry, s0, e0);
+    const int upto = total + wave_scan_add(((e0 - s0 + T4_BM - 1) / T4_BM) * n_tiles, lane);
+    if (wave == 0 && g0 + lane < p.e) {
+      meta_end[g0 + lane] = e0;
+      meta_upto[g0 + lane] = upto;
+    }
+    total = wave_bcast(upto, 63);
+  }
+  __syncthreads();
+  const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
+  const int xcd = blockIdx.x % kNumXcd, slot = blockIdx.x / kNumXcd;
+  const int wgs_per_xcd = gridDim.x / kNumXcd;
+  auto tile_at = [&](int i) -> T4Tile {
+    const int l = slot + i * wgs_per_xcd;
+    int lane_now = lane;   // laundered: keeps the table addresses out of the registers that live across the K loop
+    asm volatile("" : "+v"(lane_now));
+    return t4_locate(meta_end, meta_upto, p.e, l < per_xcd ? xcd * per_xcd + l : -1, total, n_tiles, lane_now);
+  };
+  T4Tile cur = tile_at(0);
+  if (!cur.valid) return;
+
+  // K slabs per tile, rounded up to even (the staging parities alternate per slab); slabs past K read zeros
+  const int k_slabs = 2 * ((p.k + 2 * T4_BK - 1) / (2 * T4_BK));
+  const long long w_elems = (long long)p.k * p.n;
+  auto x_rsrc = [&](const T4Tile &t) {
+    return t4_rsrc(reinterpret_cast<const int8_t *>(p.x) + (long long)t.m0 * p.k, (long long)(p.m - t.m0) * p.k);
+  };
+  auto w_rsrc = [&](const T4Tile &t) {
+    return t4_rsrc(p.w + (long long)t.grp * w_elems + (long long)t.n0 * p.k, (long long)(p.n - t.n0) * p.k);
+  };
+
+  // ---- global -> staging registers -------------------------------------------------------------------
+  // One quad = 1 KiB per wave = 8 rows x 128 B; lane L serves row L / 8, chunk position L % 8, so it
+  // fetches logical chunk (L % 8) ^ swizzle(row).  The row of quad u is 32 u + 8 wave + d_row, so neither
+  // the swizzle ((row >> 1) & 7) nor the MFMA row permutation (row & 31) depends on u.  Everything that
+  // can run past a tensor is in the per-lane offset (the only part the buffer unit range-checks).
+  const int d_row0 = 8 * wave + (lane >> 3);
+  const int d_chunk = (lane & 7) ^ ((d_row0 >> 1) & 7);
+  const unsigned a_voff0 = (unsigned)d_row0 * (unsigned)p.k + d_chunk * 16;
+  const unsigned b_voff0 = (unsigned)t4_col_of_q(d_row0) * (unsigned)p.k + d_chunk * 16;   // LDS row rho feeds MFMA row rho % 32
+  const unsigned rows32 = 32u * (unsigned)p.k;
+
+  // ---- fragment addressing ---------------------------------------------------------------------------
+  // lane (l32, hh) reads row l32 of a 32-row block, logical chunk 2 q + hh of K quarter q.  The row
+  // swizzle only depends on l32, and the chunk positions of the four quarters differ by an XOR with
+  // q << 5 in the byte address.
+  const int swz = (l32 >> 1) & 7;
+  const unsigned x_lane = (unsigned)((wave_m * T4_WT + l32) * T4_BK + ((hh ^ swz) << 4));
+  const unsigned w_lane = (unsigned)(T4_OP_STAGE + (wave_n * T4_WT + l32) * T4_BK + ((hh ^ swz) << 4));
+
+  unsigned char *st_lane = smem + wave * 1024 + lane * 16;
+  unsigned char *ep_stage = smem + T4_EP_OFF + wave * T4_EP_WAVE;
+
+  const std::integral_constant<int, 0> c0;
+  const std::integral_constant<int, 1> c1;
+  const std::integral_constant<int, 2> c2;
+  const std::integral_constant<int, 3> c3;
+
+  v16i acc[T4_F][T4_F];   // [f: weight block][i: x block]
+  v4i stg[2][2][T4_LD];   // staging quads: [slab parity][operand: 0 x, 1 w][u]
+  v4i wf[2][T4_F], xf[2][T4_F];
+
+  T4Tile nxt = cur;        // tile that follows `cur` in this workgroup's walk (loads run ahead into it)
+  __amdgpu_buffer_rsrc_t rx_c = x_rsrc(cur), rw_c = w_rsrc(cur), rx_n = rx_c, rw_n = rw_c;
+
+  // slab s of the current tile, or slab s - k_slabs of the next one
+  auto load_one = [&](int s, auto par_c, auto op_c, auto u_c) {
+    constexpr int P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
+    const bool ahead = s >= k_slabs;
+    const unsigned kbase = (unsigned)(ahead ? s - k_slabs : s) * T4_BK;
+    const bool dead = (ahead && !nxt.valid) || kbase + d_chunk * 16 >= (unsigned)p.k;   // K tail, slabs past K, no next tile
+    const unsigned kill = dead ? T4_OOB : 0u;
+    if constexpr (OP == 0)
+      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rx_n : rx_c, (a_voff0 + U * rows32) | kill, kbase, 0);
+    else
+      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rw_n : rw_c, (b_voff0 + U * rows32) | kill, kbase, 0);
+  };
+  // write quad (op, u) of slab s to its LDS stage and refill it with slab s + 2
+  auto cycle_one = [&](int s, auto par_c, auto op_c, auto u_c) {
+    constexpr int P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
+    *reinterpret_cast<v4i *>(st_lane + (s & 1) * T4_STAGE + OP * T4_OP_STAGE + U * 4096) = stg[P][OP][U];
+    load_one(s + 2, par_c, op_c, u_c);
+  };
+  // (qx = q << 5 arrives in a scalar the compiler cannot see through: hoisting the XORs out of the K
+  // loop would park eight more addresses in registers that the loop does not have)
+  auto read_w = [&](int stage, unsigned qx, auto set_c, auto f_c) {
+    constexpr int S = decltype(set_c)::value, F = decltype(f_c)::value;
+    wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_STAGE + (w_lane ^ qx) + F * 32 * T4_BK);
+  };
+  auto read_x = [&](int stage, unsigned qx, auto set_c, auto i_c) {
+    constexpr int S = decltype(set_c)::value, I = decltype(i_c)::value;
+    xf[S][I] = *reinterpret_cast<const v4i *>(smem + stage * T4_STAGE + (x_lane ^ qx) + I * 32 * T4_BK);
+  };
+  auto opaque_q = [](int q) {
+    unsigned qx = (unsigned)q << 5;
+    asm volatile("" : "+s"(qx));
+    return qx;
+  };
+
+  // ---- stream prologue (once per workgroup): slabs 0 and 1 requested; slab 0 and group 0 of slab 1
+  // written to LDS and refilled; quarter-0 fragments of slab 0 read -------------------------------------
+  {
+    auto for_u = [&](auto fn) {
+      fn(std::integral_constant<int, 0>{}); fn(std::integral_constant<int, 1>{}); fn(std::integral_constant<int, 2>{});
+      fn(std::integral_constant<int, 3>{}); fn(std::integral_constant<int, 4>{}); fn(std::integral_constant<int, 5>{});
+      fn(std::integral_constant<int, 6>{}); fn(std::integral_constant<int, 7>{});
+    };
+    // (nxt == cur here, and slabs 0 .. 3 are below k_slabs >= 4, so every request goes to `cur`)
+    for_u([&](auto u) { load_one(0, c0, c0, u); });
+    for_u([&](auto u) { load_one(0, c0, c1, u); });
+    for_u([&](auto u) { load_one(1, c1, c0, u); });
+    for_u([&](auto u) { load_one(1, c1, c1, u); });
+    for_u([&](auto u) { cycle_one(0, c0, c0, u); });
+    for_u([&](auto u) { cycle_one(0, c0, c1, u); });
+    cycle_one(1, c1, c0, c0); cycle_one(1, c1, c0, c1);
+    cycle_one(1, c1, c1, c0); cycle_one(1, c1, c1, c1);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    t4_barrier();
+  }
+
+  for (int ti = 0;; ++ti) {
+    // the tile after this one: the operand stream crosses into it during the last slabs
+    nxt = tile_at(ti + 1);
+    if (nxt.valid) { rx_n = x_rsrc(nxt); rw_n = w_rsrc(nxt); }
+
+    // Epilogue operands of this tile (scale and bias of its 256 columns, per-token scale of its 256
+    // rows) go straight from memory into this tile's LDS table (two tables, alternating per tile: the
+    // other one may still be read by a wave that is finishing the previous epilogue).  The K-loop
+    // barriers publish them long before the epilogue reads them.
+    unsigned char *table = smem + T4_PARAM_OFF + (ti & 1) * T4_PARAM_BYTES;
+    {
+      const unsigned lds = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char *)table + wave * 256;
+      const int col = cur.n0 + tid, row = cur.m0 + tid;
+      const long long pg = p.scale_per_group ? (long long)cur.grp * p.n : 0;
+      if (p.scale_dtype == DT_NONE) {
+        reinterpret_cast<float *>(table)[tid] = 1.0f;
+      } else {
+        const int esz = p.scale_dtype == DT_F32 ? 4 : p.scale_dtype == DT_BF16 ? 2 : 8;
+        const long long first = p.scale_is_scalar ? 0 : (pg + cur.n0) * esz;
+        const v4i rs = t4_raw_rsrc(reinterpret_cast<const unsigned char *>(p.scale) + first,
+                                   p.scale_is_scalar ? esz : (long long)(p.n - cur.n0) * esz);
+        const unsigned voff = col < p.n ? (p.scale_is_scalar ? 0u : (unsigned)(tid * esz)) : T4_OOB;
+        if (p.scale_dtype == DT_BF16) t4_dma_b16(rs, lds, voff);
+        else t4_dma_b32(rs, lds, voff);
+      }
+      if (p.bias == nullptr) {
+        reinterpret_cast<int *>(table + 1024)[tid] = 0;
+      } else {
+        const v4i rb = t4_raw_rsrc(p.bias + pg + cur.n0, (long long)(p.n - cur.n0) * 4);
+        t4_dma_b32(rb, lds + 1024, col < p.n ? (unsigned)(tid * 4) : T4_OOB);
+      }
+      if (p.per_token == nullptr) {
+        reinterpret_cast<float *>(table + 2048)[tid] = 1.0f;
+      } else {
+        const v4i rp = t4_raw_rsrc(p.per_token + cur.m0, (long long)(p.m - cur.m0) * 4);
+        t4_dma_b32(rp, lds + 2048, row < cur.g_end ? (unsigned)(tid * 4) : T4_OOB);
+      }
+    }
+
+    // rows of this tile that exist, and the 32-row blocks of this wave that hold any of them
+    const int rows_here = min(T4_BM, cur.g_end - cur.m0);
+    const int rows_wave = rows_here - wave_m * T4_WT;
+    const int fm_active = max(0, min(T4_F, (rows_wave + 31) / 32));
+
+#pragma unroll
+    for (int f = 0; f < T4_F; ++f)
+#pragma unroll
+      for (int i = 0; i < T4_F; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[f][i][r] = 0;
+    // quarter-0 fragments of slab 0 (read here rather than behind the previous tile's last slab, so that
+    // the epilogue does not have to keep them alive)
+    read_w(0, 0, c0, c0); read_w(0, 0, c0, c1); read_w(0, 0, c0, c2); read_w(0, 0, c0, c3);
+    read_x(0, 0, c0, c0); read_x(0, 0, c0, c1); read_x(0, 0, c0, c2); read_x(0, 0, c0, c3);
+
+    {
+      // One K quarter: the MFMAs of fragment set CUR; meanwhile the fragments of (rstage, rq) are read
+      // into set NXT and staging group G (x and w quads 2 G, 2 G + 1) of slab ss goes to LDS and is
+      // refilled.  LDS operations keep their source order; the scheduling groups pin one memory
+      // operation behind each of the first MFMAs.
+      auto quarter = [&](auto cur_c, auto nxt_c, int rstage, int rq_index, int ss, auto par_c, auto g_c) {
+        constexpr int G = decltype(g_c)::value;
+        constexpr int S = decltype(cur_c)::value;
+        const unsigned rq = opaque_q(rq_index);
+        const std::integral_constant<int, 2 * G> ua;
+        const std::integral_constant<int, 2 * G + 1> ub;
+        read_w(rstage, rq, nxt_c, c0); read_x(rstage, rq, nxt_c, c0);
+        cycle_one(ss, par_c, c0, ua);
+        read_x(rstage, rq, nxt_c, c1); read_x(rstage, rq, nxt_c, c2);
+        cycle_one(ss, par_c, c0, ub);
+        read_x(rstage, rq, nxt_c, c3); read_w(rstage, rq, nxt_c, c1);
+        cycle_one(ss, par_c, c1, ua);
+        read_w(rstage, rq, nxt_c, c2); read_w(rstage, rq, nxt_c, c3);
+        cycle_one(ss, par_c, c1, ub);
+#pragma unroll
+        for (int f = 0; f < T4_F; ++f)
+#pragma unroll
+          for (int i = 0; i < T4_F; ++i)
+            acc[f][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[S][f], xf[S][i], acc[f][i], 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // DS read
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // DS write
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // VMEM read
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      // One K slab kt (LDS stage kt & 1).  On entry the quarter-0 fragments are in fragment set 0 and
+      // group 0 of slab kt+1 is in LDS; PAR is the staging parity of slab kt+1.
+      auto period = [&](int kt, auto par_c) {
+        constexpr int PAR = decltype(par_c)::value;
+        const std::integral_constant<int, PAR ^ 1> other;
+        const int stage = kt & 1;
+        quarter(c0, c1, stage, 1, kt + 1, par_c, c1);
+        quarter(c1, c0, stage, 2, kt + 1, par_c, c2);
+        quarter(c0, c1, stage, 3, kt + 1, par_c, c3);
+        // slab kt+1 is in LDS (this wave's part) and the quarter-3 fragments are in registers: after the
+        // barrier every wave's part is visible and nobody reads this stage any more
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        t4_barrier();
+        quarter(c1, c0, stage ^ 1, 0, kt + 2, other, c0);
+      };
+      for (int kt = 0; kt < k_slabs; kt += 2) {
+        period(kt, c1);
+        period(kt + 1, c0);
+      }
+    }
+
+
+    // ---- fused dequant epilogue ----------------------------------------------------------------------
+    // acc[f][i][r] is output row 32 i + l32, column 32 f + 16 (r / 8) + 8 hh + (r % 8) of the wave tile.
+    // Per 32-row block and 128-byte column piece: dequantise, park in this wave's LDS region (rows of
+    // 128 payload bytes at a 144-byte pitch), read back with lanes along columns, store full 128-byte
+    // row segments.  The operand ring is live (it already holds the next tile), so only the small
+    // region behind it is used.  The table was published by the barriers of the slabs since kt == 2.
+    {
+      // (lane-derived values are laundered through an empty asm: otherwise every LDS address below is
+      // loop invariant, gets computed before the tile loop and has to survive the K loop in a register
+      // the K loop does not have)
+      int e_l32 = l32, e_hh = hh, e_lane = lane;
+      asm volatile("" : "+v"(e_l32), "+v"(e_hh), "+v"(e_lane));
+      const int n_base = cur.n0 + wave_n * T4_WT;
+      const int m_base = cur.m0 + wave_m * T4_WT;
+      unsigned *tb_scale = reinterpret_cast<unsigned *>(table) + wave_n * T4_WT;
+      const int *tb_bias = reinterpret_cast<const int *>(table + 1024) + wave_n * T4_WT;
+      const float *tb_pt = reinterpret_cast<const float *>(table + 2048) + wave_m * T4_WT;
+      if (p.scale_dtype == DT_BF16) {
+        // the table holds raw 16-bit patterns: widen them in place (one entry per thread)
+        unsigned *mine = reinterpret_cast<unsigned *>(table) + tid;
+        *mine = *mine << 16;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        t4_barrier();
+      }
+      auto run_pass = [&](auto i_c, auto piece_c) {
+        constexpr bool raw = MODE == 2;
+        constexpr int I = decltype(i_c)::value;
+        constexpr int PIECE = decltype(piece_c)::value;    // 16-bit outputs: 64-column half; int32: 32-column block
+        constexpr int esize = raw ? 4 : 2;
+        constexpr int f_lo = raw ? PIECE : 2 * PIECE, f_hi = raw ? PIECE + 1 : 2 * PIECE + 2;
+        if (I >= fm_active) return;
+        const float pt = tb_pt[32 * I + e_l32];
+        unsigned char *dst = ep_stage + e_l32 * T4_EP_PITCH;
+#pragma unroll
+        for (int f = f_lo; f < f_hi; ++f) {
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            const int cw = 32 * f + 16 * s2 + 8 * e_hh;          // column inside the wave tile
+            const int cs = cw - 32 * f_lo;                       // column inside the staged piece
+            const uint4 s_lo = *reinterpret_cast<const uint4 *>(tb_scale + cw);
+            const uint4 s_hi = *reinterpret_cast<const uint4 *>(tb_scale + cw + 4);
+            const int4 b_lo = *reinterpret_cast<const int4 *>(tb_bias + cw);
+            const int4 b_hi = *reinterpret_cast<const int4 *>(tb_bias + cw + 4);
+            const unsigned sraw[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
+            const int bi[8] = {b_lo.x, b_lo.y, b_lo.z, b_lo.w, b_hi.x, b_hi.y, b_hi.z, b_hi.w};
+            // accumulators leave the accumulation file here and not earlier (pinned: read ahead of time
+            // they would not fit into the architectural file next to the staging registers)
+            int a8[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a8[j]) : "a"(acc[f][I][8 * s2 + j]));
+            if constexpr (raw) {
+              int *d = reinterpret_cast<int *>(dst + cs * 4);
+              *reinterpret_cast<int4 *>(d) = make_int4(a8[0] + bi[0], a8[1] + bi[1], a8[2] + bi[2], a8[3] + bi[3]);
+              *reinterpret_cast<int4 *>(d + 4) = make_int4(a8[4] + bi[4], a8[5] + bi[5], a8[6] + bi[6], a8[7] + bi[7]);
+            } else {
+              float v[8];
+#pragma unroll
+              for (int j = 0; j < 8; ++j) v[j] = dequant(a8[j] + bi[j], __uint_as_float(sraw[j]), pt);
+              uint4 q;
+              if constexpr (MODE == 0) {
+                q.x = pack_bf16x2(v[0], v[1]); q.y = pack_bf16x2(v[2], v[3]);
+                q.z = pack_bf16x2(v[4], v[5]); q.w = pack_bf16x2(v[6], v[7]);
+              } else {
+                // the float32 product is rounded before the conversion (the golden's order); left visible,
+                // multiply and conversion are merged into one mixed-precision instruction that rounds once
+#pragma unroll
+                for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(v[j]));
+                q.x = f32_to_f16_rne(v[0]) | ((unsigned)f32_to_f16_rne(v[1]) << 16);
+                q.y = f32_to_f16_rne(v[2]) | ((unsigned)f32_to_f16_rne(v[3]) << 16);
+                q.z = f32_to_f16_rne(v[4]) | ((unsigned)f32_to_f16_rne(v[5]) << 16);
+                q.w = f32_to_f16_rne(v[6]) | ((unsigned)f32_to_f16_rne(v[7]) << 16);
+              }
+              *reinterpret_cast<uint4 *>(dst + cs * 2) = q;
+            }
+          }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const int piece = e_lane & 7;
+        const int col = (raw ? 32 * PIECE : 64 * PIECE) + (raw ? 4 : 8) * piece;   // first column of the piece in the wave tile
+        const int n_first = n_base + col;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int row = 32 * I + 8 * t + (e_lane >> 3);
+          const uint4 q = *reinterpret_cast<const uint4 *>(ep_stage + (8 * t + (e_lane >> 3)) * T4_EP_PITCH + piece * 16);
+          if (row < rows_wave && n_first < p.n) {
+            unsigned char *o = reinterpret_cast<unsigned char *>(p.out) + ((long long)(m_base + row) * p.n + n_first) * esize;
+            *reinterpret_cast<uint4 *>(o) = q;
+          }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      auto for_i = [&](auto fn) { fn(c0); fn(c1); fn(c2); fn(c3); };
+      if constexpr (MODE == 2) {
+        for_i([&](auto i) { run_pass(i, c0); run_pass(i, c1); run_pass(i, c2); run_pass(i, c3); });
+      } else {
+        for_i([&](auto i) { run_pass(i, c0); run_pass(i, c1); });
+      }
+    }
+
+    if (!nxt.valid) break;
+    cur = nxt;
+    rx_c = rx_n;
+    rw_c = rw_n;
+  }
+}
+
+template <int MODE>
+static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t stream) {
+  auto kern = gmm_w8a8_tile4_nk_kernel<MODE>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, T4_LDS_BYTES);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(T4_NW * 64), T4_LDS_BYTES, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_tile4_w8a8_nk(const GmmParams &p, hipStream_t stream) {
+  // the operand stream runs up to four slabs ahead inside one tile; the group table lives in LDS
+  if (p.k < 4 * T4_BK || p.e > T4_MAX_E) return hipErrorInvalidValue;
+  const long long n_tiles = (p.n + T4_BN - 1) / T4_BN;
+  const long long m_tiles_ub = (p.m + T4_BM - 1) / T4_BM + p.e;   // every non-empty group adds at most one partial tile
+  const long long total_ub = m_tiles_ub * n_tiles;
+  long long grid = ((total_ub + kNumXcd - 1) / kNumXcd) * kNumXcd;
+  if (grid > T4_MAX_WGS) grid = T4_MAX_WGS;
+  if (grid <= 0) return hipSuccess;
+  switch (p.out_dtype) {
+    case DT_BF16: return t4_launch<0>(p, (unsigned)grid, stream);
+    case DT_F16: return t4_launch<1>(p, (unsigned)grid, stream);
+    case DT_I32: return t4_launch<2>(p, (unsigned)grid, stream);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+}  // namespace msco

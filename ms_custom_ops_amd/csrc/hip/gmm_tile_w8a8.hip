@@ -537,6 +537,9 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream
       return nk ? launch_cfg<64, 128, 2, 2, true>(p, stream) : launch_cfg<64, 128, 2, 2, false>(p, stream);
     case TILE_128x256:   // two 4-wave workgroups per CU; [N,K] weights only
       return nk ? launch_cfg<128, 256, 1, 4, true, 3>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
+    case TILE_256x256_W4:   // needs [N,K] weights, at least four 128-byte K slabs per tile, a group table that fits in LDS
+      if (nk && p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, stream);
+      return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     default:
       return hipErrorInvalidValue;
   }
@@ -548,13 +551,14 @@ const char *tile_cfg_name(int tile_cfg) {
     case TILE_128x128: return "128x128x64";
     case TILE_64x128: return "64x128x64";
     case TILE_128x256: return "128x256x64";
+    case TILE_256x256_W4: return "256x256x128_w4";
     default: return "?";
   }
 }
 
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn) {
   switch (tile_cfg) {
-    case TILE_256x256: *bm = 256; *bn = 256; break;
+    case TILE_256x256: case TILE_256x256_W4: *bm = 256; *bn = 256; break;
     case TILE_128x128: *bm = 128; *bn = 128; break;
     case TILE_128x256: *bm = 128; *bn = 256; break;
     default: *bm = 64; *bn = 128; break;

@@ -21,7 +21,10 @@ using namespace msco;
 enum Family : int { FAM_NONE = 0, FAM_TILE = 1, FAM_SKINNY = 2, FAM_GENERIC = 3 };
 
 // values of msco_gmm_desc::kernel_override
-enum Override : int { OV_AUTO = 0, OV_TILE_256 = 1, OV_TILE_128 = 2, OV_TILE_64 = 3, OV_SKINNY = 4, OV_GENERIC = 5 };
+enum Override : int {
+  OV_AUTO = 0, OV_TILE_256 = 1, OV_TILE_128 = 2, OV_TILE_64 = 3, OV_SKINNY = 4, OV_GENERIC = 5,
+  OV_TILE_256_W4 = 6   // persistent four-wave 256 x 256 kernel ([E,N,K] weights; other layouts fall back to OV_TILE_256)
+};
 
 constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned
 constexpr int kTargetWorkgroups = 512;  // skinny kernels with a K split: aim for this many workgroups (2 per CU)
@@ -64,7 +67,7 @@ int check_desc(const msco_gmm_desc &d) {
   if (d.group_list_dtype != MSCO_DT_NONE && d.group_list_dtype != MSCO_DT_I32 && d.group_list_dtype != MSCO_DT_I64)
     return MSCO_ERR_UNSUPPORTED;
   if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
-  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_GENERIC) return MSCO_ERR_INVALID_ARG;
+  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_256_W4) return MSCO_ERR_INVALID_ARG;
   if (is_w8a8(d)) {
     if (d.out_dtype != MSCO_DT_BF16 && d.out_dtype != MSCO_DT_F16 && d.out_dtype != MSCO_DT_I32)
       return MSCO_ERR_UNSUPPORTED;
@@ -118,7 +121,8 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t rows_per_group = m / (e > 0 ? e : 1);
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     if (rows_per_group >= 192 && tiles(256, 256) >= 256) {
-      op->tile_cfg = TILE_256x256;
+      // [E,N,K] weights take the persistent four-wave kernel when a tile has at least four 128-byte K slabs
+      op->tile_cfg = (d.transpose_b && k >= 512 && e <= 1024) ? TILE_256x256_W4 : TILE_256x256;
     } else if (rows_per_group >= 96 && tiles(128, 128) >= 256) {
       op->tile_cfg = TILE_128x128;
     } else if (tiles(128, 128) >= 512) {
@@ -129,6 +133,7 @@ void choose_plan(msco_gmm_op *op) {
   }
   switch (d.kernel_override) {
     case OV_TILE_256: family = FAM_TILE; op->tile_cfg = TILE_256x256; break;
+    case OV_TILE_256_W4: family = FAM_TILE; op->tile_cfg = TILE_256x256_W4; break;
     case OV_TILE_128: family = FAM_TILE; op->tile_cfg = TILE_128x128; break;
     case OV_TILE_64: family = FAM_TILE; op->tile_cfg = TILE_64x128; break;
     case OV_SKINNY: family = FAM_SKINNY; break;

@@ -15,7 +15,7 @@ from oracle import gmm_oracle as O
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 FAMILIES = [("generic", cabi.OV_GENERIC), ("skinny", cabi.OV_SKINNY), ("tile64", cabi.OV_TILE_64),
-            ("tile128", cabi.OV_TILE_128), ("tile256", cabi.OV_TILE_256)]
+            ("tile128", cabi.OV_TILE_128), ("tile256", cabi.OV_TILE_256), ("tile256_w4", cabi.OV_TILE_256_W4)]
 
 
 def _inputs(seed, m, k, n, e):
@@ -158,6 +158,50 @@ def test_dense_equal_groups_without_group_list(device):
     for _, ov in FAMILIES:
         got, _ = run_w8a8(x, w, None, None, scale, None, override=ov)
         assert np.array_equal(got, ref)
+
+
+# ------------------------------------------------------------- persistent four-wave tile kernel
+W4 = cabi.OV_TILE_256_W4
+
+
+def test_w4_ragged_groups_k_tail_and_odd_slab_count(device):
+    # K = 1296: ten full 128-byte slabs and a 16-byte tail, an odd slab count (padded with a slab of
+    # zeros); N = 400 leaves a partial n-tile; groups: empty, 1 row, exactly 256, 257, a few hundred
+    rng, x, w, bias, scale, pt = _inputs(20, 1100, 1296, 400, 8)
+    gl = [0, 1, 257, 257, 514, 600, 1099, 1100]
+    info = _check(x, w, gl, bias, scale, pt, transpose_b=True, override=W4)
+    assert "256x256x128_w4" in info
+
+
+def test_w4_workgroups_walk_several_tiles(device):
+    # 18 m-tiles x 16 n-tiles = 288 tiles for at most 256 persistent workgroups: some walk two tiles,
+    # so the operand stream crosses a tile boundary, also into a tile of another group
+    rng, x, w, bias, scale, pt = _inputs(21, 4200, 640, 4096, 3)
+    info = _check(x, w, [1500, 1501, 4200], bias, scale, pt, transpose_b=True, override=W4)
+    assert "256x256x128_w4" in info
+
+
+def test_w4_scale_wire_formats_f16_out_and_absent_operands(device):
+    from gpu_utils import run_w8a8
+    rng, x, w, bias, scale, pt = _inputs(22, 700, 512, 528, 4)
+    gl = [100, 300, 300, 700]
+    kw = dict(transpose_b=True, override=W4)
+    ref = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt)
+    got, info = run_w8a8(x, w, gl, bias, O.encode_scale_int64(scale), pt, scale_dtype=cabi.DT_I64, **kw)
+    assert "256x256x128_w4" in info and np.array_equal(got, ref)
+    sb = O.f32_to_bf16_bits(scale)
+    got, _ = run_w8a8(x, w, gl, bias, sb, pt, scale_dtype=cabi.DT_BF16, **kw)
+    assert np.array_equal(got, O.grouped_matmul_w8a8(x, w, gl, bias, O.bf16_bits_to_f32(sb), pt))
+    # one [N] row shared by all groups; a single scalar; no bias; no per-token scale
+    got, _ = run_w8a8(x, w, gl, bias[0], scale[0], pt, scale_per_group=0, **kw)
+    assert np.array_equal(got, O.grouped_matmul_w8a8(x, w, gl, np.tile(bias[:1], (4, 1)), np.tile(scale[:1], (4, 1)), pt))
+    got, _ = run_w8a8(x, w, gl, None, scale[0, :1], None, scale_per_group=0, scale_is_scalar=1, **kw)
+    assert np.array_equal(got, O.grouped_matmul_w8a8(x, w, gl, None, np.full((4, 528), scale[0, 0], np.float32), None))
+    got, _ = run_w8a8(x, w, gl, bias, scale, pt, out="f16", **kw)
+    assert np.array_equal(got, O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt, out_dtype="f16").view(np.uint16))
+    # counts instead of cumulative ends, int32 list, rows past the last boundary stay untouched
+    counts = [100, 0, 250, 300]
+    _check(x, w, counts, bias, scale, pt, transpose_b=True, override=W4, group_list_type=1, gl_dtype=np.int32)
 
 
 # ------------------------------------------------------------------------------- weight-only path
