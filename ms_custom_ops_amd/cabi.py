@@ -70,6 +70,9 @@ def load():
         lib.msco_status_string.argtypes = [ctypes.c_int]
         lib.msco_gmm_abi_version.restype = ctypes.c_int
         lib.msco_gmm_abi_version.argtypes = []
+        lib.msco_transpose_2d.restype = ctypes.c_int
+        lib.msco_transpose_2d.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                          ctypes.c_int32, ctypes.c_void_p]
         _lib = lib
     return _lib
 
@@ -81,6 +84,12 @@ def status_string(status: int) -> str:
 def _check(where: str, status: int):
     if status != 0:
         raise BackendError(where, status, status_string(status))
+
+
+def transpose_2d(src: int, dst: int, batch: int, rows: int, cols: int, elem_bytes: int, stream: Optional[int] = None):
+    """src [batch, rows, cols] -> dst [batch, cols, rows] on the device (the weight prepack: [E,K,N] -> [E,N,K])."""
+    _check("msco_transpose_2d", load().msco_transpose_2d(ctypes.c_void_p(src), ctypes.c_void_p(dst), batch, rows, cols,
+                                                         elem_bytes, ctypes.c_void_p(stream if stream else None)))
 
 
 class GmmOp:

@@ -304,9 +304,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         if (p.scale_dtype == DT_BF16) t4_dma_b16(rs, lds, voff);
         else t4_dma_b32(rs, lds, voff);
       }
-      if (p.bias == nullptr) {
-        reinterpret_cast<int *>(table + 1024)[tid] = 0;
-      } else {
+      if (p.bias != nullptr) {
         const v4i rb = t4_raw_rsrc(p.bias + pg + cur.n0, (long long)(p.n - cur.n0) * 4);
         t4_dma_b32(rb, lds + 1024, col < p.n ? (unsigned)(tid * 4) : T4_OOB);
       }
@@ -407,6 +405,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
       asm volatile("" : "+v"(e_l32), "+v"(e_hh), "+v"(e_lane));
       const int n_base = cur.n0 + wave_n * T4_WT;
       const int m_base = cur.m0 + wave_m * T4_WT;
+      const bool has_bias = p.bias != nullptr;
       unsigned *tb_scale = reinterpret_cast<unsigned *>(table) + wave_n * T4_WT;
       const int *tb_bias = reinterpret_cast<const int *>(table + 1024) + wave_n * T4_WT;
       const float *tb_pt = reinterpret_cast<const float *>(table + 2048) + wave_m * T4_WT;
@@ -417,79 +416,101 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         t4_barrier();
       }
-      auto run_pass = [&](auto i_c, auto piece_c) {
+      // One column piece of the wave tile (16-bit outputs: a 64-column half; int32: a 32-column block):
+      // its scales are read once and kept in registers for the four 32-row blocks.  A wave's LDS
+      // operations execute in order, so the staging writes, the read-back and the next block's writes
+      // need no waits between them beyond the data dependencies the compiler tracks.
+      auto run_piece = [&](auto piece_c) {
         constexpr bool raw = MODE == 2;
-        constexpr int I = decltype(i_c)::value;
-        constexpr int PIECE = decltype(piece_c)::value;    // 16-bit outputs: 64-column half; int32: 32-column block
+        constexpr int PIECE = decltype(piece_c)::value;
         constexpr int esize = raw ? 4 : 2;
-        constexpr int f_lo = raw ? PIECE : 2 * PIECE, f_hi = raw ? PIECE + 1 : 2 * PIECE + 2;
-        if (I >= fm_active) return;
-        const float pt = tb_pt[32 * I + e_l32];
+        constexpr int NF = raw ? 1 : 2;                                   // 32-column MFMA blocks in the piece
+        constexpr int f_lo = NF * PIECE;
+        unsigned sraw[NF][2][8];
+        if constexpr (!raw) {
+#pragma unroll
+          for (int ff = 0; ff < NF; ++ff)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+              const int cw = 32 * (f_lo + ff) + 16 * s2 + 8 * e_hh;
+              const uint4 s_lo = *reinterpret_cast<const uint4 *>(tb_scale + cw);
+              const uint4 s_hi = *reinterpret_cast<const uint4 *>(tb_scale + cw + 4);
+              sraw[ff][s2][0] = s_lo.x; sraw[ff][s2][1] = s_lo.y; sraw[ff][s2][2] = s_lo.z; sraw[ff][s2][3] = s_lo.w;
+              sraw[ff][s2][4] = s_hi.x; sraw[ff][s2][5] = s_hi.y; sraw[ff][s2][6] = s_hi.z; sraw[ff][s2][7] = s_hi.w;
+            }
+        }
+        const int piece = e_lane & 7;
+        const int col = (raw ? 32 * PIECE : 64 * PIECE) + (raw ? 4 : 8) * piece;   // first column of this lane's read-back piece
+        const int n_first = n_base + col;
         unsigned char *dst = ep_stage + e_l32 * T4_EP_PITCH;
+        const unsigned char *src = ep_stage + (e_lane >> 3) * T4_EP_PITCH + piece * 16;
+        auto block = [&](auto i_c) {
+          constexpr int I = decltype(i_c)::value;
+          if (I >= fm_active) return;
+          const float pt = tb_pt[32 * I + e_l32];
 #pragma unroll
-        for (int f = f_lo; f < f_hi; ++f) {
+          for (int ff = 0; ff < NF; ++ff) {
 #pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) {
-            const int cw = 32 * f + 16 * s2 + 8 * e_hh;          // column inside the wave tile
-            const int cs = cw - 32 * f_lo;                       // column inside the staged piece
-            const uint4 s_lo = *reinterpret_cast<const uint4 *>(tb_scale + cw);
-            const uint4 s_hi = *reinterpret_cast<const uint4 *>(tb_scale + cw + 4);
-            const int4 b_lo = *reinterpret_cast<const int4 *>(tb_bias + cw);
-            const int4 b_hi = *reinterpret_cast<const int4 *>(tb_bias + cw + 4);
-            const unsigned sraw[8] = {s_lo.x, s_lo.y, s_lo.z, s_lo.w, s_hi.x, s_hi.y, s_hi.z, s_hi.w};
-            const int bi[8] = {b_lo.x, b_lo.y, b_lo.z, b_lo.w, b_hi.x, b_hi.y, b_hi.z, b_hi.w};
-            // accumulators leave the accumulation file here and not earlier (pinned: read ahead of time
-            // they would not fit into the architectural file next to the staging registers)
-            int a8[8];
+            for (int s2 = 0; s2 < 2; ++s2) {
+              const int f = f_lo + ff;
+              const int cw = 32 * f + 16 * s2 + 8 * e_hh;          // column inside the wave tile
+              const int cs = cw - 32 * f_lo;                       // column inside the staged piece
+              // accumulators leave the accumulation file here and not earlier (pinned: read ahead of time
+              // they would not fit into the architectural file next to the staging registers)
+              int a8[8];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a8[j]) : "a"(acc[f][I][8 * s2 + j]));
-            if constexpr (raw) {
-              int *d = reinterpret_cast<int *>(dst + cs * 4);
-              *reinterpret_cast<int4 *>(d) = make_int4(a8[0] + bi[0], a8[1] + bi[1], a8[2] + bi[2], a8[3] + bi[3]);
-              *reinterpret_cast<int4 *>(d + 4) = make_int4(a8[4] + bi[4], a8[5] + bi[5], a8[6] + bi[6], a8[7] + bi[7]);
-            } else {
-              float v[8];
-#pragma unroll
-              for (int j = 0; j < 8; ++j) v[j] = dequant(a8[j] + bi[j], __uint_as_float(sraw[j]), pt);
-              uint4 q;
-              if constexpr (MODE == 0) {
-                q.x = pack_bf16x2(v[0], v[1]); q.y = pack_bf16x2(v[2], v[3]);
-                q.z = pack_bf16x2(v[4], v[5]); q.w = pack_bf16x2(v[6], v[7]);
-              } else {
-                // the float32 product is rounded before the conversion (the golden's order); left visible,
-                // multiply and conversion are merged into one mixed-precision instruction that rounds once
-#pragma unroll
-                for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(v[j]));
-                q.x = f32_to_f16_rne(v[0]) | ((unsigned)f32_to_f16_rne(v[1]) << 16);
-                q.y = f32_to_f16_rne(v[2]) | ((unsigned)f32_to_f16_rne(v[3]) << 16);
-                q.z = f32_to_f16_rne(v[4]) | ((unsigned)f32_to_f16_rne(v[5]) << 16);
-                q.w = f32_to_f16_rne(v[6]) | ((unsigned)f32_to_f16_rne(v[7]) << 16);
+              for (int j = 0; j < 8; ++j) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a8[j]) : "a"(acc[f][I][8 * s2 + j]));
+              if (has_bias) {
+                const int4 b_lo = *reinterpret_cast<const int4 *>(tb_bias + cw);
+                const int4 b_hi = *reinterpret_cast<const int4 *>(tb_bias + cw + 4);
+                a8[0] += b_lo.x; a8[1] += b_lo.y; a8[2] += b_lo.z; a8[3] += b_lo.w;
+                a8[4] += b_hi.x; a8[5] += b_hi.y; a8[6] += b_hi.z; a8[7] += b_hi.w;
               }
-              *reinterpret_cast<uint4 *>(dst + cs * 2) = q;
+              if constexpr (raw) {
+                int *d = reinterpret_cast<int *>(dst + cs * 4);
+                *reinterpret_cast<int4 *>(d) = make_int4(a8[0], a8[1], a8[2], a8[3]);
+                *reinterpret_cast<int4 *>(d + 4) = make_int4(a8[4], a8[5], a8[6], a8[7]);
+              } else {
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = dequant(a8[j], __uint_as_float(sraw[ff][s2][j]), pt);
+                uint4 q;
+                if constexpr (MODE == 0) {
+                  q.x = pack_bf16x2(v[0], v[1]); q.y = pack_bf16x2(v[2], v[3]);
+                  q.z = pack_bf16x2(v[4], v[5]); q.w = pack_bf16x2(v[6], v[7]);
+                } else {
+                  // the float32 product is rounded before the conversion (the golden's order); left visible,
+                  // multiply and conversion are merged into one mixed-precision instruction that rounds once
+#pragma unroll
+                  for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(v[j]));
+                  q.x = f32_to_f16_rne(v[0]) | ((unsigned)f32_to_f16_rne(v[1]) << 16);
+                  q.y = f32_to_f16_rne(v[2]) | ((unsigned)f32_to_f16_rne(v[3]) << 16);
+                  q.z = f32_to_f16_rne(v[4]) | ((unsigned)f32_to_f16_rne(v[5]) << 16);
+                  q.w = f32_to_f16_rne(v[6]) | ((unsigned)f32_to_f16_rne(v[7]) << 16);
+                }
+                *reinterpret_cast<uint4 *>(dst + cs * 2) = q;
+              }
             }
           }
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const int piece = e_lane & 7;
-        const int col = (raw ? 32 * PIECE : 64 * PIECE) + (raw ? 4 : 8) * piece;   // first column of the piece in the wave tile
-        const int n_first = n_base + col;
+          // read back row-major: lane -> (row 8 t + lane / 8, 16-byte column piece lane % 8)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int row = 32 * I + 8 * t + (e_lane >> 3);
-          const uint4 q = *reinterpret_cast<const uint4 *>(ep_stage + (8 * t + (e_lane >> 3)) * T4_EP_PITCH + piece * 16);
-          if (row < rows_wave && n_first < p.n) {
-            unsigned char *o = reinterpret_cast<unsigned char *>(p.out) + ((long long)(m_base + row) * p.n + n_first) * esize;
-            *reinterpret_cast<uint4 *>(o) = q;
+          for (int t = 0; t < 4; ++t) {
+            const int row = 32 * I + 8 * t + (e_lane >> 3);
+            const uint4 q = *reinterpret_cast<const uint4 *>(src + 8 * t * T4_EP_PITCH);
+            if (row < rows_wave && n_first < p.n) {
+              unsigned char *o = reinterpret_cast<unsigned char *>(p.out) + ((long long)(m_base + row) * p.n + n_first) * esize;
+              *reinterpret_cast<uint4 *>(o) = q;
+            }
           }
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_sched_barrier(0);
+        };
+        block(c0); block(c1); block(c2); block(c3);
       };
-      auto for_i = [&](auto fn) { fn(c0); fn(c1); fn(c2); fn(c3); };
+      run_piece(c0);
+      run_piece(c1);
       if constexpr (MODE == 2) {
-        for_i([&](auto i) { run_pass(i, c0); run_pass(i, c1); run_pass(i, c2); run_pass(i, c3); });
-      } else {
-        for_i([&](auto i) { run_pass(i, c0); run_pass(i, c1); });
+        run_piece(c2);
+        run_piece(c3);
       }
     }
 
