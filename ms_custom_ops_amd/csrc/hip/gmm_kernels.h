@@ -18,6 +18,9 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream
 const char *tile_cfg_name(int tile_cfg);
 hipError_t launch_tile4_w8a8_nk(const GmmParams &p, hipStream_t stream);
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn);
+// K split across workgroups (p.split_k > 1; four-wave tile shapes only): partial tiles and arrival counters
+size_t tile_count_bound(int tile_cfg, int64_t m, int64_t n, int64_t e);
+size_t tile_workspace_bytes(int tile_cfg, int64_t m, int64_t n, int64_t e, int split_k);
 
 // Skinny (decode) kernels: one workgroup streams a 128-column weight strip of one group over a K
 // range; waves split K and reduce through LDS, workgroups split K and reduce through the workspace.

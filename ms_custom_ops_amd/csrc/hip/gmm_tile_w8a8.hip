@@ -150,8 +150,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     const int t = wave_scan_add(((e0 - s0 + BM - 1) / BM) * n_tiles, lane);
     total += wave_bcast(t, 63);
   }
+  // K split across workgroups (small problems): the slices of one tile sit next to each other in the
+  // grid, on the same XCD
+  const int split = p.split_k > 1 ? p.split_k : 1;
   const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
-  const int local = blockIdx.x / kNumXcd;
+  const int slot = blockIdx.x / kNumXcd;
+  const int local = slot / split, ks = slot - local * split;
   if (local >= per_xcd) return;
   const int lid = (blockIdx.x % kNumXcd) * per_xcd + local;
   if (lid >= total) return;
@@ -183,7 +187,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
 
   const int m0 = g_start + mt * BM;
   const int n0 = nt * BN;
-  const int k_slabs = (p.k + BK - 1) / BK;
+  const int k_slabs_all = (p.k + BK - 1) / BK;
+  const int per_slice = (k_slabs_all + split - 1) / split;
+  const int k_first = ks * per_slice;                                   // first slab of this workgroup's K slice
+  const int k_slabs = max(0, min(k_slabs_all, k_first + per_slice) - k_first);
 
   // Epilogue operands of this tile (scale and bias of its columns, per-token scale of its rows) are
   // requested now, parked in registers during the main loop and handed over through LDS, so that
@@ -231,7 +238,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   }
   auto issue_direct = [&](int kt) {
     const int stage = kt % NSTAGE;
-    const unsigned kbase = kt * BK;
+    const unsigned kbase = (k_first + kt) * BK;
     // K tail, and whole slabs past K (requested by the last steps of the branch-free loop): read as zero
     const unsigned kill = (kbase + d_c * 16 >= (unsigned)p.k) ? OOB : 0u;
 #pragma unroll
@@ -262,10 +269,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   unsigned rkn[NK ? 1 : KN_RING][8];
   auto load_kn = [&](int kt, int slot) {
     if constexpr (!NK) {
-      const unsigned voff = (kt * BK + 8 * kn_k8 >= p.k) ? OOB : bkn_voff;
+      const int kabs = (k_first + kt) * BK;
+      const unsigned voff = (kabs + 8 * kn_k8 >= p.k) ? OOB : bkn_voff;
 #pragma unroll
       for (int r = 0; r < 8; ++r)
-        rkn[slot][r] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff, (kt * BK + r) * p.n, 0);
+        rkn[slot][r] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff, (kabs + r) * p.n, 0);
     }
   };
   auto store_kn = [&](int kt, int slot) {
@@ -406,6 +414,43 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     if (kt + 1 < k_slabs) step(kt + 1, std::integral_constant<int, 1>{});
   }
   if (PINGPONG && !behind) phase_barrier();
+
+  // ---- K split: partial tiles meet in the workspace, the last slice to arrive adds them up ----------
+  // Every slice parks its accumulators (register by register, so the stores are contiguous across the
+  // workgroup), takes a ticket on the tile's counter, and all but the last one leave.  int32 addition
+  // is associative, so the result does not depend on the arrival order.  Agent-scope relaxed atomics
+  // keep the exchange in L2 without cache-wide fences; the counter resets itself for the next launch.
+  if (split > 1) {
+    __shared__ unsigned s_ticket;
+    constexpr int TILE_INTS = BM * BN;
+    int *base = p.partial + (long long)lid * split * TILE_INTS;
+    int *mine = base + (long long)ks * TILE_INTS + tid;
+#pragma unroll
+    for (int f = 0; f < FN; ++f)
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          __hip_atomic_store(mine + ((f * FM + i) * 16 + r) * NT, acc[f][i][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(&p.counters[lid], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != (unsigned)(split - 1)) return;
+    if (tid == 0) __hip_atomic_store(&p.counters[lid], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (int s = 0; s < split; ++s) {
+      if (s == ks) continue;
+      const int *other = base + (long long)s * TILE_INTS + tid;
+#pragma unroll
+      for (int f = 0; f < FN; ++f)
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[f][i][r] += __hip_atomic_load(other + ((f * FM + i) * 16 + r) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+
   float *ep_scale = reinterpret_cast<float *>(smem + PARAM_OFF);
   int *ep_bias = reinterpret_cast<int *>(smem + PARAM_OFF + 1024);
   float *ep_pt = reinterpret_cast<float *>(smem + PARAM_OFF + 2048);
@@ -521,7 +566,7 @@ static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
   const long long n_tiles = (p.n + BN - 1) / BN;
   const long long m_tiles_ub = (p.m + BM - 1) / BM + p.e;   // every non-empty group adds at most one partial tile
   const long long total_ub = m_tiles_ub * n_tiles;
-  const long long grid = ((total_ub + kNumXcd - 1) / kNumXcd) * kNumXcd;
+  const long long grid = ((total_ub + kNumXcd - 1) / kNumXcd) * kNumXcd * (p.split_k > 1 ? p.split_k : 1);
   if (grid <= 0) return hipSuccess;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(WAVES_M * WAVES_N * 64), lds, stream, p);
   return hipGetLastError();
@@ -554,6 +599,20 @@ const char *tile_cfg_name(int tile_cfg) {
     case TILE_256x256_W4: return "256x256x128_w4";
     default: return "?";
   }
+}
+
+// upper bound of the number of tiles (the real number depends on group_list, which only the device reads)
+size_t tile_count_bound(int tile_cfg, int64_t m, int64_t n, int64_t e) {
+  int bm, bn;
+  tile_cfg_dims(tile_cfg, &bm, &bn);
+  return (size_t)(((m + bm - 1) / bm + e) * ((n + bn - 1) / bn));
+}
+
+size_t tile_workspace_bytes(int tile_cfg, int64_t m, int64_t n, int64_t e, int split_k) {
+  if (split_k <= 1) return 0;
+  int bm, bn;
+  tile_cfg_dims(tile_cfg, &bm, &bn);
+  return tile_count_bound(tile_cfg, m, n, e) * (size_t)split_k * bm * bn * 4;
 }
 
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn) {

@@ -30,6 +30,9 @@ constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-st
 constexpr int kTargetWorkgroups = 512;  // skinny kernels with a K split: aim for this many workgroups (2 per CU)
 constexpr int kMaxSplitK = 8;             // keeps the last arriver's reduction to two rounds of loads
 constexpr int kNumCUs = 256;
+constexpr int kTileTargetWorkgroups = 256;   // tile kernels with a K split: aim for this many workgroups (one per CU)
+constexpr int kTileSplitMaxTiles = 128;      // ... and only split below this many tiles (measured: beyond it the partial-tile exchange costs more than it hides)
+constexpr int kTileMinSlabs = 4;               // 64-byte K slabs every slice keeps at least
 
 int env_int(const char *name, int fallback) {
   const char *v = std::getenv(name);
@@ -147,6 +150,21 @@ void choose_plan(msco_gmm_op *op) {
   if (family == FAM_TILE) {
     const int forced = env_int("MSCO_TILE_CFG", -1);
     if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO) op->tile_cfg = forced;
+    // Few tiles (M of a few hundred rows): split K across workgroups until about kTileTargetWorkgroups of them
+    // stream operands; every slice keeps at least kTileMinSlabs 64-byte K slabs.  Small tile shapes only.
+    if (op->tile_cfg == TILE_128x128 || op->tile_cfg == TILE_64x128) {
+      int bm, bn;
+      tile_cfg_dims(op->tile_cfg, &bm, &bn);
+      const int64_t t = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+      const int target = env_int("MSCO_TILE_TARGET_WGS", kTileTargetWorkgroups);
+      int want = t <= kTileSplitMaxTiles ? (int)((target + t / 2) / std::max<int64_t>(t, 1)) : 1;
+      const int cap = (int)std::max<int64_t>(1, ((k + 63) / 64) / kTileMinSlabs);
+      want = std::max(1, std::min(std::min(want, kMaxSplitK), cap));
+      const int forced_split = env_int("MSCO_TILE_SPLIT_K", 0);
+      if (forced_split > 0) want = std::min(forced_split, cap);
+      op->split_k = want;
+      op->workspace_bytes = tile_workspace_bytes(op->tile_cfg, m, n, e, op->split_k);
+    }
   }
   if (family == FAM_SKINNY) {
     // grid.y enumerates (group, 16-row chunk)
@@ -238,8 +256,9 @@ int msco_gmm_plan(msco_gmm_handle h, int64_t m, int64_t k, int64_t n, int64_t e,
   std::lock_guard<std::mutex> lock(h->mu);
   h->m = m; h->k = k; h->n = n; h->e = e;
   choose_plan(h);
-  if (h->family == FAM_SKINNY && h->split_k > 1) {
-    const size_t need = skinny_counter_count(m, n, e, h->skinny_cols);
+  if ((h->family == FAM_SKINNY || h->family == FAM_TILE) && h->split_k > 1) {
+    const size_t need = h->family == FAM_TILE ? tile_count_bound(h->tile_cfg, m, n, e)
+                                              : skinny_counter_count(m, n, e, h->skinny_cols);
     if (need > h->counters_cap) {
       if (h->counters) (void)hipFree(h->counters);
       h->counters = nullptr;

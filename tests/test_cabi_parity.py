@@ -160,6 +160,14 @@ def test_dense_equal_groups_without_group_list(device):
         assert np.array_equal(got, ref)
 
 
+@pytest.mark.parametrize("transpose_b", [False, True])
+def test_few_tiles_split_k_across_workgroups(device, transpose_b):
+    # 2 x 8 tiles of 64 x 128: the plan splits K across workgroups; partial tiles meet in the workspace
+    rng, x, w, bias, scale, pt = _inputs(23, 100, 2064, 1024, 2)
+    info = _check(x, w, [37, 100], bias, scale, pt, transpose_b=transpose_b, override=cabi.OV_AUTO)
+    assert "tile_64x128" in info and "split_k=1 " not in info
+
+
 # ------------------------------------------------------------- persistent four-wave tile kernel
 W4 = cabi.OV_TILE_256_W4
 
