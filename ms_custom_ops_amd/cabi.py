@@ -27,7 +27,8 @@ IN_COUNT = 8
 OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC, OV_TILE_256_W4 = range(7)
 
 EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco_gmm_plan_info", "msco_gmm_destroy",
-                    "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d")
+                    "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
+                    "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_token_unpermute")
 
 
 class GmmDesc(ctypes.Structure):
@@ -73,6 +74,13 @@ def load():
         lib.msco_transpose_2d.restype = ctypes.c_int
         lib.msco_transpose_2d.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                           ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_moe_init_routing_v2_workspace_bytes.restype = ctypes.c_size_t
+        lib.msco_moe_init_routing_v2_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]
+        lib.msco_moe_init_routing_v2.restype = ctypes.c_int
+        lib.msco_moe_init_routing_v2.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_size_t] + [ctypes.c_int64] * 4 + \
+                                                [ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_moe_token_unpermute.restype = ctypes.c_int
+        lib.msco_moe_token_unpermute.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int64] * 3 + [ctypes.c_int32, ctypes.c_void_p]
         _lib = lib
     return _lib
 
@@ -90,6 +98,28 @@ def transpose_2d(src: int, dst: int, batch: int, rows: int, cols: int, elem_byte
     """src [batch, rows, cols] -> dst [batch, cols, rows] on the device (the weight prepack: [E,K,N] -> [E,N,K])."""
     _check("msco_transpose_2d", load().msco_transpose_2d(ctypes.c_void_p(src), ctypes.c_void_p(dst), batch, rows, cols,
                                                          elem_bytes, ctypes.c_void_p(stream if stream else None)))
+
+
+def moe_init_routing_v2_workspace_bytes(num_rows: int, k: int, expert_num: int) -> int:
+    return int(load().msco_moe_init_routing_v2_workspace_bytes(num_rows, k, expert_num))
+
+
+def moe_init_routing_v2(x: int, expert_idx: int, expanded_x: int, expanded_row_idx: int, tokens: Optional[int],
+                        before_capacity: Optional[int], workspace: int, workspace_bytes: int, num_rows: int, hidden: int,
+                        k: int, expert_num: int, elem_bytes: int, flag: int, stream: Optional[int] = None):
+    """Raw-pointer call of msco_moe_init_routing_v2 (see include/msco_moe.h)."""
+    vp = lambda v: ctypes.c_void_p(v if v else None)
+    _check("msco_moe_init_routing_v2", load().msco_moe_init_routing_v2(
+        vp(x), vp(expert_idx), vp(expanded_x), vp(expanded_row_idx), vp(tokens), vp(before_capacity), vp(workspace),
+        workspace_bytes, num_rows, hidden, k, expert_num, elem_bytes, flag, vp(stream)))
+
+
+def moe_token_unpermute(permuted: int, sorted_indices: int, probs: int, out: int, num_tokens: int, top_k: int, hidden: int,
+                        dtype: int, stream: Optional[int] = None):
+    """Raw-pointer call of msco_moe_token_unpermute (see include/msco_moe.h)."""
+    vp = lambda v: ctypes.c_void_p(v if v else None)
+    _check("msco_moe_token_unpermute", load().msco_moe_token_unpermute(vp(permuted), vp(sorted_indices), vp(probs), vp(out),
+                                                                       num_tokens, top_k, hidden, dtype, vp(stream)))
 
 
 class GmmOp:

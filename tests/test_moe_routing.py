@@ -1,0 +1,192 @@
+"""moe_init_routing_v2 and moe_token_unpermute: oracle pins (CPU) and GPU parity through the C ABI.
+
+The oracle restates the reference goldens (tests/st/test_custom_moe_init_routing_v2.py:33-93,
+tests/st/test_custom_moe_token_unpermute.py:37-47).  Bar on the GPU: integer outputs and gathered rows
+bit-exact; the un-permutation bit-exact too, because the kernel rounds where the golden rounds (the
+reference's own tolerance is rtol = atol = 1e-3)."""
+import numpy as np
+import pytest
+import torch
+
+from ms_custom_ops_amd import cabi
+from oracle import moe_oracle as M
+
+
+# ----------------------------------------------------------------------------------- oracle pins (CPU)
+def test_routing_oracle_tiny_case_by_hand():
+    # 3 tokens, k = 2, 3 experts: flat expert ids [2, 0, 1, 2, 0, 0]; stable order of flat positions: 1, 4, 5 | 2 | 0, 3
+    x = np.arange(12, dtype=np.float16).reshape(3, 4)
+    ex, idx, tok = M.moe_init_routing_v2(x, np.array([[2, 0], [1, 2], [0, 0]], dtype=np.int32), 3, 1)
+    assert idx.tolist() == [4, 0, 3, 5, 1, 2]
+    assert np.array_equal(ex, x[[0, 2, 2, 1, 0, 1]])
+    assert tok.tolist() == [3, 4, 6]
+    assert M.moe_init_routing_v2(x, np.array([[2, 0], [1, 2], [0, 0]], dtype=np.int32), 3, 2)[2].tolist() == [3, 1, 2]
+
+
+@pytest.mark.parametrize("n_rows,k,e", [(1, 1, 1), (17, 2, 8), (130, 6, 64), (64, 8, 256)])
+def test_routing_oracle_against_independent_sort_and_invariants(n_rows, k, e):
+    rng = np.random.default_rng(n_rows)
+    x = rng.uniform(-1, 1, (n_rows, 16)).astype(np.float16)
+    idx = rng.integers(0, e, (n_rows, k)).astype(np.int32)
+    ex, ridx, cum = M.moe_init_routing_v2(x, idx, e, 1)
+    ex2, ridx2, counts = M.moe_init_routing_v2_by_loops(x, idx, e)
+    assert np.array_equal(ex, ex2) and np.array_equal(ridx, ridx2) and np.array_equal(cum, np.cumsum(counts))
+    assert sorted(ridx.tolist()) == list(range(n_rows * k))                       # a permutation
+    flat = idx.reshape(-1)
+    dest_expert = np.empty(n_rows * k, dtype=np.int64)
+    dest_expert[ridx] = flat
+    assert np.all(np.diff(dest_expert) >= 0)                                      # rows end up sorted by expert
+    for e_id in range(e):                                                         # stable inside every expert
+        pos = np.nonzero(flat == e_id)[0]
+        assert np.all(np.diff(ridx[pos]) > 0)
+    assert np.array_equal(ex[ridx], np.repeat(x, k, axis=0))                      # every entry got its token's row
+    assert cum[-1] == n_rows * k
+
+
+def test_unpermute_oracle_against_scalar_loops_and_closed_forms():
+    rng = np.random.default_rng(3)
+    t, k, h = 9, 4, 32
+    pt = rng.standard_normal((t * k, h)).astype(np.float16)
+    pr = rng.standard_normal((t, k)).astype(np.float16)
+    si = rng.permutation(t * k).astype(np.int32)
+    got = M.moe_token_unpermute(pt, si, pr)
+    # scalar loops with an independent half implementation (torch): round the product, then the running sum
+    ref = torch.zeros(t, h, dtype=torch.float16)
+    tp, tr = torch.from_numpy(pt), torch.from_numpy(pr)
+    for i in range(t):
+        for kk in range(k):
+            prod = (tr[i, kk].float() * tp[int(si[i * k + kk])].float()).half()
+            ref[i] = (ref[i].float() + prod.float()).half()
+    assert np.array_equal(got.view(np.uint16), ref.numpy().view(np.uint16))
+    # K = 1 with probability one is a plain gather; all-ones data sums to K exactly
+    assert np.array_equal(M.moe_token_unpermute(pt[:t], si[:t] % t, np.ones((t, 1), np.float16)), pt[:t][si[:t] % t])
+    ones = M.moe_token_unpermute(np.ones((t * k, h), np.float16), si, np.ones((t, k), np.float16))
+    assert np.all(ones == k)
+    # bfloat16 variant against torch's bfloat16 arithmetic
+    pb = torch.randn(t * k, h).bfloat16()
+    rb = torch.randn(t, k).bfloat16()
+    ref_b = torch.zeros(t, h, dtype=torch.bfloat16)
+    for i in range(t):
+        for kk in range(k):
+            prod = (rb[i, kk].float() * pb[int(si[i * k + kk])].float()).bfloat16()
+            ref_b[i] = (ref_b[i].float() + prod.float()).bfloat16()
+    got_b = M.moe_token_unpermute_bf16(pb.view(torch.int16).numpy().view(np.uint16), si, rb.view(torch.int16).numpy().view(np.uint16))
+    assert np.array_equal(got_b, ref_b.view(torch.int16).numpy().view(np.uint16))
+
+
+def test_c_abi_exports_the_moe_entry_points_and_rejects_bad_shapes():
+    lib = cabi.load()
+    for name in ("msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_token_unpermute"):
+        assert hasattr(lib, name)
+    assert cabi.moe_init_routing_v2_workspace_bytes(4096, 2, 8) == (8 * 8 + 8192) * 4
+    # argument checks happen before anything touches a device
+    with pytest.raises(cabi.BackendError):
+        cabi.moe_token_unpermute(1, 1, 1, 1, 4, 8, 1001, cabi.DT_F16)        # hidden not a multiple of 8
+    with pytest.raises(cabi.BackendError):
+        cabi.moe_init_routing_v2(1, 1, 1, 1, 1, None, 1, 1 << 20, 4, 1024, 2, 2000, 2, 1)   # more than 1024 experts
+
+
+# ----------------------------------------------------------------------------------- GPU parity
+def _route_gpu(x, idx, e, flag):
+    n_rows, h = x.shape
+    k = idx.shape[1]
+    dev = "cuda:0"
+    view = {1: np.int8, 2: np.int16, 4: np.int32}[x.dtype.itemsize]
+    tx = torch.from_numpy(np.ascontiguousarray(x).view(view)).to(dev)
+    ti = torch.from_numpy(idx).to(dev)
+    ex = torch.full((n_rows * k, h), 77, dtype=tx.dtype, device=dev)
+    ridx = torch.full((n_rows * k,), -5, dtype=torch.int32, device=dev)
+    tok = torch.full((e,), -5, dtype=torch.int32, device=dev)
+    cap = torch.full((e,), -5, dtype=torch.int32, device=dev)
+    wsb = cabi.moe_init_routing_v2_workspace_bytes(n_rows, k, e)
+    ws = torch.empty(max(wsb, 1), dtype=torch.uint8, device=dev)
+    for _ in range(2):   # twice: nothing may depend on what the previous call left in the workspace
+        cabi.moe_init_routing_v2(tx.data_ptr(), ti.data_ptr(), ex.data_ptr(), ridx.data_ptr(), tok.data_ptr(), cap.data_ptr(),
+                                 ws.data_ptr(), wsb, n_rows, h, k, e, x.dtype.itemsize, flag, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return ex.cpu().numpy().view(x.dtype), ridx.cpu().numpy(), tok.cpu().numpy(), cap.cpu().numpy()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_rows,h,k,e,flag", [(1, 1024, 1, 1, 1), (10, 2048, 8, 8, 1), (1001, 1024, 2, 8, 2),
+                                              (513, 1024, 6, 64, 1), (300, 7168, 4, 256, 1)])
+def test_init_routing_matches_the_golden(n_rows, h, k, e, flag):
+    np.random.seed(0)                                                             # the reference test's stream (:102-104)
+    x = np.random.uniform(-1, 1, size=(n_rows, h)).astype(np.float16)
+    idx = np.random.randint(0, e, size=(n_rows, k)).astype(np.int32)
+    ex, ridx, tok, cap = _route_gpu(x, idx, e, flag)
+    ref_x, ref_idx, ref_tok = M.moe_init_routing_v2(x, idx, e, flag)
+    assert np.array_equal(ridx, ref_idx)
+    assert np.array_equal(tok, ref_tok)
+    assert np.array_equal(ex.view(np.uint16), ref_x.view(np.uint16))
+    assert np.all(cap == 0)
+
+
+@pytest.mark.gpu
+def test_init_routing_skewed_experts_int8_rows_and_mixtral_shape():
+    # Zipf-skewed expert popularity with empty experts, int8 activations (the quantised input of the grouped matmul)
+    rng = np.random.default_rng(5)
+    e, k, n_rows, h = 64, 6, 2048, 2048
+    pop = 1.0 / np.arange(1, e + 1) ** 1.2
+    idx = np.stack([rng.choice(e, size=k, replace=False, p=pop / pop.sum()) for _ in range(n_rows)]).astype(np.int32)
+    idx[idx == 63] = 0                                                            # expert 63 stays empty
+    x = rng.integers(-127, 128, (n_rows, h), dtype=np.int8)
+    ex, ridx, tok, _ = _route_gpu(x, idx, e, 1)
+    ref_x, ref_idx, ref_tok = M.moe_init_routing_v2(x, idx, e, 1)
+    assert np.array_equal(ridx, ref_idx) and np.array_equal(tok, ref_tok) and np.array_equal(ex, ref_x)
+    assert tok[-1] == tok[-2] == n_rows * k
+    # the routing of the headline matmul workload: 4096 tokens, top-2 of 8 experts
+    idx = np.argsort(-rng.standard_normal((4096, 8)), axis=1)[:, :2].astype(np.int32)
+    x = rng.integers(-127, 128, (4096, 4096), dtype=np.int8)
+    ex, ridx, tok, _ = _route_gpu(x, idx, 8, 1)
+    ref_x, ref_idx, ref_tok = M.moe_init_routing_v2(x, idx, 8, 1)
+    assert np.array_equal(ridx, ref_idx) and np.array_equal(tok, ref_tok) and np.array_equal(ex, ref_x)
+
+
+def _unpermute_gpu(pt_bits, si, pr_bits, dtype):
+    dev = "cuda:0"
+    t, k = pr_bits.shape
+    h = pt_bits.shape[1]
+    tp = torch.from_numpy(pt_bits.view(np.int16)).to(dev)
+    ts = torch.from_numpy(si).to(dev)
+    tr = torch.from_numpy(pr_bits.view(np.int16)).to(dev)
+    out = torch.full((t, h), 0x7FC0, dtype=torch.int16, device=dev)
+    cabi.moe_token_unpermute(tp.data_ptr(), ts.data_ptr(), tr.data_ptr(), out.data_ptr(), t, k, h, dtype,
+                             torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return out.cpu().numpy().view(np.uint16)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("token_num", [1, 16, 1001])
+@pytest.mark.parametrize("hidden", [7168, 2048])
+@pytest.mark.parametrize("top_k", [8, 2])
+def test_token_unpermute_matches_the_golden(token_num, hidden, top_k):
+    np.random.seed(token_num + hidden)
+    pt = np.random.randn(token_num * top_k, hidden).astype(np.float16)            # inputs as the reference test draws them (:66-70)
+    si = np.arange(token_num * top_k, dtype=np.int32)
+    np.random.shuffle(si)
+    pr = np.random.randn(token_num, top_k).astype(np.float16)
+    got = _unpermute_gpu(pt.view(np.uint16), si, pr.view(np.uint16), cabi.DT_F16)
+    ref = M.moe_token_unpermute(pt, si, pr)
+    assert np.allclose(got.view(np.float16), ref, rtol=1e-3, atol=1e-3)           # the reference's tolerance
+    assert np.array_equal(got, ref.view(np.uint16))                               # and bit-exact
+
+
+@pytest.mark.gpu
+def test_token_unpermute_bf16_and_round_trip_with_routing():
+    rng = np.random.default_rng(11)
+    t, k, h = 257, 4, 1024
+    pt = (rng.standard_normal((t * k, h)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    pr = (rng.standard_normal((t, k)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    si = rng.permutation(t * k).astype(np.int32)
+    got = _unpermute_gpu(pt, si, pr, cabi.DT_BF16)
+    assert np.array_equal(got, M.moe_token_unpermute_bf16(pt, si, pr))
+    # routing followed by un-permutation with weights 1, 0, 0, 0 returns every token's own row
+    x = rng.standard_normal((t, h)).astype(np.float16)
+    idx = rng.integers(0, 8, (t, k)).astype(np.int32)
+    ex, ridx, _, _ = _route_gpu(x, idx, 8, 1)
+    probs = np.zeros((t, k), np.float16)
+    probs[:, 0] = 1
+    back = _unpermute_gpu(ex.view(np.uint16), ridx, probs.view(np.uint16), cabi.DT_F16)
+    assert np.array_equal(back, x.view(np.uint16))
