@@ -13,6 +13,12 @@ Drop-in for the grouped / dense quantized matmul entries of ms_custom_ops
     quant_batch_matmul(x1, x2, scale, offset=None, bias=None, pertoken_scale=None,
                        transpose_x1=False, transpose_x2=False, x2_format="ND", output_dtype=float16)
 
+and for the two MoE steps on either side of the grouped matmul:
+
+    moe_init_routing_v2(x, expert_idx, active_num, expert_capacity, expert_num, drop_pad_mode,
+                        expert_tokens_count_or_cumsum_flag, expert_tokens_before_capacity_flag)
+    moe_token_unpermute(permuted_tokens, sorted_indices, probs, padded_mode=False, restore_shape=None)
+
 Tensors are PyTorch-ROCm tensors on the GPU; PyTorch only provides device memory and the current
 stream.  The compiled operator layer (``ms_custom_ops_amd.ms_custom_ops``, pybind11) validates and
 plans, and the HIP backend behind the C ABI (``lib/libmsco_gmm.so``) does the work.  There is no
@@ -38,7 +44,8 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
         "ms_custom_ops_amd: the compiled operator module is missing; run `python ms_custom_ops_amd/build.py` "
         "(needs hipcc for gfx950 and g++). There is no fallback implementation.") from exc
 
-__all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "set_context", "get_context", "exec_mode",
+__all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "moe_init_routing_v2", "moe_token_unpermute",
+           "set_context", "get_context", "exec_mode",
            "GRAPH_MODE", "PYNATIVE_MODE", "dtype_to_type_id", "type_id_to_dtype", "plan_cache_stats", "trans_data"]
 
 GRAPH_MODE = 0
@@ -172,6 +179,32 @@ def quant_batch_matmul(x1, x2, scale, offset=None, bias=None, pertoken_scale=Non
         return _C._graph_run("quant_batch_matmul", args)[0].owner
     return _C.quant_batch_matmul(_wrap(x1), _wrap(x2), _wrap(scale), _wrap(offset), _wrap(bias), _wrap(pertoken_scale),
                                  bool(transpose_x1), bool(transpose_x2), str(x2_format), od).owner
+
+
+def moe_init_routing_v2(x, expert_idx, active_num, expert_capacity, expert_num, drop_pad_mode,
+                        expert_tokens_count_or_cumsum_flag, expert_tokens_before_capacity_flag):
+    """Dropless MoE routing in front of the grouped matmul (ops/c_api/moe_init_routing_v2/moe_init_routing_v2.cc:238-242):
+    returns (expanded_x, expanded_row_idx, expert_tokens_count_or_cumsum, expert_tokens_before_capacity)."""
+    if _mode == GRAPH_MODE:
+        args = [_wrap(x), _wrap(expert_idx), int(active_num), int(expert_capacity), int(expert_num), int(drop_pad_mode),
+                int(expert_tokens_count_or_cumsum_flag), bool(expert_tokens_before_capacity_flag)]
+        outs = _C._graph_run("moe_init_routing_v2", args)
+    else:
+        outs = _C.moe_init_routing_v2(_wrap(x), _wrap(expert_idx), int(active_num), int(expert_capacity), int(expert_num),
+                                      int(drop_pad_mode), int(expert_tokens_count_or_cumsum_flag),
+                                      bool(expert_tokens_before_capacity_flag))
+    return tuple(o.owner for o in outs)
+
+
+def moe_token_unpermute(permuted_tokens, sorted_indices, probs, padded_mode=False, restore_shape=None):
+    """Weighted un-permutation behind the grouped matmul
+    (ops/c_api/moe_token_unpermute/moe_token_unpermute.cc:152-156): out[i] = sum_k probs[i, k] * permuted_tokens[sorted_indices[i*K + k]]."""
+    if _mode == GRAPH_MODE:
+        args = [_wrap(permuted_tokens), _wrap(sorted_indices), _wrap(probs), bool(padded_mode),
+                None if restore_shape is None else str(tuple(restore_shape))]
+        return _C._graph_run("moe_token_unpermute", args)[0].owner
+    return _C.moe_token_unpermute(_wrap(permuted_tokens), _wrap(sorted_indices), _wrap(probs), bool(padded_mode),
+                                  None if restore_shape is None else [int(v) for v in restore_shape]).owner
 
 
 def trans_data(tensor, transdata_type=1):
