@@ -32,8 +32,10 @@ I8, I32, I64, U64, F16, F32, BF16 = 32, 34, 35, 40, 42, 43, 45
 
 # ------------------------------------------------------------------------------------- C ABI surface
 def test_header_symbols_are_exported():
-    header = open(os.path.join(REPO, "include", "msco_gmm.h")).read()
-    declared = set(re.findall(r"MSCO_API\s+[\w\s\*]+?\b(msco_\w+)\s*\(", header))
+    declared = set()
+    for name in sorted(os.listdir(os.path.join(REPO, "include"))):   # every header: msco_gmm.h, msco_moe.h
+        header = open(os.path.join(REPO, "include", name)).read()
+        declared |= set(re.findall(r"MSCO_API\s+[\w\s\*]+?\b(msco_\w+)\s*\(", header))
     assert declared == set(cabi.EXPORTED_SYMBOLS)
     lib = cabi.load()
     for name in declared:
