@@ -163,6 +163,57 @@ def cpu_baseline(wl, budget_s=15.0):
                       "numpy float32 dot per group + dequant epilogue + bf16 cast"}
 
 
+def moe_neighbours(steps, warmup):
+    """The routing step in front of the grouped matmul and the un-permutation behind it, on the shapes of the
+    headline MoE layer: HBM-bound row copies, reported as algorithmic bytes per second."""
+    import torch
+    from ms_custom_ops_amd import cabi
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    out = []
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for a, b in ev:
+            a.record()
+            fn()
+            b.record()
+        torch.cuda.synchronize()
+        return sum(a.elapsed_time(b) for a, b in ev) / steps * 1e-3
+
+    # routing: 4096 tokens x top-2 of 8 experts, int8 activations of width K = 4096 (the x of c3)
+    rows, k, e, h = 4096, 2, 8, 4096
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    x = torch.randint(-127, 128, (rows, h), dtype=torch.int8, device=dev, generator=g)
+    idx = torch.argsort(torch.randn(rows, e, device=dev, generator=g), dim=1, descending=True)[:, :k].to(torch.int32).contiguous()
+    ex = torch.empty((rows * k, h), dtype=torch.int8, device=dev)
+    ridx = torch.empty(rows * k, dtype=torch.int32, device=dev)
+    tok = torch.empty(e, dtype=torch.int32, device=dev)
+    wsb = cabi.moe_init_routing_v2_workspace_bytes(rows, k, e)
+    ws = torch.empty(max(wsb, 1), dtype=torch.uint8, device=dev)
+    sec = timed(lambda: cabi.moe_init_routing_v2(x.data_ptr(), idx.data_ptr(), ex.data_ptr(), ridx.data_ptr(), tok.data_ptr(), None,
+                                                 ws.data_ptr(), wsb, rows, h, k, e, 1, 1, st))
+    byts = rows * h + rows * k * h + rows * k * 4 * 2 + e * 4          # x read once, expanded_x written, indices in and out
+    out.append({"workload": f"moe_init_routing_v2: {rows} tokens x top-{k} of {e} experts, int8 rows of {h}", "launch_us": sec * 1e6,
+                "gbs": byts / sec / 1e9, "hbm_frac": byts / sec / 1e9 / PEAK_HBM_GBS, "bytes_per_launch": byts})
+
+    # un-permutation: 4096 tokens x top-8, float16 rows of 7168 (the reference op's largest supported shape class)
+    t, k, h = 4096, 8, 7168
+    pt = torch.randn((t * k, h), dtype=torch.float16, device=dev, generator=g)
+    si = torch.randperm(t * k, device=dev, generator=g).to(torch.int32)
+    pr = torch.randn((t, k), dtype=torch.float16, device=dev, generator=g)
+    o = torch.empty((t, h), dtype=torch.float16, device=dev)
+    sec = timed(lambda: cabi.moe_token_unpermute(pt.data_ptr(), si.data_ptr(), pr.data_ptr(), o.data_ptr(), t, k, h, cabi.DT_F16, st))
+    byts = t * k * h * 2 + t * h * 2 + t * k * (4 + 2)
+    out.append({"workload": f"moe_token_unpermute: {t} tokens x top-{k}, float16 rows of {h}", "launch_us": sec * 1e6,
+                "gbs": byts / sec / 1e9, "hbm_frac": byts / sec / 1e9 / PEAK_HBM_GBS, "bytes_per_launch": byts})
+    return out
+
+
 def measured_traffic(workload, layout, kernel):
     """HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs (scaled by
     the same counters' reading for a copy of known size); None when no measurement of this kernel is on file."""
@@ -268,6 +319,7 @@ def main():
             del p2
             torch.cuda.empty_cache()
         result["sweep"] = sweep
+        result["moe_neighbours"] = moe_neighbours(max(20, min(100, args.steps)), 10)
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(wl)

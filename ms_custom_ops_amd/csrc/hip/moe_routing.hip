@@ -4,8 +4,8 @@
 //   init_routing   1. per block of 1024 entries: histogram of the expert ids (LDS atomics)
 //                  2. one workgroup: per expert, exclusive scan over the blocks, then over the experts;
 //                     writes the count / cumulative-count output
-//                  3. per block, one wavefront walks its entries 64 at a time in flat order and ranks
-//                     them among equal expert ids with ballots, which keeps the sort stable
+//                  3. per block, sixteen wavefronts rank 64 consecutive entries each among equal expert ids with
+//                     ballots; a prefix over the sixteen chunks keeps the flat order, so the sort is stable
 //                  4. one workgroup per output row copies x[token] with 16-byte loads and stores
 //   unpermute      one workgroup per token: 16 bytes of every selected row per lane, the running sum kept
 //                  in the element type and rounded exactly where the golden rounds it
@@ -70,33 +70,44 @@ __global__ void __launch_bounds__(1024) route_scan_kernel(int *block_hist, int *
   }
 }
 
-__global__ void __launch_bounds__(64) route_rank_kernel(const int *expert_idx, const int *block_first, int *expanded_row_idx,
-                                                        int *sorted_src, long long n, int expert_num) {
-  __shared__ int next[kMaxExperts];
-  const int lane = threadIdx.x;
-  for (int e = lane; e < expert_num; e += 64) next[e] = block_first[(long long)blockIdx.x * expert_num + e];
+// One block of 1024 entries, sixteen wavefronts of 64 consecutive entries each.  A wavefront ranks its entries among
+// equal expert ids with ballots (one round per distinct id in the chunk) and leaves the chunk's per-expert counts
+// in LDS; a prefix over the sixteen chunks turns the counts into first positions; rank + first position is the
+// output row.  Chunks, and positions inside a chunk, are taken in flat order, so the sort is stable.
+__global__ void __launch_bounds__(1024) route_rank_kernel(const int *expert_idx, const int *block_first, int *expanded_row_idx,
+                                                          int *sorted_src, long long n, int expert_num) {
+  extern __shared__ int chunk_first[];   // [16][expert_num]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int *mine = chunk_first + wave * expert_num;
+  for (int e = lane; e < expert_num; e += 64) mine[e] = 0;
+  const long long i = (long long)blockIdx.x * kRouteBlock + threadIdx.x;
+  const bool live = i < n;
+  const int e = live ? clamp_expert(expert_idx[i], expert_num) : -1;
+  unsigned long long todo = __ballot(live);
+  int rank = 0;
+  while (todo) {
+    const int leader = __ffsll((long long)todo) - 1;
+    const int e0 = __shfl(e, leader);
+    const unsigned long long same = __ballot(e == e0) & todo;
+    if (e == e0) rank = __popcll(same & ((1ull << lane) - 1ull));
+    if (lane == leader) mine[e0] = __popcll(same);      // after the zero fill above: one wavefront's LDS operations stay in order
+    todo &= ~same;
+  }
   __syncthreads();
-  const long long first = (long long)blockIdx.x * kRouteBlock;
-  for (int c = 0; c < kRouteBlock / 64; ++c) {
-    const long long i = first + c * 64 + lane;
-    const bool live = i < n;
-    const int e = live ? clamp_expert(expert_idx[i], expert_num) : -1;
-    unsigned long long todo = __ballot(live);
-    int dest = 0;
-    while (todo) {
-      const int leader = __ffsll((long long)todo) - 1;
-      const int e0 = __shfl(e, leader);
-      const unsigned long long same = __ballot(e == e0) & todo;
-      if (e == e0 && live) dest = next[e0] + __popcll(same & ((1ull << lane) - 1ull));
-      __syncthreads();                                   // one wavefront: orders the LDS read above and the update below
-      if (lane == leader) next[e0] += __popcll(same);
-      __syncthreads();
-      todo &= ~same;
+  for (int x = threadIdx.x; x < expert_num; x += 1024) {
+    int running = block_first[(long long)blockIdx.x * expert_num + x];
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int c = chunk_first[w * expert_num + x];
+      chunk_first[w * expert_num + x] = running;
+      running += c;
     }
-    if (live) {
-      expanded_row_idx[i] = dest;
-      sorted_src[dest] = (int)i;
-    }
+  }
+  __syncthreads();
+  if (live) {
+    const int dest = mine[e] + rank;
+    expanded_row_idx[i] = dest;
+    sorted_src[dest] = (int)i;
   }
 }
 
@@ -119,36 +130,90 @@ __device__ __forceinline__ float from_elem(unsigned short b) {
   return BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b);
 }
 
-template <bool BF16>
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+
+// K: top_k as a compile-time constant (the row indices, the probabilities and the K row pieces of a pass are then all
+// requested before the first one is used; with a run-time loop every step waits for two dependent loads), 0: any top_k
+template <bool BF16, int K>
 __global__ void __launch_bounds__(256) unpermute_kernel(const unsigned short *permuted, const int *sorted_indices,
-                                                        const unsigned short *probs, unsigned short *out, int top_k,
+                                                        const unsigned short *probs, unsigned short *out, int top_k_arg,
                                                         long long hidden) {
   const long long token = blockIdx.x;
-  for (long long h0 = (long long)threadIdx.x * 8; h0 < hidden; h0 += 256 * 8) {
-    unsigned short acc[8];
+  const int top_k = K > 0 ? K : top_k_arg;
+  constexpr int KK = K > 0 ? K : 1;
+  long long rows[KK];
+  unsigned short pbs[KK];
+  if constexpr (K > 0) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] = 0;
-    for (int kk = 0; kk < top_k; ++kk) {
-      const long long row = sorted_indices[token * top_k + kk];
-      const float p = from_elem<BF16>(probs[token * top_k + kk]);
-      const uint4 q = *reinterpret_cast<const uint4 *>(permuted + row * hidden + h0);
-      const unsigned w[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const unsigned short v = (unsigned short)(w[j >> 1] >> (16 * (j & 1)));
-        // product rounded to the element type, then the running sum rounded to it: two float32 operations,
-        // kept apart (no fused multiply-add) because the golden rounds in between
-        float prod = p * from_elem<BF16>(v);
-        asm volatile("" : "+v"(prod));
-        const float prod_r = from_elem<BF16>(to_elem<BF16>(prod));
-        float sum = from_elem<BF16>(acc[j]) + prod_r;
-        asm volatile("" : "+v"(sum));
-        acc[j] = to_elem<BF16>(sum);
-      }
+    for (int kk = 0; kk < K; ++kk) {
+      rows[kk] = sorted_indices[token * K + kk];
+      pbs[kk] = probs[token * K + kk];
     }
+  }
+  // blockIdx.y walks the row in pieces of 2048 elements: one pass per workgroup, so nothing waits for a previous pass
+  for (long long h0 = ((long long)blockIdx.y * 256 + threadIdx.x) * 8; h0 < hidden; h0 += (long long)gridDim.y * 256 * 8) {
+    uint4 pieces[KK];
+    if constexpr (K > 0) {
+#pragma unroll
+      for (int kk = 0; kk < K; ++kk) pieces[kk] = *reinterpret_cast<const uint4 *>(permuted + rows[kk] * hidden + h0);
+    }
+    // running sums, kept as the float32 value of the already rounded element
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+    auto step = [&](int kk) {
+      unsigned short pbits;
+      uint4 q;
+      if constexpr (K > 0) {
+        pbits = pbs[kk];
+        q = pieces[kk];
+      } else {
+        pbits = probs[token * top_k + kk];
+        q = *reinterpret_cast<const uint4 *>(permuted + (long long)sorted_indices[token * top_k + kk] * hidden + h0);
+      }
+      const unsigned w[4] = {q.x, q.y, q.z, q.w};
+      // The golden rounds the product to the element type, then the running sum (both computed in float32).
+      // The two steps are kept apart -- no fused multiply-add, no mixed-precision merge -- by empty asm statements.
+      if constexpr (!BF16) {
+        // float16: the packed half multiply rounds the exact product once, which is what rounding the (exact)
+        // float32 product gives; the sum goes through float32 because numpy's does (double rounding included)
+        const h2_t p2 = {__builtin_bit_cast(_Float16, pbits), __builtin_bit_cast(_Float16, pbits)};
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          h2_t prod = __builtin_bit_cast(h2_t, w[d]) * p2;
+          asm volatile("" : "+v"(prod));
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            float sum = acc[2 * d + u] + (float)prod[u];
+            asm volatile("" : "+v"(sum));
+            acc[2 * d + u] = (float)(_Float16)sum;
+          }
+        }
+      } else {
+        const float p = bf16_bits_to_f32(pbits);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const unsigned short v = (unsigned short)(w[j >> 1] >> (16 * (j & 1)));
+          float prod = p * bf16_bits_to_f32(v);
+          asm volatile("" : "+v"(prod));
+          float sum = acc[j] + bf16_bits_to_f32(f32_to_bf16_rne(prod));
+          asm volatile("" : "+v"(sum));
+          acc[j] = bf16_bits_to_f32(f32_to_bf16_rne(sum));
+        }
+      }
+        };
+    if constexpr (K > 0) {
+#pragma unroll
+      for (int kk = 0; kk < K; ++kk) step(kk);
+    } else {
+      for (int kk = 0; kk < top_k; ++kk) step(kk);
+    }
+    unsigned short ob[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ob[j] = to_elem<BF16>(acc[j]);   // exact: acc already holds an element-type value
     uint4 o;
-    o.x = acc[0] | ((unsigned)acc[1] << 16); o.y = acc[2] | ((unsigned)acc[3] << 16);
-    o.z = acc[4] | ((unsigned)acc[5] << 16); o.w = acc[6] | ((unsigned)acc[7] << 16);
+    o.x = ob[0] | ((unsigned)ob[1] << 16); o.y = ob[2] | ((unsigned)ob[3] << 16);
+    o.z = ob[4] | ((unsigned)ob[5] << 16); o.w = ob[6] | ((unsigned)ob[7] << 16);
     *reinterpret_cast<uint4 *>(out + token * hidden + h0) = o;
   }
 }
@@ -194,8 +259,8 @@ int msco_moe_init_routing_v2(const void *x, const int32_t *expert_idx, void *exp
   hipLaunchKernelGGL(route_hist_kernel, dim3((unsigned)blocks), dim3(256), 0, s, expert_idx, block_hist, n, (int)expert_num);
   hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, block_hist, expert_tokens_count_or_cumsum,
                      expert_tokens_before_capacity, (int)blocks, (int)expert_num, (int)count_or_cumsum_flag);
-  hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(64), 0, s, expert_idx, block_hist, expanded_row_idx,
-                     sorted_src, n, (int)expert_num);
+  hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(1024), (size_t)16 * expert_num * sizeof(int), s, expert_idx,
+                     block_hist, expanded_row_idx, sorted_src, n, (int)expert_num);
   hipLaunchKernelGGL(route_gather_kernel, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned char *>(x), sorted_src,
                      static_cast<unsigned char *>(expanded_x), (long long)hidden * elem_bytes, (int)k);
   return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
@@ -213,10 +278,21 @@ int msco_moe_token_unpermute(const void *permuted_tokens, const int32_t *sorted_
   const auto *pt = static_cast<const unsigned short *>(permuted_tokens);
   const auto *pr = static_cast<const unsigned short *>(probs);
   auto *o = static_cast<unsigned short *>(out);
-  if (dtype == MSCO_DT_BF16)
-    hipLaunchKernelGGL(unpermute_kernel<true>, dim3((unsigned)num_tokens), dim3(256), 0, s, pt, sorted_indices, pr, o, (int)top_k, (long long)hidden);
-  else
-    hipLaunchKernelGGL(unpermute_kernel<false>, dim3((unsigned)num_tokens), dim3(256), 0, s, pt, sorted_indices, pr, o, (int)top_k, (long long)hidden);
+  const dim3 grid((unsigned)num_tokens, (unsigned)((hidden + 2047) / 2048 > 16 ? 16 : (hidden + 2047) / 2048)), block(256);
+  const bool bf = dtype == MSCO_DT_BF16;
+#define MSCO_UNPERMUTE(K)                                                                                               \
+  do {                                                                                                                  \
+    if (bf) hipLaunchKernelGGL((unpermute_kernel<true, K>), grid, block, 0, s, pt, sorted_indices, pr, o, (int)top_k, (long long)hidden);  \
+    else hipLaunchKernelGGL((unpermute_kernel<false, K>), grid, block, 0, s, pt, sorted_indices, pr, o, (int)top_k, (long long)hidden);    \
+  } while (0)
+  switch (top_k) {
+    case 1: MSCO_UNPERMUTE(1); break;
+    case 2: MSCO_UNPERMUTE(2); break;
+    case 4: MSCO_UNPERMUTE(4); break;
+    case 8: MSCO_UNPERMUTE(8); break;
+    default: MSCO_UNPERMUTE(0); break;
+  }
+#undef MSCO_UNPERMUTE
   return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
 }
 

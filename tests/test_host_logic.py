@@ -181,15 +181,17 @@ def test_quant_batch_matmul_infer():
 
 # ------------------------------------------------------------------------------------- registration surface
 def test_registry_and_module_surface():
-    assert set(_C._registered_graph_ops()) == {"grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul"}
-    for name in ("grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul"):
+    ops = ("grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "moe_init_routing_v2", "moe_token_unpermute")
+    assert set(_C._registered_graph_ops()) == set(ops)
+    for name in ops:
         assert callable(getattr(_C, name)) and callable(getattr(mco, name))
     header = open(os.path.join(REPO, "ms_custom_ops_amd", "csrc", "ops", "framework", "module.h")).read()
     for token in ("REG_GRAPH_MODE_OP", "MS_CUSTOM_OPS_EXTENSION_MODULE", "class ModuleRegistry", "RegisterAll"):
         assert token in header
 
 
-@pytest.mark.parametrize("op", ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul"])
+@pytest.mark.parametrize("op", ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "moe_init_routing_v2",
+                                "moe_token_unpermute"])
 def test_yaml_prototype_agrees_with_pybind_signature(op):
     """The prototype and the pybind definition must agree on names, order and defaults
     (the reference's rule, docs/ops_develop_guide.md:378)."""
