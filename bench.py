@@ -2,7 +2,7 @@
 """Benchmark of the grouped W8A8 matmul path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout kn|nk] [--no-sweep] [--no-cpu]
-    python bench.py --probe c3|c2_m16|...|copy [--layout kn|nk] [--steps K]     (for rocprofv3 counter runs)
+    python bench.py --probe c3|c2_m16|...|copy|moe [--layout kn|nk] [--steps K]     (for rocprofv3 counter runs)
 
 A step is one pass of the hot path over one batch of synthetic input (inputs resident in HBM before
 the timed region).  The headline workload is the Mixtral-shaped MoE configuration (E=8, top-2 over
@@ -48,7 +48,7 @@ def parse():
                     help="weight storage the op sees: nk=[E,N,K] (prepacked once, the default), kn=[E,K,N] as generated")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--probe", default=None, help="workload name or `copy`: untimed launches only, for counter collection")
+    ap.add_argument("--probe", default=None, help="workload name, `copy` or `moe` (the routing / un-permutation pair): launches only, for counter collection")
     return ap.parse_args()
 
 
@@ -237,6 +237,9 @@ def probe(args):
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"probe": "copy", "bytes_read": COPY_BYTES, "bytes_written": COPY_BYTES, "launches": args.steps}))
+        return
+    if args.probe == "moe":
+        print(json.dumps({"probe": "moe", "moe_neighbours": moe_neighbours(args.steps, 5)}))
         return
     wl = workloads.make(args.probe)
     prob = DeviceProblem(wl, args.layout)
