@@ -70,12 +70,23 @@ typedef enum msco_dtype {
   MSCO_DT_F32 = 7
 } msco_dtype;
 
+/* Storage of the weight tensor.  The reference keeps its weights in the device's own blocked format (FRACTAL_NZ,
+ * produced once by trans_data, ops/c_api/trans_data/trans_data.cc:203-223; grouped_matmul forces it,
+ * ops/c_api/grouped_matmul/grouped_matmul.cc:216-232); MSCO_WL_PACKED is this backend's counterpart: per group
+ * ceil(N/16) column groups of ceil(K/64) blocks of 1024 bytes, zero outside K x N; byte 16 l + i (l = 0..63,
+ * i = 0..15) of block (a, b) holds w[k = 64 b + 16 (l / 16) + i][n = 16 a + (l % 16)].  Decode shapes stream it at
+ * the rate of a contiguous read. */
+enum {
+  MSCO_WL_ROW_MAJOR = 0,       /* [E,K,N], or [E,N,K] when transpose_b */
+  MSCO_WL_PACKED = 1           /* e * msco_packed_weight_bytes(k, n) bytes written by msco_pack_weight */
+};
+
 /* Positional inputs of msco_gmm_launch.  Slots 0..6 follow the order the reference passes to its
  * kernel object (grouped_matmul.cc:201-207,301-307); slot 7 is the V4 antiquant offset
  * (grouped_matmul_v4_cops.cc:94-97). */
 enum {
   MSCO_IN_X = 0,               /* [M,K] int8 (W8A8) or bf16/f16 (W8A16) */
-  MSCO_IN_WEIGHT = 1,          /* [E,K,N] int8, or [E,N,K] when transpose_b */
+  MSCO_IN_WEIGHT = 1,          /* [E,K,N] int8, or [E,N,K] when transpose_b, or packed (weight_layout) */
   MSCO_IN_BIAS = 2,            /* [E,N] int32, optional */
   MSCO_IN_SCALE = 3,           /* [E,N] f32 / bf16 / int64|uint64 carrying f32 bits in the low word; optional */
   MSCO_IN_GROUP_LIST = 4,      /* [E] int32 / int64; NULL = E equal groups of M/E rows (dense / batched) */
@@ -103,7 +114,8 @@ typedef struct msco_gmm_desc {
   int32_t scale_per_group;   /* 1: scale/bias are [E,N]; 0: one [N] (or [1]) row shared by all groups */
   int32_t scale_is_scalar;   /* 1: scale holds a single element broadcast over N */
   int32_t kernel_override;   /* 0 auto; else force a kernel family (see msco_gmm_plan_info), for tests */
-  int32_t reserved[5];
+  int32_t weight_layout;     /* MSCO_WL_ROW_MAJOR: as transpose_b says; MSCO_WL_PACKED: written by msco_pack_weight */
+  int32_t reserved[4];
 } msco_gmm_desc;
 
 typedef struct msco_gmm_op *msco_gmm_handle;
@@ -135,6 +147,14 @@ MSCO_API int msco_gmm_destroy(msco_gmm_handle h);
  * the HIP kernels read x rows K-contiguous, so the op layer materialises x1 transposed once. */
 MSCO_API int msco_transpose_2d(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols,
                                int32_t elem_bytes, void *stream);
+
+/* Weight prepack, once at load time -- the counterpart of the reference's trans_data ND -> FRACTAL_NZ step
+ * (ops/c_api/trans_data/trans_data.cc:203-223, shape contract ops/c_api/trans_data/trans_data.md:45-99).
+ * src is [e,k,n] int8 (or [e,n,k] when src_transposed); dst receives e * msco_packed_weight_bytes(k, n) bytes in the
+ * MSCO_WL_PACKED layout.  Enqueues on the stream, allocates nothing. */
+MSCO_API size_t msco_packed_weight_bytes(int64_t k, int64_t n);
+MSCO_API int msco_pack_weight(const void *src, void *dst, int64_t e, int64_t k, int64_t n, int32_t src_transposed,
+                              void *stream);
 
 /* Static text for a status code. */
 MSCO_API const char *msco_status_string(int status);

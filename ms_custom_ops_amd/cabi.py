@@ -26,8 +26,12 @@ IN_COUNT = 8
 # msco_gmm_desc.kernel_override
 OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC, OV_TILE_256_W4 = range(7)
 
+# msco_gmm_desc.weight_layout
+WL_ROW_MAJOR, WL_PACKED = 0, 1
+
 EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco_gmm_plan_info", "msco_gmm_destroy",
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
+                    "msco_packed_weight_bytes", "msco_pack_weight",
                     "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_token_unpermute")
 
 
@@ -35,7 +39,7 @@ class GmmDesc(ctypes.Structure):
     _fields_ = [(name, ctypes.c_int32) for name in (
         "abi_version", "x_dtype", "weight_dtype", "out_dtype", "group_list_dtype", "group_list_type", "bias_dtype",
         "scale_dtype", "per_token_dtype", "antiquant_dtype", "has_antiquant_offset", "transpose_b", "scale_per_group",
-        "scale_is_scalar", "kernel_override")] + [("reserved", ctypes.c_int32 * 5)]
+        "scale_is_scalar", "kernel_override", "weight_layout")] + [("reserved", ctypes.c_int32 * 4)]
 
 
 class BackendError(RuntimeError):
@@ -74,6 +78,11 @@ def load():
         lib.msco_transpose_2d.restype = ctypes.c_int
         lib.msco_transpose_2d.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
                                           ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_packed_weight_bytes.restype = ctypes.c_size_t
+        lib.msco_packed_weight_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64]
+        lib.msco_pack_weight.restype = ctypes.c_int
+        lib.msco_pack_weight.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64,
+                                         ctypes.c_int32, ctypes.c_void_p]
         lib.msco_moe_init_routing_v2_workspace_bytes.restype = ctypes.c_size_t
         lib.msco_moe_init_routing_v2_workspace_bytes.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64]
         lib.msco_moe_init_routing_v2.restype = ctypes.c_int
@@ -98,6 +107,18 @@ def transpose_2d(src: int, dst: int, batch: int, rows: int, cols: int, elem_byte
     """src [batch, rows, cols] -> dst [batch, cols, rows] on the device (the weight prepack: [E,K,N] -> [E,N,K])."""
     _check("msco_transpose_2d", load().msco_transpose_2d(ctypes.c_void_p(src), ctypes.c_void_p(dst), batch, rows, cols,
                                                          elem_bytes, ctypes.c_void_p(stream if stream else None)))
+
+
+def packed_weight_bytes(k: int, n: int) -> int:
+    """Bytes of one group's K x N int8 weights in the packed layout."""
+    return int(load().msco_packed_weight_bytes(k, n))
+
+
+def pack_weight(src: int, dst: int, e: int, k: int, n: int, src_transposed: bool = False, stream: Optional[int] = None):
+    """src [e,k,n] int8 (or [e,n,k] when src_transposed) -> dst, e * packed_weight_bytes(k, n) bytes in the packed
+    layout that GmmOp(weight_layout=WL_PACKED) reads."""
+    _check("msco_pack_weight", load().msco_pack_weight(ctypes.c_void_p(src), ctypes.c_void_p(dst), e, k, n,
+                                                       int(bool(src_transposed)), ctypes.c_void_p(stream if stream else None)))
 
 
 def moe_init_routing_v2_workspace_bytes(num_rows: int, k: int, expert_num: int) -> int:

@@ -17,7 +17,23 @@ __device__ __forceinline__ int group_of_row(const GmmParams &p, int m) {
   return -1;
 }
 
-template <bool NK>
+// byte offset of w[k][n] inside one group's weights; LAYOUT 0 [K,N], 1 [N,K], 2 packed (1 KiB blocks of 16 columns x
+// 64 K bytes: byte 16 l + i of block (n / 16, k / 64) holds k % 64 = 16 (l / 16) + i, n % 16 = l % 16)
+template <int LAYOUT>
+__device__ __forceinline__ long long weight_offset(const GmmParams &p, int k, int n) {
+  if (LAYOUT == 0) return (long long)k * p.n + n;
+  if (LAYOUT == 1) return (long long)n * p.k + k;
+  const long long k_blocks = (p.k + 63) / 64;
+  const int kk = k & 63;
+  return ((long long)(n >> 4) * k_blocks + (k >> 6)) * 1024 + ((kk >> 4) * 16 + (n & 15)) * 16 + (kk & 15);
+}
+template <int LAYOUT>
+__device__ __forceinline__ long long weight_group_bytes(const GmmParams &p) {
+  if (LAYOUT == 2) return (long long)((p.n + 15) / 16) * ((p.k + 63) / 64) * 1024;
+  return (long long)p.k * p.n;
+}
+
+template <int LAYOUT>
 __global__ void __launch_bounds__(256) gmm_w8a8_generic_kernel(const GmmParams p) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (long long)p.m * p.n) return;
@@ -28,14 +44,9 @@ __global__ void __launch_bounds__(256) gmm_w8a8_generic_kernel(const GmmParams p
     return;
   }
   const int8_t *x = reinterpret_cast<const int8_t *>(p.x) + (long long)m * p.k;
-  const int8_t *w = p.w + (long long)g * p.k * p.n;
+  const int8_t *w = p.w + (long long)g * weight_group_bytes<LAYOUT>(p);
   int acc = 0;
-  if (NK) {
-    const int8_t *wr = w + (long long)n * p.k;
-    for (int k = 0; k < p.k; ++k) acc += (int)x[k] * (int)wr[k];
-  } else {
-    for (int k = 0; k < p.k; ++k) acc += (int)x[k] * (int)w[(long long)k * p.n + n];
-  }
+  for (int k = 0; k < p.k; ++k) acc += (int)x[k] * (int)w[weight_offset<LAYOUT>(p, k, n)];
   acc += load_bias(p, g, n);
   const float f = dequant(acc, load_scale(p, g, n), p.per_token ? p.per_token[m] : 1.0f);
   store_out(p, idx, acc, f);
@@ -47,6 +58,7 @@ __device__ __forceinline__ float load_half_like(const void *ptr, long long i, in
 }
 
 // out[m,n] = s[g,n] * (sum_k x[m,k] * w[g,k,n] + o[g,n] * sum_k x[m,k]), float32 accumulation.
+template <int LAYOUT>
 __global__ void __launch_bounds__(256) gmm_a16w8_generic_kernel(const GmmParams p) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (long long)p.m * p.n) return;
@@ -57,11 +69,11 @@ __global__ void __launch_bounds__(256) gmm_a16w8_generic_kernel(const GmmParams 
     out[idx] = 0;
     return;
   }
-  const int8_t *w = p.w + (long long)g * p.k * p.n;
+  const int8_t *w = p.w + (long long)g * weight_group_bytes<LAYOUT>(p);
   float acc = 0.0f, xsum = 0.0f;
   for (int k = 0; k < p.k; ++k) {
     const float xv = load_half_like(p.x, (long long)m * p.k + k, p.x_dtype);
-    acc = fmaf(xv, (float)w[(long long)k * p.n + n], acc);
+    acc = fmaf(xv, (float)w[weight_offset<LAYOUT>(p, k, n)], acc);
     xsum += xv;
   }
   const float s = p.aq_scale ? load_half_like(p.aq_scale, (long long)g * p.n + n, p.x_dtype) : 1.0f;
@@ -107,23 +119,29 @@ hipError_t launch_transpose_2d(const void *src, void *dst, long long batch, long
   return hipGetLastError();
 }
 
-hipError_t launch_generic_w8a8(const GmmParams &p, bool nk, hipStream_t stream) {
+hipError_t launch_generic_w8a8(const GmmParams &p, int layout, hipStream_t stream) {
   const long long total = (long long)p.m * p.n;
   if (total == 0) return hipSuccess;
   const unsigned grid = (unsigned)((total + 255) / 256);
-  if (nk) {
-    hipLaunchKernelGGL(gmm_w8a8_generic_kernel<true>, dim3(grid), dim3(256), 0, stream, p);
+  if (layout == 2) {
+    hipLaunchKernelGGL(gmm_w8a8_generic_kernel<2>, dim3(grid), dim3(256), 0, stream, p);
+  } else if (layout == 1) {
+    hipLaunchKernelGGL(gmm_w8a8_generic_kernel<1>, dim3(grid), dim3(256), 0, stream, p);
   } else {
-    hipLaunchKernelGGL(gmm_w8a8_generic_kernel<false>, dim3(grid), dim3(256), 0, stream, p);
+    hipLaunchKernelGGL(gmm_w8a8_generic_kernel<0>, dim3(grid), dim3(256), 0, stream, p);
   }
   return hipGetLastError();
 }
 
-hipError_t launch_generic_a16w8(const GmmParams &p, hipStream_t stream) {
+hipError_t launch_generic_a16w8(const GmmParams &p, int layout, hipStream_t stream) {
   const long long total = (long long)p.m * p.n;
   if (total == 0) return hipSuccess;
   const unsigned grid = (unsigned)((total + 255) / 256);
-  hipLaunchKernelGGL(gmm_a16w8_generic_kernel, dim3(grid), dim3(256), 0, stream, p);
+  if (layout == 2) {
+    hipLaunchKernelGGL(gmm_a16w8_generic_kernel<2>, dim3(grid), dim3(256), 0, stream, p);
+  } else {
+    hipLaunchKernelGGL(gmm_a16w8_generic_kernel<0>, dim3(grid), dim3(256), 0, stream, p);
+  }
   return hipGetLastError();
 }
 

@@ -31,9 +31,18 @@ size_t skinny_workspace_bytes(int64_t m, int64_t n, int64_t e, int split_k, int 
 size_t skinny_counter_count(int64_t m, int64_t n, int64_t e, int cols);
 size_t a16w8_workspace_bytes(int64_t m, int64_t n, int64_t e, int split_k);
 
+// Decode kernels for weights in the packed layout (gmm_stream.hip): 4 waves, strips of up to 256 columns, K slices of
+// at most 128 blocks of 64 bytes (split_k chosen accordingly); workspace and counters as for the 4-wave skinny kernel.
+hipError_t launch_stream_w8a8(const GmmParams &p, hipStream_t stream);
+int stream_blocks_per_wave(int64_t k, int split_k);
+size_t packed_weight_bytes(int64_t k, int64_t n);   // bytes of one group's weights in the packed layout
+hipError_t launch_pack_weight(const void *src, void *dst, long long e, long long k, long long n, bool src_nk,
+                              hipStream_t stream);
+
 // Shape-agnostic fallback kernels (one output element per thread), any K / N.
-hipError_t launch_generic_w8a8(const GmmParams &p, bool nk, hipStream_t stream);
-hipError_t launch_generic_a16w8(const GmmParams &p, hipStream_t stream);
+// layout: 0 [E,K,N], 1 [E,N,K], 2 packed
+hipError_t launch_generic_w8a8(const GmmParams &p, int layout, hipStream_t stream);
+hipError_t launch_generic_a16w8(const GmmParams &p, int layout, hipStream_t stream);
 
 // Batched 2-D transpose, src [batch, rows, cols] -> dst [batch, cols, rows].
 hipError_t launch_transpose_2d(const void *src, void *dst, long long batch, long long rows, long long cols,

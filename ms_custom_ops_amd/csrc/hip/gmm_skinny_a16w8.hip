@@ -114,7 +114,7 @@ __global__ void __launch_bounds__(AW_THREADS, 4) gmm_a16w8_skinny_kernel(const G
     const unsigned voff = (k_ok && cols_ok) ? (unsigned)(k0 * p.n + n0 + 16 * c16) : kBufferOob;
     v4i r[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff, i * p.n, 0);
+    for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff, i * p.n, kStreamAux);
     const v4i a = k_ok ? *reinterpret_cast<const v4i *>(xrow + k0) : v4i{0, 0, 0, 0};
 #pragma unroll
     for (int c4 = 0; c4 < 4; ++c4) {

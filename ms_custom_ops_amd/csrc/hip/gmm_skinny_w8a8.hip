@@ -91,7 +91,7 @@ __global__ void __launch_bounds__(SK_THREADS, NK ? 3 : 4) gmm_w8a8_skinny_kernel
       const unsigned voff = (k_ok && cols_ok) ? (unsigned)(k0 * p.n + n0 + 16 * c16) : kBufferOob;
       v4i r[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff, i * p.n, 0);
+      for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, voff, i * p.n, kStreamAux);
       const i64 a = k_ok ? *reinterpret_cast<const i64 *>(xrow + k0) : 0;
 #pragma unroll
       for (int c4 = 0; c4 < 4; ++c4) {
@@ -310,7 +310,7 @@ __global__ void __launch_bounds__(W16_THREADS) gmm_w8a8_skinny16_kernel(const Gm
       const unsigned voff = (k_ok && cols_ok) ? (unsigned)(k0 * p.n + n0 + 8 * c16) : kBufferOob;
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        rk[s][i] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rw, voff, i * p.n, 0));
+        rk[s][i] = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(rw, voff, i * p.n, kStreamAux));
       ak[s] = k_ok ? *reinterpret_cast<const i64 *>(xrow + k0) : 0;
     }
   };

@@ -1,0 +1,303 @@
+// Grouped decode kernels for weights in the packed layout (gfx950): HBM-bound weight streaming at the
+// rate of a plain contiguous read.
+//
+// Packed layout of one group's weights (K x N int8): ceil(N/16) column groups, each ceil(K/64) blocks of
+// 1024 bytes, zero outside K x N.  Byte 16 l + i (l = 0..63, i = 0..15) of block (a, b) is
+//     w[k = 64 b + 16 (l / 16) + i][n = 16 a + (l % 16)],
+// so one 16-byte load per lane of 1024 consecutive bytes IS the B operand of v_mfma_i32_16x16x64_i8
+// (lane l: column l % 16, K bytes 16 (l / 16) ..), and the blocks of a column group and the column groups
+// of a strip follow each other in memory.  Measured on MI355X a workgroup whose waves take neighbouring
+// 1 KiB pieces of one contiguous region streams at about 7 TB/s, against 6.2 TB/s for the best walk of
+// 256-byte row segments of a row-major matrix and 5.5 TB/s for any walk of a [N,K] matrix whose row pitch
+// is a power of two -- which is why this layout exists.
+//
+// Work decomposition (both kernels): a workgroup (4 waves) owns one 16-row chunk of one group, one strip
+// of up to 16 column groups (256 columns; fewer for small weight sets, so that every CU gets a strip without
+// splitting K) and one K slice of at most 128 blocks.  It walks its strip in memory
+// order: column group after column group, wave w taking blocks w, w + 4, ... of the slice, eight loads in
+// flight per wave across column-group boundaries.  A wave meets the same K blocks in every column group,
+// so its x fragments are loaded once and stay in registers; the inner step is one 16-byte load and one
+// MFMA, nothing else.  Per column group a wave parks its partial tile in LDS; afterwards the four waves'
+// tiles are added in wave order.  K split across workgroups, arrival counter and epilogue are those of the
+// row-major decode kernels.
+#include <type_traits>
+#include <utility>
+
+#include "gmm_common.h"
+#include "gmm_kernels.h"
+
+namespace msco {
+
+namespace {
+// f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>), in order
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+constexpr int ST_WAVES = 4;
+constexpr int ST_THREADS = ST_WAVES * 64;
+constexpr int ST_COLS = kSkinnyCols;                  // 256 columns = 16 column groups per strip
+constexpr int ST_GROUPS = ST_COLS / 16;
+constexpr int ST_TILE_INTS = kSkinnyRows * ST_COLS;   // one partial tile
+constexpr size_t ST_LDS = (size_t)ST_WAVES * ST_GROUPS * 64 * 16 + 16;   // red[wave][column group][lane] + ticket
+typedef long long i64;
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+__host__ __device__ inline long long packed_group_bytes(long long k, long long n) {
+  return ((n + 15) / 16) * ((k + 63) / 64) * 1024;
+}
+}  // namespace
+
+// ---- packing -------------------------------------------------------------------------------------------
+// One thread per 16 destination bytes.  NK: source [E,N,K] (16 K-contiguous bytes), else [E,K,N].
+template <bool NK>
+__global__ void __launch_bounds__(256) pack_weight_kernel(const int8_t *src, int8_t *dst, long long e, int k, int n) {
+  const long long per_group = packed_group_bytes(k, n) / 16;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= e * per_group) return;
+  const long long g = idx / per_group, r = idx % per_group;
+  const int l = (int)(r & 63);
+  const long long blk = r >> 6;
+  const int kblocks = (k + 63) / 64;
+  const int a = (int)(blk / kblocks), b = (int)(blk % kblocks);
+  const int col = 16 * a + (l & 15), k0 = 64 * b + 16 * (l >> 4);
+  const int8_t *s = src + g * (long long)k * n;
+  int8_t v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int kk = k0 + i;
+    v[i] = (col < n && kk < k) ? (NK ? s[(long long)col * k + kk] : s[(long long)kk * n + col]) : (int8_t)0;
+  }
+  *reinterpret_cast<uint4 *>(dst + idx * 16) = *reinterpret_cast<const uint4 *>(v);
+}
+
+hipError_t launch_pack_weight(const void *src, void *dst, long long e, long long k, long long n, bool src_nk,
+                              hipStream_t stream) {
+  const long long total = e * (packed_group_bytes(k, n) / 16);
+  if (total == 0) return hipSuccess;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  if (src_nk) {
+    hipLaunchKernelGGL(pack_weight_kernel<true>, dim3(grid), dim3(256), 0, stream, static_cast<const int8_t *>(src),
+                       static_cast<int8_t *>(dst), e, (int)k, (int)n);
+  } else {
+    hipLaunchKernelGGL(pack_weight_kernel<false>, dim3(grid), dim3(256), 0, stream, static_cast<const int8_t *>(src),
+                       static_cast<int8_t *>(dst), e, (int)k, (int)n);
+  }
+  return hipGetLastError();
+}
+
+size_t packed_weight_bytes(int64_t k, int64_t n) { return (size_t)packed_group_bytes(k, n); }
+
+// ---- W8A8 ----------------------------------------------------------------------------------------------
+// NB = K blocks a wave meets per column group (the slice has at most 4 NB blocks); 4, 8, 16 or 32.
+template <int NB>
+__global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const GmmParams p) {
+  extern __shared__ __align__(16) unsigned char st_smem[];
+  v4i(*red)[ST_GROUPS][64] = reinterpret_cast<v4i(*)[ST_GROUPS][64]>(st_smem);   // [wave][column group][lane]
+  unsigned *s_ticket = reinterpret_cast<unsigned *>(st_smem + ST_LDS - 16);
+  constexpr int D = NB < 8 ? NB : 8;   // loads in flight per wave
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c16 = lane & 15, h = lane >> 4;
+  const int strip = blockIdx.x, ks = blockIdx.z;
+  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;   // first chunks of all groups are dispatched first
+
+  int g_start = 0, g_end = 0;
+  for (int g = 0; g <= grp; ++g) {
+    g_start = g_end;
+    g_end = group_end(p, g, g_start);
+  }
+  const int m0 = g_start + mc * kSkinnyRows;
+  const int chunk_rows = min(kSkinnyRows, g_end - m0);
+  if (chunk_rows <= 0) return;
+
+  const int n0 = strip * p.strip_groups * 16;
+  const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
+  const int cg_count = min(p.strip_groups, col_groups - strip * p.strip_groups);   // column groups of this strip that exist
+  const long long group_bytes = (long long)col_groups * k_blocks * 1024;
+  const __amdgpu_buffer_rsrc_t rw = buffer_over(p.w + (long long)grp * group_bytes, group_bytes);   // planned only below 2^31
+  const int per_split = (k_blocks + p.split_k - 1) / p.split_k;
+  const int kb_begin = ks * per_split;
+  const int kb_end = min(k_blocks, kb_begin + per_split);
+
+  // the wave's blocks kb_begin + wave + 4 j: x fragments (zero past the slice or past K, which also cancels
+  // whatever a masked weight load returns) and byte offsets inside a column group
+  const int8_t *xrow = reinterpret_cast<const int8_t *>(p.x) + (long long)min(m0 + c16, g_end - 1) * p.k;
+  v4i xf[NB];
+  unsigned voff[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const int kb = kb_begin + wave + ST_WAVES * j;
+    const int k0 = kb * 64 + 16 * h;   // K % 16 == 0: 16 K bytes all inside or all outside
+    const bool ok = kb < kb_end && k0 < p.k;
+    xf[j] = ok ? *reinterpret_cast<const v4i *>(xrow + k0) : v4i{0, 0, 0, 0};
+    voff[j] = kb < kb_end ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob;
+  }
+
+  v4i ring[D];
+  const int cg_base = strip * p.strip_groups * k_blocks * 1024;   // byte offset of the strip's first column group
+  auto issue = [&](int cg, auto j_c, auto slot_c) {
+    constexpr int J = decltype(j_c)::value, SLOT = decltype(slot_c)::value;
+    const unsigned vo = cg < cg_count ? voff[J] : kBufferOob;
+    ring[SLOT] = __builtin_amdgcn_raw_buffer_load_b128(rw, vo, cg_base + cg * k_blocks * 1024, kStreamAux);
+  };
+  static_for<NB>([&](auto j_c) {
+    constexpr int J = decltype(j_c)::value;
+    if constexpr (J < D) issue(0, j_c, j_c);
+  });
+  for (int cg = 0; cg < cg_count; ++cg) {
+    v4i a0 = v4i{0, 0, 0, 0}, a1 = v4i{0, 0, 0, 0};
+    static_for<NB>([&](auto j_c) {
+      constexpr int J = decltype(j_c)::value;
+      constexpr int SLOT = J % D;
+      if constexpr (J & 1) a1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[J], ring[SLOT], a1, 0, 0, 0);
+      else a0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[J], ring[SLOT], a0, 0, 0, 0);
+      if constexpr (J + D < NB) issue(cg, std::integral_constant<int, J + D>{}, std::integral_constant<int, SLOT>{});
+      else issue(cg + 1, std::integral_constant<int, J + D - NB>{}, std::integral_constant<int, SLOT>{});
+    });
+    red[wave][cg][lane] = a0 + a1;
+  }
+  __syncthreads();
+
+  // ---- the four waves' tiles, added in wave order: thread (wave, lane) ends up with column groups
+  // wave + 4 e (e = 0..3) of its lane position, rows 4h..4h+3, column 16 (wave + 4 e) + c ----------------
+  v4i v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int cg = wave + 4 * e;
+    v4i s = v4i{0, 0, 0, 0};
+    if (cg < cg_count) {
+      s = red[0][cg][lane];
+#pragma unroll
+      for (int w = 1; w < ST_WAVES; ++w) s += red[w][cg][lane];
+    }
+    v[e] = s;
+  }
+  const bool rows_ok = 4 * h < chunk_rows;  // at least one of the lane's 4 rows is part of the chunk
+
+  if (p.split_k > 1) {
+    // cross-workgroup reduction through the workspace with agent-scope relaxed atomics (no cache-wide
+    // fences); slice s, 64-bit word e of thread t at ((s * 8 + e) * 256 + t); the last arriver adds up
+    const long long tile = ((long long)grp * p.max_chunks + mc) * p.n_strips + strip;
+    i64 *base = reinterpret_cast<i64 *>(p.partial) + tile * p.split_k * (ST_TILE_INTS / 2);
+    if (rows_ok) {
+      i64 *mine = base + (long long)ks * (ST_TILE_INTS / 2) + tid;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const i64 word = (i64)(((unsigned long long)(unsigned)v[e >> 1][2 * (e & 1) + 1] << 32) |
+                               (unsigned)v[e >> 1][2 * (e & 1)]);
+        __hip_atomic_store(mine + e * ST_THREADS, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) *s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*s_ticket != (unsigned)(p.split_k - 1)) return;
+    if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (rows_ok) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = v4i{0, 0, 0, 0};
+      for (int s0 = 0; s0 < p.split_k; s0 += 4) {
+        i64 t[4][8];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int s = min(s0 + u, p.split_k - 1);
+          const i64 *src = base + (long long)s * (ST_TILE_INTS / 2) + tid;
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            t[u][e] = __hip_atomic_load(src + e * ST_THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (s0 + u < p.split_k) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              v[e >> 1][2 * (e & 1)] += (int)(unsigned)(unsigned long long)t[u][e];
+              v[e >> 1][2 * (e & 1) + 1] += (int)(unsigned)((unsigned long long)t[u][e] >> 32);
+            }
+          }
+      }
+    }
+  }
+
+  // ---- epilogue: v[e] = rows 4h..4h+3 of column 16 (wave + 4 e) + c ---------------------------------------
+  float pt[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) pt[r] = (p.per_token && 4 * h + r < chunk_rows) ? p.per_token[m0 + 4 * h + r] : 1.0f;
+  unsigned short(*tile_out)[ST_COLS + 8] = reinterpret_cast<unsigned short(*)[ST_COLS + 8]>(st_smem);
+  __syncthreads();  // every wave is done reading red[]
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int cl = 16 * (wave + 4 * e) + c16;  // column inside the strip
+    const int n = n0 + cl;
+    if (wave + 4 * e < cg_count && n < p.n && rows_ok) {
+      const int bias = load_bias(p, grp, n);
+      if (p.out_dtype == DT_I32) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (4 * h + r < chunk_rows)
+            reinterpret_cast<int *>(p.out)[(long long)(m0 + 4 * h + r) * p.n + n] = v[e][r] + bias;
+      } else {
+        const float sc = load_scale(p, grp, n);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float f = dequant(v[e][r] + bias, sc, pt[r]);
+          tile_out[4 * h + r][cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+        }
+      }
+    }
+  }
+  if (p.out_dtype == DT_I32) return;
+  __syncthreads();
+  // whole-row stores: 16 rows x 32 pieces of 8 columns, two pieces per thread
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int item = tid + ST_THREADS * u;
+    const int row = item >> 5, c8 = (item & 31) * 8;
+    const int n = n0 + c8;
+    if (row < chunk_rows && c8 < 16 * cg_count && n < p.n) {  // N % 16 == 0: 8 columns all inside or all outside
+      const uint4 q = *reinterpret_cast<const uint4 *>(&tile_out[row][c8]);
+      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned short *>(p.out) + (long long)(m0 + row) * p.n + n) = q;
+    }
+  }
+}
+
+int stream_blocks_per_wave(int64_t k, int split_k) {
+  const int64_t k_blocks = (k + 63) / 64;
+  const int64_t per_split = (k_blocks + split_k - 1) / split_k;
+  return (int)((per_split + ST_WAVES - 1) / ST_WAVES);
+}
+
+template <int NB>
+static hipError_t stream_launch_w8a8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
+  auto kern = gmm_w8a8_stream_kernel<NB>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)ST_LDS);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(ST_THREADS), ST_LDS, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_stream_w8a8(const GmmParams &p, hipStream_t stream) {
+  if (p.m == 0) return hipSuccess;
+  const int nb = stream_blocks_per_wave(p.k, p.split_k);
+  if (nb > 32 || p.strip_groups < 1 || p.strip_groups > ST_GROUPS) return hipErrorInvalidValue;   // the plan splits K until a slice has at most 128 blocks
+  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  if (nb > 16) return stream_launch_w8a8<32>(p, grid, stream);
+  if (nb > 8) return stream_launch_w8a8<16>(p, grid, stream);
+  if (nb > 4) return stream_launch_w8a8<8>(p, grid, stream);
+  return stream_launch_w8a8<4>(p, grid, stream);
+}
+
+}  // namespace msco

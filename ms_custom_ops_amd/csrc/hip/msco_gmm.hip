@@ -52,6 +52,7 @@ struct msco_gmm_op {
   int skinny_wide16 = 0;
   int skinny_cols = kSkinnyCols;
   int n_strips = 0;
+  int strip_groups = 16;
   size_t workspace_bytes = 0;
   unsigned *counters = nullptr;
   size_t counters_cap = 0;
@@ -63,6 +64,9 @@ namespace {
 
 bool is_w8a8(const msco_gmm_desc &d) { return d.x_dtype == MSCO_DT_I8; }
 bool is_a16w8(const msco_gmm_desc &d) { return d.x_dtype == MSCO_DT_BF16 || d.x_dtype == MSCO_DT_F16; }
+bool is_packed(const msco_gmm_desc &d) { return d.weight_layout == MSCO_WL_PACKED; }
+// 0 [E,K,N], 1 [E,N,K], 2 packed
+int layout_of(const msco_gmm_desc &d) { return is_packed(d) ? 2 : (d.transpose_b ? 1 : 0); }
 
 int check_desc(const msco_gmm_desc &d) {
   if (d.abi_version != MSCO_GMM_ABI_VERSION) return MSCO_ERR_INVALID_ARG;
@@ -71,6 +75,7 @@ int check_desc(const msco_gmm_desc &d) {
     return MSCO_ERR_UNSUPPORTED;
   if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
   if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_256_W4) return MSCO_ERR_INVALID_ARG;
+  if (d.weight_layout != MSCO_WL_ROW_MAJOR && d.weight_layout != MSCO_WL_PACKED) return MSCO_ERR_INVALID_ARG;
   if (is_w8a8(d)) {
     if (d.out_dtype != MSCO_DT_BF16 && d.out_dtype != MSCO_DT_F16 && d.out_dtype != MSCO_DT_I32)
       return MSCO_ERR_UNSUPPORTED;
@@ -85,7 +90,7 @@ int check_desc(const msco_gmm_desc &d) {
   if (is_a16w8(d)) {
     if (d.out_dtype != d.x_dtype) return MSCO_ERR_UNSUPPORTED;       // weight-only output keeps x's dtype
     if (d.antiquant_dtype != d.x_dtype) return MSCO_ERR_UNSUPPORTED; // scale / offset share x's dtype
-    if (d.transpose_b) return MSCO_ERR_UNSUPPORTED;
+    if (d.transpose_b && d.weight_layout == MSCO_WL_ROW_MAJOR) return MSCO_ERR_UNSUPPORTED;
     if (d.bias_dtype != MSCO_DT_NONE || d.scale_dtype != MSCO_DT_NONE || d.per_token_dtype != MSCO_DT_NONE)
       return MSCO_ERR_UNSUPPORTED;
     return MSCO_OK;
@@ -114,9 +119,14 @@ void choose_plan(msco_gmm_op *op) {
   int family;
   if (!aligned) {
     family = FAM_GENERIC;
+  } else if (is_packed(d)) {
+    // packed weights: the streaming decode kernel up to kSkinnyMaxRows rows; larger M has no MFMA kernel for this
+    // layout yet and runs the generic one
+    family = (m <= kSkinnyMaxRows && is_w8a8(d)) ? FAM_SKINNY : FAM_GENERIC;
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
-  } else if (m <= kSkinnyMaxRows) {
+  } else if (m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) {
+    // a single group of more than two 16-row chunks would stream the weights once per chunk: the small tile takes it
     family = FAM_SKINNY;
   } else {
     family = FAM_TILE;
@@ -134,7 +144,9 @@ void choose_plan(msco_gmm_op *op) {
       op->tile_cfg = TILE_64x128;
     }
   }
-  switch (d.kernel_override) {
+  if (is_packed(d)) {
+    if (d.kernel_override == OV_GENERIC) family = FAM_GENERIC;
+  } else switch (d.kernel_override) {
     case OV_TILE_256: family = FAM_TILE; op->tile_cfg = TILE_256x256; break;
     case OV_TILE_256_W4: family = FAM_TILE; op->tile_cfg = TILE_256x256_W4; break;
     case OV_TILE_128: family = FAM_TILE; op->tile_cfg = TILE_128x128; break;
@@ -144,7 +156,8 @@ void choose_plan(msco_gmm_op *op) {
     default: break;
   }
   // the MFMA kernels address x and one group's weights through 32-bit buffer offsets
-  const bool fits32 = k * n < ((int64_t)1 << 31) && m * k < ((int64_t)1 << 31);
+  const bool fits32 = (is_packed(d) ? (int64_t)packed_weight_bytes(k, n) : k * n) < ((int64_t)1 << 31) &&
+                      m * k < ((int64_t)1 << 31);
   if ((family == FAM_TILE || family == FAM_SKINNY) && !(aligned && fits32)) family = FAM_GENERIC;
   if (family == FAM_TILE && !is_w8a8(d)) family = FAM_SKINNY;
   if (family == FAM_TILE) {
@@ -177,12 +190,27 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t active = std::max<int64_t>(
       1, std::min<int64_t>(e * op->max_chunks, std::min<int64_t>(m, e) + m / kSkinnyRows));
     const int64_t tiles128 = ((n + 127) / 128) * active;
-    int wide16 = is_w8a8(d) && tiles128 <= kNumCUs;
+    int wide16 = is_w8a8(d) && tiles128 <= kNumCUs && !is_packed(d);
     const int forced_variant = env_int("MSCO_SKINNY_WIDE16", -1);
     if (forced_variant >= 0 && is_w8a8(d)) wide16 = forced_variant != 0;
     op->skinny_wide16 = wide16;
     int want, cap;
-    if (wide16) {
+    if (is_packed(d)) {
+      // Packed weights: strips as wide as still give every CU a workgroup without splitting K (a slice holds at
+      // most 128 blocks of 64 bytes), then a K split up to about two workgroups per CU.
+      const int64_t col_groups = (n + 15) / 16, k_blocks = (k + 63) / 64;
+      const int floor_split = (int)((k_blocks + 127) / 128);
+      int groups = 16;
+      while (groups > 1 && ((col_groups + groups - 1) / groups) * active * floor_split < kNumCUs) groups /= 2;
+      op->strip_groups = groups;
+      op->n_strips = (int)((col_groups + groups - 1) / groups);
+      op->skinny_cols = groups * 16;
+      const int64_t base = (int64_t)op->n_strips * active;
+      want = (int)(kTargetWorkgroups / std::max<int64_t>(base, 1));
+      cap = std::max<int>(1, (int)(k_blocks / 16));      // a slice keeps at least 16 blocks
+      want = std::max(floor_split, std::min(std::min(want, kMaxSplitK), cap));
+      cap = kMaxSplitK * 64;
+    } else if (wide16) {
       // at most one 16-wave workgroup per CU, every wave keeps at least one block
       want = (int)(kNumCUs / std::max<int64_t>(tiles128, 1));
       cap = std::max<int>(1, (int)(d.transpose_b ? (k + 63) / 64 : (k + 31) / 32) / 16);
@@ -198,10 +226,18 @@ void choose_plan(msco_gmm_op *op) {
     want = std::max(1, std::min(want, cap));
     const int forced = env_int("MSCO_SKINNY_SPLIT_K", 0);
     if (forced > 0) want = std::min(forced, cap);
+    if (is_packed(d)) want = std::max(want, (int)(((k + 63) / 64 + 127) / 128));   // also under a forced split
     op->split_k = want;
-    op->skinny_cols = wide16 ? 128 : kSkinnyCols;
-    op->workspace_bytes = is_w8a8(d) ? skinny_workspace_bytes(m, n, e, op->split_k, op->skinny_cols)
-                                     : a16w8_workspace_bytes(m, n, e, op->split_k);
+    if (!is_packed(d)) op->skinny_cols = wide16 ? 128 : kSkinnyCols;
+    if (is_packed(d)) {
+      // the packed-layout kernels keep a full 16 x 256 partial tile per (strip, K slice) whatever the strip's width
+      op->workspace_bytes = op->split_k > 1 ? skinny_counter_count(m, n, e, op->skinny_cols) * (size_t)op->split_k *
+                                                kSkinnyRows * kSkinnyCols * 4
+                                            : 0;
+    } else {
+      op->workspace_bytes = is_w8a8(d) ? skinny_workspace_bytes(m, n, e, op->split_k, op->skinny_cols)
+                                       : a16w8_workspace_bytes(m, n, e, op->split_k);
+    }
   }
   op->family = family;
 
@@ -210,10 +246,10 @@ void choose_plan(msco_gmm_op *op) {
   std::snprintf(buf, sizeof(buf),
                 "msco_gmm plan: kernel=%s%s%s%s layout=%s m=%lld k=%lld n=%lld e=%lld split_k=%d strips=%d "
                 "workspace=%zu",
-                is_w8a8(d) ? "w8a8_" : "a16w8_", fam,
+                is_w8a8(d) ? "w8a8_" : "a16w8_", (family == FAM_SKINNY && is_packed(d)) ? "stream" : fam,
                 family == FAM_TILE ? (std::string("_") + tile_cfg_name(op->tile_cfg)).c_str() : "",
                 (family == FAM_SKINNY && op->skinny_wide16) ? "_16w" : "",
-                d.transpose_b ? "[E,N,K]" : "[E,K,N]", (long long)m, (long long)k, (long long)n, (long long)e,
+                is_packed(d) ? "packed" : d.transpose_b ? "[E,N,K]" : "[E,K,N]", (long long)m, (long long)k, (long long)n, (long long)e,
                 op->split_k, op->n_strips, op->workspace_bytes);
   op->info = buf;
 }
@@ -330,17 +366,19 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   p.split_k = h->split_k;
   p.n_strips = h->n_strips;
   p.max_chunks = h->max_chunks;
+  p.strip_groups = h->strip_groups;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t err = hipSuccess;
   const bool nk = d.transpose_b != 0;
+  const int layout = layout_of(d);
   if (is_w8a8(d)) {
     if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, s);
-    else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
-    else err = launch_generic_w8a8(p, nk, s);
+    else if (h->family == FAM_SKINNY) err = layout == 2 ? launch_stream_w8a8(p, s) : launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
+    else err = launch_generic_w8a8(p, layout, s);
   } else {
     if (h->family == FAM_SKINNY) err = launch_skinny_a16w8(p, s);
-    else err = launch_generic_a16w8(p, s);
+    else err = launch_generic_a16w8(p, layout, s);
   }
   return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
 }
@@ -353,6 +391,20 @@ int msco_transpose_2d(const void *src, void *dst, int64_t batch, int64_t rows, i
   if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) return MSCO_ERR_UNSUPPORTED;
   const hipError_t err =
     launch_transpose_2d(src, dst, batch, rows, cols, elem_bytes, static_cast<hipStream_t>(stream));
+  return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
+}
+
+size_t msco_packed_weight_bytes(int64_t k, int64_t n) {
+  if (k <= 0 || n <= 0) return 0;
+  return packed_weight_bytes(k, n);
+}
+
+int msco_pack_weight(const void *src, void *dst, int64_t e, int64_t k, int64_t n, int32_t src_transposed, void *stream) {
+  if (e < 0 || k < 0 || n < 0 || k > INT32_MAX || n > INT32_MAX) return MSCO_ERR_SHAPE;
+  if (e * k * n == 0) return MSCO_OK;
+  if (src == nullptr || dst == nullptr) return MSCO_ERR_INVALID_ARG;
+  if ((e * (int64_t)(packed_weight_bytes(k, n) / 16) + 255) / 256 > 0x7FFFFFFFll) return MSCO_ERR_SHAPE;
+  const hipError_t err = launch_pack_weight(src, dst, e, k, n, src_transposed != 0, static_cast<hipStream_t>(stream));
   return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
 }
 

@@ -47,7 +47,7 @@ __all__ = [
     "f32_to_bf16_bits", "bf16_bits_to_f32", "f32_to_f16", "int32_matmul_exact", "int32_matmul_bruteforce",
     "group_bounds", "grouped_int32_acc", "dequant_epilogue", "grouped_matmul_w8a8", "golden_np_qbmm",
     "golden_grouped_w8a8", "golden_v4_pertoken", "golden_v4_perchannel_bias", "golden_v4_a16w8",
-    "quant_batch_matmul_oracle", "a16w8_grouped_f64", "encode_scale_int64", "encode_scale_int64_qbmm",
+    "quant_batch_matmul_oracle", "a16w8_grouped_f64", "encode_scale_int64", "encode_scale_int64_qbmm", "pack_weights",
     "decode_scale_int64", "random_group_list", "count_compare", "bf16_ulp_check",
 ]
 
@@ -387,3 +387,20 @@ def bf16_ulp_check(out_bits, ref_bits):
     with np.errstate(divide="ignore", invalid="ignore"):
         rel = np.where(r != 0, err / np.abs(r), np.where(err == 0, 0.0, np.inf))
     return (float(rel.max()) if rel.size else 0.0), int(bad.sum())
+
+
+def pack_weights(w):
+    """[E,K,N] int8 -> the backend's packed weight layout, as a flat int8 array per group: [E, bytes].
+
+    This layout has no counterpart in the reference (whose blocked weight format, FRACTAL_NZ, is produced by its
+    closed trans_data kernel); it is restated here from the layout's definition so that the device-side packing can be
+    checked: per group ceil(N/16) column groups of ceil(K/64) blocks of 1024 bytes, zero outside K x N; byte
+    16 l + i (l = 0..63, i = 0..15) of block (a, b) holds w[k = 64 b + 16 (l // 16) + i][n = 16 a + (l % 16)].
+    Pinned in tests/test_oracle_pins.py by a per-byte loop over the definition."""
+    w = np.asarray(w, dtype=np.int8)
+    e, k, n = w.shape
+    kb, ng = (k + 63) // 64, (n + 15) // 16
+    wp = np.zeros((e, kb * 64, ng * 16), dtype=np.int8)
+    wp[:, :k, :n] = w
+    # k = 64 b + 16 q + i, n = 16 a + c  ->  [e, a, b, q, c, i]
+    return np.ascontiguousarray(wp.reshape(e, kb, 4, 16, ng, 16).transpose(0, 4, 1, 2, 5, 3)).reshape(e, -1)

@@ -278,3 +278,23 @@ def test_a16w8_closed_forms_and_c_cross_check():
     gold = O.golden_v4_a16w8(x.astype(np.float32), w, s, o, ends)
     big = np.abs(got[:30]) > 1.0
     np.testing.assert_allclose(gold[big], got[:30][big], rtol=1e-3)
+
+
+def test_pack_weights_follows_the_layout_definition_byte_by_byte():
+    """The packed weight layout is this backend's own (the reference's blocked format comes out of its closed trans_data
+    kernel): the vectorised restatement is checked against a per-byte loop over the definition, padding included."""
+    rng = np.random.default_rng(3)
+    for e, k, n in [(1, 64, 16), (2, 70, 20), (1, 200, 33)]:
+        w = rng.integers(-128, 128, (e, k, n), dtype=np.int8)
+        packed = O.pack_weights(w)
+        kb, ng = (k + 63) // 64, (n + 15) // 16
+        assert packed.shape == (e, ng * kb * 1024)
+        for g in range(e):
+            for a in range(ng):
+                for b in range(kb):
+                    blk = packed[g, (a * kb + b) * 1024:(a * kb + b + 1) * 1024]
+                    for l in range(64):
+                        for i in range(16):
+                            kk, nn = 64 * b + 16 * (l // 16) + i, 16 * a + (l % 16)
+                            want = w[g, kk, nn] if (kk < k and nn < n) else 0
+                            assert blk[16 * l + i] == want

@@ -1,0 +1,101 @@
+"""The packed weight layout: the device-side packing against the layout's numpy restatement, and GPU parity of the kernels
+that read it (the streaming decode kernel, the generic kernel for everything else) against the CPU oracle, through the
+C ABI.  Bar as for the row-major layouts: int32 accumulators and bf16 outputs bit-exact."""
+import numpy as np
+import pytest
+
+from ms_custom_ops_amd import cabi
+from oracle import gmm_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(seed, m, k, n, e):
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (e, k, n), dtype=np.int8)
+    bias = rng.integers(-1000, 1001, (e, n)).astype(np.int32)
+    scale = rng.uniform(1e-3, 1e-2, (e, n)).astype(np.float32)
+    pt = rng.uniform(1e-3, 1e-2, m).astype(np.float32)
+    return x, w, bias, scale, pt
+
+
+def _check(x, w, gl, bias, scale, pt, *, src_transposed=False, override=cabi.OV_AUTO, group_list_type=0):
+    from gpu_utils import run_w8a8
+    _, ends = O.group_bounds(gl, group_list_type)
+    last = int(ends[-1])
+    ref_acc = O.grouped_matmul_w8a8(x, w, gl, bias, group_list_type=group_list_type, out_dtype="i32")
+    ref_bits = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt, group_list_type=group_list_type)
+    acc, info = run_w8a8(x, w, gl, bias, out="i32", transpose_b=src_transposed, override=override, packed=True,
+                         group_list_type=group_list_type, launches=2)
+    assert np.array_equal(acc[:last], ref_acc[:last]), info
+    assert (acc[last:] == -7777).all(), info                       # rows past the last boundary stay untouched
+    bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", transpose_b=src_transposed, override=override, packed=True,
+                          group_list_type=group_list_type, launches=2)
+    assert np.array_equal(bits[:last], ref_bits[:last]), info
+    return info
+
+
+@pytest.mark.parametrize("e,k,n,src_transposed", [(1, 64, 16, False), (3, 200, 40, False), (2, 4096, 272, True),
+                                                  (8, 130, 1000, True)])
+def test_device_packing_matches_the_layout_definition(device, e, k, n, src_transposed):
+    import torch
+    from gpu_utils import pack_on_device, to_dev
+    w = np.random.default_rng(7).integers(-128, 128, (e, k, n), dtype=np.int8)
+    src = np.ascontiguousarray(w.transpose(0, 2, 1)) if src_transposed else w
+    got = pack_on_device(to_dev(src), e, k, n, src_transposed)
+    torch.cuda.synchronize()
+    assert cabi.packed_weight_bytes(k, n) == ((n + 15) // 16) * ((k + 63) // 64) * 1024
+    assert np.array_equal(got.cpu().numpy().reshape(e, -1), O.pack_weights(w))
+
+
+@pytest.mark.parametrize("m,k,n,e,gl", [
+    (16, 4096, 512, 1, [16]),                                   # one strip walk per column group pair, no K split
+    (13, 1024, 272, 2, [5, 13]),                                # N tail inside the last strip, short K
+    (40, 2048, 1040, 4, [0, 17, 17, 40]),                       # empty groups, a group of two 16-row chunks
+    (16, 4096 + 64 * 5, 256, 1, [16]),                          # K blocks not a multiple of the four waves
+    (33, 720, 48, 3, [16, 16, 33]),                             # K not a multiple of 64: zero-padded last block
+    (16, 11008, 4096, 1, [16]),                                 # K beyond one slice: split across workgroups
+    (16, 64, 16, 1, [16]),                                      # a single block
+    (20, 4096, 3584, 8, [2, 4, 4, 9, 12, 15, 18, 20]),          # MoE decode shape (quarter width), full-width strips
+    (9, 8192, 512, 2, [4, 9]),                                  # 32 blocks per wave
+])
+def test_streaming_decode_kernel_is_bit_exact(device, m, k, n, e, gl):
+    x, w, bias, scale, pt = _inputs(11, m, k, n, e)
+    info = _check(x, w, gl, bias, scale, pt)
+    assert "w8a8_stream" in info and "layout=packed" in info
+
+
+@pytest.mark.parametrize("split", [2, 3, 8])
+def test_streaming_decode_with_forced_k_split(device, split, monkeypatch):
+    monkeypatch.setenv("MSCO_SKINNY_SPLIT_K", str(split))
+    x, w, bias, scale, pt = _inputs(12, 21, 2048, 528, 2)
+    info = _check(x, w, [10, 21], bias, scale, pt, src_transposed=True)
+    assert f"split_k={split} " in info
+
+
+def test_counts_and_rows_past_the_last_boundary(device):
+    x, w, bias, scale, pt = _inputs(13, 48, 1024, 256, 4)
+    _check(x, w, [10, 0, 20, 5], bias, scale, pt, group_list_type=1)    # 35 of 48 rows belong to a group
+
+
+@pytest.mark.parametrize("m,gl", [(64, [30, 64]), (200, [90, 200])])
+def test_larger_m_runs_the_generic_kernel_on_packed_weights(device, m, gl):
+    x, w, bias, scale, pt = _inputs(14, m, 512, 256, 2)
+    info = _check(x, w, gl, bias, scale, pt, override=cabi.OV_GENERIC if m <= 64 else cabi.OV_AUTO)
+    assert "generic" in info and "layout=packed" in info
+
+
+def test_wire_formats_on_packed_weights(device):
+    """bf16 scale, int64-encoded scale, a single shared scale row, fp16 output."""
+    from gpu_utils import run_w8a8
+    x, w, bias, scale, pt = _inputs(15, 16, 1024, 256, 2)
+    gl = [7, 16]
+    sb = O.f32_to_bf16_bits(scale)
+    got, _ = run_w8a8(x, w, gl, None, sb, pt, out="bf16", scale_dtype=cabi.DT_BF16, packed=True)
+    assert np.array_equal(got, O.grouped_matmul_w8a8(x, w, gl, None, O.bf16_bits_to_f32(sb), pt))
+    got, _ = run_w8a8(x, w, gl, bias, O.encode_scale_int64(scale), pt, out="bf16", scale_dtype=cabi.DT_I64, packed=True)
+    assert np.array_equal(got, O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt))
+    got, _ = run_w8a8(x, w, gl, bias[0], scale[0], pt, out="f16", scale_per_group=0, packed=True)
+    ref = O.grouped_matmul_w8a8(x, w, gl, np.tile(bias[:1], (2, 1)), np.tile(scale[:1], (2, 1)), pt, out_dtype="f16")
+    assert np.array_equal(got, ref.view(np.uint16))
