@@ -34,6 +34,8 @@ size_t a16w8_workspace_bytes(int64_t m, int64_t n, int64_t e, int split_k);
 // Decode kernels for weights in the packed layout (gmm_stream.hip): 4 waves, strips of up to 256 columns, K slices of
 // at most 128 blocks of 64 bytes (split_k chosen accordingly); workspace and counters as for the 4-wave skinny kernel.
 hipError_t launch_stream_w8a8(const GmmParams &p, hipStream_t stream);
+hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream);   // K slices of at most 64 blocks
+size_t stream_a16w8_tile_bytes();   // workspace bytes of one (strip, K slice) partial tile of the weight-only kernel
 int stream_blocks_per_wave(int64_t k, int split_k);
 size_t packed_weight_bytes(int64_t k, int64_t n);   // bytes of one group's weights in the packed layout
 hipError_t launch_pack_weight(const void *src, void *dst, long long e, long long k, long long n, bool src_nk,

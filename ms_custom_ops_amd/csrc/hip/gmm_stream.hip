@@ -300,4 +300,265 @@ hipError_t launch_stream_w8a8(const GmmParams &p, hipStream_t stream) {
   return stream_launch_w8a8<4>(p, grid, stream);
 }
 
+// ---- weight-only (bf16 / f16 activations) ------------------------------------------------------------------
+// The 16 K bytes a lane holds of a block feed two v_mfma_f32_16x16x32_{bf16,f16}: bytes 0..7 and bytes 8..15, each
+// turned into exact 16-bit values of (w + 128) (v_cvt_f32_ubyteN on w ^ 0x80, then a 16-bit pack).  The x fragments
+// follow the same K order: for block b, lane (c, q), step s the 8 values x[c][64 b + 16 q + 8 s ..].  As in the
+// row-major weight-only kernel the row sums of x (one MFMA against ones per fragment, once per workgroup) fold the
+// offset and the +128 into the epilogue:  out = s * (sum_k x (w + 128) + (o - 128) sum_k x).
+namespace {
+constexpr int SA_TILE_WORDS = kSkinnyRows * ST_COLS / 2 + 128;   // 64-bit words: partial tile + 4 row sums per lane slot
+constexpr size_t SA_LDS = (size_t)ST_WAVES * ST_GROUPS * 64 * 16 + (size_t)ST_WAVES * 64 * 16 + 16;
+
+template <bool BF16>
+__device__ __forceinline__ unsigned sa_pack2(float lo, float hi) {
+  if constexpr (BF16) {
+    // both values are integers below 256: the upper 16 bits of the float32 pattern are the exact bf16
+    return perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+  } else {
+    return __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+  }
+}
+template <int B>
+__device__ __forceinline__ float sa_ubyte(unsigned w) {
+  return (float)((w >> (8 * B)) & 0xFFu);   // v_cvt_f32_ubyteB
+}
+// 8 consecutive K bytes (two dwords, already + 128) -> the 8 16-bit values of one MFMA operand
+template <bool BF16>
+__device__ __forceinline__ v4i sa_frag(unsigned lo, unsigned hi) {
+  v4i f;
+  f[0] = (int)sa_pack2<BF16>(sa_ubyte<0>(lo), sa_ubyte<1>(lo));
+  f[1] = (int)sa_pack2<BF16>(sa_ubyte<2>(lo), sa_ubyte<3>(lo));
+  f[2] = (int)sa_pack2<BF16>(sa_ubyte<0>(hi), sa_ubyte<1>(hi));
+  f[3] = (int)sa_pack2<BF16>(sa_ubyte<2>(hi), sa_ubyte<3>(hi));
+  return f;
+}
+template <bool BF16>
+__device__ __forceinline__ v4f sa_mfma(const v4i &a, const v4i &b, const v4f &c) {
+  if constexpr (BF16) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+}
+template <bool BF16>
+__device__ __forceinline__ float sa_half_like(unsigned short b) {
+  return BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b);
+}
+}  // namespace
+
+template <bool BF16, int NB>
+__global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const GmmParams p) {
+  extern __shared__ __align__(16) unsigned char st_smem[];
+  v4f(*red)[ST_GROUPS][64] = reinterpret_cast<v4f(*)[ST_GROUPS][64]>(st_smem);   // [wave][column group][lane]
+  v4f(*red_rs)[64] = reinterpret_cast<v4f(*)[64]>(st_smem + (size_t)ST_WAVES * ST_GROUPS * 64 * 16);
+  unsigned *s_ticket = reinterpret_cast<unsigned *>(st_smem + SA_LDS - 16);
+  constexpr int D = NB < 8 ? NB : 8;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c16 = lane & 15, h = lane >> 4;
+  const int strip = blockIdx.x, ks = blockIdx.z;
+  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
+
+  int g_start = 0, g_end = 0;
+  for (int g = 0; g <= grp; ++g) {
+    g_start = g_end;
+    g_end = group_end(p, g, g_start);
+  }
+  const int m0 = g_start + mc * kSkinnyRows;
+  const int chunk_rows = min(kSkinnyRows, g_end - m0);
+  if (chunk_rows <= 0) return;
+
+  const int n0 = strip * p.strip_groups * 16;
+  const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
+  const int cg_count = min(p.strip_groups, col_groups - strip * p.strip_groups);
+  const long long group_bytes = (long long)col_groups * k_blocks * 1024;
+  const __amdgpu_buffer_rsrc_t rw = buffer_over(p.w + (long long)grp * group_bytes, group_bytes);
+  const int per_split = (k_blocks + p.split_k - 1) / p.split_k;
+  const int kb_begin = ks * per_split;
+  const int kb_end = min(k_blocks, kb_begin + per_split);
+
+  const unsigned short *xrow = reinterpret_cast<const unsigned short *>(p.x) + (long long)min(m0 + c16, g_end - 1) * p.k;
+  const unsigned ones = BF16 ? 0x3F803F80u : 0x3C003C00u;
+  const v4i ones_frag = v4i{(int)ones, (int)ones, (int)ones, (int)ones};
+  v4i xf[NB][2];
+  unsigned voff[NB];
+  v4f rs = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    const int kb = kb_begin + wave + ST_WAVES * j;
+    const int k0 = kb * 64 + 16 * h;   // K % 16 == 0: the 16 K positions are all inside or all outside
+    const bool ok = kb < kb_end && k0 < p.k;
+    xf[j][0] = ok ? *reinterpret_cast<const v4i *>(xrow + k0) : v4i{0, 0, 0, 0};
+    xf[j][1] = ok ? *reinterpret_cast<const v4i *>(xrow + k0 + 8) : v4i{0, 0, 0, 0};
+    voff[j] = kb < kb_end ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob;
+    rs = sa_mfma<BF16>(xf[j][0], ones_frag, rs);
+    rs = sa_mfma<BF16>(xf[j][1], ones_frag, rs);
+  }
+
+  v4i ring[D];
+  const int cg_base = strip * p.strip_groups * k_blocks * 1024;
+  auto issue = [&](int cg, auto j_c, auto slot_c) {
+    constexpr int J = decltype(j_c)::value, SLOT = decltype(slot_c)::value;
+    const unsigned vo = cg < cg_count ? voff[J] : kBufferOob;
+    ring[SLOT] = __builtin_amdgcn_raw_buffer_load_b128(rw, vo, cg_base + cg * k_blocks * 1024, kStreamAux);
+  };
+  static_for<NB>([&](auto j_c) {
+    constexpr int J = decltype(j_c)::value;
+    if constexpr (J < D) issue(0, j_c, j_c);
+  });
+  for (int cg = 0; cg < cg_count; ++cg) {
+    v4f a0 = v4f{0.f, 0.f, 0.f, 0.f}, a1 = v4f{0.f, 0.f, 0.f, 0.f};
+    static_for<NB>([&](auto j_c) {
+      constexpr int J = decltype(j_c)::value;
+      constexpr int SLOT = J % D;
+      const v4i r = ring[SLOT];
+      const unsigned d0 = (unsigned)r[0] ^ 0x80808080u, d1 = (unsigned)r[1] ^ 0x80808080u;   // w + 128 as unsigned bytes
+      const unsigned d2 = (unsigned)r[2] ^ 0x80808080u, d3 = (unsigned)r[3] ^ 0x80808080u;
+      a0 = sa_mfma<BF16>(xf[J][0], sa_frag<BF16>(d0, d1), a0);
+      a1 = sa_mfma<BF16>(xf[J][1], sa_frag<BF16>(d2, d3), a1);
+      if constexpr (J + D < NB) issue(cg, std::integral_constant<int, J + D>{}, std::integral_constant<int, SLOT>{});
+      else issue(cg + 1, std::integral_constant<int, J + D - NB>{}, std::integral_constant<int, SLOT>{});
+    });
+    red[wave][cg][lane] = a0 + a1;
+  }
+  red_rs[wave][lane] = rs;
+  __syncthreads();
+
+  // the four waves' tiles and row sums, added in wave order (reproducible run to run)
+  v4f v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int cg = wave + 4 * e;
+    v4f s = v4f{0.f, 0.f, 0.f, 0.f};
+    if (cg < cg_count) {
+      s = red[0][cg][lane];
+#pragma unroll
+      for (int w = 1; w < ST_WAVES; ++w) s += red[w][cg][lane];
+    }
+    v[e] = s;
+  }
+  v4f xs = red_rs[0][lane];
+#pragma unroll
+  for (int w = 1; w < ST_WAVES; ++w) xs += red_rs[w][lane];
+  const bool rows_ok = 4 * h < chunk_rows;
+
+  if (p.split_k > 1) {
+    // float32 partials through the workspace, added in slice order by the last arriver.  Slice s: word e (0..7) of
+    // thread t at (s * SA_TILE_WORDS + e * 256 + t); row sums of wave 0's lanes at (... + 2048 + 2 lane + {0, 1})
+    const long long tile = ((long long)grp * p.max_chunks + mc) * p.n_strips + strip;
+    i64 *base = reinterpret_cast<i64 *>(p.partial) + tile * p.split_k * SA_TILE_WORDS;
+    auto pack = [](float lo, float hi) {
+      return (i64)(((unsigned long long)__float_as_uint(hi) << 32) | __float_as_uint(lo));
+    };
+    if (rows_ok) {
+      i64 *mine = base + (long long)ks * SA_TILE_WORDS;
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        __hip_atomic_store(mine + e * ST_THREADS + tid, pack(v[e >> 1][2 * (e & 1)], v[e >> 1][2 * (e & 1) + 1]),
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (wave == 0) {
+        __hip_atomic_store(mine + 2048 + 2 * lane, pack(xs[0], xs[1]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + 2048 + 2 * lane + 1, pack(xs[2], xs[3]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) *s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*s_ticket != (unsigned)(p.split_k - 1)) return;
+    if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (rows_ok) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = v4f{0.f, 0.f, 0.f, 0.f};
+      xs = v4f{0.f, 0.f, 0.f, 0.f};
+      for (int s0 = 0; s0 < p.split_k; s0 += 4) {
+        i64 t[4][10];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int s = min(s0 + u, p.split_k - 1);
+          const i64 *src = base + (long long)s * SA_TILE_WORDS;
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            t[u][e] = __hip_atomic_load(src + e * ST_THREADS + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          t[u][8] = __hip_atomic_load(src + 2048 + 2 * lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          t[u][9] = __hip_atomic_load(src + 2048 + 2 * lane + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (s0 + u < p.split_k) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              v[e >> 1][2 * (e & 1)] += __uint_as_float((unsigned)(unsigned long long)t[u][e]);
+              v[e >> 1][2 * (e & 1) + 1] += __uint_as_float((unsigned)((unsigned long long)t[u][e] >> 32));
+            }
+            xs[0] += __uint_as_float((unsigned)(unsigned long long)t[u][8]);
+            xs[1] += __uint_as_float((unsigned)((unsigned long long)t[u][8] >> 32));
+            xs[2] += __uint_as_float((unsigned)(unsigned long long)t[u][9]);
+            xs[3] += __uint_as_float((unsigned)((unsigned long long)t[u][9] >> 32));
+          }
+      }
+    }
+  }
+
+  // ---- epilogue: v[e] = rows 4h..4h+3 of column 16 (wave + 4 e) + c --------------------------------------------
+  unsigned short(*tile_out)[ST_COLS + 8] = reinterpret_cast<unsigned short(*)[ST_COLS + 8]>(st_smem);
+  __syncthreads();   // every wave is done reading red[]
+  const unsigned short *sc = reinterpret_cast<const unsigned short *>(p.aq_scale);
+  const unsigned short *of = reinterpret_cast<const unsigned short *>(p.aq_offset);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int cl = 16 * (wave + 4 * e) + c16;
+    const int n = n0 + cl;
+    if (wave + 4 * e < cg_count && n < p.n && rows_ok) {
+      const float s = sc ? sa_half_like<BF16>(sc[(long long)grp * p.n + n]) : 1.0f;
+      const float o = of ? sa_half_like<BF16>(of[(long long)grp * p.n + n]) : 0.0f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float f = fmaf(o - 128.0f, xs[r], v[e][r]) * s;
+        tile_out[4 * h + r][cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int item = tid + ST_THREADS * u;
+    const int row = item >> 5, c8 = (item & 31) * 8;
+    const int n = n0 + c8;
+    if (row < chunk_rows && c8 < 16 * cg_count && n < p.n) {
+      const uint4 q = *reinterpret_cast<const uint4 *>(&tile_out[row][c8]);
+      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned short *>(p.out) + (long long)(m0 + row) * p.n + n) = q;
+    }
+  }
+}
+
+size_t stream_a16w8_tile_bytes() { return (size_t)SA_TILE_WORDS * 8; }
+
+template <bool BF16, int NB>
+static hipError_t stream_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
+  auto kern = gmm_a16w8_stream_kernel<BF16, NB>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)SA_LDS);
+    if (e != hipSuccess) return e;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(ST_THREADS), SA_LDS, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream) {
+  if (p.m == 0) return hipSuccess;
+  const int nb = stream_blocks_per_wave(p.k, p.split_k);
+  if (nb > 16 || p.strip_groups < 1 || p.strip_groups > ST_GROUPS) return hipErrorInvalidValue;   // slices of at most 64 blocks
+  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  const bool bf = p.x_dtype == DT_BF16;
+  if (nb > 8) return bf ? stream_launch_a16w8<true, 16>(p, grid, stream) : stream_launch_a16w8<false, 16>(p, grid, stream);
+  if (nb > 4) return bf ? stream_launch_a16w8<true, 8>(p, grid, stream) : stream_launch_a16w8<false, 8>(p, grid, stream);
+  return bf ? stream_launch_a16w8<true, 4>(p, grid, stream) : stream_launch_a16w8<false, 4>(p, grid, stream);
+}
+
 }  // namespace msco

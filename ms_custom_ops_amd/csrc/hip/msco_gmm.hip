@@ -120,9 +120,9 @@ void choose_plan(msco_gmm_op *op) {
   if (!aligned) {
     family = FAM_GENERIC;
   } else if (is_packed(d)) {
-    // packed weights: the streaming decode kernel up to kSkinnyMaxRows rows; larger M has no MFMA kernel for this
-    // layout yet and runs the generic one
-    family = (m <= kSkinnyMaxRows && is_w8a8(d)) ? FAM_SKINNY : FAM_GENERIC;
+    // packed weights: the streaming decode kernels (W8A8 up to kSkinnyMaxRows rows, weight-only at any M, like its
+    // row-major counterpart); W8A8 with larger M has no MFMA kernel for this layout yet and runs the generic one
+    family = (m <= kSkinnyMaxRows || is_a16w8(d)) ? FAM_SKINNY : FAM_GENERIC;
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
   } else if (m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) {
@@ -199,7 +199,8 @@ void choose_plan(msco_gmm_op *op) {
       // Packed weights: strips as wide as still give every CU a workgroup without splitting K (a slice holds at
       // most 128 blocks of 64 bytes), then a K split up to about two workgroups per CU.
       const int64_t col_groups = (n + 15) / 16, k_blocks = (k + 63) / 64;
-      const int floor_split = (int)((k_blocks + 127) / 128);
+      const int slice_blocks = is_w8a8(d) ? 128 : 64;
+      const int floor_split = (int)((k_blocks + slice_blocks - 1) / slice_blocks);
       int groups = 16;
       while (groups > 1 && ((col_groups + groups - 1) / groups) * active * floor_split < kNumCUs) groups /= 2;
       op->strip_groups = groups;
@@ -226,14 +227,17 @@ void choose_plan(msco_gmm_op *op) {
     want = std::max(1, std::min(want, cap));
     const int forced = env_int("MSCO_SKINNY_SPLIT_K", 0);
     if (forced > 0) want = std::min(forced, cap);
-    if (is_packed(d)) want = std::max(want, (int)(((k + 63) / 64 + 127) / 128));   // also under a forced split
+    if (is_packed(d)) {   // also under a forced split
+      const int slice_blocks = is_w8a8(d) ? 128 : 64;
+      want = std::max(want, (int)(((k + 63) / 64 + slice_blocks - 1) / slice_blocks));
+    }
     op->split_k = want;
     if (!is_packed(d)) op->skinny_cols = wide16 ? 128 : kSkinnyCols;
     if (is_packed(d)) {
       // the packed-layout kernels keep a full 16 x 256 partial tile per (strip, K slice) whatever the strip's width
-      op->workspace_bytes = op->split_k > 1 ? skinny_counter_count(m, n, e, op->skinny_cols) * (size_t)op->split_k *
-                                                kSkinnyRows * kSkinnyCols * 4
-                                            : 0;
+      const size_t tile_bytes = is_w8a8(d) ? (size_t)kSkinnyRows * kSkinnyCols * 4 : stream_a16w8_tile_bytes();
+      op->workspace_bytes =
+        op->split_k > 1 ? skinny_counter_count(m, n, e, op->skinny_cols) * (size_t)op->split_k * tile_bytes : 0;
     } else {
       op->workspace_bytes = is_w8a8(d) ? skinny_workspace_bytes(m, n, e, op->split_k, op->skinny_cols)
                                        : a16w8_workspace_bytes(m, n, e, op->split_k);
@@ -377,7 +381,7 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
     else if (h->family == FAM_SKINNY) err = layout == 2 ? launch_stream_w8a8(p, s) : launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
     else err = launch_generic_w8a8(p, layout, s);
   } else {
-    if (h->family == FAM_SKINNY) err = launch_skinny_a16w8(p, s);
+    if (h->family == FAM_SKINNY) err = layout == 2 ? launch_stream_a16w8(p, s) : launch_skinny_a16w8(p, s);
     else err = launch_generic_a16w8(p, layout, s);
   }
   return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;

@@ -99,3 +99,58 @@ def test_wire_formats_on_packed_weights(device):
     got, _ = run_w8a8(x, w, gl, bias[0], scale[0], pt, out="f16", scale_per_group=0, packed=True)
     ref = O.grouped_matmul_w8a8(x, w, gl, np.tile(bias[:1], (2, 1)), np.tile(scale[:1], (2, 1)), pt, out_dtype="f16")
     assert np.array_equal(got, ref.view(np.uint16))
+
+
+# ------------------------------------------------------------------------------- weight-only path on packed weights
+def _weight_only_case(seed, m, k, n, e, gl, dtype):
+    rng = np.random.default_rng(seed)
+    half = np.float16 if dtype == "f16" else None
+    def to_bits(a):
+        return a.astype(np.float16).view(np.uint16) if half else O.f32_to_bf16_bits(a.astype(np.float32))
+    def to_f(b):
+        return b.view(np.float16).astype(np.float32) if half else O.bf16_bits_to_f32(b)
+    x = to_bits(rng.standard_normal((m, k)))
+    w = rng.integers(-127, 128, (e, k, n), dtype=np.int8)
+    s = to_bits(rng.uniform(1e-3, 1e-2, (e, n)))
+    o = to_bits(rng.integers(-8, 9, (e, n)).astype(np.float32))
+    xf, sf, of = to_f(x), to_f(s), to_f(o)
+    exact = O.a16w8_grouped_f64(xf, w, sf, of, gl)
+    starts, ends = O.group_bounds(gl)
+    mag = np.zeros_like(exact)
+    for g in range(e):
+        a, b = int(starts[g]), int(ends[g])
+        mag[a:b] = np.abs(xf[a:b].astype(np.float64)) @ (np.abs(w[g].astype(np.float64) + of[g]) * np.abs(sf[g]))
+    return x, w, s, o, exact, mag, to_f, int(ends[-1])
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("m,k,n,e,gl", [
+    (32, 1024, 3584, 8, [3, 7, 7, 12, 20, 25, 30, 32]),     # the weight-only decode configuration at quarter size
+    (16, 4096, 272, 1, [16]),                               # 16 blocks per wave, N tail
+    (40, 720, 48, 2, [17, 40]),                             # K not a multiple of 64, groups of two chunks
+    (9, 8192 + 320, 256, 2, [4, 9]),                        # K beyond one slice: split across workgroups
+])
+def test_weight_only_streaming_kernel_within_tolerance(device, dtype, m, k, n, e, gl):
+    """Tolerance (floating point, as for the row-major weight-only kernel): |out - exact| <= ulp * |exact| +
+    1e-5 * sum_k |x (w + o) s|, ulp = 2**-7 (bf16) or 2**-10 (f16), against the float64 value of the reference's
+    a16w8 golden (tests/st/test_grouped_matmul_v4_cops.py:166-174)."""
+    from gpu_utils import run_a16w8
+    x, w, s, o, exact, mag, to_f, last = _weight_only_case(21, m, k, n, e, gl, dtype)
+    bits, info = run_a16w8(x, w, s, o, gl, dtype=dtype, packed=True)
+    assert "a16w8_stream" in info and "layout=packed" in info
+    got = to_f(bits).astype(np.float64)
+    ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
+    assert (np.abs(got[:last] - exact[:last]) <= ulp * np.abs(exact[:last]) + 1e-5 * mag[:last]).all(), info
+    # and the same inputs through the row-major kernel agree to the same bound (two float32 summation orders)
+    bits_rm, _ = run_a16w8(x, w, s, o, gl, dtype=dtype)
+    assert (np.abs(to_f(bits_rm).astype(np.float64)[:last] - got[:last]) <= 2 * ulp * np.abs(exact[:last]) + 2e-5 * mag[:last]).all()
+
+
+def test_weight_only_generic_kernel_on_packed_weights(device):
+    from gpu_utils import run_a16w8
+    x, w, s, o, exact, mag, to_f, last = _weight_only_case(22, 12, 200, 48, 2, [5, 12], "bf16")
+    # K % 16 != 0 has no MFMA path: generic kernel, packed indexing
+    bits, info = run_a16w8(x, w, s, o, [5, 12], packed=True)
+    assert "generic" in info
+    got = to_f(bits).astype(np.float64)
+    assert (np.abs(got[:last] - exact[:last]) <= 2.0 ** -7 * np.abs(exact[:last]) + 1e-5 * mag[:last]).all(), info
