@@ -15,7 +15,8 @@ Prints ONE JSON line.  Besides the contract keys it carries
   roofline      the dominant kernel's achieved algorithmic rate against the MI355X peak,
   cpu_baseline  the numpy restatement of the reference golden timed on this box's host cores,
   sweep         the other configurations (dense decode / prefill sweep, skewed MoE, weight-only
-                decode) as TOPS and GB/s with their roofline fractions.
+                decode) as TOPS and GB/s with their roofline fractions; decode shapes also on weights
+                prepacked to the blocked layout (layout "packed").
 --probe runs a few untimed launches of one workload (or, for `copy`, of a plain device-to-device copy
 of COPY_BYTES bytes, the reference a counter reading is scaled by) so that a profiler sees nothing else.
 """
@@ -33,6 +34,8 @@ sys.path.insert(0, REPO)
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 ROTATE_BYTES = 768e6      # HBM-bound cases rotate over weight copies totalling more than the 256 MB Infinity Cache
+LAYOUT_TEXT = {"nk": "prepacked once to [E,N,K]", "kn": "[E,K,N] as generated",
+               "packed": "prepacked once to the blocked layout"}
 COPY_BYTES = 1 << 29      # --probe copy: one launch reads and writes this many bytes
 TRAFFIC_FILE = os.path.join(REPO, "ms_custom_ops_amd", "measured_traffic.json")
 
@@ -44,8 +47,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=40,
                     help="untimed steps; the GPU clock needs a few tens of launches to settle")
     ap.add_argument("--workload", default="c3")
-    ap.add_argument("--layout", default="nk", choices=["kn", "nk"],
-                    help="weight storage the op sees: nk=[E,N,K] (prepacked once, the default), kn=[E,K,N] as generated")
+    ap.add_argument("--layout", default="nk", choices=["kn", "nk", "packed"],
+                    help="weight storage the op sees: nk=[E,N,K] (prepacked once, the default), kn=[E,K,N] as generated, "
+                         "packed=the blocked layout of msco_pack_weight (decode shapes)")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--probe", default=None, help="workload name, `copy` or `moe` (the routing / un-permutation pair): launches only, for counter collection")
@@ -79,6 +83,19 @@ class DeviceProblem:
             torch.cuda.synchronize()
             self.prepack_ms = a.elapsed_time(b)
             w0 = packed
+        elif layout == "packed":
+            # one-time prepack into the backend's blocked layout (the counterpart of the reference's trans_data step)
+            packed = torch.empty(wl.e * cabi.packed_weight_bytes(wl.k, wl.n), dtype=torch.int8, device=dev)
+            st = torch.cuda.current_stream().cuda_stream
+            cabi.pack_weight(w0.data_ptr(), packed.data_ptr(), wl.e, wl.k, wl.n, False, st)   # warm
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            cabi.pack_weight(w0.data_ptr(), packed.data_ptr(), wl.e, wl.k, wl.n, False, st)
+            b.record()
+            torch.cuda.synchronize()
+            self.prepack_ms = a.elapsed_time(b)
+            w0 = packed
         # extra weight copies (random bytes; only the timing uses them) defeat the Infinity Cache
         self.w = [w0] + [torch.randint(-127, 128, w0.shape, dtype=torch.int8, device=dev) for _ in range(copies - 1)]
         self.gl = t(wl.group_list)
@@ -86,13 +103,15 @@ class DeviceProblem:
         if self.a16:
             self.scale, self.offset = t(wl.scale.view(np.int16)), t(wl.offset.view(np.int16))
             self.op = cabi.GmmOp(x_dtype=cabi.DT_BF16, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,
-                                 antiquant_dtype=cabi.DT_BF16, has_antiquant_offset=1)
+                                 antiquant_dtype=cabi.DT_BF16, has_antiquant_offset=1,
+                                 weight_layout=cabi.WL_PACKED if layout == "packed" else cabi.WL_ROW_MAJOR)
         else:
             self.scale, self.pt, self.bias = t(wl.scale), t(wl.per_token), t(wl.bias)
             self.op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,
                                  scale_dtype=cabi.DT_F32, per_token_dtype=cabi.DT_F32,
                                  bias_dtype=cabi.DT_I32 if self.bias is not None else cabi.DT_NONE,
-                                 transpose_b=int(nk))
+                                 transpose_b=int(nk),
+                                 weight_layout=cabi.WL_PACKED if layout == "packed" else cabi.WL_ROW_MAJOR)
         self.ws_bytes = self.op.plan(wl.m, wl.k, wl.n, wl.e)
         self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
         self.stream = torch.cuda.current_stream().cuda_stream
@@ -109,20 +128,22 @@ class DeviceProblem:
         self.op.launch(ins, self.out.data_ptr(), self.ws.data_ptr(), self.ws_bytes, self.stream)
 
     def time(self, steps, warmup):
-        """Returns (wall seconds of `steps` steps, mean per-launch seconds from HIP events on the launch stream)."""
+        """Returns (wall seconds of `steps` steps, mean per-launch seconds: one pair of HIP events on the launch stream
+        around the `steps` back-to-back launches, so the figure is the launch-to-launch period of a running stream and
+        agrees with a profiler's kernel durations)."""
         torch = self.torch
         for _ in range(warmup):
             self.step()
         torch.cuda.synchronize()
-        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
-        for a, b in ev:
-            a.record()
+        first.record()
+        for _ in range(steps):
             self.step()
-            b.record()
+        last.record()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
-        per_launch = sum(a.elapsed_time(b) for a, b in ev) / steps * 1e-3
+        per_launch = first.elapsed_time(last) / steps * 1e-3
         return wall, per_launch
 
 
@@ -176,13 +197,13 @@ def moe_neighbours(steps, warmup):
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
-        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-        for a, b in ev:
-            a.record()
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        first.record()
+        for _ in range(steps):
             fn()
-            b.record()
+        last.record()
         torch.cuda.synchronize()
-        return sum(a.elapsed_time(b) for a, b in ev) / steps * 1e-3
+        return first.elapsed_time(last) / steps * 1e-3
 
     # routing: 4096 tokens x top-2 of 8 experts, int8 activations of width K = 4096 (the x of c3)
     rows, k, e, h = 4096, 2, 8, 4096
@@ -293,7 +314,7 @@ def main():
         "ms_per_step": step_s * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8 (int32 accumulate, bf16 out)", "data": "synthetic",
         "config": {"workload": f"{wl.name}: grouped W8A8, E={wl.e}, rows={work['rows']}, K={wl.k}, N={wl.n}, "
-                               f"weights {'prepacked once to [E,N,K]' if args.layout == 'nk' else '[E,K,N] as generated'}, "
+                               f"weights {LAYOUT_TEXT[args.layout]}, "
                                "routing top-2 of softmax(N(0,1))",
                    "plan": plan, "prepack_ms": prob.prepack_ms},
         "hbm_gbs": work["bytes"] / step_s / 1e9, "hbm_frac": work["bytes"] / step_s / 1e9 / PEAK_HBM_GBS,
@@ -308,7 +329,8 @@ def main():
         other = "kn" if args.layout == "nk" else "nk"
         for name, layout in [("c3", other), ("c2_m2048", "nk"), ("c2_m2048", "kn"), ("c4", "nk"), ("c4", "kn"),
                              ("c1", "nk"), ("c1", "kn"), ("c2_m256", "nk"), ("c2_m256", "kn"), ("c2_m16", "nk"),
-                             ("c2_m16", "kn"), ("c2_m1", "kn"), ("c5", "kn")]:
+                             ("c2_m16", "kn"), ("c2_m16", "packed"), ("c2_m1", "kn"), ("c2_m1", "packed"), ("c5", "kn"),
+                             ("c5", "packed")]:
             w2 = workloads.make(name)
             w_bytes = w2.w.nbytes
             hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5")
@@ -318,7 +340,7 @@ def main():
             wk, tops, gbs = rates(w2, sec)
             sweep.append({"workload": name, "layout": layout, "launch_us": sec * 1e6, "tops": tops,
                           "int8_frac": tops / PEAK_INT8_TOPS, "gbs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS,
-                          "weight_copies_rotated": copies, "kernel": p2.op.plan_info().split("kernel=")[1].split(" m=")[0]})
+                          "weight_copies_rotated": copies, "prepack_ms": p2.prepack_ms, "kernel": p2.op.plan_info().split("kernel=")[1].split(" m=")[0]})
             del p2
             torch.cuda.empty_cache()
         result["sweep"] = sweep
