@@ -207,10 +207,50 @@ def moe_token_unpermute(permuted_tokens, sorted_indices, probs, padded_mode=Fals
                                   None if restore_shape is None else [int(v) for v in restore_shape]).owner
 
 
-def trans_data(tensor, transdata_type=1):
-    """Weight pre-pass hook.  The reference converts weights to the Ascend FRACTAL_NZ format before
-    grouped_matmul (tests/st/test_grouped_matmul.py:131-133); the HIP kernels read weights as stored,
-    so this returns its input unchanged and exists only so that such call sites keep working."""
+def trans_data(tensor, transdata_type=1, nd_shape=None, transposed=False):
+    """Weight prepack, once at load time (ops/c_api/trans_data/trans_data.cc:203-223; the reference converts weights to the
+    device's blocked FRACTAL_NZ format before grouped_matmul, tests/st/test_grouped_matmul.py:131-133, and
+    grouped_matmul_v4_cops takes them with weight_format="FRACTAL_NZ", tests/st/test_grouped_matmul_v4_cops.py:514-519).
+
+    transdata_type 1 (ND_TO_FRACTAL_NZ): an int8 weight [E, K, N] (or [K, N]) on the GPU becomes an int8 tensor
+    [E, N/16, ceil(K/64), 1024] (or [N/16, ceil(K/64), 1024]) in this backend's blocked layout; N must be a multiple
+    of 16.  `grouped_matmul` recognises such a tensor by its shape, `grouped_matmul_v4_cops` takes it with
+    weight_format="FRACTAL_NZ".  Decode shapes stream it at the rate of a contiguous read.  The blocked layout is
+    defined on (k, n), not on rows and columns of whatever was stored: a weight kept as [E, N, K] (what transpose_b=True
+    describes) is packed with transposed=True, and the packed tensor is then passed with transpose_b=False.
+    transdata_type 0 (FRACTAL_NZ_TO_ND): the inverse; a torch tensor carries no logical shape besides its own, so
+    `nd_shape` ([E, K, N] or [K, N]) says what to cut the zero padding back to (default: the padded shape);
+    transposed=True returns [E, N, K].
+    Tensors of other dtypes are returned unchanged: only int8 weights have a blocked form here."""
     if transdata_type not in (0, 1):
         raise ValueError("transdata_type must be 0 (FRACTAL_NZ_TO_ND) or 1 (ND_TO_FRACTAL_NZ)")
-    return tensor
+    if not isinstance(tensor, torch.Tensor) or tensor.dtype != torch.int8:
+        return tensor
+    from . import cabi
+    if transdata_type == 1:
+        if tensor.dim() not in (2, 3):
+            raise ValueError(f"For TransData, an int8 weight must be [K, N] or [E, K, N], but got {tuple(tensor.shape)}")
+        if not tensor.is_cuda:
+            raise RuntimeError("For TransData, the input must be on the GPU (the operators have no CPU path)")
+        w = tensor.contiguous()
+        lead = (w.shape[0],) if w.dim() == 3 else ()
+        e = w.shape[0] if w.dim() == 3 else 1
+        k, n = (int(w.shape[-1]), int(w.shape[-2])) if transposed else (int(w.shape[-2]), int(w.shape[-1]))
+        if n % 16 != 0:
+            raise ValueError(f"For TransData, the N dimension must be aligned to 16, but got {n}")
+        out = torch.empty(lead + (n // 16, (k + 63) // 64, 1024), dtype=torch.int8, device=w.device)
+        with torch.cuda.device(w.device):
+            cabi.pack_weight(w.data_ptr(), out.data_ptr(), e, k, n, bool(transposed), torch.cuda.current_stream().cuda_stream)
+        return out
+    if tensor.dim() not in (3, 4) or tensor.shape[-1] != 1024:
+        raise ValueError("For TransData, FRACTAL_NZ_TO_ND takes a tensor made by ND_TO_FRACTAL_NZ "
+                         f"([E, N/16, ceil(K/64), 1024] or [N/16, ceil(K/64), 1024]), but got {tuple(tensor.shape)}")
+    lead = tuple(tensor.shape[:-3])
+    ng, kb = int(tensor.shape[-3]), int(tensor.shape[-2])
+    # byte 16 l + i of block (a, b): k = 64 b + 16 (l // 16) + i, n = 16 a + (l % 16)  ->  [.., a, b, q, c, i] -> [.., b, q, i, a, c]
+    d = len(lead)
+    v = tensor.contiguous().view(lead + (ng, kb, 4, 16, 16))
+    nd = v.permute(*range(d), d + 1, d + 2, d + 4, d + 0, d + 3).reshape(lead + (kb * 64, ng * 16))
+    if nd_shape is not None:
+        nd = nd[..., :int(nd_shape[-2]), :int(nd_shape[-1])]
+    return (nd.transpose(-1, -2) if transposed else nd).contiguous()

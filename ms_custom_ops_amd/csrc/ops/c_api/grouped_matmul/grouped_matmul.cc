@@ -8,7 +8,8 @@
 //
 // Differences, all on the side of doing less or saying so:
 //   * only the quantized path (int8 x and weight) exists on this backend; float16 x raises;
-//   * weights are consumed as stored ([E,K,N], or [E,N,K] with transpose_b): there is no FRACTAL_NZ
+//   * weights are consumed as stored ([E,K,N], or [E,N,K] with transpose_b), or prepacked by trans_data into the
+//     backend's blocked layout ([E, N/16, ceil(K/64), 1024] int8) -- the counterpart of the reference's FRACTAL_NZ
 //     pre-pass, and x_format = 1 raises;
 //   * `output_dtype` is an extra, trailing, optional argument: None keeps the reference's float16
 //     output, bfloat16 selects the bf16 epilogue.
@@ -45,7 +46,7 @@ void CheckInputRank(const ShapeVector &x_shape, const ShapeVector &weight_shape,
   if (x_shape.size() != kDim2) {
     MS_LOG_EXCEPTION << "For GroupedMatmul, input 'x' must be 2D, but got:" << x_shape.size();
   }
-  if (weight_shape.size() != kDim3) {
+  if (weight_shape.size() != kDim3 && !IsPackedWeightShape(weight_shape, kDim4)) {
     MS_LOG_EXCEPTION << "For GroupedMatmul, input 'weight' must be 3D, but got:" << weight_shape.size();
   }
   if (group_list_shape.size() != kDim1) {
@@ -60,8 +61,14 @@ ShapeVector InferGroupedMatmulOutputShape(const ShapeVector &x_shape, const Shap
   const int64_t m = transpose_a ? x_shape[kIndex1] : x_shape[kIndex0];
   const int64_t k = transpose_a ? x_shape[kIndex0] : x_shape[kIndex1];
   const int64_t e = weight_shape[kIndex0];
-  const int64_t n = transpose_b ? weight_shape[kIndex1] : weight_shape[kIndex2];
-  const int64_t wk = transpose_b ? weight_shape[kIndex2] : weight_shape[kIndex1];
+  const bool packed = IsPackedWeightShape(weight_shape, kDim4);   // [E, N / 16, ceil(K / 64), 1024] from trans_data
+  if (packed && transpose_b) {
+    MS_LOG_EXCEPTION << "For GroupedMatmul, a weight prepacked by trans_data carries its own layout; 'transpose_b' must "
+                        "be false.";
+  }
+  const int64_t n = packed ? weight_shape[kIndex1] * 16 : (transpose_b ? weight_shape[kIndex1] : weight_shape[kIndex2]);
+  const int64_t wk = packed ? (weight_shape[kIndex2] == (k + 63) / 64 ? k : weight_shape[kIndex2] * 64)
+                            : (transpose_b ? weight_shape[kIndex2] : weight_shape[kIndex1]);
   if (k != wk) {
     MS_LOG_EXCEPTION << "For GroupedMatmul, input 'x' and 'weight' must have the same dimension of 'k', but got:" << k
                      << " and " << wk;
@@ -160,6 +167,7 @@ static msco_gmm_desc MakeGroupedMatmulDesc(const TensorList &in, TypeId out_dtyp
   d.scale_dtype = in[MSCO_IN_SCALE].is_defined() ? ToBackendDtype(in[MSCO_IN_SCALE].data_type()) : MSCO_DT_NONE;
   d.per_token_dtype = in[MSCO_IN_PER_TOKEN_SCALE].is_defined() ? MSCO_DT_F32 : MSCO_DT_NONE;
   d.transpose_b = transpose_b ? 1 : 0;
+  d.weight_layout = IsPackedWeightShape(in[MSCO_IN_WEIGHT].shape(), kDim4) ? MSCO_WL_PACKED : MSCO_WL_ROW_MAJOR;
   d.scale_per_group = 1;
   return d;
 }
@@ -167,6 +175,7 @@ static msco_gmm_desc MakeGroupedMatmulDesc(const TensorList &in, TypeId out_dtyp
 static GmmProblem MakeGroupedMatmulProblem(const TensorList &in, bool transpose_b) {
   const auto &xs = in[MSCO_IN_X].shape();
   const auto &ws = in[MSCO_IN_WEIGHT].shape();
+  if (IsPackedWeightShape(ws, kDim4)) return GmmProblem{xs[0], xs[1], ws[1] * 16, ws[0]};
   return GmmProblem{xs[0], xs[1], transpose_b ? ws[1] : ws[2], ws[0]};
 }
 

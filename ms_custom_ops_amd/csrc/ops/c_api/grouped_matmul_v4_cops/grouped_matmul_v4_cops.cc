@@ -39,9 +39,9 @@ const ms::Tensor &At(const TensorVec &v, size_t i) {
 }
 
 void CheckV4Support(const V4Args &a) {
-  if (a.weight_format != kNdFormat) {
-    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", weight_format '" << a.weight_format
-                     << "' is an Ascend memory format; the HIP backend takes weights as stored (ND).";
+  if (a.weight_format != kNdFormat && a.weight_format != kFractalNzFormat) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", weight_format must be 'ND' or 'FRACTAL_NZ', but got '"
+                     << a.weight_format << "'.";
   }
   if (a.act_type != 0 || !a.activation_input.empty() || !a.activation_quant_scale.empty() ||
       !a.activation_quant_offset.empty()) {
@@ -72,7 +72,7 @@ void CheckV4Support(const V4Args &a) {
 void LaunchOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias, const ms::Tensor &scale,
                const ms::Tensor &aq_scale, const ms::Tensor &aq_offset, const ms::Tensor &per_token,
                const ms::Tensor &group_list, int64_t group_list_type, const ms::Tensor &out, int64_t m, int64_t k,
-               int64_t n, int64_t e, void *stream) {
+               int64_t n, int64_t e, bool packed, void *stream) {
   const std::string op_name = "GroupedMatmulV4";
   const TypeId xt = x.data_type();
   msco_gmm_desc d{};
@@ -83,6 +83,7 @@ void LaunchOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias,
   d.group_list_dtype = group_list.is_defined() ? ToBackendDtype(group_list.data_type()) : MSCO_DT_NONE;
   d.group_list_type = static_cast<int32_t>(group_list_type);
   d.scale_per_group = 1;
+  d.weight_layout = packed ? MSCO_WL_PACKED : MSCO_WL_ROW_MAJOR;
   const void *addrs[MSCO_IN_COUNT] = {nullptr};
   addrs[MSCO_IN_X] = x.GetDataPtr();
   addrs[MSCO_IN_WEIGHT] = w.GetDataPtr();
@@ -156,14 +157,17 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
   if (a.group_type == kGroupTypeSingleOutput) {
     const auto &x = a.x[0];
     const auto &w = a.weight[0];
-    if (x.shape().size() != kDim2 || w.shape().size() != kDim3) {
+    const bool packed = a.weight_format == kFractalNzFormat;   // [E, N / 16, ceil(K / 64), 1024] from trans_data
+    if (x.shape().size() != kDim2 || (packed ? !IsPackedWeightShape(w.shape(), kDim4) : w.shape().size() != kDim3)) {
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", with group_type 0 'x' must be [M, K] and 'weight' "
-                         << "[E, K, N], but got " << x.shape() << " and " << w.shape();
+                         << (packed ? "[E, N/16, ceil(K/64), 1024] (prepacked by trans_data)" : "[E, K, N]") << ", but got "
+                         << x.shape() << " and " << w.shape();
     }
-    const int64_t m = x.shape()[0], k = x.shape()[1], e = w.shape()[0], n = w.shape()[2];
-    if (w.shape()[1] != k) {
+    const int64_t m = x.shape()[0], k = x.shape()[1], e = w.shape()[0], n = packed ? w.shape()[1] * 16 : w.shape()[2];
+    const int64_t wk = packed ? (w.shape()[2] == (k + 63) / 64 ? k : w.shape()[2] * 64) : w.shape()[1];
+    if (wk != k) {
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", the K dimension of 'x' and 'weight' must be equal, "
-                         << "but got " << k << " and " << w.shape()[1];
+                         << "but got " << k << " and " << wk;
     }
     if (!a.group_list.is_defined()) {
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", group_type 0 needs 'group_list'.";
@@ -173,7 +177,7 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
                          << " elements, but got " << a.group_list.data_type() << " " << a.group_list.shape();
     }
     LaunchOne(x, w, At(a.bias, 0), At(a.scale, 0), At(a.antiquant_scale, 0), At(a.antiquant_offset, 0),
-              At(a.per_token_scale, 0), a.group_list, a.group_list_type, outputs.at(0), m, k, n, e, stream);
+              At(a.per_token_scale, 0), a.group_list, a.group_list_type, outputs.at(0), m, k, n, e, packed, stream);
     return;
   }
   if (a.group_type != kGroupTypeMultiOutput) {
@@ -184,18 +188,21 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
   for (size_t i = 0; i < a.x.size(); ++i) {
     const auto &x = a.x[i];
     const auto &w = a.weight[i];
-    if (w.shape().size() != kDim2 || x.shape().size() < kDim2) {
-      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", with group_type -1 every weight must be [K, N] "
+    const bool packed = a.weight_format == kFractalNzFormat;   // [N / 16, ceil(K / 64), 1024] from trans_data
+    if ((packed ? !IsPackedWeightShape(w.shape(), kDim3) : w.shape().size() != kDim2) || x.shape().size() < kDim2) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", with group_type -1 every weight must be "
+                         << (packed ? "[N/16, ceil(K/64), 1024] (prepacked by trans_data) " : "[K, N] ")
                          << "and every x at least 2D, but got " << x.shape() << " and " << w.shape();
     }
-    const int64_t k = x.shape().back(), n = w.shape()[1];
-    if (w.shape()[0] != k) {
+    const int64_t k = x.shape().back(), n = packed ? w.shape()[0] * 16 : w.shape()[1];
+    const int64_t wk = packed ? (w.shape()[1] == (k + 63) / 64 ? k : w.shape()[1] * 64) : w.shape()[0];
+    if (wk != k) {
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", the K dimension of 'x' and 'weight' must be equal, "
-                         << "but got " << k << " and " << w.shape()[0];
+                         << "but got " << k << " and " << wk;
     }
     const int64_t rows = k > 0 ? x.numel() / k : 0;
     LaunchOne(x, w, At(a.bias, i), At(a.scale, i), At(a.antiquant_scale, i), At(a.antiquant_offset, i),
-              At(a.per_token_scale, i), ms::Tensor(), 0, outputs.at(i), rows, k, n, 1, stream);
+              At(a.per_token_scale, i), ms::Tensor(), 0, outputs.at(i), rows, k, n, 1, packed, stream);
   }
 }
 }  // namespace
@@ -268,7 +275,7 @@ std::vector<ms::Tensor> grouped_matmul_v4_cops_custom(
   const int64_t &group_list_type, const int64_t &act_type, const std::string &weight_format,
   const std::optional<int64_t> &output_dtype) {
   auto output_types = InferOutputTypes(x, weight, scale, output_dtype);
-  auto output_shapes = InferOutputShapes(x, weight, group_list, group_type);
+  auto output_shapes = InferOutputShapes(x, weight, group_list, group_type, weight_format);
   if (output_types.size() != output_shapes.size()) {
     MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName
                        << ", the number of output types must be equal to the number of output shapes, "

@@ -50,8 +50,20 @@ TypeIdList InferOutputTypes(const TensorVec &x, const TensorVec &weight, const s
 }
 
 ShapeArray InferOutputShapes(const TensorVec &x, const TensorVec &weight, const std::optional<ms::Tensor> &group_list,
-                             const int64_t &group_type) {
+                             const int64_t &group_type, const std::string &weight_format) {
   ShapeArray output_shapes;
+  // FRACTAL_NZ on this backend: weights prepacked by trans_data, int8 [E, N / 16, ceil(K / 64), 1024] (no E for the
+  // per-matrix form); N comes from the number of 16-column groups
+  const bool packed = weight_format == kFractalNzFormat;
+  auto n_of = [&](const ms::Tensor &w, size_t rank) -> int64_t {
+    if (!packed) return w.shape().back();
+    if (!IsPackedWeightShape(w.shape(), rank) || w.data_type() != kNumberTypeInt8) {
+      MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", weight_format 'FRACTAL_NZ' takes Int8 weights "
+                         << "prepacked by trans_data (last dimension 1024, rank " << rank << "), but got " << w.data_type()
+                         << " " << w.shape();
+    }
+    return w.shape()[rank - kDim3] * 16;
+  };
   if (group_type == kGroupTypeMultiOutput) {
     if (x.size() != weight.size()) {
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName
@@ -63,7 +75,7 @@ ShapeArray InferOutputShapes(const TensorVec &x, const TensorVec &weight, const 
       if (res_shape.empty() || weight[i].shape().empty()) {
         MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", 'x' and 'weight' must not be scalars.";
       }
-      res_shape.back() = weight[i].shape().back();
+      res_shape.back() = n_of(weight[i], kDim3);
       output_shapes.emplace_back(std::move(res_shape));
     }
     return output_shapes;
@@ -78,7 +90,7 @@ ShapeArray InferOutputShapes(const TensorVec &x, const TensorVec &weight, const 
     MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", 'x' must be at least 2D, but got " << x_shape;
   }
   const int64_t m = x_shape[x_shape.size() - kIndex2];
-  int64_t n = w_shape.back();
+  int64_t n = n_of(weight[0], kDim4);
   if (weight[0].data_type() == kNumberTypeInt4) n <<= 1;
   const int64_t group_list_size = group_list.has_value() ? group_list.value().shape()[0] : 1;
   if (group_type == kGroupTypeSingleOutput) {
@@ -140,7 +152,9 @@ ShapeArray GroupedMatmulV4CopsFuncImpl::InferShape(const KernelTensorList &input
                          << gl->shape().size();
     }
   }
-  return InferOutputShapes(inputs[kXIndex].sequence, inputs[kWeightIndex].sequence, gl, group_type);
+  const std::string weight_format =
+    inputs[kWeightFormatIndex].IsNone() ? std::string(kNdFormat) : inputs[kWeightFormatIndex].GetValueWithCheck<std::string>();
+  return InferOutputShapes(inputs[kXIndex].sequence, inputs[kWeightIndex].sequence, gl, group_type, weight_format);
 }
 
 TypeIdList GroupedMatmulV4CopsFuncImpl::InferType(const KernelTensorList &inputs) const {

@@ -4,6 +4,7 @@
 #ifndef MS_CUSTOM_OPS_OPS_C_API_GROUPED_MATMUL_V4_COPS_FUNC_IMPL_H_
 #define MS_CUSTOM_OPS_OPS_C_API_GROUPED_MATMUL_V4_COPS_FUNC_IMPL_H_
 
+#include <string>
 #include <optional>
 #include <vector>
 
@@ -37,7 +38,7 @@ using TensorVec = std::vector<ms::Tensor>;
 TypeIdList InferOutputTypes(const TensorVec &x, const TensorVec &weight, const std::optional<TensorVec> &scale,
                             const std::optional<int64_t> &output_dtype);
 ShapeArray InferOutputShapes(const TensorVec &x, const TensorVec &weight, const std::optional<ms::Tensor> &group_list,
-                             const int64_t &group_type);
+                             const int64_t &group_type, const std::string &weight_format = "ND");
 
 // Graph mode sees the twelve list inputs flattened into one positional list; group_info[i] is the
 // length of list i (0 = None, which still occupies one slot), as the reference's tuple-unfolding

@@ -25,11 +25,18 @@ constexpr size_t kIndex3{3};
 constexpr size_t kDim1{1};
 constexpr size_t kDim2{2};
 constexpr size_t kDim3{3};
+constexpr size_t kDim4{4};
 constexpr size_t kNumber1{1};
 constexpr size_t kNumber2{2};
 
 constexpr auto kFractalNzFormat = "FRACTAL_NZ";
 constexpr auto kNdFormat = "ND";
+// Weights prepacked by trans_data(..., ND_TO_FRACTAL_NZ) travel as int8 tensors whose last dimension is one 1024-byte
+// block: [E, N / 16, ceil(K / 64), 1024], or [N / 16, ceil(K / 64), 1024] for a single matrix.
+constexpr int64_t kPackedBlockBytes = 1024;
+inline bool IsPackedWeightShape(const std::vector<int64_t> &shape, size_t rank) {
+  return shape.size() == rank && shape.back() == kPackedBlockBytes;
+}
 
 enum class DataFormat : int32_t { ND = 0, FRACTAL_NZ = 1 };
 

@@ -18,7 +18,7 @@ def _t(a):
 
 
 def custom_grouped_matmul(m, k, n, e, trans_b=True, with_bias=True, with_pertoken_scale=False, scale_dtype="float32",
-                          out_dtype=None, seed=0):
+                          out_dtype=None, seed=0, prepack=False):
     """Same input recipe as the reference's custom_grouped_matmul (test_grouped_matmul.py:85-159)."""
     rng = np.random.default_rng(seed)
     x = rng.uniform(-20, 20, size=[m, k]).astype(np.int8)
@@ -29,7 +29,16 @@ def custom_grouped_matmul(m, k, n, e, trans_b=True, with_bias=True, with_pertoke
     gl = O.random_group_list(m, e, rng).astype(np.int32)
 
     w_dev = np.transpose(w, (0, 2, 1)) if trans_b else w
-    weight = ms_custom_ops.trans_data(_t(w_dev), transdata_type=1)   # a no-op hook on this backend
+    if prepack:
+        # the reference's flow (weight to the device's blocked format first, test_grouped_matmul.py:131-133): the packed
+        # tensor carries its own layout, so the op is then called with transpose_b = False
+        weight = ms_custom_ops.trans_data(_t(w_dev), transdata_type=1, transposed=trans_b)
+        assert tuple(weight.shape) == (e, n // 16, (k + 63) // 64, 1024)
+        back = ms_custom_ops.trans_data(weight, transdata_type=0, nd_shape=(e, k, n), transposed=trans_b)
+        assert torch.equal(back, _t(w_dev))
+        trans_b = False
+    else:
+        weight = _t(w_dev)
     scale = _t(s) if scale_dtype == "float32" else _t(O.encode_scale_int64(s))
     out = ms_custom_ops.grouped_matmul(_t(x), weight, _t(gl), _t(b), scale, _t(ps), None, False, trans_b,
                                        output_dtype=out_dtype)
@@ -103,3 +112,34 @@ def test_plan_cache_hits_on_repeated_shapes(device):
         custom_grouped_matmul(64, 64, 128, 8, seed=3)
     h1, m1, size = ms_custom_ops.plan_cache_stats()
     assert m1 - m0 == 1 and h1 - h0 == 2 and size >= 1
+
+
+@pytest.mark.parametrize("m", [24, 1000])
+@pytest.mark.parametrize("trans_b", [True, False])
+@pytest.mark.parametrize("exec_mode", MODES)
+def test_gmm_on_weights_prepacked_by_trans_data(device, m, trans_b, exec_mode):
+    """trans_data(ND_TO_FRACTAL_NZ) then grouped_matmul, as the reference's callers do (test_grouped_matmul.py:131-147):
+    decode-sized M takes the streaming kernel, large M the generic one; both bit-exact."""
+    with ms_custom_ops.exec_mode(exec_mode):
+        custom_grouped_matmul(m, 192, 128, 8, trans_b=trans_b, with_pertoken_scale=True, prepack=True)
+        custom_grouped_matmul(m, 192, 128, 8, trans_b=trans_b, out_dtype=torch.bfloat16, prepack=True)
+
+
+def test_trans_data_rules(device):
+    w = torch.zeros(8, 64, 40, dtype=torch.int8, device="cuda")
+    with pytest.raises(ValueError, match="N dimension must be aligned to 16"):
+        ms_custom_ops.trans_data(w, 1)
+    with pytest.raises(ValueError, match="transdata_type must be 0"):
+        ms_custom_ops.trans_data(w, 2)
+    with pytest.raises(ValueError, match="FRACTAL_NZ_TO_ND takes a tensor made by"):
+        ms_custom_ops.trans_data(w, 0)
+    f = torch.zeros(8, 64, 48, dtype=torch.float16, device="cuda")
+    assert ms_custom_ops.trans_data(f, 1) is f                      # only int8 weights have a blocked form
+    packed = ms_custom_ops.trans_data(torch.zeros(8, 64, 48, dtype=torch.int8, device="cuda"), 1)
+    x = torch.zeros(4, 64, dtype=torch.int8, device="cuda")
+    gl = torch.full((8,), 4, dtype=torch.int32, device="cuda")
+    s = torch.ones(8, 48, device="cuda")
+    with pytest.raises(RuntimeError, match="'transpose_b' must be false"):
+        ms_custom_ops.grouped_matmul(x, packed, gl, None, s, None, None, False, True)
+    with pytest.raises(RuntimeError, match="same dimension of 'k'"):
+        ms_custom_ops.grouped_matmul(torch.zeros(4, 128, dtype=torch.int8, device="cuda"), packed, gl, None, s)

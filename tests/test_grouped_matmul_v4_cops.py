@@ -128,13 +128,57 @@ def test_v4_multi_output_group_type_minus_one(device, mode):
         assert np.array_equal(r.view(torch.int16).cpu().numpy().view(np.uint16), ref)
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("weight_format", ["ND", "FRACTAL_NZ"])
+def test_v4_fractal_nz(device, mode, weight_format):
+    """The reference's test_ops_grouped_mamtul_v4_fractal_nz (test_grouped_matmul_v4_cops.py:486-520) on the quantized
+    path: the weight goes through trans_data(ND_TO_FRACTAL_NZ) and the op is told weight_format="FRACTAL_NZ";
+    group_type -1 with one [16, 256] x [256, 128] problem as there, and the grouped form (group_type 0)."""
+    rng = np.random.default_rng(1)
+    x0 = rng.integers(-127, 128, (16, 256), dtype=np.int8)
+    w0 = rng.integers(-127, 128, (256, 128), dtype=np.int8)
+    s0 = rng.uniform(1e-3, 1e-2, 128).astype(np.float32)
+    prep = (lambda t: ms_custom_ops.trans_data(t, transdata_type=1)) if weight_format == "FRACTAL_NZ" else (lambda t: t)
+    with ms_custom_ops.exec_mode(mode):
+        res = ms_custom_ops.grouped_matmul_v4_cops([_t(x0)], [prep(_t(w0))], None, [_t(s0)], split_item=0, group_type=-1,
+                                                   weight_format=weight_format, output_dtype=torch.bfloat16)
+    assert tuple(res[0].shape) == (16, 128)
+    assert np.array_equal(res[0].view(torch.int16).cpu().numpy().view(np.uint16), O.quant_batch_matmul_oracle(x0, w0, s0))
+
+    x = rng.integers(-127, 128, (40, 320), dtype=np.int8)
+    w = rng.integers(-127, 128, (8, 320, 272), dtype=np.int8)
+    s = rng.uniform(1e-3, 1e-2, (8, 272)).astype(np.float32)
+    pt = rng.uniform(1e-3, 1e-2, 40).astype(np.float32)
+    gl = np.array([3, 3, 10, 17, 22, 30, 30, 40], dtype=np.int64)
+    with ms_custom_ops.exec_mode(mode):
+        out = ms_custom_ops.grouped_matmul_v4_cops([_t(x)], [prep(_t(w))], None, [_t(s)], None, None, None, [_t(pt)], _t(gl),
+                                                   split_item=3, group_type=0, weight_format=weight_format,
+                                                   output_dtype=torch.bfloat16)[0]
+        acc = ms_custom_ops.grouped_matmul_v4_cops([_t(x)], [prep(_t(w))], group_list=_t(gl), split_item=3, group_type=0,
+                                                   weight_format=weight_format)[0]
+    ref_bits, ref_acc = O.grouped_matmul_w8a8(x, w, gl, None, s, pt, return_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), ref_acc)
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), ref_bits)
+    # weight-only path on the same prepacked weights
+    xb = _t(rng.standard_normal((40, 320)).astype(np.float32), torch.bfloat16)
+    aq = _t(rng.uniform(1e-3, 1e-2, (8, 272)).astype(np.float32), torch.bfloat16)
+    ao = _t(rng.integers(-8, 9, (8, 272)).astype(np.float32), torch.bfloat16)
+    with ms_custom_ops.exec_mode(mode):
+        wo = ms_custom_ops.grouped_matmul_v4_cops([xb], [prep(_t(w))], None, None, None, [aq], [ao], None, _t(gl),
+                                                  split_item=3, group_type=0, weight_format=weight_format)[0]
+    exact = O.a16w8_grouped_f64(xb.float().cpu().numpy(), w, aq.float().cpu().numpy(), ao.float().cpu().numpy(), gl)
+    np.testing.assert_allclose(wo.float().cpu().numpy(), exact, rtol=2 ** -6, atol=0.05)
+
+
 def test_v4_errors(device):
     x = torch.zeros(32, 64, dtype=torch.int8, device="cuda")
     w = torch.zeros(8, 64, 128, dtype=torch.int8, device="cuda")
     gl = torch.full((8,), 4, dtype=torch.int64, device="cuda")
     f = ms_custom_ops.grouped_matmul_v4_cops
-    with pytest.raises(RuntimeError, match="weight_format 'FRACTAL_NZ'"):
+    with pytest.raises(ValueError, match="weight_format 'FRACTAL_NZ' takes Int8 weights prepacked by trans_data"):
         f([x], [w], group_list=gl, split_item=3, group_type=0, weight_format="FRACTAL_NZ")
+    with pytest.raises(RuntimeError, match="weight_format must be 'ND' or 'FRACTAL_NZ'"):
+        f([x], [w], group_list=gl, split_item=3, group_type=0, weight_format="NC1HWC0")
     with pytest.raises(RuntimeError, match="fused activation is not implemented"):
         f([x], [w], group_list=gl, split_item=3, group_type=0, act_type=1)
     with pytest.raises(RuntimeError, match="quantized paths only"):
