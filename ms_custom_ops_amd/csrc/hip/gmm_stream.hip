@@ -300,6 +300,213 @@ hipError_t launch_stream_w8a8(const GmmParams &p, hipStream_t stream) {
   return stream_launch_w8a8<4>(p, grid, stream);
 }
 
+// ---- W8A8, more than 16 rows per group (packed weights) -----------------------------------------------------
+// Same streaming idea for 16 TCH rows per workgroup (TCH = 2, 4, 8): a workgroup owns one chunk of 16 TCH rows of one
+// group, a strip of four column groups (64 columns) and one K slice; wave w takes K blocks w, w + 4, ...  Per K block
+// a wave loads its TCH x fragments (16 rows x 64 K bytes each) and the four weight blocks and issues 4 TCH MFMAs into
+// accumulators that stay in registers for the whole slice.  At the end the four waves add their tiles into one LDS
+// tile with ds_add (int32: exact in any order), K slices of different workgroups meet in the workspace as in the
+// kernels above, and the epilogue stages the 16 TCH x 64 output tile in LDS for whole-row stores.  Operand delivery
+// from L2 bounds this kernel, not the matrix pipe: per K block a wave moves (TCH + 4) KiB for 4 TCH MFMAs.
+namespace {
+constexpr int SM_GROUPS = 4;                    // column groups per strip
+constexpr int SM_COLS = SM_GROUPS * 16;
+template <int TCH>
+struct SmShape {
+  static constexpr int kRows = 16 * TCH;
+  static constexpr int kFrags = SM_GROUPS * TCH;              // 16 x 16 int32 fragments of the tile
+  static constexpr int kTileInts = kRows * SM_COLS;
+  static constexpr size_t kLds = (size_t)kTileInts * 4 + 16;   // int32 tile (later the 16-bit output tile) + ticket
+};
+}  // namespace
+
+template <int TCH>
+__global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_streamm_kernel(const GmmParams p) {
+  using S = SmShape<TCH>;
+  extern __shared__ __align__(16) unsigned char st_smem[];
+  int *tile = reinterpret_cast<int *>(st_smem);   // fragment (cg, t), lane, r at ((cg * TCH + t) * 64 + lane) * 4 + r
+  unsigned *s_ticket = reinterpret_cast<unsigned *>(st_smem + S::kLds - 16);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c16 = lane & 15, h = lane >> 4;
+  const int strip = blockIdx.x, ks = blockIdx.z;
+  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
+
+  int g_start = 0, g_end = 0;
+  for (int g = 0; g <= grp; ++g) {
+    g_start = g_end;
+    g_end = group_end(p, g, g_start);
+  }
+  const int m0 = g_start + mc * S::kRows;
+  const int chunk_rows = min(S::kRows, g_end - m0);
+  if (chunk_rows <= 0) return;
+
+  for (int i = tid; i < S::kTileInts / 4; i += ST_THREADS) reinterpret_cast<v4i *>(tile)[i] = v4i{0, 0, 0, 0};
+
+  const int n0 = strip * SM_COLS;
+  const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
+  const int cg_count = min(SM_GROUPS, col_groups - strip * SM_GROUPS);
+  const long long group_bytes = (long long)col_groups * k_blocks * 1024;
+  const __amdgpu_buffer_rsrc_t rw = buffer_over(p.w + (long long)grp * group_bytes, group_bytes);
+  const __amdgpu_buffer_rsrc_t rx = buffer_over(p.x, (long long)p.m * p.k);   // planned only when M * K < 2^31
+  const int per_split = (k_blocks + p.split_k - 1) / p.split_k;
+  const int kb_begin = ks * per_split;
+  const int kb_end = min(k_blocks, kb_begin + per_split);
+  const int cg_base = strip * SM_GROUPS * k_blocks * 1024;
+
+  // row of fragment t in this lane (clamped into the group: rows past the chunk are computed and never stored)
+  unsigned xoff[TCH];
+#pragma unroll
+  for (int t = 0; t < TCH; ++t) xoff[t] = (unsigned)(min(m0 + 16 * t + c16, g_end - 1) * p.k + 16 * h);
+
+  v4i acc[SM_GROUPS][TCH];
+#pragma unroll
+  for (int cg = 0; cg < SM_GROUPS; ++cg)
+#pragma unroll
+    for (int t = 0; t < TCH; ++t) acc[cg][t] = v4i{0, 0, 0, 0};
+
+  auto fetch = [&](int kb, v4i (&xf)[TCH], v4i (&wv)[SM_GROUPS]) {
+    const bool live = kb < kb_end;
+    const bool k_ok = live && kb * 64 + 16 * h < p.k;   // K % 16 == 0: 16 K bytes all inside or all outside
+#pragma unroll
+    for (int cg = 0; cg < SM_GROUPS; ++cg)
+      wv[cg] = __builtin_amdgcn_raw_buffer_load_b128(rw, (live && cg < cg_count) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
+                                                     cg_base + cg * k_blocks * 1024, 0);
+#pragma unroll
+    for (int t = 0; t < TCH; ++t)
+      xf[t] = __builtin_amdgcn_raw_buffer_load_b128(rx, k_ok ? xoff[t] + (unsigned)(kb * 64) : kBufferOob, 0, 0);
+  };
+  auto multiply = [&](const v4i (&xf)[TCH], const v4i (&wv)[SM_GROUPS]) {
+#pragma unroll
+    for (int cg = 0; cg < SM_GROUPS; ++cg)
+#pragma unroll
+      for (int t = 0; t < TCH; ++t) acc[cg][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(xf[t], wv[cg], acc[cg][t], 0, 0, 0);
+  };
+  {
+    // two K blocks in flight per wave: the loads of the next block are issued before this one is multiplied
+    v4i xa[TCH], wa[SM_GROUPS], xb[TCH], wb[SM_GROUPS];
+    int kb = kb_begin + wave;
+    fetch(kb, xa, wa);
+    for (; kb < kb_end; kb += 2 * ST_WAVES) {
+      fetch(kb + ST_WAVES, xb, wb);   // past the slice: masked, zeros
+      multiply(xa, wa);
+      fetch(kb + 2 * ST_WAVES, xa, wa);
+      multiply(xb, wb);
+    }
+  }
+
+  __syncthreads();   // the tile is zeroed
+#pragma unroll
+  for (int cg = 0; cg < SM_GROUPS; ++cg)
+#pragma unroll
+    for (int t = 0; t < TCH; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        __hip_atomic_fetch_add(tile + ((cg * TCH + t) * 64 + lane) * 4 + r, acc[cg][t][r], __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+  __syncthreads();
+
+  // thread tid owns fragments f = j * 4 + wave (j = 0..TCH-1) at its lane position: rows 16 t + 4 h + r, column 16 cg + c
+  constexpr int OWN = S::kFrags / ST_WAVES;   // = TCH
+  v4i v[OWN];
+#pragma unroll
+  for (int j = 0; j < OWN; ++j) v[j] = reinterpret_cast<const v4i *>(tile)[(j * ST_WAVES + wave) * 64 + lane];
+
+  if (p.split_k > 1) {
+    // slice s, fragment word (j, half) of thread t at ((s * OWN + j) * 2 + half) * 256 + t, 64-bit words
+    const long long tile_id = ((long long)grp * p.max_chunks + mc) * p.n_strips + strip;
+    i64 *base = reinterpret_cast<i64 *>(p.partial) + tile_id * p.split_k * (S::kTileInts / 2);
+    i64 *mine = base + (long long)ks * (S::kTileInts / 2) + tid;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        const i64 word = (i64)(((unsigned long long)(unsigned)v[j][2 * hf + 1] << 32) | (unsigned)v[j][2 * hf]);
+        __hip_atomic_store(mine + (j * 2 + hf) * ST_THREADS, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (tid == 0) *s_ticket = __hip_atomic_fetch_add(&p.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*s_ticket != (unsigned)(p.split_k - 1)) return;
+    if (tid == 0) __hip_atomic_store(&p.counters[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) v[j] = v4i{0, 0, 0, 0};
+    for (int s = 0; s < p.split_k; ++s) {
+      const i64 *src = base + (long long)s * (S::kTileInts / 2) + tid;
+      i64 t2[OWN][2];
+#pragma unroll
+      for (int j = 0; j < OWN; ++j)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+          t2[j][hf] = __hip_atomic_load(src + (j * 2 + hf) * ST_THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int j = 0; j < OWN; ++j)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          v[j][2 * hf] += (int)(unsigned)(unsigned long long)t2[j][hf];
+          v[j][2 * hf + 1] += (int)(unsigned)((unsigned long long)t2[j][hf] >> 32);
+        }
+    }
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------------------
+  unsigned short(*tile_out)[SM_COLS + 8] = reinterpret_cast<unsigned short(*)[SM_COLS + 8]>(st_smem);
+  __syncthreads();   // every thread holds its part of the int32 tile: the LDS tile can be reused
+#pragma unroll
+  for (int j = 0; j < OWN; ++j) {
+    const int f = j * ST_WAVES + wave, cg = f / TCH, t = f % TCH;
+    const int cl = 16 * cg + c16, n = n0 + cl;
+    if (cg < cg_count && n < p.n) {
+      const int bias = load_bias(p, grp, n);
+      const float sc = p.out_dtype == DT_I32 ? 1.0f : load_scale(p, grp, n);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = 16 * t + 4 * h + r;
+        if (row < chunk_rows) {
+          if (p.out_dtype == DT_I32) {
+            reinterpret_cast<int *>(p.out)[(long long)(m0 + row) * p.n + n] = v[j][r] + bias;
+          } else {
+            const float f32 = dequant(v[j][r] + bias, sc, p.per_token ? p.per_token[m0 + row] : 1.0f);
+            tile_out[row][cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f32) : f32_to_f16_rne(f32);
+          }
+        }
+      }
+    }
+  }
+  if (p.out_dtype == DT_I32) return;
+  __syncthreads();
+  // whole-row stores: 16 TCH rows x 8 pieces of 8 columns
+  for (int item = tid; item < S::kRows * 8; item += ST_THREADS) {
+    const int row = item >> 3, c8 = (item & 7) * 8;
+    const int n = n0 + c8;
+    if (row < chunk_rows && c8 < 16 * cg_count && n < p.n) {
+      const uint4 q = *reinterpret_cast<const uint4 *>(&tile_out[row][c8]);
+      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned short *>(p.out) + (long long)(m0 + row) * p.n + n) = q;
+    }
+  }
+}
+
+int streamm_chunk_rows(int tch) { return 16 * tch; }
+size_t streamm_tile_bytes(int tch) { return (size_t)16 * tch * SM_COLS * 4; }
+
+template <int TCH>
+static hipError_t streamm_launch(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
+  hipLaunchKernelGGL(gmm_w8a8_streamm_kernel<TCH>, grid, dim3(ST_THREADS), SmShape<TCH>::kLds, stream, p);
+  return hipGetLastError();
+}
+
+// tch = 16-row fragments per chunk (2, 4 or 8); p.max_chunks counts chunks of 16 tch rows, p.n_strips strips of 64 columns
+hipError_t launch_streamm_w8a8(const GmmParams &p, int tch, hipStream_t stream) {
+  if (p.m == 0) return hipSuccess;
+  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  if (tch == 8) return streamm_launch<8>(p, grid, stream);
+  if (tch == 4) return streamm_launch<4>(p, grid, stream);
+  if (tch == 2) return streamm_launch<2>(p, grid, stream);
+  return hipErrorInvalidValue;
+}
+
 // ---- weight-only (bf16 / f16 activations) ------------------------------------------------------------------
 // The 16 K bytes a lane holds of a block feed two v_mfma_f32_16x16x32_{bf16,f16}: bytes 0..7 and bytes 8..15, each
 // turned into exact 16-bit values of (w + 128) (v_cvt_f32_ubyteN on w ^ 0x80, then a 16-bit pack).  The x fragments

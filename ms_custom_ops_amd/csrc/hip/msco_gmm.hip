@@ -53,6 +53,7 @@ struct msco_gmm_op {
   int skinny_cols = kSkinnyCols;
   int n_strips = 0;
   int strip_groups = 16;
+  int stream_tch = 1;        // packed W8A8: 16-row fragments per chunk (1: gmm_w8a8_stream_kernel, 2/4/8: the multi-row kernel)
   size_t workspace_bytes = 0;
   unsigned *counters = nullptr;
   size_t counters_cap = 0;
@@ -120,9 +121,9 @@ void choose_plan(msco_gmm_op *op) {
   if (!aligned) {
     family = FAM_GENERIC;
   } else if (is_packed(d)) {
-    // packed weights: the streaming decode kernels (W8A8 up to kSkinnyMaxRows rows, weight-only at any M, like its
-    // row-major counterpart); W8A8 with larger M has no MFMA kernel for this layout yet and runs the generic one
-    family = (m <= kSkinnyMaxRows || is_a16w8(d)) ? FAM_SKINNY : FAM_GENERIC;
+    // packed weights: the streaming kernels at any M (W8A8 with more than 16 rows per group: the multi-row variant;
+    // there is no tile kernel for this layout yet, so large M re-streams the weights from L2 once per 128 rows)
+    family = FAM_SKINNY;
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
   } else if (m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) {
@@ -179,23 +180,40 @@ void choose_plan(msco_gmm_op *op) {
       op->workspace_bytes = tile_workspace_bytes(op->tile_cfg, m, n, e, op->split_k);
     }
   }
+  op->stream_tch = 1;
+  if (family == FAM_SKINNY && is_packed(d) && is_w8a8(d)) {
+    // rows a group is expected to hold (shapes only): 16-row chunks up to 16 rows, else chunks of 32 / 64 / 128 rows
+    const int64_t rows = e == 1 ? m : (m + e - 1) / e;
+    op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
+  }
   if (family == FAM_SKINNY) {
-    // grid.y enumerates (group, 16-row chunk)
-    op->max_chunks = (int)((m + kSkinnyRows - 1) / kSkinnyRows);
+    // grid.y enumerates (group, chunk of 16 * stream_tch rows)
+    const int64_t chunk_rows = (int64_t)kSkinnyRows * op->stream_tch;
+    op->max_chunks = (int)((m + chunk_rows - 1) / chunk_rows);
     if (op->max_chunks < 1) op->max_chunks = 1;
     if (e * op->max_chunks > 65535) family = FAM_GENERIC;
   }
   if (family == FAM_SKINNY) {
     // Only shapes enter: the number of (group, chunk) pairs that can hold rows is estimated from M and E.
     const int64_t active = std::max<int64_t>(
-      1, std::min<int64_t>(e * op->max_chunks, std::min<int64_t>(m, e) + m / kSkinnyRows));
+      1, std::min<int64_t>(e * op->max_chunks, std::min<int64_t>(m, e) + m / (kSkinnyRows * op->stream_tch)));
     const int64_t tiles128 = ((n + 127) / 128) * active;
     int wide16 = is_w8a8(d) && tiles128 <= kNumCUs && !is_packed(d);
     const int forced_variant = env_int("MSCO_SKINNY_WIDE16", -1);
     if (forced_variant >= 0 && is_w8a8(d)) wide16 = forced_variant != 0;
     op->skinny_wide16 = wide16;
     int want, cap;
-    if (is_packed(d)) {
+    if (is_packed(d) && op->stream_tch > 1) {
+      // multi-row kernel: strips of four column groups, K split until about two workgroups per CU stream operands
+      const int64_t col_groups = (n + 15) / 16, k_blocks = (k + 63) / 64;
+      op->strip_groups = 4;
+      op->n_strips = (int)((col_groups + 3) / 4);
+      op->skinny_cols = 64;
+      const int64_t base = (int64_t)op->n_strips * active;
+      want = (int)(kTargetWorkgroups / std::max<int64_t>(base, 1));
+      cap = std::max<int>(1, (int)(k_blocks / 16));      // a slice keeps at least 16 blocks
+      want = std::max(1, std::min(std::min(want, kMaxSplitK), cap));
+    } else if (is_packed(d)) {
       // Packed weights: strips as wide as still give every CU a workgroup without splitting K (a slice holds at
       // most 128 blocks of 64 bytes), then a K split up to about two workgroups per CU.
       const int64_t col_groups = (n + 15) / 16, k_blocks = (k + 63) / 64;
@@ -227,7 +245,7 @@ void choose_plan(msco_gmm_op *op) {
     want = std::max(1, std::min(want, cap));
     const int forced = env_int("MSCO_SKINNY_SPLIT_K", 0);
     if (forced > 0) want = std::min(forced, cap);
-    if (is_packed(d)) {   // also under a forced split
+    if (is_packed(d) && op->stream_tch == 1) {   // also under a forced split
       const int slice_blocks = is_w8a8(d) ? 128 : 64;
       want = std::max(want, (int)(((k + 63) / 64 + slice_blocks - 1) / slice_blocks));
     }
@@ -235,9 +253,12 @@ void choose_plan(msco_gmm_op *op) {
     if (!is_packed(d)) op->skinny_cols = wide16 ? 128 : kSkinnyCols;
     if (is_packed(d)) {
       // the packed-layout kernels keep a full 16 x 256 partial tile per (strip, K slice) whatever the strip's width
-      const size_t tile_bytes = is_w8a8(d) ? (size_t)kSkinnyRows * kSkinnyCols * 4 : stream_a16w8_tile_bytes();
-      op->workspace_bytes =
-        op->split_k > 1 ? skinny_counter_count(m, n, e, op->skinny_cols) * (size_t)op->split_k * tile_bytes : 0;
+      const size_t tile_bytes = !is_w8a8(d)           ? stream_a16w8_tile_bytes()
+                                : op->stream_tch > 1 ? streamm_tile_bytes(op->stream_tch)
+                                                     : (size_t)kSkinnyRows * kSkinnyCols * 4;
+      const size_t tiles = op->stream_tch > 1 ? (size_t)e * op->max_chunks * op->n_strips
+                                              : skinny_counter_count(m, n, e, op->skinny_cols);
+      op->workspace_bytes = op->split_k > 1 ? tiles * (size_t)op->split_k * tile_bytes : 0;
     } else {
       op->workspace_bytes = is_w8a8(d) ? skinny_workspace_bytes(m, n, e, op->split_k, op->skinny_cols)
                                        : a16w8_workspace_bytes(m, n, e, op->split_k);
@@ -250,7 +271,7 @@ void choose_plan(msco_gmm_op *op) {
   std::snprintf(buf, sizeof(buf),
                 "msco_gmm plan: kernel=%s%s%s%s layout=%s m=%lld k=%lld n=%lld e=%lld split_k=%d strips=%d "
                 "workspace=%zu",
-                is_w8a8(d) ? "w8a8_" : "a16w8_", (family == FAM_SKINNY && is_packed(d)) ? "stream" : fam,
+                is_w8a8(d) ? "w8a8_" : "a16w8_", (family == FAM_SKINNY && is_packed(d)) ? (op->stream_tch > 1 ? "stream_rows" : "stream") : fam,
                 family == FAM_TILE ? (std::string("_") + tile_cfg_name(op->tile_cfg)).c_str() : "",
                 (family == FAM_SKINNY && op->skinny_wide16) ? "_16w" : "",
                 is_packed(d) ? "packed" : d.transpose_b ? "[E,N,K]" : "[E,K,N]", (long long)m, (long long)k, (long long)n, (long long)e,
@@ -378,7 +399,8 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   const int layout = layout_of(d);
   if (is_w8a8(d)) {
     if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, s);
-    else if (h->family == FAM_SKINNY) err = layout == 2 ? launch_stream_w8a8(p, s) : launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
+    else if (h->family == FAM_SKINNY && layout == 2) err = h->stream_tch > 1 ? launch_streamm_w8a8(p, h->stream_tch, s) : launch_stream_w8a8(p, s);
+    else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
     else err = launch_generic_w8a8(p, layout, s);
   } else {
     if (h->family == FAM_SKINNY) err = layout == 2 ? launch_stream_a16w8(p, s) : launch_skinny_a16w8(p, s);

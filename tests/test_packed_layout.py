@@ -79,10 +79,24 @@ def test_counts_and_rows_past_the_last_boundary(device):
     _check(x, w, [10, 0, 20, 5], bias, scale, pt, group_list_type=1)    # 35 of 48 rows belong to a group
 
 
-@pytest.mark.parametrize("m,gl", [(64, [30, 64]), (200, [90, 200])])
-def test_larger_m_runs_the_generic_kernel_on_packed_weights(device, m, gl):
-    x, w, bias, scale, pt = _inputs(14, m, 512, 256, 2)
-    info = _check(x, w, gl, bias, scale, pt, override=cabi.OV_GENERIC if m <= 64 else cabi.OV_AUTO)
+@pytest.mark.parametrize("m,k,n,e,gl", [
+    (32, 1024, 128, 1, [32]),                                   # two 16-row fragments per chunk
+    (17, 512, 80, 1, [17]),                                     # one row into the second fragment, N tail
+    (64, 2048, 272, 1, [64]),                                   # four fragments, K split across workgroups
+    (128, 4096, 256, 1, [128]),                                 # eight fragments (the dense 128-row configuration's M and K)
+    (300, 720, 144, 2, [100, 300]),                             # chunks of 128 rows, K not a multiple of 64
+    (500, 512, 64, 8, [0, 40, 40, 200, 210, 350, 480, 490]),    # ragged groups, empty groups, rows past the last boundary
+    (1000, 256, 1040, 4, [250, 500, 750, 1000]),                # several chunks per group, 17 strips
+])
+def test_multi_row_streaming_kernel_is_bit_exact(device, m, k, n, e, gl):
+    x, w, bias, scale, pt = _inputs(16, m, k, n, e)
+    info = _check(x, w, gl, bias, scale, pt, src_transposed=(e == 8))
+    assert "w8a8_stream_rows" in info and "layout=packed" in info
+
+
+def test_forced_generic_kernel_on_packed_weights(device):
+    x, w, bias, scale, pt = _inputs(14, 64, 512, 256, 2)
+    info = _check(x, w, [30, 64], bias, scale, pt, override=cabi.OV_GENERIC)
     assert "generic" in info and "layout=packed" in info
 
 
