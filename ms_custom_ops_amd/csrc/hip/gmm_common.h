@@ -118,6 +118,19 @@ __device__ __forceinline__ void group_rows_chunk(const GmmParams &p, int g0, int
   carry = wave_bcast(e_l, 63);
 }
 
+// [start, end) of group `grp`, wave-uniform, by the wave-parallel walk above: one round of loads per 64 groups instead
+// of grp + 1 dependent ones.  Every lane of the wave must call it (the scans use cross-lane moves).
+__device__ __forceinline__ void group_range(const GmmParams &p, int grp, int lane, int &g_start, int &g_end) {
+  int carry = 0, start = 0, end = 0;
+  int g0 = 0;
+  for (;; g0 += 64) {
+    group_rows_chunk(p, g0, lane, carry, start, end);
+    if (grp < g0 + 64) break;
+  }
+  g_start = wave_bcast(start, grp - g0);
+  g_end = wave_bcast(end, grp - g0);
+}
+
 // ---- number formats ----------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
 

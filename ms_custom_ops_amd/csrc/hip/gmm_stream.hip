@@ -108,11 +108,8 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
   const int strip = blockIdx.x, ks = blockIdx.z;
   const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;   // first chunks of all groups are dispatched first
 
-  int g_start = 0, g_end = 0;
-  for (int g = 0; g <= grp; ++g) {
-    g_start = g_end;
-    g_end = group_end(p, g, g_start);
-  }
+  int g_start, g_end;
+  group_range(p, grp, lane, g_start, g_end);
   const int m0 = g_start + mc * kSkinnyRows;
   const int chunk_rows = min(kSkinnyRows, g_end - m0);
   if (chunk_rows <= 0) return;
@@ -333,11 +330,8 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_streamm_kernel(const G
   const int strip = blockIdx.x, ks = blockIdx.z;
   const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
 
-  int g_start = 0, g_end = 0;
-  for (int g = 0; g <= grp; ++g) {
-    g_start = g_end;
-    g_end = group_end(p, g, g_start);
-  }
+  int g_start, g_end;
+  group_range(p, grp, lane, g_start, g_end);
   const int m0 = g_start + mc * S::kRows;
   const int chunk_rows = min(S::kRows, g_end - m0);
   if (chunk_rows <= 0) return;
@@ -568,11 +562,8 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
   const int strip = blockIdx.x, ks = blockIdx.z;
   const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
 
-  int g_start = 0, g_end = 0;
-  for (int g = 0; g <= grp; ++g) {
-    g_start = g_end;
-    g_end = group_end(p, g, g_start);
-  }
+  int g_start, g_end;
+  group_range(p, grp, lane, g_start, g_end);
   const int m0 = g_start + mc * kSkinnyRows;
   const int chunk_rows = min(kSkinnyRows, g_end - m0);
   if (chunk_rows <= 0) return;

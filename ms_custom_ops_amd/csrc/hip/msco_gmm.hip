@@ -27,6 +27,7 @@ enum Override : int {
 };
 
 constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned
+constexpr int64_t kSkinnyMaxChunkSlots = 1024;   // (group, 16-row chunk) slots up to which many small groups take the decode kernels
 constexpr int kTargetWorkgroups = 512;  // skinny kernels with a K split: aim for this many workgroups (2 per CU)
 constexpr int kMaxSplitK = 8;             // keeps the last arriver's reduction to two rounds of loads
 constexpr int kNumCUs = 256;
@@ -126,7 +127,10 @@ void choose_plan(msco_gmm_op *op) {
     family = FAM_SKINNY;
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
-  } else if (m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) {
+  } else if ((m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) || (e > 1 && (m + e - 1) / e <= kSkinnyRows && e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots)) {
+    // decode: few rows in total, or groups of about one 16-row chunk each (the weights stream once per chunk).  The
+    // grid enumerates every (group, chunk) a malformed-to-the-limit group_list could fill; beyond a thousand slots
+    // the empty workgroups cost more than the tile kernel's partial tiles.
     // a single group of more than two 16-row chunks would stream the weights once per chunk: the small tile takes it
     family = FAM_SKINNY;
   } else {
@@ -185,6 +189,9 @@ void choose_plan(msco_gmm_op *op) {
     // rows a group is expected to hold (shapes only): 16-row chunks up to 16 rows, else chunks of 32 / 64 / 128 rows
     const int64_t rows = e == 1 ? m : (m + e - 1) / e;
     op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
+    // fewer, larger chunks when the (group, chunk) grid would be mostly empty slots
+    while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > env_int("MSCO_STREAM_MAX_SLOTS", (int)kSkinnyMaxChunkSlots))
+      op->stream_tch = op->stream_tch == 1 ? 2 : op->stream_tch * 2;
   }
   if (family == FAM_SKINNY) {
     // grid.y enumerates (group, chunk of 16 * stream_tch rows)
