@@ -330,10 +330,10 @@ def main():
         for name, layout in [("c3", other), ("c2_m2048", "nk"), ("c2_m2048", "kn"), ("c4", "nk"), ("c4", "kn"),
                              ("c1", "nk"), ("c1", "kn"), ("c2_m256", "nk"), ("c2_m256", "kn"), ("c2_m16", "nk"),
                              ("c2_m16", "kn"), ("c2_m16", "packed"), ("c2_m1", "kn"), ("c2_m1", "packed"), ("c5", "kn"),
-                             ("c5", "packed")]:
+                             ("c5", "packed"), ("c3_decode", "kn"), ("c3_decode", "packed")]:
             w2 = workloads.make(name)
             w_bytes = w2.w.nbytes
-            hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5")
+            hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5", "c3_decode")
             copies = max(1, int(np.ceil(ROTATE_BYTES / w_bytes))) if hbm_bound_guess else 1
             p2 = DeviceProblem(w2, layout, copies)
             _, sec = p2.time(max(20, min(200, args.steps)), args.warmup)

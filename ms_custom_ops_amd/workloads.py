@@ -13,6 +13,8 @@ c2_m{M}     dense linear,  K=4096 N=11008, M in {1, 16, 256, 2048}, int32 bias i
 c3          MoE E=8 top-2 over 4096 tokens (8192 rows), K=4096 N=14336
 c4          MoE E=64 top-6 over 8192 tokens (49152 rows), Zipf(1.2) expert popularity, K=2048 N=2816
 c5          weight-only decode, E=8 top-2 over 16 tokens (32 rows), bf16 x, K=4096 N=14336
+c3_decode   the c3 layer at decode time: E=8 top-2 over 16 tokens (32 rows), int8 x, K=4096 N=14336 (not one of the
+            published configurations: c3's weights with c5's routing, the W8A8 counterpart of c5)
 """
 from __future__ import annotations
 
@@ -102,6 +104,14 @@ def make(name: str, *, scale_down: int = 1) -> Workload:
         return Workload(name, "w8a8", m, k, n, e, x, w, s, pt, bias, None, gl)
     if name == "c3":
         t, e, top_k = 4096 // sd, 8, 2
+        k, n = 4096 // sd, 14336 // sd
+        m = t * top_k
+        x = _int8((m, k)); w = _int8((e, k, n)); s = _scale((e, n)); pt = _scale((m,))
+        logits = np.random.randn(t, e)
+        gl, _, _ = route_topk(logits, top_k, e)
+        return Workload(name, "w8a8", m, k, n, e, x, w, s, pt, None, None, gl)
+    if name == "c3_decode":
+        t, e, top_k = 16, 8, 2
         k, n = 4096 // sd, 14336 // sd
         m = t * top_k
         x = _int8((m, k)); w = _int8((e, k, n)); s = _scale((e, n)); pt = _scale((m,))

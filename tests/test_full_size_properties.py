@@ -23,13 +23,13 @@ def _sha(a):
     return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
 
 
-def _launch(tx, tw, tg, ts, tp, tb, m, k, n, e, out_dt, nk=False, override=0):
+def _launch(tx, tw, tg, ts, tp, tb, m, k, n, e, out_dt, nk=False, override=0, packed=False):
     raw = out_dt == cabi.DT_I32
     op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=out_dt, group_list_dtype=cabi.DT_I64,
                     bias_dtype=cabi.DT_I32 if tb is not None else 0,
                     scale_dtype=0 if (raw or ts is None) else cabi.DT_F32,
                     per_token_dtype=0 if (raw or tp is None) else cabi.DT_F32, transpose_b=int(nk),
-                    kernel_override=override)
+                    kernel_override=override, weight_layout=cabi.WL_PACKED if packed else cabi.WL_ROW_MAJOR)
     ws = op.plan(m, k, n, e)
     tws = torch.empty(max(ws, 1), dtype=torch.uint8, device="cuda:0")
     out = torch.empty((m, n), dtype=torch.int32 if raw else torch.int16, device="cuda:0")
@@ -77,6 +77,17 @@ def test_full_size_workload_bit_exact_and_checksums(device, name):
     twt = tw.transpose(1, 2).contiguous()
     acc_nk, info = _launch(tx, twt, tg, None, None, None, wl.m, wl.k, wl.n, wl.e, cabi.DT_I32, nk=True)
     assert torch.equal(acc_nk, acc), info
+    del acc_nk
+
+    # ... and so does the packed layout (decode and mid-size configurations: the kernels that read it stream the
+    # weights once per chunk of rows, which is not how the 8192- and 49152-row configurations are meant to run)
+    if wl.m <= 256:
+        from gpu_utils import pack_on_device
+        twp = pack_on_device(twt, wl.e, wl.k, wl.n, True)
+        acc_p, info = _launch(tx, twp, tg, None, None, None, wl.m, wl.k, wl.n, wl.e, cabi.DT_I32, packed=True)
+        assert "stream" in info and torch.equal(acc_p, acc), info
+        bits_p, info = _launch(tx, twp, tg, ts, tp, tb, wl.m, wl.k, wl.n, wl.e, cabi.DT_BF16, packed=True)
+        assert _sha(bits_p.cpu().numpy().view(np.uint16)) == dig["bf16"], info
 
 
 def test_full_size_c5_weight_only_against_sampled_exact_rows(device):
@@ -90,6 +101,22 @@ def test_full_size_c5_weight_only_against_sampled_exact_rows(device):
     for g in range(wl.e):
         a, b = int(starts[g]), int(ends[g])
         mag[a:b] = np.abs(xf[a:b].astype(np.float64)) @ (np.abs(wl.w[g].astype(np.float64) + of[g]) * np.abs(sf[g]))
-    bits, info = run_a16w8(wl.x, wl.w, wl.scale, wl.offset, wl.group_list)
-    got = O.bf16_bits_to_f32(bits).astype(np.float64)
-    assert (np.abs(got - exact) <= 2.0 ** -7 * np.abs(exact) + 1e-5 * mag).all(), info
+    for packed in (False, True):
+        bits, info = run_a16w8(wl.x, wl.w, wl.scale, wl.offset, wl.group_list, packed=packed)
+        got = O.bf16_bits_to_f32(bits).astype(np.float64)
+        assert (np.abs(got - exact) <= 2.0 ** -7 * np.abs(exact) + 1e-5 * mag).all(), info
+        assert ("a16w8_stream" in info) == packed
+
+
+def test_full_size_w8a8_moe_decode_both_layouts(device):
+    """c3's weights at decode time (32 rows over 8 experts) at full size: row-major and packed weights against the
+    oracle, bit-exact (the oracle needs 32 x 4096 x 14336 multiply-adds: cheap)."""
+    from gpu_utils import run_w8a8
+    wl = workloads.make("c3_decode")
+    ref_bits, ref_acc = O.grouped_matmul_w8a8(wl.x, wl.w, wl.group_list, None, wl.scale, wl.per_token, return_acc=True)
+    for packed in (False, True):
+        acc, info = run_w8a8(wl.x, wl.w, wl.group_list, out="i32", packed=packed)
+        assert np.array_equal(acc, ref_acc), info
+        bits, info = run_w8a8(wl.x, wl.w, wl.group_list, None, wl.scale, wl.per_token, packed=packed)
+        assert np.array_equal(bits, ref_bits), info
+        assert ("w8a8_stream" in info) == packed
