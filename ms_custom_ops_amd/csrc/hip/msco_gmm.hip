@@ -145,6 +145,10 @@ void choose_plan(msco_gmm_op *op) {
       op->tile_cfg = TILE_128x128;
     } else if (tiles(128, 128) >= 512) {
       op->tile_cfg = TILE_128x128;
+    } else if (d.transpose_b && rows_per_group >= 192 && tiles(128, 128) > kTileSplitMaxTiles) {
+      // [E,N,K] weights, a few hundred rows: 128 x 128 tiles on at least half of the CUs beat twice as many 64 x 128
+      // tiles (measured: M = 256, N = 11008: 32 us against 44 us); with fewer tiles the K split of the small tile wins
+      op->tile_cfg = TILE_128x128;
     } else {
       op->tile_cfg = TILE_64x128;
     }
