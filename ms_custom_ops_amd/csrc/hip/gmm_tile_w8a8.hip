@@ -423,15 +423,19 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   if (split > 1) {
     __shared__ unsigned s_ticket;
     constexpr int TILE_INTS = BM * BN;
-    int *base = p.partial + (long long)lid * split * TILE_INTS;
-    int *mine = base + (long long)ks * TILE_INTS + tid;
+    constexpr int WORDS = FN * FM * 8;   // 64-bit words per thread: accumulator registers (r, r + 1) travel together
+    typedef long long i64;
+    i64 *base = reinterpret_cast<i64 *>(p.partial) + (long long)lid * split * (TILE_INTS / 2);
+    i64 *mine = base + (long long)ks * (TILE_INTS / 2) + tid;
 #pragma unroll
     for (int f = 0; f < FN; ++f)
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          __hip_atomic_store(mine + ((f * FM + i) * 16 + r) * NT, acc[f][i][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int r = 0; r < 16; r += 2) {
+          const i64 word = (i64)(((unsigned long long)(unsigned)acc[f][i][r + 1] << 32) | (unsigned)acc[f][i][r]);
+          __hip_atomic_store(mine + ((f * FM + i) * 8 + r / 2) * NT, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     if (tid == 0) s_ticket = __hip_atomic_fetch_add(&p.counters[lid], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -440,14 +444,21 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     if (tid == 0) __hip_atomic_store(&p.counters[lid], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     for (int s = 0; s < split; ++s) {
       if (s == ks) continue;
-      const int *other = base + (long long)s * TILE_INTS + tid;
+      const i64 *other = base + (long long)s * (TILE_INTS / 2) + tid;
+      // all loads of a slice are issued before the first add: one memory round trip per slice, not one per word
+      i64 t[WORDS];
+#pragma unroll
+      for (int u = 0; u < WORDS; ++u) t[u] = __hip_atomic_load(other + u * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
       for (int f = 0; f < FN; ++f)
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
-          for (int r = 0; r < 16; ++r)
-            acc[f][i][r] += __hip_atomic_load(other + ((f * FM + i) * 16 + r) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int r = 0; r < 16; r += 2) {
+            const unsigned long long w = (unsigned long long)t[(f * FM + i) * 8 + r / 2];
+            acc[f][i][r] += (int)(unsigned)w;
+            acc[f][i][r + 1] += (int)(unsigned)(w >> 32);
+          }
     }
   }
 

@@ -231,7 +231,8 @@ void choose_plan(msco_gmm_op *op) {
       const int slice_blocks = is_w8a8(d) ? 128 : 64;
       const int floor_split = (int)((k_blocks + slice_blocks - 1) / slice_blocks);
       int groups = 16;
-      while (groups > 1 && ((col_groups + groups - 1) / groups) * active * floor_split < kNumCUs) groups /= 2;
+      const int min_wgs = env_int("MSCO_STREAM_MIN_WGS", kNumCUs);
+      while (groups > 1 && ((col_groups + groups - 1) / groups) * active * floor_split < min_wgs) groups /= 2;
       op->strip_groups = groups;
       op->n_strips = (int)((col_groups + groups - 1) / groups);
       op->skinny_cols = groups * 16;
