@@ -233,6 +233,8 @@ void choose_plan(msco_gmm_op *op) {
       int groups = 16;
       const int min_wgs = env_int("MSCO_STREAM_MIN_WGS", kNumCUs);
       while (groups > 1 && ((col_groups + groups - 1) / groups) * active * floor_split < min_wgs) groups /= 2;
+      const int forced_groups = env_int("MSCO_STREAM_GROUPS", 0);
+      if (forced_groups >= 1 && forced_groups <= 16) groups = forced_groups;
       op->strip_groups = groups;
       op->n_strips = (int)((col_groups + groups - 1) / groups);
       op->skinny_cols = groups * 16;
