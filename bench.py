@@ -327,7 +327,8 @@ def main():
     if not args.no_sweep:
         sweep = []
         other = "kn" if args.layout == "nk" else "nk"
-        for name, layout in [("c3", other), ("c2_m2048", "nk"), ("c2_m2048", "kn"), ("c4", "nk"), ("c4", "kn"),
+        for name, layout in [("c3", other), ("c3", "packed"), ("c2_m2048", "nk"), ("c2_m2048", "kn"), ("c2_m2048", "packed"),
+                             ("c4", "nk"), ("c4", "kn"), ("c4", "packed"),
                              ("c1", "nk"), ("c1", "kn"), ("c2_m256", "nk"), ("c2_m256", "kn"), ("c2_m16", "nk"),
                              ("c2_m16", "kn"), ("c2_m16", "packed"), ("c2_m1", "kn"), ("c2_m1", "packed"), ("c5", "kn"),
                              ("c5", "packed"), ("c3_decode", "kn"), ("c3_decode", "packed")]:

@@ -139,8 +139,13 @@ __device__ __forceinline__ T4Tile t4_locate(const int *meta_end, const int *meta
 
 }  // namespace
 
-// MODE: output type, 0 bf16, 1 f16, 2 int32 (raw accumulators plus bias)
-template <int MODE>
+// MODE: output type, 0 bf16, 1 f16, 2 int32 (raw accumulators plus bias).
+// PK: weights in the packed layout (1 KiB blocks of 16 columns x 64 K bytes, byte 16 l + i of block (a, b) =
+// w[k = 64 b + 16 (l / 16) + i][n = 16 a + l % 16]) instead of [E,N,K].  A slab of a tile is then 16 column groups x 2
+// blocks; staging quad (u, wave) is block 4 u + wave = (column group 2 u + wave / 2, K block wave % 2) and goes to LDS as
+// it is, so only the global offsets and the weight fragment addresses differ: MFMA row r of a 32-row block is column
+// t4_col_of_q(r), K quarter q is K block q / 2, 16-byte chunks 2 (q % 2) + hh.
+template <int MODE, bool PK>
 __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const GmmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -186,8 +191,14 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   auto x_rsrc = [&](const T4Tile &t) {
     return t4_rsrc(reinterpret_cast<const int8_t *>(p.x) + (long long)t.m0 * p.k, (long long)(p.m - t.m0) * p.k);
   };
+  const int k_blocks = (p.k + 63) / 64, col_groups = (p.n + 15) / 16;   // packed layout
   auto w_rsrc = [&](const T4Tile &t) {
-    return t4_rsrc(p.w + (long long)t.grp * w_elems + (long long)t.n0 * p.k, (long long)(p.n - t.n0) * p.k);
+    if constexpr (PK) {
+      const long long cg_bytes = (long long)k_blocks * 1024;
+      return t4_rsrc(p.w + ((long long)t.grp * col_groups + t.n0 / 16) * cg_bytes, (long long)(col_groups - t.n0 / 16) * cg_bytes);
+    } else {
+      return t4_rsrc(p.w + (long long)t.grp * w_elems + (long long)t.n0 * p.k, (long long)(p.n - t.n0) * p.k);
+    }
   };
 
   // ---- global -> staging registers -------------------------------------------------------------------
@@ -198,8 +209,10 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   const int d_row0 = 8 * wave + (lane >> 3);
   const int d_chunk = (lane & 7) ^ ((d_row0 >> 1) & 7);
   const unsigned a_voff0 = (unsigned)d_row0 * (unsigned)p.k + d_chunk * 16;
-  const unsigned b_voff0 = (unsigned)t4_col_of_q(d_row0) * (unsigned)p.k + d_chunk * 16;   // LDS row rho feeds MFMA row rho % 32
+  const unsigned b_voff0 = PK ? (unsigned)(((wave >> 1) * k_blocks + (wave & 1)) * 1024 + lane * 16)
+                              : (unsigned)t4_col_of_q(d_row0) * (unsigned)p.k + d_chunk * 16;   // LDS row rho feeds MFMA row rho % 32
   const unsigned rows32 = 32u * (unsigned)p.k;
+  const unsigned b_step = PK ? 2u * (unsigned)k_blocks * 1024u : rows32;   // staging quad u -> u + 1: two column groups / 32 rows
 
   // ---- fragment addressing ---------------------------------------------------------------------------
   // lane (l32, hh) reads row l32 of a 32-row block, logical chunk 2 q + hh of K quarter q.  The row
@@ -207,7 +220,8 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   // q << 5 in the byte address.
   const int swz = (l32 >> 1) & 7;
   const unsigned x_lane = (unsigned)((wave_m * T4_WT + l32) * T4_BK + ((hh ^ swz) << 4));
-  const unsigned w_lane = (unsigned)(T4_OP_STAGE + (wave_n * T4_WT + l32) * T4_BK + ((hh ^ swz) << 4));
+  const unsigned w_lane = PK ? (unsigned)(T4_OP_STAGE + wave_n * 16384 + (l32 >> 4) * 2048 + hh * 256 + (t4_col_of_q(l32) & 15) * 16)
+                             : (unsigned)(T4_OP_STAGE + (wave_n * T4_WT + l32) * T4_BK + ((hh ^ swz) << 4));
 
   unsigned char *st_lane = smem + wave * 1024 + lane * 16;
   unsigned char *ep_stage = smem + T4_EP_OFF + wave * T4_EP_WAVE;
@@ -231,10 +245,16 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     const unsigned kbase = (unsigned)(ahead ? s - k_slabs : s) * T4_BK;
     const bool dead = (ahead && !nxt.valid) || kbase + d_chunk * 16 >= (unsigned)p.k;   // K tail, slabs past K, no next tile
     const unsigned kill = dead ? T4_OOB : 0u;
-    if constexpr (OP == 0)
+    if constexpr (OP == 0) {
       stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rx_n : rx_c, (a_voff0 + U * rows32) | kill, kbase, 0);
-    else
-      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rw_n : rw_c, (b_voff0 + U * rows32) | kill, kbase, 0);
+    } else if constexpr (PK) {
+      // K block 2 slab + wave % 2 of column groups 2 U + wave / 2; blocks past K do not exist (the last one is zero padded)
+      const unsigned kb = 2u * (unsigned)(ahead ? s - k_slabs : s) + (unsigned)(wave & 1);
+      const unsigned kill_w = ((ahead && !nxt.valid) || kb >= (unsigned)k_blocks) ? T4_OOB : 0u;
+      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rw_n : rw_c, (b_voff0 + U * b_step) | kill_w, kbase * 16, 0);
+    } else {
+      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rw_n : rw_c, (b_voff0 + U * b_step) | kill, kbase, 0);
+    }
   };
   // write quad (op, u) of slab s to its LDS stage and refill it with slab s + 2
   auto cycle_one = [&](int s, auto par_c, auto op_c, auto u_c) {
@@ -246,7 +266,12 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   // loop would park eight more addresses in registers that the loop does not have)
   auto read_w = [&](int stage, unsigned qx, auto set_c, auto f_c) {
     constexpr int S = decltype(set_c)::value, F = decltype(f_c)::value;
-    wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_STAGE + (w_lane ^ qx) + F * 32 * T4_BK);
+    if constexpr (PK) {
+      // qx = q << 5: K block q / 2 is 1024 bytes on, chunk pair q % 2 another 512
+      wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_STAGE + (w_lane + (qx >> 6) * 1024 + ((qx >> 5) & 1) * 512) + F * 4096);
+    } else {
+      wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_STAGE + (w_lane ^ qx) + F * 32 * T4_BK);
+    }
   };
   auto read_x = [&](int stage, unsigned qx, auto set_c, auto i_c) {
     constexpr int S = decltype(set_c)::value, I = decltype(i_c)::value;
@@ -521,9 +546,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   }
 }
 
-template <int MODE>
+template <int MODE, bool PK>
 static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t stream) {
-  auto kern = gmm_w8a8_tile4_nk_kernel<MODE>;
+  auto kern = gmm_w8a8_tile4_nk_kernel<MODE, PK>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -535,7 +560,7 @@ static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t strea
   return hipGetLastError();
 }
 
-hipError_t launch_tile4_w8a8_nk(const GmmParams &p, hipStream_t stream) {
+hipError_t launch_tile4_w8a8_nk(const GmmParams &p, bool packed, hipStream_t stream) {
   // the operand stream runs up to four slabs ahead inside one tile; the group table lives in LDS
   if (p.k < 4 * T4_BK || p.e > T4_MAX_E) return hipErrorInvalidValue;
   const long long n_tiles = (p.n + T4_BN - 1) / T4_BN;
@@ -545,9 +570,9 @@ hipError_t launch_tile4_w8a8_nk(const GmmParams &p, hipStream_t stream) {
   if (grid > T4_MAX_WGS) grid = T4_MAX_WGS;
   if (grid <= 0) return hipSuccess;
   switch (p.out_dtype) {
-    case DT_BF16: return t4_launch<0>(p, (unsigned)grid, stream);
-    case DT_F16: return t4_launch<1>(p, (unsigned)grid, stream);
-    case DT_I32: return t4_launch<2>(p, (unsigned)grid, stream);
+    case DT_BF16: return packed ? t4_launch<0, true>(p, (unsigned)grid, stream) : t4_launch<0, false>(p, (unsigned)grid, stream);
+    case DT_F16: return packed ? t4_launch<1, true>(p, (unsigned)grid, stream) : t4_launch<1, false>(p, (unsigned)grid, stream);
+    case DT_I32: return packed ? t4_launch<2, true>(p, (unsigned)grid, stream) : t4_launch<2, false>(p, (unsigned)grid, stream);
     default: return hipErrorInvalidValue;
   }
 }

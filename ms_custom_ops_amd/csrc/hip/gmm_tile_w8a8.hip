@@ -594,7 +594,7 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream
     case TILE_128x256:   // two 4-wave workgroups per CU; [N,K] weights only
       return nk ? launch_cfg<128, 256, 1, 4, true, 3>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     case TILE_256x256_W4:   // needs [N,K] weights, at least four 128-byte K slabs per tile, a group table that fits in LDS
-      if (nk && p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, stream);
+      if (nk && p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, false, stream);
       return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     default:
       return hipErrorInvalidValue;

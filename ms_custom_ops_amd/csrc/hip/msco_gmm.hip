@@ -122,9 +122,14 @@ void choose_plan(msco_gmm_op *op) {
   if (!aligned) {
     family = FAM_GENERIC;
   } else if (is_packed(d)) {
-    // packed weights: the streaming kernels at any M (W8A8 with more than 16 rows per group: the multi-row variant;
-    // there is no tile kernel for this layout yet, so large M re-streams the weights from L2 once per 128 rows)
+    // packed weights: the streaming kernels (W8A8 with more than 16 rows per group: the multi-row variant), and for
+    // prefill-sized W8A8 problems the persistent tile kernel
     family = FAM_SKINNY;
+    const int64_t rows_per_group = m / (e > 0 ? e : 1);
+    if (is_w8a8(d) && rows_per_group >= 192 && ((m + 255) / 256) * ((n + 255) / 256) >= 256 && k >= 512 && e <= 1024) {
+      family = FAM_TILE;                 // prefill: the persistent tile kernel reads the packed blocks directly
+      op->tile_cfg = TILE_256x256_W4;
+    }
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
   } else if ((m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) || (e > 1 && (m + e - 1) / e <= kSkinnyRows && e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots)) {
@@ -155,6 +160,11 @@ void choose_plan(msco_gmm_op *op) {
   }
   if (is_packed(d)) {
     if (d.kernel_override == OV_GENERIC) family = FAM_GENERIC;
+    if (d.kernel_override == OV_SKINNY) family = FAM_SKINNY;
+    if (d.kernel_override == OV_TILE_256_W4 && is_w8a8(d) && k >= 512 && e <= 1024) {
+      family = FAM_TILE;
+      op->tile_cfg = TILE_256x256_W4;
+    }
   } else switch (d.kernel_override) {
     case OV_TILE_256: family = FAM_TILE; op->tile_cfg = TILE_256x256; break;
     case OV_TILE_256_W4: family = FAM_TILE; op->tile_cfg = TILE_256x256_W4; break;
@@ -171,7 +181,7 @@ void choose_plan(msco_gmm_op *op) {
   if (family == FAM_TILE && !is_w8a8(d)) family = FAM_SKINNY;
   if (family == FAM_TILE) {
     const int forced = env_int("MSCO_TILE_CFG", -1);
-    if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO) op->tile_cfg = forced;
+    if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO && !is_packed(d)) op->tile_cfg = forced;
     // Few tiles (M of a few hundred rows): split K across workgroups until about kTileTargetWorkgroups of them
     // stream operands; every slice keeps at least kTileMinSlabs 64-byte K slabs.  Small tile shapes only.
     if (op->tile_cfg == TILE_128x128 || op->tile_cfg == TILE_64x128) {
@@ -412,7 +422,7 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   const bool nk = d.transpose_b != 0;
   const int layout = layout_of(d);
   if (is_w8a8(d)) {
-    if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, s);
+    if (h->family == FAM_TILE) err = layout == 2 ? launch_tile4_w8a8_nk(p, true, s) : launch_tile_w8a8(p, h->tile_cfg, nk, s);
     else if (h->family == FAM_SKINNY && layout == 2) err = h->stream_tch > 1 ? launch_streamm_w8a8(p, h->stream_tch, s) : launch_stream_w8a8(p, s);
     else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
     else err = launch_generic_w8a8(p, layout, s);

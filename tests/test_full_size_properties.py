@@ -79,15 +79,17 @@ def test_full_size_workload_bit_exact_and_checksums(device, name):
     assert torch.equal(acc_nk, acc), info
     del acc_nk
 
-    # ... and so does the packed layout (decode and mid-size configurations: the kernels that read it stream the
-    # weights once per chunk of rows, which is not how the 8192- and 49152-row configurations are meant to run)
-    if wl.m <= 256:
-        from gpu_utils import pack_on_device
-        twp = pack_on_device(twt, wl.e, wl.k, wl.n, True)
-        acc_p, info = _launch(tx, twp, tg, None, None, None, wl.m, wl.k, wl.n, wl.e, cabi.DT_I32, packed=True)
-        assert "stream" in info and torch.equal(acc_p, acc), info
-        bits_p, info = _launch(tx, twp, tg, ts, tp, tb, wl.m, wl.k, wl.n, wl.e, cabi.DT_BF16, packed=True)
-        assert _sha(bits_p.cpu().numpy().view(np.uint16)) == dig["bf16"], info
+    # ... and so does the packed layout: streaming kernels for the decode and few-hundred-row configurations, the
+    # persistent tile kernel for the prefill ones
+    from gpu_utils import pack_on_device
+    twp = pack_on_device(twt, wl.e, wl.k, wl.n, True)
+    del twt
+    acc_p, info = _launch(tx, twp, tg, None, None, None, wl.m, wl.k, wl.n, wl.e, cabi.DT_I32, packed=True)
+    assert ("tile_256x256x128_w4" if wl.m >= 2048 else "stream") in info and "layout=packed" in info, info
+    assert torch.equal(acc_p, acc), info
+    del acc_p
+    bits_p, info = _launch(tx, twp, tg, ts, tp, tb, wl.m, wl.k, wl.n, wl.e, cabi.DT_BF16, packed=True)
+    assert _sha(bits_p.cpu().numpy().view(np.uint16)) == dig["bf16"], info
 
 
 def test_full_size_c5_weight_only_against_sampled_exact_rows(device):

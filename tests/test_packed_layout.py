@@ -94,6 +94,28 @@ def test_multi_row_streaming_kernel_is_bit_exact(device, m, k, n, e, gl):
     assert "w8a8_stream_rows" in info and "layout=packed" in info
 
 
+@pytest.mark.parametrize("m,k,n,e,gl", [
+    (256, 512, 256, 1, [256]),                                  # one tile, four slabs
+    (300, 640, 272, 2, [100, 300]),                             # partial tiles, N tail inside a column group pair
+    (700, 576, 528, 4, [100, 300, 300, 700]),                   # odd number of 64-byte K blocks: the last slab is half empty
+    (2048, 1024, 768, 3, [1, 1030, 2048]),                      # workgroups walk several tiles
+    (1500, 720, 1040, 8, [0, 40, 300, 300, 900, 1210, 1480, 1490]),   # K not a multiple of 64, ragged and empty groups
+])
+def test_persistent_tile_kernel_on_packed_weights_is_bit_exact(device, m, k, n, e, gl):
+    x, w, bias, scale, pt = _inputs(17, m, k, n, e)
+    info = _check(x, w, gl, bias, scale, pt, override=cabi.OV_TILE_256_W4)
+    assert "tile_256x256x128_w4" in info and "layout=packed" in info
+
+
+def test_prefill_sized_problems_on_packed_weights_take_the_tile_kernel(device):
+    from gpu_utils import run_w8a8
+    x, w, bias, scale, pt = _inputs(18, 4096, 512, 4096, 8)
+    gl = [500, 1000, 1600, 2000, 2600, 3000, 3500, 4096]
+    got, info = run_w8a8(x, w, gl, None, scale, pt, packed=True)
+    assert "tile_256x256x128_w4" in info and "layout=packed" in info
+    assert np.array_equal(got, O.grouped_matmul_w8a8(x, w, gl, None, scale, pt))
+
+
 def test_forced_generic_kernel_on_packed_weights(device):
     x, w, bias, scale, pt = _inputs(14, 64, 512, 256, 2)
     info = _check(x, w, [30, 64], bias, scale, pt, override=cabi.OV_GENERIC)
