@@ -1,22 +1,22 @@
 #!/usr/bin/env python3
 """Benchmark of the grouped W8A8 matmul path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout kn|nk] [--no-sweep] [--no-cpu]
-    python bench.py --probe c3|c2_m16|...|copy|moe [--layout kn|nk] [--steps K]     (for rocprofv3 counter runs)
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout packed|nk|kn] [--no-sweep] [--no-cpu]
+    python bench.py --probe c3|c2_m16|...|copy|moe [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs)
 
 A step is one pass of the hot path over one batch of synthetic input (inputs resident in HBM before
 the timed region).  The headline workload is the Mixtral-shaped MoE configuration (E=8, top-2 over
 4096 tokens = 8192 rows, K=4096, N=14336); `value` is its int8 throughput.  The weights are generated
-[E,K,N] as the configuration states and prepacked once, on the device, to the backend's [E,N,K] layout
-(the reference prepacks weights too, to its FRACTAL_NZ format, before the op runs); the prepack is
-outside the timed region and its duration is reported as `prepack_ms`.  `--layout kn` times the op on
-the unpacked [E,K,N] weights instead; the sweep always carries both.
+[E,K,N] as the configuration states and prepacked once, on the device, to the backend's blocked layout
+(msco_pack_weight; the reference prepacks weights too, to its FRACTAL_NZ format, before the op runs); the
+prepack is outside the timed region and its duration is reported as `prepack_ms`.  `--layout nk` times the op
+on weights transposed once to [E,N,K], `--layout kn` on the unpacked [E,K,N] weights; the sweep always carries
+all three.
 Prints ONE JSON line.  Besides the contract keys it carries
   roofline      the dominant kernel's achieved algorithmic rate against the MI355X peak,
   cpu_baseline  the numpy restatement of the reference golden timed on this box's host cores,
   sweep         the other configurations (dense decode / prefill sweep, skewed MoE, weight-only
-                decode) as TOPS and GB/s with their roofline fractions; decode shapes also on weights
-                prepacked to the blocked layout (layout "packed").
+                decode) as TOPS and GB/s with their roofline fractions, per weight layout.
 --probe runs a few untimed launches of one workload (or, for `copy`, of a plain device-to-device copy
 of COPY_BYTES bytes, the reference a counter reading is scaled by) so that a profiler sees nothing else.
 """
@@ -47,9 +47,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=40,
                     help="untimed steps; the GPU clock needs a few tens of launches to settle")
     ap.add_argument("--workload", default="c3")
-    ap.add_argument("--layout", default="nk", choices=["kn", "nk", "packed"],
-                    help="weight storage the op sees: nk=[E,N,K] (prepacked once, the default), kn=[E,K,N] as generated, "
-                         "packed=the blocked layout of msco_pack_weight (decode shapes)")
+    ap.add_argument("--layout", default="packed", choices=["kn", "nk", "packed"],
+                    help="weight storage the op sees: packed=the blocked layout of msco_pack_weight (prepacked once, the default), "
+                         "nk=[E,N,K] (prepacked once by a transpose), kn=[E,K,N] as generated")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--probe", default=None, help="workload name, `copy` or `moe` (the routing / un-permutation pair): launches only, for counter collection")
@@ -326,9 +326,9 @@ def main():
 
     if not args.no_sweep:
         sweep = []
-        other = "kn" if args.layout == "nk" else "nk"
-        for name, layout in [("c3", other), ("c3", "packed"), ("c2_m2048", "nk"), ("c2_m2048", "kn"), ("c2_m2048", "packed"),
-                             ("c4", "nk"), ("c4", "kn"), ("c4", "packed"),
+        others = [l for l in ("packed", "nk", "kn") if l != args.layout]
+        for name, layout in [("c3", others[0]), ("c3", others[1]), ("c2_m2048", "packed"), ("c2_m2048", "nk"), ("c2_m2048", "kn"),
+                             ("c4", "packed"), ("c4", "nk"), ("c4", "kn"), ("c1", "packed"), ("c2_m256", "packed"),
                              ("c1", "nk"), ("c1", "kn"), ("c2_m256", "nk"), ("c2_m256", "kn"), ("c2_m16", "nk"),
                              ("c2_m16", "kn"), ("c2_m16", "packed"), ("c2_m1", "kn"), ("c2_m1", "packed"), ("c5", "kn"),
                              ("c5", "packed"), ("c3_decode", "kn"), ("c3_decode", "packed")]:

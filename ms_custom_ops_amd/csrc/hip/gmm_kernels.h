@@ -13,8 +13,8 @@ enum TileCfg : int {
   TILE_CFG_COUNT = 5
 };
 
-// MFMA tile kernel for W8A8 (prefill shapes).  nk: weights stored [E,N,K].
-hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream_t stream);
+// MFMA tile kernel for W8A8 (prefill shapes).  nk: weights stored [E,N,K]; packed: the packed layout (nk is ignored).
+hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool packed, hipStream_t stream);
 const char *tile_cfg_name(int tile_cfg);
 hipError_t launch_tile4_w8a8_nk(const GmmParams &p, bool packed, hipStream_t stream);   // weights [E,N,K] or packed
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn);

@@ -104,8 +104,13 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // STAGES = depth of the LDS ring of the operands that are loaded straight into LDS (STAGES - 1 slabs in flight)
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES>
+// PK (with NK): weights in the packed layout (1 KiB blocks of 16 columns x 64 K bytes, byte 16 l + i of block (a, b) =
+// w[k = 64 b + 16 (l / 16) + i][n = 16 a + l % 16]).  A 64-byte K slab of the tile is then one block per column group:
+// the LDS-direct load of a block copies it as it lies, and a weight fragment is read at block (column / 16), chunk
+// 2 kk + hh, row (column % 16) -- conflict free without a swizzle.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES, bool PK = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel(const GmmParams p) {
+  static_assert(!PK || NK, "packed weights use the LDS-direct weight path");
   constexpr int NSTAGE = STAGES;
   constexpr int AHEAD = STAGES - 1;                 // slabs requested ahead of the one being multiplied
   static_assert(NK || STAGES == 4, "the [K,N] register ring is three slabs deep");
@@ -211,8 +216,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   const int8_t *wg = p.w + (long long)grp * w_elems;
   const __amdgpu_buffer_rsrc_t rx =
     make_rsrc(reinterpret_cast<const int8_t *>(p.x) + (long long)m0 * p.k, (long long)(p.m - m0) * p.k);
-  const __amdgpu_buffer_rsrc_t rw = NK ? make_rsrc(wg + (long long)n0 * p.k, (long long)(p.n - n0) * p.k)
-                                       : make_rsrc(wg + n0, w_elems - n0);
+  const int pk_blocks = (p.k + 63) / 64, pk_groups = (p.n + 15) / 16;   // packed layout: K blocks per column group, column groups
+  const __amdgpu_buffer_rsrc_t rw =
+    PK   ? make_rsrc(p.w + ((long long)grp * pk_groups + n0 / 16) * pk_blocks * 1024, (long long)(pk_groups - n0 / 16) * pk_blocks * 1024)
+    : NK ? make_rsrc(wg + (long long)n0 * p.k, (long long)(p.n - n0) * p.k)
+         : make_rsrc(wg + n0, w_elems - n0);
 
   // ---- operands loaded straight into LDS (x rows, [N,K] weights) -----------------------------
   // One wave instruction fills 1 KiB of LDS = 16 rows x 64 B, lane L writing bytes [16 L, 16 L + 16).
@@ -233,7 +241,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     for (int u = 0; u < B_LD; ++u) {
       const int blk = wave * B_LD + u;
       const int rho = blk * 16 + d_row;
-      b_voff[u] = (unsigned)((rho & ~31) + col_of_q(rho & 31)) * (unsigned)p.k + d_c * 16;
+      if constexpr (PK) b_voff[u] = (unsigned)(blk * pk_blocks * 1024 + lane * 16);   // column group blk of the tile
+      else b_voff[u] = (unsigned)((rho & ~31) + col_of_q(rho & 31)) * (unsigned)p.k + d_c * 16;
     }
   }
   auto issue_direct = [&](int kt) {
@@ -250,7 +259,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
 #pragma unroll
       for (int u = 0; u < B_LD; ++u) {
         const int blk = wave * B_LD + u;
-        buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill, kbase);
+        if constexpr (PK) {
+          // K block k_first + kt of the column group; blocks past K do not exist (the last one is zero padded)
+          const unsigned kill_w = (k_first + kt >= pk_blocks) ? OOB : 0u;
+          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, (k_first + kt) * 1024);
+        } else {
+          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill, kbase);
+        }
       }
     }
   };
@@ -298,7 +313,11 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   };
   auto read_w = [&](int kt, int f, int kk) -> v4i {
     const int rho = wave_n * WTN + 32 * f + l32;
-    if constexpr (NK) {
+    if constexpr (PK) {
+      const unsigned char *b = lds_b + (kt % NSTAGE) * B_STAGE;
+      const int col = wave_n * WTN + 32 * f + col_of_q(l32);   // MFMA row l32 of block f is this column of the tile
+      return *reinterpret_cast<const v4i *>(b + (col >> 4) * 1024 + (2 * kk + hh) * 256 + (col & 15) * 16);
+    } else if constexpr (NK) {
       const unsigned char *b = lds_b + (kt % NSTAGE) * B_STAGE;
       return *reinterpret_cast<const v4i *>(b + rho * BK + (((2 * kk + hh) ^ swz64(rho)) << 4));
     } else {
@@ -561,12 +580,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
 }
 
 // ---- host launcher ---------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4, bool PK = false>
 static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
   const size_t loop_lds = (size_t)STAGES * BM * BK + (size_t)(NK ? STAGES : KN_STAGES) * BN * BK;
   const size_t epi_lds = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * 144;   // epilogue staging, 144-byte row pitch
   const size_t lds = (loop_lds > epi_lds ? loop_lds : epi_lds) + 3 * 1024;   // + epilogue operand table
-  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES>;
+  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES, PK>;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -583,7 +602,18 @@ static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, hipStream_t stream) {
+hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool packed, hipStream_t stream) {
+  if (packed) {
+    switch (tile_cfg) {
+      case TILE_128x128: return launch_cfg<128, 128, 2, 2, true, 4, true>(p, stream);
+      case TILE_64x128: return launch_cfg<64, 128, 2, 2, true, 4, true>(p, stream);
+      case TILE_256x256_W4:
+        if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, true, stream);
+        return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
+      case TILE_256x256: case TILE_128x256: return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
+      default: return hipErrorInvalidValue;
+    }
+  }
   switch (tile_cfg) {
     case TILE_256x256:
       return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);

@@ -119,24 +119,21 @@ void choose_plan(msco_gmm_op *op) {
   op->tile_cfg = TILE_256x256;
 
   int family;
+  // packed weights are K-contiguous per column like [E,N,K]: the same tile kernels read them
+  const bool k_major = d.transpose_b != 0 || is_packed(d);
+  const bool many_small_groups = e > 1 && (m + e - 1) / e <= kSkinnyRows &&
+                                 e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots;
   if (!aligned) {
     family = FAM_GENERIC;
-  } else if (is_packed(d)) {
-    // packed weights: the streaming kernels (W8A8 with more than 16 rows per group: the multi-row variant), and for
-    // prefill-sized W8A8 problems the persistent tile kernel
-    family = FAM_SKINNY;
-    const int64_t rows_per_group = m / (e > 0 ? e : 1);
-    if (is_w8a8(d) && rows_per_group >= 192 && ((m + 255) / 256) * ((n + 255) / 256) >= 256 && k >= 512 && e <= 1024) {
-      family = FAM_TILE;                 // prefill: the persistent tile kernel reads the packed blocks directly
-      op->tile_cfg = TILE_256x256_W4;
-    }
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
-  } else if ((m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) || (e > 1 && (m + e - 1) / e <= kSkinnyRows && e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots)) {
+  } else if (is_packed(d) ? (m <= kSkinnyMaxRows || many_small_groups)
+                          : ((m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) || many_small_groups)) {
     // decode: few rows in total, or groups of about one 16-row chunk each (the weights stream once per chunk).  The
     // grid enumerates every (group, chunk) a malformed-to-the-limit group_list could fill; beyond a thousand slots
-    // the empty workgroups cost more than the tile kernel's partial tiles.
-    // a single group of more than two 16-row chunks would stream the weights once per chunk: the small tile takes it
+    // the empty workgroups cost more than the tile kernel's partial tiles.  On row-major weights a single group of
+    // more than two 16-row chunks would stream the weights once per chunk and takes the small tile instead; on packed
+    // weights the multi-row streaming kernel covers up to 64 rows in one pass.
     family = FAM_SKINNY;
   } else {
     family = FAM_TILE;
@@ -144,28 +141,21 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t rows_per_group = m / (e > 0 ? e : 1);
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     if (rows_per_group >= 192 && tiles(256, 256) >= 256) {
-      // [E,N,K] weights take the persistent four-wave kernel when a tile has at least four 128-byte K slabs
-      op->tile_cfg = (d.transpose_b && k >= 512 && e <= 1024) ? TILE_256x256_W4 : TILE_256x256;
+      // K-major weights take the persistent four-wave kernel when a tile has at least four 128-byte K slabs
+      op->tile_cfg = (k_major && k >= 512 && e <= 1024) ? TILE_256x256_W4 : TILE_256x256;
     } else if (rows_per_group >= 96 && tiles(128, 128) >= 256) {
       op->tile_cfg = TILE_128x128;
     } else if (tiles(128, 128) >= 512) {
       op->tile_cfg = TILE_128x128;
-    } else if (d.transpose_b && rows_per_group >= 192 && tiles(128, 128) > kTileSplitMaxTiles) {
-      // [E,N,K] weights, a few hundred rows: 128 x 128 tiles on at least half of the CUs beat twice as many 64 x 128
+    } else if (k_major && rows_per_group >= 192 && tiles(128, 128) > kTileSplitMaxTiles) {
+      // K-major weights, a few hundred rows: 128 x 128 tiles on at least half of the CUs beat twice as many 64 x 128
       // tiles (measured: M = 256, N = 11008: 32 us against 44 us); with fewer tiles the K split of the small tile wins
       op->tile_cfg = TILE_128x128;
     } else {
       op->tile_cfg = TILE_64x128;
     }
   }
-  if (is_packed(d)) {
-    if (d.kernel_override == OV_GENERIC) family = FAM_GENERIC;
-    if (d.kernel_override == OV_SKINNY) family = FAM_SKINNY;
-    if (d.kernel_override == OV_TILE_256_W4 && is_w8a8(d) && k >= 512 && e <= 1024) {
-      family = FAM_TILE;
-      op->tile_cfg = TILE_256x256_W4;
-    }
-  } else switch (d.kernel_override) {
+  switch (d.kernel_override) {
     case OV_TILE_256: family = FAM_TILE; op->tile_cfg = TILE_256x256; break;
     case OV_TILE_256_W4: family = FAM_TILE; op->tile_cfg = TILE_256x256_W4; break;
     case OV_TILE_128: family = FAM_TILE; op->tile_cfg = TILE_128x128; break;
@@ -181,7 +171,7 @@ void choose_plan(msco_gmm_op *op) {
   if (family == FAM_TILE && !is_w8a8(d)) family = FAM_SKINNY;
   if (family == FAM_TILE) {
     const int forced = env_int("MSCO_TILE_CFG", -1);
-    if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO && !is_packed(d)) op->tile_cfg = forced;
+    if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO) op->tile_cfg = forced;
     // Few tiles (M of a few hundred rows): split K across workgroups until about kTileTargetWorkgroups of them
     // stream operands; every slice keeps at least kTileMinSlabs 64-byte K slabs.  Small tile shapes only.
     if (op->tile_cfg == TILE_128x128 || op->tile_cfg == TILE_64x128) {
@@ -422,7 +412,7 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   const bool nk = d.transpose_b != 0;
   const int layout = layout_of(d);
   if (is_w8a8(d)) {
-    if (h->family == FAM_TILE) err = layout == 2 ? launch_tile4_w8a8_nk(p, true, s) : launch_tile_w8a8(p, h->tile_cfg, nk, s);
+    if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, layout == 2, s);
     else if (h->family == FAM_SKINNY && layout == 2) err = h->stream_tch > 1 ? launch_streamm_w8a8(p, h->stream_tch, s) : launch_stream_w8a8(p, s);
     else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
     else err = launch_generic_w8a8(p, layout, s);

@@ -79,13 +79,13 @@ def test_full_size_workload_bit_exact_and_checksums(device, name):
     assert torch.equal(acc_nk, acc), info
     del acc_nk
 
-    # ... and so does the packed layout: streaming kernels for the decode and few-hundred-row configurations, the
-    # persistent tile kernel for the prefill ones
+    # ... and so does the packed layout: streaming kernels for the decode configurations, the small tile kernels for a
+    # few hundred rows, the persistent tile kernel for the prefill ones
     from gpu_utils import pack_on_device
     twp = pack_on_device(twt, wl.e, wl.k, wl.n, True)
     del twt
     acc_p, info = _launch(tx, twp, tg, None, None, None, wl.m, wl.k, wl.n, wl.e, cabi.DT_I32, packed=True)
-    assert ("tile_256x256x128_w4" if wl.m >= 2048 else "stream") in info and "layout=packed" in info, info
+    assert ("tile_256x256x128_w4" if wl.m >= 2048 else "stream" if wl.m <= 64 else "tile_") in info and "layout=packed" in info, info
     assert torch.equal(acc_p, acc), info
     del acc_p
     bits_p, info = _launch(tx, twp, tg, ts, tp, tb, wl.m, wl.k, wl.n, wl.e, cabi.DT_BF16, packed=True)

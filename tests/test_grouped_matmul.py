@@ -119,7 +119,7 @@ def test_plan_cache_hits_on_repeated_shapes(device):
 @pytest.mark.parametrize("exec_mode", MODES)
 def test_gmm_on_weights_prepacked_by_trans_data(device, m, trans_b, exec_mode):
     """trans_data(ND_TO_FRACTAL_NZ) then grouped_matmul, as the reference's callers do (test_grouped_matmul.py:131-147):
-    decode-sized M takes the streaming kernel, larger M its multi-row variant; both bit-exact."""
+    decode-sized M takes the streaming kernels, larger M the tile kernels; both bit-exact."""
     with ms_custom_ops.exec_mode(exec_mode):
         custom_grouped_matmul(m, 192, 128, 8, trans_b=trans_b, with_pertoken_scale=True, prepack=True)
         custom_grouped_matmul(m, 192, 128, 8, trans_b=trans_b, out_dtype=torch.bfloat16, prepack=True)

@@ -89,9 +89,30 @@ def test_counts_and_rows_past_the_last_boundary(device):
     (1000, 256, 1040, 4, [250, 500, 750, 1000]),                # several chunks per group, 17 strips
 ])
 def test_multi_row_streaming_kernel_is_bit_exact(device, m, k, n, e, gl):
+    """Planned by itself up to 64 rows; forced here for the larger cases (which the plan gives to the tile kernels)."""
     x, w, bias, scale, pt = _inputs(16, m, k, n, e)
-    info = _check(x, w, gl, bias, scale, pt, src_transposed=(e == 8))
+    info = _check(x, w, gl, bias, scale, pt, src_transposed=(e == 8), override=cabi.OV_AUTO if m <= 64 else cabi.OV_SKINNY)
     assert "w8a8_stream_rows" in info and "layout=packed" in info
+
+
+@pytest.mark.parametrize("family,override", [("64x128", cabi.OV_TILE_64), ("128x128", cabi.OV_TILE_128), ("256x256x64", cabi.OV_TILE_256)])
+@pytest.mark.parametrize("m,k,n,e,gl,split", [
+    (333, 256, 384, 8, [5, 5, 40, 100, 100, 230, 300, 333], 0),     # ragged and empty groups
+    (300, 160, 272, 1, [300], 0),                                   # K and N tails
+    (128, 2048, 512, 1, [128], 0),                                  # few tiles: K split across workgroups
+    (200, 720, 144, 2, [90, 200], 2),                               # forced K split, K not a multiple of 64
+])
+def test_eight_wave_and_small_tile_kernels_on_packed_weights(device, monkeypatch, family, override, m, k, n, e, gl, split):
+    monkeypatch.setenv("MSCO_TILE_SPLIT_K", str(split))
+    x, w, bias, scale, pt = _inputs(19, m, k, n, e)
+    info = _check(x, w, gl, bias, scale, pt, override=override)
+    assert f"tile_{family}" in info and "layout=packed" in info
+
+
+def test_a_few_hundred_rows_on_packed_weights_take_the_small_tiles(device):
+    x, w, bias, scale, pt = _inputs(20, 256, 1024, 4096, 1)
+    info = _check(x, w, [256], bias, scale, pt)
+    assert "w8a8_tile_" in info and "layout=packed" in info
 
 
 @pytest.mark.parametrize("m,k,n,e,gl", [
