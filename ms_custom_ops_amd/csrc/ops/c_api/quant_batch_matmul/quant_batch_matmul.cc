@@ -31,16 +31,33 @@ constexpr size_t kQbmmInputX2Format = 8;
 constexpr size_t kQbmmInputDtype = 9;
 constexpr int64_t kFloat16 = 42;
 
+// x2 as the shape rules see it.  With x2_format "FRACTAL_NZ" x2 is a weight prepacked by trans_data, int8
+// [..., N / 16, ceil(K / 64), 1024]; its logical shape is [..., K, N] with K taken from x1.
+static ShapeVector QbmmLogicalX2Shape(const ShapeVector &x1_shape, const ShapeVector &x2_shape, bool transpose_x1,
+                                      bool transpose_x2, const std::string &x2_format) {
+  if (x2_format != kFractalNzFormat) return x2_shape;
+  if (x2_shape.size() < kDim3 || x2_shape.back() != kPackedBlockBytes || x1_shape.size() < kDim2) {
+    MS_EXCEPTION_VALUE << "For quant_batch_matmul, x2_format 'FRACTAL_NZ' takes an x2 prepacked by trans_data "
+                       << "([..., N/16, ceil(K/64), 1024]), but got " << x2_shape;
+  }
+  if (transpose_x2) {
+    MS_EXCEPTION_VALUE << "For quant_batch_matmul, an x2 prepacked by trans_data carries its own layout; 'transpose_x2' "
+                       << "must be false.";
+  }
+  const int64_t k = transpose_x1 ? x1_shape[x1_shape.size() - kDim2] : x1_shape.back();
+  const int64_t kb = x2_shape[x2_shape.size() - kDim2];
+  ShapeVector logical(x2_shape.begin(), x2_shape.end() - kDim3);
+  logical.push_back(kb == (k + 63) / 64 ? k : kb * 64);   // a mismatch surfaces as the usual K error
+  logical.push_back(x2_shape[x2_shape.size() - kDim3] * 16);
+  return logical;
+}
+
 static void CheckQbmmInputs(const ms::Tensor &x1, const ms::Tensor &x2, const ms::Tensor &scale,
                             const ms::Tensor &offset, const ms::Tensor &bias, const ms::Tensor &pertoken,
                             const std::string &x2_format, TypeId out_dtype, const BatchMatMulDims &d) {
   if (x2_format != kNdFormat && x2_format != kFractalNzFormat) {
     MS_LOG_EXCEPTION << "For quant_batch_matmul, the 'x2_format' is only support ['ND', 'FRACTAL_NZ'], but got "
                      << x2_format;
-  }
-  if (x2_format == kFractalNzFormat) {
-    MS_LOG_EXCEPTION << "For quant_batch_matmul, x2_format 'FRACTAL_NZ' is an Ascend memory format; the HIP backend "
-                        "takes x2 as stored (ND).";
   }
   if (x1.data_type() != kNumberTypeInt8 || x2.data_type() != kNumberTypeInt8) {
     MS_LOG_EXCEPTION << "For quant_batch_matmul, 'x1' and 'x2' must be int8, but got " << x1.data_type() << " and "
@@ -72,7 +89,7 @@ static void CheckQbmmInputs(const ms::Tensor &x1, const ms::Tensor &x2, const ms
 // One backend launch: x [rows, K], weight [e, K, N] (or [e, N, K]), e equal groups of rows / e.
 static void LaunchDense(const std::string &op_name, const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &scale,
                         const ms::Tensor &bias, const ms::Tensor &pertoken, const ms::Tensor &out, int64_t rows,
-                        int64_t k, int64_t n, int64_t e, bool transpose_x2, void *stream) {
+                        int64_t k, int64_t n, int64_t e, bool transpose_x2, bool packed, void *stream) {
   msco_gmm_desc d{};
   d.abi_version = MSCO_GMM_ABI_VERSION;
   d.x_dtype = MSCO_DT_I8;
@@ -84,6 +101,7 @@ static void LaunchDense(const std::string &op_name, const ms::Tensor &x, const m
   d.scale_dtype = raw ? MSCO_DT_NONE : ToBackendDtype(scale.data_type());
   d.per_token_dtype = (!raw && pertoken.is_defined()) ? MSCO_DT_F32 : MSCO_DT_NONE;
   d.transpose_b = transpose_x2 ? 1 : 0;
+  d.weight_layout = packed ? MSCO_WL_PACKED : MSCO_WL_ROW_MAJOR;
   d.scale_per_group = 0;
   d.scale_is_scalar = scale.numel() == 1 ? 1 : 0;
   auto plan = GmmPlanCache::GetInstance().GetOrCreate(op_name, d, GmmProblem{rows, k, n, e}, stream);
@@ -106,7 +124,10 @@ void RunQuantBatchMatmul(const ms::Tensor &x1_in, const ms::Tensor &x2, const ms
                          const ms::Tensor &offset, const ms::Tensor &bias, const ms::Tensor &pertoken,
                          bool transpose_x1, bool transpose_x2, const std::string &x2_format, const ms::Tensor &out) {
   const std::string op_name = "QuantBatchMatmul";
-  const BatchMatMulDims d = BatchMatMulSplitDims(x1_in.shape(), x2.shape(), transpose_x1, transpose_x2, op_name);
+  const bool packed = x2_format == kFractalNzFormat;
+  const BatchMatMulDims d = BatchMatMulSplitDims(
+    x1_in.shape(), QbmmLogicalX2Shape(x1_in.shape(), x2.shape(), transpose_x1, transpose_x2, x2_format), transpose_x1,
+    transpose_x2, op_name);
   CheckQbmmInputs(x1_in, x2, scale, offset, bias, pertoken, x2_format, out.data_type(), d);
   CheckContiguous(op_name, {x1_in, x2, scale, bias, pertoken}, true);
   CheckContiguous(op_name, {out}, false);
@@ -128,12 +149,12 @@ void RunQuantBatchMatmul(const ms::Tensor &x1_in, const ms::Tensor &x2, const ms
   const bool shared_rows = !pertoken.is_defined() || bo == 1;
   if (b2 == 1 && shared_rows) {
     // every batch of x1 multiplies the same x2: one dense problem with B*M rows
-    LaunchDense(op_name, x1, x2, scale, bias, pertoken, out, b1 * d.m, d.k, d.n, 1, transpose_x2, stream);
+    LaunchDense(op_name, x1, x2, scale, bias, pertoken, out, b1 * d.m, d.k, d.n, 1, transpose_x2, packed, stream);
     return;
   }
   if (d.x1_batch == d.x2_batch && shared_rows) {
     // batch b of x1 meets batch b of x2: B equal groups
-    LaunchDense(op_name, x1, x2, scale, bias, pertoken, out, bo * d.m, d.k, d.n, bo, transpose_x2, stream);
+    LaunchDense(op_name, x1, x2, scale, bias, pertoken, out, bo * d.m, d.k, d.n, bo, transpose_x2, packed, stream);
     return;
   }
   // general broadcasting: one dense launch per output batch
@@ -148,8 +169,10 @@ void RunQuantBatchMatmul(const ms::Tensor &x1_in, const ms::Tensor &x2, const ms
       s1 *= d.x1_batch[ax];
       s2 *= d.x2_batch[ax];
     }
-    LaunchDense(op_name, x1.Slice(i1 * d.m * d.k, {d.m, d.k}), x2.Slice(i2 * d.k * d.n, {d.k, d.n}), scale, bias,
-                pertoken, out.Slice(idx * d.m * d.n, {d.m, d.n}), d.m, d.k, d.n, 1, transpose_x2, stream);
+    const int64_t x2_elems = packed ? (d.n / 16) * ((d.k + 63) / 64) * kPackedBlockBytes : d.k * d.n;   // one matrix of x2
+    LaunchDense(op_name, x1.Slice(i1 * d.m * d.k, {d.m, d.k}),
+                packed ? x2.Slice(i2 * x2_elems, {d.n / 16, (d.k + 63) / 64, kPackedBlockBytes}) : x2.Slice(i2 * x2_elems, {d.k, d.n}),
+                scale, bias, pertoken, out.Slice(idx * d.m * d.n, {d.m, d.n}), d.m, d.k, d.n, 1, transpose_x2, packed, stream);
   }
 }
 
@@ -161,8 +184,12 @@ class QuantBatchMatmulCustomOpFuncImpl : public OpFuncImpl {
   ShapeArray InferShape(const KernelTensorList &inputs) const override {
     const bool transpose_x1 = inputs[kQbmmInputTransposeX1].GetValueWithCheck<bool>();
     const bool transpose_x2 = inputs[kQbmmInputTransposeX2].GetValueWithCheck<bool>();
-    return {BatchMatMulMakeShape(inputs[kQbmmInputX1].GetShape(), inputs[kQbmmInputX2].GetShape(), transpose_x1,
-                                 transpose_x2, kQbmmMatSize, "QuantBatchMatmul")};
+    const std::string x2_format = inputs[kQbmmInputX2Format].IsNone() ? std::string(kNdFormat)
+                                                                      : inputs[kQbmmInputX2Format].GetValueWithCheck<std::string>();
+    return {BatchMatMulMakeShape(inputs[kQbmmInputX1].GetShape(),
+                                 QbmmLogicalX2Shape(inputs[kQbmmInputX1].GetShape(), inputs[kQbmmInputX2].GetShape(),
+                                                    transpose_x1, transpose_x2, x2_format),
+                                 transpose_x1, transpose_x2, kQbmmMatSize, "QuantBatchMatmul")};
   }
   TypeIdList InferType(const KernelTensorList &inputs) const override {
     TypeId output_type = kNumberTypeFloat16;
@@ -209,7 +236,8 @@ ms::Tensor quant_batch_matmul_custom(const ms::Tensor &x1, const ms::Tensor &x2,
                                      const std::optional<ms::Tensor> &pertoken_scale, bool transpose_x1,
                                      bool transpose_x2, const std::string &x2_format, const int64_t output_dtype) {
   auto output_shape =
-    BatchMatMulMakeShape(x1.shape(), x2.shape(), transpose_x1, transpose_x2, kQbmmMatSize, "QuantBatchMatmul");
+    BatchMatMulMakeShape(x1.shape(), QbmmLogicalX2Shape(x1.shape(), x2.shape(), transpose_x1, transpose_x2, x2_format),
+                         transpose_x1, transpose_x2, kQbmmMatSize, "QuantBatchMatmul");
   auto out = AllocateTensor(static_cast<TypeId>(output_dtype), output_shape);
   RunQuantBatchMatmul(x1, x2, scale, GetTensorOrEmpty(offset), GetTensorOrEmpty(bias),
                       GetTensorOrEmpty(pertoken_scale), transpose_x1, transpose_x2, x2_format, out);

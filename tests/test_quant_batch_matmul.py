@@ -39,6 +39,33 @@ def test_custom_quant_batch_matmul_basic(device, exec_mode, dtype):
         assert np.array_equal(_bits(out), O.quant_batch_matmul_oracle(x1, x2, scale))
 
 
+@pytest.mark.parametrize("exec_mode", MODES)
+def test_custom_quant_batch_matmul_bfp16_nz(device, exec_mode):
+    """The reference's test_custom_quant_batch_matmul_bfp16_nz (tests/st/test_quant_batch_matmul.py:86-118): x2 goes
+    through trans_data(ND_TO_FRACTAL_NZ) and the op is told x2_format="FRACTAL_NZ"; batched, then one shared x2 and a
+    decode-sized x1."""
+    rng = np.random.default_rng(5)
+    batch, m, k, n = 2, 128, 256, 128
+    x1 = rng.integers(-5, 5, (batch, m, k)).astype(np.int8)
+    x2 = rng.integers(-5, 5, (batch, k, n)).astype(np.int8)
+    scale = np.ones([n]).astype(np.float32)
+    expected = np.matmul(x1.astype(np.int32), x2.astype(np.int32)) * scale
+    with ms_custom_ops.exec_mode(exec_mode):
+        x2_nz = ms_custom_ops.trans_data(_t(x2), transdata_type=1)
+        out = ms_custom_ops.quant_batch_matmul(_t(x1), x2_nz, _t(scale), x2_format="FRACTAL_NZ", output_dtype=torch.bfloat16)
+    assert tuple(x2_nz.shape) == (batch, n // 16, k // 64, 1024) and out.shape == (batch, m, n)
+    assert np.allclose(expected, out.float().cpu().numpy(), 0.01)                 # reference's bar
+    assert np.array_equal(_bits(out), O.quant_batch_matmul_oracle(x1, x2, scale))
+    # one x2 for every batch of x1, 16 rows each: the streaming decode kernel on packed weights
+    x1d = rng.integers(-127, 128, (3, 16, 320)).astype(np.int8)
+    w = rng.integers(-127, 128, (320, 272)).astype(np.int8)
+    sc = rng.uniform(1e-3, 1e-2, 272).astype(np.float32)
+    with ms_custom_ops.exec_mode(exec_mode):
+        out = ms_custom_ops.quant_batch_matmul(_t(x1d), ms_custom_ops.trans_data(_t(w), 1), _t(sc), x2_format="FRACTAL_NZ",
+                                               output_dtype=torch.bfloat16)
+    assert np.array_equal(_bits(out), O.quant_batch_matmul_oracle(x1d.reshape(-1, 320), w, sc).reshape(3, 16, 272))
+
+
 def test_default_output_dtype_is_float16(device):
     x1 = torch.ones(16, 32, dtype=torch.int8, device="cuda")
     x2 = torch.ones(32, 16, dtype=torch.int8, device="cuda")
@@ -150,8 +177,10 @@ def test_qbmm_errors(device):
     q = ms_custom_ops.quant_batch_matmul
     with pytest.raises(RuntimeError, match="'x2_format' is only support"):
         q(x1, x2, s, x2_format="NCHW")
-    with pytest.raises(RuntimeError, match="FRACTAL_NZ"):
+    with pytest.raises(ValueError, match="'FRACTAL_NZ' takes an x2 prepacked by trans_data"):
         q(x1, x2, s, x2_format="FRACTAL_NZ")
+    with pytest.raises(ValueError, match="'transpose_x2' must be false"):
+        q(x1, ms_custom_ops.trans_data(x2, 1), s, transpose_x2=True, x2_format="FRACTAL_NZ")
     with pytest.raises(RuntimeError, match="'offset' is not implemented"):
         q(x1, x2, s, offset=s)
     with pytest.raises(RuntimeError, match="'output_dtype' must be"):
