@@ -5,6 +5,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+#include <utility>
+
 namespace msco {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -239,6 +242,16 @@ __device__ __forceinline__ void transpose16x8(const uint2 (&r)[16], v4i (&frag)[
     transpose4x4(r[4 * q].y, r[4 * q + 1].y, r[4 * q + 2].y, r[4 * q + 3].y, c0, c1, c2, c3);
     frag[4][q] = (int)c0; frag[5][q] = (int)c1; frag[6][q] = (int)c2; frag[7][q] = (int)c3;
   }
+}
+
+// f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>), in order
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 }  // namespace msco

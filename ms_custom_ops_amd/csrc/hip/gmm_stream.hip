@@ -29,16 +29,6 @@
 namespace msco {
 
 namespace {
-// f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>), in order
-template <typename F, int... I>
-__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F &&f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 constexpr int ST_WAVES = 4;
 constexpr int ST_THREADS = ST_WAVES * 64;
 constexpr int ST_COLS = kSkinnyCols;                  // 256 columns = 16 column groups per strip

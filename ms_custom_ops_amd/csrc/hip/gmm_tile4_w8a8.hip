@@ -14,7 +14,15 @@
 //     multiply, written to the LDS stage that the last barrier retired, and the registers are refilled
 //     right behind the write.  One load, one LDS write and two fragment reads are issued per four
 //     MFMAs: a burst of either would stall the in-order issue of the only wave on the SIMD.
-//   * One workgroup barrier per slab (2048 MFMA cycles).  Two LDS stages of 64 KiB.
+//   * One workgroup barrier per slab (2048 MFMA cycles).  Two LDS stages of 64 KiB (x stages 0 and 1, then weight
+//     stages 0 and 1, so that stage and block offsets fit the offset field of the LDS instructions).
+//   * A wave that is alone on its SIMD issues one instruction about every six cycles, whatever its kind (measured
+//     with chains of independent VALU, scalar and no-op instructions), so every address computation, scalar select
+//     and wait between the MFMAs costs as much issue time as a memory instruction.  The K loop therefore has two
+//     bodies: a steady-state one for slabs whose look-ahead stays inside the tile and inside K (stage, K quarter
+//     and staging parity are compile-time constants, every LDS access is a base register plus an immediate, loads
+//     need no tail masks: 346 instructions per 128 MFMAs) and a general one for the last slabs, whose loads run into
+//     the next tile or past K (546 instructions).
 //   * LDS rows are 128 B; 16-byte chunk c of row r sits at chunk position c ^ ((r >> 1) & 7), which
 //     makes both the staging writes and the 16-lane fragment reads bank-conflict free.
 //   * Persistent workgroups.  A workgroup walks its share of the tiles and the operand stream never
@@ -23,7 +31,12 @@
 //   * Weights are the MFMA's first operand and x the second, so a lane owns output row m and runs of 8
 //     consecutive columns; the fused dequant epilogue is staged through a small LDS region next to the
 //     ring (32 rows at a time) and stores full 128-byte row segments.
-//   * Partial m-tiles (the last tile of a group) skip the 32-row MFMA blocks that hold no rows.
+//   * The epilogue is issue bound as well (about 1150 VALU instructions per wave): its stores go through a buffer
+//     descriptor over the rows that exist (no predicates, one address add per store) and the LDS round trip of one
+//     32-row block hides under the arithmetic of the next.
+//   * Partial m-tiles (the last tile of a group) are multiplied in full (a loop variant or branches that skip the
+//     32-row blocks without rows make the register allocator shuffle or spill the 256 accumulators); their epilogue
+//     only touches the blocks that hold rows.
 #include "gmm_common.h"
 #include "gmm_kernels.h"
 
@@ -38,8 +51,9 @@ constexpr int T4_NW = 4;                         // wavefronts: 2 (m) x 2 (n)
 constexpr int T4_WT = 128;                       // wave tile edge
 constexpr int T4_F = 4;                          // 32 x 32 MFMA blocks per wave tile edge
 constexpr int T4_OP_STAGE = T4_BM * T4_BK;       // one operand's share of a stage (32 KiB)
-constexpr int T4_STAGE = 2 * T4_OP_STAGE;        // x rows, then weight rows
-constexpr int T4_RING = 2 * T4_STAGE;            // 128 KiB
+constexpr int T4_W_BASE = 2 * T4_OP_STAGE;       // x stages 0 and 1, then weight stages 0 and 1: a stage and a block offset
+                                                 // together fit the 16-bit offset field of an LDS instruction
+constexpr int T4_RING = 2 * T4_W_BASE;           // 128 KiB
 constexpr int T4_LD = T4_BM / 8 / T4_NW;         // staging quads (8 rows x 128 B per wave) per operand and slab
 constexpr int T4_EP_PITCH = 144;                 // epilogue staging: 128 payload bytes per row
 constexpr int T4_PARAM_OFF = T4_RING;            // epilogue operand tables (scale, bias, per-token; two tiles) behind the ring
@@ -206,24 +220,38 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   // fetches logical chunk (L % 8) ^ swizzle(row).  The row of quad u is 32 u + 8 wave + d_row, so neither
   // the swizzle ((row >> 1) & 7) nor the MFMA row permutation (row & 31) depends on u.  Everything that
   // can run past a tensor is in the per-lane offset (the only part the buffer unit range-checks).
-  const int d_row0 = 8 * wave + (lane >> 3);
-  const int d_chunk = (lane & 7) ^ ((d_row0 >> 1) & 7);
-  const unsigned a_voff0 = (unsigned)d_row0 * (unsigned)p.k + d_chunk * 16;
-  const unsigned b_voff0 = PK ? (unsigned)(((wave >> 1) * k_blocks + (wave & 1)) * 1024 + lane * 16)
-                              : (unsigned)t4_col_of_q(d_row0) * (unsigned)p.k + d_chunk * 16;   // LDS row rho feeds MFMA row rho % 32
+  // These lane constants are worked out again at the top of every tile from a lane id the compiler cannot see
+  // through: kept across the epilogue they would cost it registers, and a spill there stalls the operand stream.
   const unsigned rows32 = 32u * (unsigned)p.k;
   const unsigned b_step = PK ? 2u * (unsigned)k_blocks * 1024u : rows32;   // staging quad u -> u + 1: two column groups / 32 rows
-
+  int d_chunk;
+  unsigned a_voff0, b_voff0;
   // ---- fragment addressing ---------------------------------------------------------------------------
   // lane (l32, hh) reads row l32 of a 32-row block, logical chunk 2 q + hh of K quarter q.  The row
   // swizzle only depends on l32, and the chunk positions of the four quarters differ by an XOR with
-  // q << 5 in the byte address.
-  const int swz = (l32 >> 1) & 7;
-  const unsigned x_lane = (unsigned)((wave_m * T4_WT + l32) * T4_BK + ((hh ^ swz) << 4));
-  const unsigned w_lane = PK ? (unsigned)(T4_OP_STAGE + wave_n * 16384 + (l32 >> 4) * 2048 + hh * 256 + (t4_col_of_q(l32) & 15) * 16)
-                             : (unsigned)(T4_OP_STAGE + (wave_n * T4_WT + l32) * T4_BK + ((hh ^ swz) << 4));
-
-  unsigned char *st_lane = smem + wave * 1024 + lane * 16;
+  // q << 5 in the byte address.  LDS writes of the staging quads go to st_x / st_w.
+  // Every LDS and buffer instruction of the steady-state K loop takes one of these registers and an immediate
+  // offset: a wave that is alone on its SIMD issues one instruction about every six cycles whatever its kind, so
+  // address arithmetic and scalar bookkeeping between the MFMAs cost as much issue time as the memory instructions.
+  unsigned x_lane, w_lane, st_x, st_w;
+  auto lane_constants = [&]() {
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    const int q32 = ln & 31, h = ln >> 5;
+    const int d_row0 = 8 * wave + (ln >> 3);
+    d_chunk = (ln & 7) ^ ((d_row0 >> 1) & 7);
+    a_voff0 = (unsigned)d_row0 * (unsigned)p.k + d_chunk * 16;
+    b_voff0 = PK ? (unsigned)(((wave >> 1) * k_blocks + (wave & 1)) * 1024 + ln * 16)
+                 : (unsigned)t4_col_of_q(d_row0) * (unsigned)p.k + d_chunk * 16;   // LDS row rho feeds MFMA row rho % 32
+    const int swz = (q32 >> 1) & 7;
+    x_lane = (unsigned)((wave_m * T4_WT + q32) * T4_BK + ((h ^ swz) << 4));
+    w_lane = PK ? (unsigned)(T4_W_BASE + wave_n * 16384 + (q32 >> 4) * 2048 + h * 256 + (t4_col_of_q(q32) & 15) * 16)
+                : (unsigned)(T4_W_BASE + (wave_n * T4_WT + q32) * T4_BK + ((h ^ swz) << 4));
+    st_x = (unsigned)(wave * 1024 + ln * 16);
+    st_w = st_x + T4_W_BASE;
+    asm volatile("" : "+v"(st_w));
+  };
+  lane_constants();
   unsigned char *ep_stage = smem + T4_EP_OFF + wave * T4_EP_WAVE;
 
   const std::integral_constant<int, 0> c0;
@@ -259,8 +287,16 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   // write quad (op, u) of slab s to its LDS stage and refill it with slab s + 2
   auto cycle_one = [&](int s, auto par_c, auto op_c, auto u_c) {
     constexpr int P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
-    *reinterpret_cast<v4i *>(st_lane + (s & 1) * T4_STAGE + OP * T4_OP_STAGE + U * 4096) = stg[P][OP][U];
+    *reinterpret_cast<v4i *>(smem + ((OP == 0 ? st_x : st_w) + (s & 1) * T4_OP_STAGE + U * 4096)) = stg[P][OP][U];
     load_one(s + 2, par_c, op_c, u_c);
+  };
+  // the same for a slab whose successor lies inside the current tile and inside K: WS = stage written, soff = scalar
+  // offset of slab s + 2 (bytes of K; 16 times that in the packed weights)
+  auto cycle_clean = [&](auto ws_c, unsigned soff, auto par_c, auto op_c, auto u_c) {
+    constexpr int WS = decltype(ws_c)::value, P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
+    *reinterpret_cast<v4i *>(smem + ((OP == 0 ? st_x : st_w) + WS * T4_OP_STAGE + U * 4096)) = stg[P][OP][U];
+    if constexpr (OP == 0) stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rx_c, a_voff0 + U * rows32, soff, 0);
+    else stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rw_c, b_voff0 + U * b_step, PK ? soff * 16 : soff, 0);
   };
   // (qx = q << 5 arrives in a scalar the compiler cannot see through: hoisting the XORs out of the K
   // loop would park eight more addresses in registers that the loop does not have)
@@ -268,14 +304,24 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     constexpr int S = decltype(set_c)::value, F = decltype(f_c)::value;
     if constexpr (PK) {
       // qx = q << 5: K block q / 2 is 1024 bytes on, chunk pair q % 2 another 512
-      wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_STAGE + (w_lane + (qx >> 6) * 1024 + ((qx >> 5) & 1) * 512) + F * 4096);
+      wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_OP_STAGE + (w_lane + (qx >> 6) * 1024 + ((qx >> 5) & 1) * 512) + F * 4096);
     } else {
-      wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_STAGE + (w_lane ^ qx) + F * 32 * T4_BK);
+      wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_OP_STAGE + (w_lane ^ qx) + F * 32 * T4_BK);
     }
   };
   auto read_x = [&](int stage, unsigned qx, auto set_c, auto i_c) {
     constexpr int S = decltype(set_c)::value, I = decltype(i_c)::value;
-    xf[S][I] = *reinterpret_cast<const v4i *>(smem + stage * T4_STAGE + (x_lane ^ qx) + I * 32 * T4_BK);
+    xf[S][I] = *reinterpret_cast<const v4i *>(smem + stage * T4_OP_STAGE + (x_lane ^ qx) + I * 32 * T4_BK);
+  };
+  // fragment reads with everything but the registers above known at compile time
+  auto read_w_clean = [&](auto stage_c, auto q_c, auto set_c, auto f_c) {
+    constexpr int ST = decltype(stage_c)::value, Q = decltype(q_c)::value, S = decltype(set_c)::value, F = decltype(f_c)::value;
+    if constexpr (PK) wf[S][F] = *reinterpret_cast<const v4i *>(smem + (w_lane + ST * T4_OP_STAGE + (Q >> 1) * 1024 + (Q & 1) * 512 + F * 4096));
+    else wf[S][F] = *reinterpret_cast<const v4i *>(smem + ((w_lane ^ (unsigned)(Q << 5)) + ST * T4_OP_STAGE + F * 4096));
+  };
+  auto read_x_clean = [&](auto stage_c, auto q_c, auto set_c, auto i_c) {
+    constexpr int ST = decltype(stage_c)::value, Q = decltype(q_c)::value, S = decltype(set_c)::value, I = decltype(i_c)::value;
+    xf[S][I] = *reinterpret_cast<const v4i *>(smem + ((x_lane ^ (unsigned)(Q << 5)) + ST * T4_OP_STAGE + I * 4096));
   };
   auto opaque_q = [](int q) {
     unsigned qx = (unsigned)q << 5;
@@ -303,11 +349,11 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     t4_barrier();
   }
-
   for (int ti = 0;; ++ti) {
     // the tile after this one: the operand stream crosses into it during the last slabs
     nxt = tile_at(ti + 1);
     if (nxt.valid) { rx_n = x_rsrc(nxt); rw_n = w_rsrc(nxt); }
+    if (ti > 0) lane_constants();
 
     // Epilogue operands of this tile (scale and bias of its 256 columns, per-token scale of its 256
     // rows) go straight from memory into this tile's LDS table (two tables, alternating per tile: the
@@ -346,36 +392,26 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     const int rows_wave = rows_here - wave_m * T4_WT;
     const int fm_active = max(0, min(T4_F, (rows_wave + 31) / 32));
 
+    // (a zero the compiler cannot see through: a constant vector of zeros gets hoisted out of the tile loop into
+    // registers the K loops do not have)
+    int zero = 0;
+    asm volatile("" : "+v"(zero));
 #pragma unroll
     for (int f = 0; f < T4_F; ++f)
 #pragma unroll
       for (int i = 0; i < T4_F; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[f][i][r] = 0;
+        for (int r = 0; r < 16; ++r) acc[f][i][r] = zero;
     // quarter-0 fragments of slab 0 (read here rather than behind the previous tile's last slab, so that
     // the epilogue does not have to keep them alive)
     read_w(0, 0, c0, c0); read_w(0, 0, c0, c1); read_w(0, 0, c0, c2); read_w(0, 0, c0, c3);
     read_x(0, 0, c0, c0); read_x(0, 0, c0, c1); read_x(0, 0, c0, c2); read_x(0, 0, c0, c3);
 
     {
-      // One K quarter: the MFMAs of fragment set CUR; meanwhile the fragments of (rstage, rq) are read
-      // into set NXT and staging group G (x and w quads 2 G, 2 G + 1) of slab ss goes to LDS and is
-      // refilled.  LDS operations keep their source order; the scheduling groups pin one memory
-      // operation behind each of the first MFMAs.
-      auto quarter = [&](auto cur_c, auto nxt_c, int rstage, int rq_index, int ss, auto par_c, auto g_c) {
-        constexpr int G = decltype(g_c)::value;
-        constexpr int S = decltype(cur_c)::value;
-        const unsigned rq = opaque_q(rq_index);
-        const std::integral_constant<int, 2 * G> ua;
-        const std::integral_constant<int, 2 * G + 1> ub;
-        read_w(rstage, rq, nxt_c, c0); read_x(rstage, rq, nxt_c, c0);
-        cycle_one(ss, par_c, c0, ua);
-        read_x(rstage, rq, nxt_c, c1); read_x(rstage, rq, nxt_c, c2);
-        cycle_one(ss, par_c, c0, ub);
-        read_x(rstage, rq, nxt_c, c3); read_w(rstage, rq, nxt_c, c1);
-        cycle_one(ss, par_c, c1, ua);
-        read_w(rstage, rq, nxt_c, c2); read_w(rstage, rq, nxt_c, c3);
-        cycle_one(ss, par_c, c1, ub);
+      // The 16 MFMAs of fragment set S; the scheduling groups pin one memory operation of the caller behind each
+      // of the first MFMAs.
+      auto mfma_quarter = [&](auto set_c) {
+        constexpr int S = decltype(set_c)::value;
 #pragma unroll
         for (int f = 0; f < T4_F; ++f)
 #pragma unroll
@@ -394,6 +430,25 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         }
         __builtin_amdgcn_sched_barrier(0);
       };
+      // One K quarter: the MFMAs of fragment set CUR; meanwhile the fragments of (rstage, rq) are read
+      // into set NXT and staging group G (x and w quads 2 G, 2 G + 1) of slab ss goes to LDS and is
+      // refilled.  LDS operations keep their source order; the scheduling groups pin one memory
+      // operation behind each of the first MFMAs.
+      auto quarter = [&](auto cur_c, auto nxt_c, int rstage, int rq_index, int ss, auto par_c, auto g_c) {
+        constexpr int G = decltype(g_c)::value;
+        const unsigned rq = opaque_q(rq_index);
+        const std::integral_constant<int, 2 * G> ua;
+        const std::integral_constant<int, 2 * G + 1> ub;
+        read_w(rstage, rq, nxt_c, c0); read_x(rstage, rq, nxt_c, c0);
+        cycle_one(ss, par_c, c0, ua);
+        read_x(rstage, rq, nxt_c, c1); read_x(rstage, rq, nxt_c, c2);
+        cycle_one(ss, par_c, c0, ub);
+        read_x(rstage, rq, nxt_c, c3); read_w(rstage, rq, nxt_c, c1);
+        cycle_one(ss, par_c, c1, ua);
+        read_w(rstage, rq, nxt_c, c2); read_w(rstage, rq, nxt_c, c3);
+        cycle_one(ss, par_c, c1, ub);
+        mfma_quarter(cur_c);
+      };
       // One K slab kt (LDS stage kt & 1).  On entry the quarter-0 fragments are in fragment set 0 and
       // group 0 of slab kt+1 is in LDS; PAR is the staging parity of slab kt+1.
       auto period = [&](int kt, auto par_c) {
@@ -409,13 +464,49 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         t4_barrier();
         quarter(c1, c0, stage ^ 1, 0, kt + 2, other, c0);
       };
-      for (int kt = 0; kt < k_slabs; kt += 2) {
+      // The same with stage, quarter and parity known at compile time, for slabs whose look-ahead stays inside the
+      // current tile and inside K (loads need neither the next tile's descriptors nor a tail mask).
+      auto quarter_clean = [&](auto cur_c, auto nxt_c, auto rstage_c, auto rq_c, auto ws_c, unsigned soff, auto par_c, auto g_c) {
+        constexpr int G = decltype(g_c)::value;
+        const std::integral_constant<int, 2 * G> ua;
+        const std::integral_constant<int, 2 * G + 1> ub;
+        read_w_clean(rstage_c, rq_c, nxt_c, c0); read_x_clean(rstage_c, rq_c, nxt_c, c0);
+        cycle_clean(ws_c, soff, par_c, c0, ua);
+        read_x_clean(rstage_c, rq_c, nxt_c, c1); read_x_clean(rstage_c, rq_c, nxt_c, c2);
+        cycle_clean(ws_c, soff, par_c, c0, ub);
+        read_x_clean(rstage_c, rq_c, nxt_c, c3); read_w_clean(rstage_c, rq_c, nxt_c, c1);
+        cycle_clean(ws_c, soff, par_c, c1, ua);
+        read_w_clean(rstage_c, rq_c, nxt_c, c2); read_w_clean(rstage_c, rq_c, nxt_c, c3);
+        cycle_clean(ws_c, soff, par_c, c1, ub);
+        mfma_quarter(cur_c);
+      };
+      // slab kt in stage ST; soff3 / soff4: K offsets of slabs kt + 3 and kt + 4
+      auto period_clean = [&](auto stage_c, auto par_c, unsigned soff3, unsigned soff4) {
+        constexpr int ST = decltype(stage_c)::value, PAR = decltype(par_c)::value;
+        const std::integral_constant<int, ST ^ 1> other_stage;
+        const std::integral_constant<int, PAR ^ 1> other;
+        quarter_clean(c0, c1, stage_c, c1, other_stage, soff3, par_c, c1);
+        quarter_clean(c1, c0, stage_c, c2, other_stage, soff3, par_c, c2);
+        quarter_clean(c0, c1, stage_c, c3, other_stage, soff3, par_c, c3);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        t4_barrier();
+        quarter_clean(c1, c0, other_stage, c0, stage_c, soff4, other, c0);
+      };
+      // iterations whose furthest request (group 0 of slab kt + 5) ends inside K
+      const int k_clean = max(0, ((p.k / T4_BK - 4) / 2) * 2);
+      int kt = 0;
+      for (; kt < k_clean; kt += 2) {
+        const unsigned kb = (unsigned)kt * T4_BK;
+        period_clean(c0, c1, kb + 3 * T4_BK, kb + 4 * T4_BK);
+        period_clean(c1, c0, kb + 4 * T4_BK, kb + 5 * T4_BK);
+      }
+      // the last slabs of the tile (their look-ahead runs into the next tile or past K) multiply every block: what
+      // lands in blocks without rows is never stored
+      for (; kt < k_slabs; kt += 2) {
         period(kt, c1);
         period(kt + 1, c0);
       }
     }
-
-
     // ---- fused dequant epilogue ----------------------------------------------------------------------
     // acc[f][i][r] is output row 32 i + l32, column 32 f + 16 (r / 8) + 8 hh + (r % 8) of the wave tile.
     // Per 32-row block and 128-byte column piece: dequantise, park in this wave's LDS region (rows of
@@ -441,104 +532,144 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         t4_barrier();
       }
-      // One column piece of the wave tile (16-bit outputs: a 64-column half; int32: a 32-column block):
-      // its scales are read once and kept in registers for the four 32-row blocks.  A wave's LDS
-      // operations execute in order, so the staging writes, the read-back and the next block's writes
-      // need no waits between them beyond the data dependencies the compiler tracks.
-      auto run_piece = [&](auto piece_c) {
-        constexpr bool raw = MODE == 2;
+      // The wave tile leaves in units of one column piece (16-bit outputs: a 64-column half; int32: a 32-column
+      // block) x one 32-row block.  A unit is dequantised into four 16-byte vectors per lane, parked in the wave's
+      // staging rows and read back with lanes along columns, so that a store covers full 128-byte row segments.
+      // The units are software pipelined: the read-back of unit u - 1 is issued before the arithmetic of unit u and
+      // stored behind it, so the LDS round trip hides under the arithmetic (a wave's LDS operations execute in
+      // order: the staging writes of unit u queue behind that read-back).  Rows past the end of the group fall
+      // outside the store descriptor, columns past N are killed in the lane offset: stores need no predicates.
+      constexpr bool raw = MODE == 2;
+      constexpr int esize = raw ? 4 : 2;
+      constexpr int NF = raw ? 1 : 2;                                   // 32-column MFMA blocks in a piece
+      constexpr int PIECES = raw ? 4 : 2;
+      constexpr int UNITS = PIECES * T4_F;
+      const unsigned pitch = (unsigned)p.n * esize;
+      const int rows_valid = max(0, min(T4_WT, rows_wave));
+      // (assembled from scalars read off lane 0: a descriptor the compiler takes for lane-dependent is applied
+      // lane group by lane group)
+      const unsigned long long out_first =
+          (unsigned long long)(reinterpret_cast<unsigned char *>(p.out) + ((long long)m_base * p.n + n_base) * esize);
+      const unsigned out_lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)out_first);
+      const unsigned out_hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(out_first >> 32));
+      const __amdgpu_buffer_rsrc_t rs_out =
+          t4_rsrc(reinterpret_cast<void *>(((unsigned long long)out_hi << 32) | out_lo),
+                  __builtin_amdgcn_readfirstlane((int)min((long long)rows_valid * pitch, 0x7FFFFFFFll)));
+      const int piece = e_lane & 7;
+      const unsigned v_row = (unsigned)(e_lane >> 3) * pitch + piece * 16;
+      unsigned char *dst = ep_stage + e_l32 * T4_EP_PITCH + 16 * e_hh * (raw ? 2 : 1);
+      const unsigned char *src = ep_stage + (e_lane >> 3) * T4_EP_PITCH + piece * 16;
+      unsigned sraw[NF][2][8];
+      uint4 q[4], rb[4];
+      auto read_back = [&]() {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) rb[t] = *reinterpret_cast<const uint4 *>(src + 8 * t * T4_EP_PITCH);
+      };
+      auto store_unit = [&](auto u_c) {
+        constexpr int U = decltype(u_c)::value, PIECE = U / T4_F, I = U % T4_F;
+        const int n_first = n_base + PIECE * (raw ? 32 : 64) + (raw ? 4 : 8) * piece;
+        const unsigned v0 = (n_first < p.n ? v_row : T4_OOB) + PIECE * 128;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, rb[t]), rs_out, v0 + (unsigned)(32 * I + 8 * t) * pitch, 0, 0);
+      };
+      auto load_scales = [&](auto piece_c) {
         constexpr int PIECE = decltype(piece_c)::value;
-        constexpr int esize = raw ? 4 : 2;
-        constexpr int NF = raw ? 1 : 2;                                   // 32-column MFMA blocks in the piece
-        constexpr int f_lo = NF * PIECE;
-        unsigned sraw[NF][2][8];
         if constexpr (!raw) {
 #pragma unroll
           for (int ff = 0; ff < NF; ++ff)
 #pragma unroll
             for (int s2 = 0; s2 < 2; ++s2) {
-              const int cw = 32 * (f_lo + ff) + 16 * s2 + 8 * e_hh;
+              const int cw = 32 * (NF * PIECE + ff) + 16 * s2 + 8 * e_hh;
               const uint4 s_lo = *reinterpret_cast<const uint4 *>(tb_scale + cw);
               const uint4 s_hi = *reinterpret_cast<const uint4 *>(tb_scale + cw + 4);
               sraw[ff][s2][0] = s_lo.x; sraw[ff][s2][1] = s_lo.y; sraw[ff][s2][2] = s_lo.z; sraw[ff][s2][3] = s_lo.w;
               sraw[ff][s2][4] = s_hi.x; sraw[ff][s2][5] = s_hi.y; sraw[ff][s2][6] = s_hi.z; sraw[ff][s2][7] = s_hi.w;
             }
         }
-        const int piece = e_lane & 7;
-        const int col = (raw ? 32 * PIECE : 64 * PIECE) + (raw ? 4 : 8) * piece;   // first column of this lane's read-back piece
-        const int n_first = n_base + col;
-        unsigned char *dst = ep_stage + e_l32 * T4_EP_PITCH;
-        const unsigned char *src = ep_stage + (e_lane >> 3) * T4_EP_PITCH + piece * 16;
-        auto block = [&](auto i_c) {
-          constexpr int I = decltype(i_c)::value;
-          if (I >= fm_active) return;
-          const float pt = tb_pt[32 * I + e_l32];
+      };
+      auto compute = [&](auto u_c) {
+        constexpr int U = decltype(u_c)::value, PIECE = U / T4_F, I = U % T4_F;
+        const float pt = tb_pt[32 * I + e_l32];
 #pragma unroll
-          for (int ff = 0; ff < NF; ++ff) {
+        for (int ff = 0; ff < NF; ++ff) {
 #pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2) {
-              const int f = f_lo + ff;
-              const int cw = 32 * f + 16 * s2 + 8 * e_hh;          // column inside the wave tile
-              const int cs = cw - 32 * f_lo;                       // column inside the staged piece
-              // accumulators leave the accumulation file here and not earlier (pinned: read ahead of time
-              // they would not fit into the architectural file next to the staging registers)
-              int a8[8];
+          for (int s2 = 0; s2 < 2; ++s2) {
+            constexpr int f_lo = NF * PIECE;
+            const int f = f_lo + ff;
+            const int cw = 32 * f + 16 * s2 + 8 * e_hh;          // column inside the wave tile
+            // accumulators leave the accumulation file here and not earlier (pinned: read ahead of time they
+            // would not fit into the architectural file next to the staging registers)
+            int a8[8];
 #pragma unroll
-              for (int j = 0; j < 8; ++j) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a8[j]) : "a"(acc[f][I][8 * s2 + j]));
-              if (has_bias) {
-                const int4 b_lo = *reinterpret_cast<const int4 *>(tb_bias + cw);
-                const int4 b_hi = *reinterpret_cast<const int4 *>(tb_bias + cw + 4);
-                a8[0] += b_lo.x; a8[1] += b_lo.y; a8[2] += b_lo.z; a8[3] += b_lo.w;
-                a8[4] += b_hi.x; a8[5] += b_hi.y; a8[6] += b_hi.z; a8[7] += b_hi.w;
-              }
-              if constexpr (raw) {
-                int *d = reinterpret_cast<int *>(dst + cs * 4);
-                *reinterpret_cast<int4 *>(d) = make_int4(a8[0], a8[1], a8[2], a8[3]);
-                *reinterpret_cast<int4 *>(d + 4) = make_int4(a8[4], a8[5], a8[6], a8[7]);
+            for (int j = 0; j < 8; ++j) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a8[j]) : "a"(acc[f][I][8 * s2 + j]));
+            if (has_bias) {
+              const int4 b_lo = *reinterpret_cast<const int4 *>(tb_bias + cw);
+              const int4 b_hi = *reinterpret_cast<const int4 *>(tb_bias + cw + 4);
+              a8[0] += b_lo.x; a8[1] += b_lo.y; a8[2] += b_lo.z; a8[3] += b_lo.w;
+              a8[4] += b_hi.x; a8[5] += b_hi.y; a8[6] += b_hi.z; a8[7] += b_hi.w;
+            }
+            if constexpr (raw) {
+              q[2 * s2] = make_uint4(a8[0], a8[1], a8[2], a8[3]);
+              q[2 * s2 + 1] = make_uint4(a8[4], a8[5], a8[6], a8[7]);
+            } else {
+              float v[8];
+#pragma unroll
+              for (int j = 0; j < 8; ++j) v[j] = dequant(a8[j], __uint_as_float(sraw[ff][s2][j]), pt);
+              uint4 r;
+              if constexpr (MODE == 0) {
+                r.x = pack_bf16x2(v[0], v[1]); r.y = pack_bf16x2(v[2], v[3]);
+                r.z = pack_bf16x2(v[4], v[5]); r.w = pack_bf16x2(v[6], v[7]);
               } else {
-                float v[8];
+                // the float32 product is rounded before the conversion (the golden's order); left visible,
+                // multiply and conversion are merged into one mixed-precision instruction that rounds once
 #pragma unroll
-                for (int j = 0; j < 8; ++j) v[j] = dequant(a8[j], __uint_as_float(sraw[ff][s2][j]), pt);
-                uint4 q;
-                if constexpr (MODE == 0) {
-                  q.x = pack_bf16x2(v[0], v[1]); q.y = pack_bf16x2(v[2], v[3]);
-                  q.z = pack_bf16x2(v[4], v[5]); q.w = pack_bf16x2(v[6], v[7]);
-                } else {
-                  // the float32 product is rounded before the conversion (the golden's order); left visible,
-                  // multiply and conversion are merged into one mixed-precision instruction that rounds once
-#pragma unroll
-                  for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(v[j]));
-                  q.x = f32_to_f16_rne(v[0]) | ((unsigned)f32_to_f16_rne(v[1]) << 16);
-                  q.y = f32_to_f16_rne(v[2]) | ((unsigned)f32_to_f16_rne(v[3]) << 16);
-                  q.z = f32_to_f16_rne(v[4]) | ((unsigned)f32_to_f16_rne(v[5]) << 16);
-                  q.w = f32_to_f16_rne(v[6]) | ((unsigned)f32_to_f16_rne(v[7]) << 16);
-                }
-                *reinterpret_cast<uint4 *>(dst + cs * 2) = q;
+                for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(v[j]));
+                r.x = f32_to_f16_rne(v[0]) | ((unsigned)f32_to_f16_rne(v[1]) << 16);
+                r.y = f32_to_f16_rne(v[2]) | ((unsigned)f32_to_f16_rne(v[3]) << 16);
+                r.z = f32_to_f16_rne(v[4]) | ((unsigned)f32_to_f16_rne(v[5]) << 16);
+                r.w = f32_to_f16_rne(v[6]) | ((unsigned)f32_to_f16_rne(v[7]) << 16);
               }
+              q[2 * ff + s2] = r;
             }
           }
-          // read back row-major: lane -> (row 8 t + lane / 8, 16-byte column piece lane % 8)
+        }
+      };
+      // staging row of a lane: 16-bit outputs, vector 2 ff + s2 holds columns 32 ff + 16 s2 + 8 hh .. + 8 (bytes 64 ff +
+      // 32 s2 + 16 hh); int32, vectors 2 s2 and 2 s2 + 1 hold columns 16 s2 + 8 hh .. + 8 (bytes 64 s2 + 32 hh, + 16)
+      auto park = [&]() {
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int row = 32 * I + 8 * t + (e_lane >> 3);
-            const uint4 q = *reinterpret_cast<const uint4 *>(src + 8 * t * T4_EP_PITCH);
-            if (row < rows_wave && n_first < p.n) {
-              unsigned char *o = reinterpret_cast<unsigned char *>(p.out) + ((long long)(m_base + row) * p.n + n_first) * esize;
-              *reinterpret_cast<uint4 *>(o) = q;
-            }
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4 *>(dst + (raw ? 64 * (j >> 1) + 16 * (j & 1) : 32 * j)) = q[j];
+      };
+      if (fm_active == T4_F) {
+        static_for<UNITS>([&](auto u_c) {
+          constexpr int U = decltype(u_c)::value;
+          if constexpr (U > 0) read_back();
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (U % T4_F == 0) load_scales(std::integral_constant<int, U / T4_F>{});
+          compute(u_c);
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (U > 0) store_unit(std::integral_constant<int, (U > 0 ? U - 1 : 0)>{});
+          park();
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        read_back();
+        store_unit(std::integral_constant<int, UNITS - 1>{});
+      } else {
+        // partial m-tile: only the 32-row blocks that hold rows, one after the other
+        static_for<UNITS>([&](auto u_c) {
+          constexpr int U = decltype(u_c)::value;
+          if constexpr (U % T4_F == 0) load_scales(std::integral_constant<int, U / T4_F>{});
+          if (U % T4_F < fm_active) {
+            compute(u_c);
+            park();
+            read_back();
+            store_unit(u_c);
           }
           __builtin_amdgcn_sched_barrier(0);
-        };
-        block(c0); block(c1); block(c2); block(c3);
-      };
-      run_piece(c0);
-      run_piece(c1);
-      if constexpr (MODE == 2) {
-        run_piece(c2);
-        run_piece(c3);
+        });
       }
     }
-
     if (!nxt.valid) break;
     cur = nxt;
     rx_c = rx_n;
