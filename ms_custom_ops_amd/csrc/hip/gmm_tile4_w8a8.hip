@@ -202,8 +202,10 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   // K slabs per tile, rounded up to even (the staging parities alternate per slab); slabs past K read zeros
   const int k_slabs = 2 * ((p.k + 2 * T4_BK - 1) / (2 * T4_BK));
   const long long w_elems = (long long)p.k * p.n;
+  // (the window ends with the group: the rows of a partial m-tile that belong to the next group read as zeros, cost no
+  // memory traffic, and multiplying zeros costs the matrix pipe far less power than multiplying somebody else's rows)
   auto x_rsrc = [&](const T4Tile &t) {
-    return t4_rsrc(reinterpret_cast<const int8_t *>(p.x) + (long long)t.m0 * p.k, (long long)(p.m - t.m0) * p.k);
+    return t4_rsrc(reinterpret_cast<const int8_t *>(p.x) + (long long)t.m0 * p.k, (long long)(t.g_end - t.m0) * p.k);
   };
   const int k_blocks = (p.k + 63) / 64, col_groups = (p.n + 15) / 16;   // packed layout
   auto w_rsrc = [&](const T4Tile &t) {

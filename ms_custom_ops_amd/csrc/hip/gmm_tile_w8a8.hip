@@ -211,11 +211,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   }
 
   // Buffer descriptors start at this tile's first x row / weight column, so per-lane offsets stay
-  // small; anything past the end of the tensor reads as zero (no clamping, no branches in the loop).
+  // small; anything past the end of the group's rows / the tensor reads as zero (no clamping, no branches in
+  // the loop; zeros instead of the next group's rows cost neither memory traffic nor matrix-pipe power).
   const long long w_elems = (long long)p.k * p.n;
   const int8_t *wg = p.w + (long long)grp * w_elems;
   const __amdgpu_buffer_rsrc_t rx =
-    make_rsrc(reinterpret_cast<const int8_t *>(p.x) + (long long)m0 * p.k, (long long)(p.m - m0) * p.k);
+    make_rsrc(reinterpret_cast<const int8_t *>(p.x) + (long long)m0 * p.k, (long long)(g_end - m0) * p.k);
   const int pk_blocks = (p.k + 63) / 64, pk_groups = (p.n + 15) / 16;   // packed layout: K blocks per column group, column groups
   const __amdgpu_buffer_rsrc_t rw =
     PK   ? make_rsrc(p.w + ((long long)grp * pk_groups + n0 / 16) * pk_blocks * 1024, (long long)(pk_groups - n0 / 16) * pk_blocks * 1024)
