@@ -1,7 +1,8 @@
 // MoE routing (stable counting sort of (token, k) entries by expert + activation gather) and weighted
 // un-permutation for gfx950.  Both are HBM-bound row copies around a small integer problem:
 //
-//   init_routing   1. per block of 1024 entries: histogram of the expert ids (LDS atomics)
+//   init_routing   (steps 1-3 are one launch for up to 16 blocks, every block repeating the small steps 1 and 2 for itself)
+//                  1. per block of 1024 entries: histogram of the expert ids (LDS atomics)
 //                  2. one workgroup: per expert, exclusive scan over the blocks, then over the experts;
 //                     writes the count / cumulative-count output
 //                  3. per block, sixteen wavefronts rank 64 consecutive entries each among equal expert ids with
@@ -87,15 +88,12 @@ __global__ void __launch_bounds__(1024) route_scan_kernel(int *block_hist, int *
 // equal expert ids with ballots (one round per distinct id in the chunk) and leaves the chunk's per-expert counts
 // in LDS; a prefix over the sixteen chunks turns the counts into first positions; rank + first position is the
 // output row.  Chunks, and positions inside a chunk, are taken in flat order, so the sort is stable.
-__global__ void __launch_bounds__(1024) route_rank_kernel(const int *expert_idx, const int *block_first, int *expanded_row_idx,
-                                                          int *sorted_src, long long n, int expert_num) {
-  extern __shared__ int chunk_first[];   // [16][expert_num]
+// (block_first: this block's row of first positions, in global memory or in LDS; e: the entry's expert id, -1 for none)
+__device__ __forceinline__ void rank_block(int *chunk_first, const int *block_first, long long i, bool live, int e,
+                                           int *expanded_row_idx, int *sorted_src, int expert_num) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int *mine = chunk_first + wave * expert_num;
-  for (int e = lane; e < expert_num; e += 64) mine[e] = 0;
-  const long long i = (long long)blockIdx.x * kRouteBlock + threadIdx.x;
-  const bool live = i < n;
-  const int e = live ? clamp_expert(expert_idx[i], expert_num) : -1;
+  for (int x = lane; x < expert_num; x += 64) mine[x] = 0;
   unsigned long long todo = __ballot(live);
   int rank = 0;
   while (todo) {
@@ -108,7 +106,7 @@ __global__ void __launch_bounds__(1024) route_rank_kernel(const int *expert_idx,
   }
   __syncthreads();
   for (int x = threadIdx.x; x < expert_num; x += 1024) {
-    int running = block_first[(long long)blockIdx.x * expert_num + x];
+    int running = block_first[x];
 #pragma unroll
     for (int w = 0; w < 16; ++w) {
       const int c = chunk_first[w * expert_num + x];
@@ -122,6 +120,72 @@ __global__ void __launch_bounds__(1024) route_rank_kernel(const int *expert_idx,
     expanded_row_idx[i] = dest;
     sorted_src[dest] = (int)i;
   }
+}
+
+__global__ void __launch_bounds__(1024) route_rank_kernel(const int *expert_idx, const int *block_first, int *expanded_row_idx,
+                                                          int *sorted_src, long long n, int expert_num) {
+  extern __shared__ int chunk_first[];   // [16][expert_num]
+  const long long i = (long long)blockIdx.x * kRouteBlock + threadIdx.x;
+  const bool live = i < n;
+  const int e = live ? clamp_expert(expert_idx[i], expert_num) : -1;
+  rank_block(chunk_first, block_first + (long long)blockIdx.x * expert_num, i, live, e, expanded_row_idx, sorted_src, expert_num);
+}
+
+// Histogram, scan and ranking in one launch for problems of at most kSmallBlocks blocks: every block histograms all
+// entries itself (a few thousand LDS atomics) instead of waiting for the other blocks, then ranks its own 1024.  At
+// this size the three launches above cost more in launch gaps than in work.
+constexpr int kSmallBlocks = 16;
+__global__ void __launch_bounds__(1024) route_small_kernel(const int *expert_idx, int *count_or_cumsum, int *before_capacity,
+                                                           int *expanded_row_idx, int *sorted_src, long long n, int expert_num,
+                                                           int flag) {
+  extern __shared__ int lds[];   // first[blocks][expert_num], chunk_first[16][expert_num], total[expert_num], base[expert_num]
+  const int blocks = gridDim.x;
+  int *first = lds;
+  int *chunk_first = first + blocks * expert_num;
+  int *total = chunk_first + 16 * expert_num;
+  int *base = total + expert_num;
+  for (int x = threadIdx.x; x < blocks * expert_num; x += 1024) first[x] = 0;
+  __syncthreads();
+  int my_e = -1;
+  for (int b = 0; b < blocks; ++b) {
+    const long long i = (long long)b * kRouteBlock + threadIdx.x;
+    if (i < n) {
+      const int e = clamp_expert(expert_idx[i], expert_num);
+      atomicAdd(&first[b * expert_num + e], 1);
+      if (b == (int)blockIdx.x) my_e = e;
+    }
+  }
+  __syncthreads();
+  const int e = threadIdx.x;
+  if (e < expert_num) {
+    int running = 0;
+    for (int b = 0; b < blocks; ++b) {
+      const int v = first[b * expert_num + e];
+      first[b * expert_num + e] = running;
+      running += v;
+    }
+    total[e] = running;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int j = 0; j < expert_num; ++j) {
+      base[j] = acc;
+      acc += total[j];
+    }
+  }
+  __syncthreads();
+  if (e < expert_num) {
+    first[blockIdx.x * expert_num + e] += base[e];
+    if (blockIdx.x == 0) {
+      if (count_or_cumsum != nullptr && flag == 1) count_or_cumsum[e] = base[e] + total[e];
+      if (count_or_cumsum != nullptr && flag == 2) count_or_cumsum[e] = total[e];
+      if (before_capacity != nullptr) before_capacity[e] = 0;
+    }
+  }
+  __syncthreads();
+  const long long i = (long long)blockIdx.x * kRouteBlock + threadIdx.x;
+  rank_block(chunk_first, first + blockIdx.x * expert_num, i, my_e >= 0, my_e, expanded_row_idx, sorted_src, expert_num);
 }
 
 __global__ void __launch_bounds__(256) route_gather_kernel(const unsigned char *x, const int *sorted_src, unsigned char *expanded_x,
@@ -269,11 +333,17 @@ int msco_moe_init_routing_v2(const void *x, const int32_t *expert_idx, void *exp
   const long long blocks = route_blocks(n);
   int *block_hist = static_cast<int *>(workspace);
   int *sorted_src = block_hist + blocks * expert_num;
-  hipLaunchKernelGGL(route_hist_kernel, dim3((unsigned)blocks), dim3(256), 0, s, expert_idx, block_hist, n, (int)expert_num);
-  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, block_hist, expert_tokens_count_or_cumsum,
-                     expert_tokens_before_capacity, (int)blocks, (int)expert_num, (int)count_or_cumsum_flag);
-  hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(1024), (size_t)16 * expert_num * sizeof(int), s, expert_idx,
-                     block_hist, expanded_row_idx, sorted_src, n, (int)expert_num);
+  const size_t small_lds = (size_t)(blocks + 16 + 2) * expert_num * sizeof(int);
+  if (blocks <= kSmallBlocks && small_lds <= 64 * 1024) {
+    hipLaunchKernelGGL(route_small_kernel, dim3((unsigned)blocks), dim3(1024), small_lds, s, expert_idx, expert_tokens_count_or_cumsum,
+                       expert_tokens_before_capacity, expanded_row_idx, sorted_src, n, (int)expert_num, (int)count_or_cumsum_flag);
+  } else {
+    hipLaunchKernelGGL(route_hist_kernel, dim3((unsigned)blocks), dim3(256), 0, s, expert_idx, block_hist, n, (int)expert_num);
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, block_hist, expert_tokens_count_or_cumsum,
+                       expert_tokens_before_capacity, (int)blocks, (int)expert_num, (int)count_or_cumsum_flag);
+    hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(1024), (size_t)16 * expert_num * sizeof(int), s, expert_idx,
+                       block_hist, expanded_row_idx, sorted_src, n, (int)expert_num);
+  }
   hipLaunchKernelGGL(route_gather_kernel, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned char *>(x), sorted_src,
                      static_cast<unsigned char *>(expanded_x), (long long)hidden * elem_bytes, (int)k);
   return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
