@@ -449,7 +449,7 @@ hipError_t launch_skinny_w8a8(const GmmParams &p, bool nk, bool wide16, hipStrea
   if (p.m == 0) return hipSuccess;
   if (wide16) {
     auto kern = nk ? gmm_w8a8_skinny16_kernel<true> : gmm_w8a8_skinny16_kernel<false>;
-    static bool attr_done[2] = {false, false};   // idempotent, so a race between first launches is harmless
+    static std::atomic<bool> attr_done[2];   // zero-initialised; the attribute call is idempotent, so a race between first launches repeats it at worst
     if (!attr_done[nk]) {
       const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)W16_LDS);

@@ -265,7 +265,7 @@ int stream_blocks_per_wave(int64_t k, int split_k) {
 template <int NB>
 static hipError_t stream_launch_w8a8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
   auto kern = gmm_w8a8_stream_kernel<NB>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)ST_LDS);
@@ -727,7 +727,7 @@ size_t stream_a16w8_tile_bytes() { return (size_t)SA_TILE_WORDS * 8; }
 template <bool BF16, int NB>
 static hipError_t stream_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
   auto kern = gmm_a16w8_stream_kernel<BF16, NB>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)SA_LDS);

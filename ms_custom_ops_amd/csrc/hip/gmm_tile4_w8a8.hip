@@ -682,7 +682,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
 template <int MODE, bool PK>
 static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t stream) {
   auto kern = gmm_w8a8_tile4_nk_kernel<MODE, PK>;
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, T4_LDS_BYTES);
