@@ -7,6 +7,7 @@
  *   ----------------------------------------------------------------------------  -----------------------------
  *   internal_v2::CreateMoeInitRoutingOp(inputs, outputs, MoeInitRoutingParam)      msco_moe_init_routing_v2
  *     ops/c_api/moe_init_routing_v2/moe_init_routing_v2.cc:132-147,179-182           (+ _workspace_bytes)
+ *   (none: fusion of the routing step with the activation quantisation)            msco_moe_init_routing_v2_quant
  *   internal_v2::CreateMoeTokenUnpermuteOp(inputs, outputs)                        msco_moe_token_unpermute
  *     ops/c_api/moe_token_unpermute/moe_token_unpermute.cc:93-99,118-121
  *
@@ -45,6 +46,22 @@ MSCO_API int msco_moe_init_routing_v2(const void *x, const int32_t *expert_idx, 
                                       int32_t *expert_tokens_before_capacity, void *workspace, size_t workspace_bytes,
                                       int64_t num_rows, int64_t hidden, int64_t k, int64_t expert_num,
                                       int32_t elem_bytes, int32_t count_or_cumsum_flag, void *stream);
+
+/* The same routing with the activations quantised on the way: what an int8 grouped matmul behind the routing step
+ * consumes.  No operator of the reference does this in one step; the arithmetic is the per-token dynamic quantisation
+ * that the reference's test applies to the activations in front of its int8-activation grouped matmul
+ * (dyn_quant, tests/st/test_grouped_matmul_w4.py:83-89), row by row, with t = sorted[j] / k:
+ *   expanded_scale[j] = float32(max_h |x[t, h]|) / 127
+ *   expanded_x[j, h]  = int8(rint(float32(x[t, h]) / expanded_scale[j]))          (rint: half to even, as np.round)
+ * x [num_rows, hidden] in x_dtype (MSCO_DT_F16 or MSCO_DT_BF16), hidden a multiple of 8; expanded_x int8 [n, hidden];
+ * expanded_scale float32 [n] (the grouped matmul's per_token_scale).  A row of zeros gets scale 0 and zeros (the
+ * golden divides 0 by 0 there).  Everything else as in msco_moe_init_routing_v2, same workspace. */
+MSCO_API int msco_moe_init_routing_v2_quant(const void *x, const int32_t *expert_idx, int8_t *expanded_x,
+                                            float *expanded_scale, int32_t *expanded_row_idx,
+                                            int32_t *expert_tokens_count_or_cumsum, int32_t *expert_tokens_before_capacity,
+                                            void *workspace, size_t workspace_bytes, int64_t num_rows, int64_t hidden,
+                                            int64_t k, int64_t expert_num, int32_t x_dtype, int32_t count_or_cumsum_flag,
+                                            void *stream);
 
 /* Weighted un-permutation: out[i, :] = sum_k probs[i, k] * permuted_tokens[sorted_indices[i * top_k + k], :],
  * accumulated in the element type exactly as the golden does (tests/st/test_custom_moe_token_unpermute.py:37-47:

@@ -32,7 +32,8 @@ WL_ROW_MAJOR, WL_PACKED = 0, 1
 EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco_gmm_plan_info", "msco_gmm_destroy",
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
                     "msco_packed_weight_bytes", "msco_pack_weight",
-                    "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_token_unpermute")
+                    "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_init_routing_v2_quant",
+                    "msco_moe_token_unpermute")
 
 
 class GmmDesc(ctypes.Structure):
@@ -88,6 +89,9 @@ def load():
         lib.msco_moe_init_routing_v2.restype = ctypes.c_int
         lib.msco_moe_init_routing_v2.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_size_t] + [ctypes.c_int64] * 4 + \
                                                 [ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_moe_init_routing_v2_quant.restype = ctypes.c_int
+        lib.msco_moe_init_routing_v2_quant.argtypes = [ctypes.c_void_p] * 8 + [ctypes.c_size_t] + [ctypes.c_int64] * 4 + \
+            [ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
         lib.msco_moe_token_unpermute.restype = ctypes.c_int
         lib.msco_moe_token_unpermute.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int64] * 3 + [ctypes.c_int32, ctypes.c_void_p]
         _lib = lib
@@ -133,6 +137,17 @@ def moe_init_routing_v2(x: int, expert_idx: int, expanded_x: int, expanded_row_i
     _check("msco_moe_init_routing_v2", load().msco_moe_init_routing_v2(
         vp(x), vp(expert_idx), vp(expanded_x), vp(expanded_row_idx), vp(tokens), vp(before_capacity), vp(workspace),
         workspace_bytes, num_rows, hidden, k, expert_num, elem_bytes, flag, vp(stream)))
+
+
+def moe_init_routing_v2_quant(x: int, expert_idx: int, expanded_x: int, expanded_scale: int, expanded_row_idx: int,
+                              tokens: Optional[int], before_capacity: Optional[int], workspace: int, workspace_bytes: int,
+                              num_rows: int, hidden: int, k: int, expert_num: int, x_dtype: int, flag: int,
+                              stream: Optional[int] = None):
+    """Raw-pointer call of msco_moe_init_routing_v2_quant (see include/msco_moe.h)."""
+    vp = lambda v: ctypes.c_void_p(v if v else None)
+    _check("msco_moe_init_routing_v2_quant", load().msco_moe_init_routing_v2_quant(
+        vp(x), vp(expert_idx), vp(expanded_x), vp(expanded_scale), vp(expanded_row_idx), vp(tokens), vp(before_capacity),
+        vp(workspace), workspace_bytes, num_rows, hidden, k, expert_num, x_dtype, flag, vp(stream)))
 
 
 def moe_token_unpermute(permuted: int, sorted_indices: int, probs: int, out: int, num_tokens: int, top_k: int, hidden: int,

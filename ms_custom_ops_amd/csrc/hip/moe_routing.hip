@@ -197,6 +197,66 @@ __global__ void __launch_bounds__(256) route_gather_kernel(const unsigned char *
   for (long long v = threadIdx.x; v < row_bytes / 16; v += 256) dst[v] = src[v];   // kept cacheable: the matmul reads it next
 }
 
+// The gather with per-row dynamic int8 quantisation on the way (tests/st/test_grouped_matmul_w4.py:83-89):
+//   scale = float32(max |x[t, :]|) / 127,   q[h] = int8(rint(float32(x[t, h]) / scale))
+// One workgroup per output row, 16 bytes (8 elements) per lane and step.  Up to four steps a lane keeps its elements
+// in registers between the maximum and the division; longer rows are read again (they are L2 hits).  |x| is ordered
+// like its bit pattern without the sign, so the maximum is taken on 15-bit integers and converted once.
+template <bool BF16>
+__global__ void __launch_bounds__(256) route_gather_quant_kernel(const unsigned short *x, const int *sorted_src, signed char *expanded_x,
+                                                                 float *expanded_scale, long long hidden, int k) {
+  __shared__ unsigned wave_max[4];
+  const long long j = blockIdx.x;
+  const long long token = sorted_src[j] / k;
+  const uint4 *src = reinterpret_cast<const uint4 *>(x + token * hidden);
+  uint2 *dst = reinterpret_cast<uint2 *>(expanded_x + j * hidden);
+  const long long vecs = hidden / 8;
+  constexpr int KEEP = 4;
+  uint4 kept[KEEP];
+  unsigned mx = 0;
+  auto fold = [&](const uint4 &v) {
+    const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      mx = max(mx, w[i] & 0x7FFFu);
+      mx = max(mx, (w[i] >> 16) & 0x7FFFu);
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < KEEP; ++u) {
+    const long long v = threadIdx.x + u * 256;
+    kept[u] = v < vecs ? src[v] : make_uint4(0, 0, 0, 0);
+    fold(kept[u]);
+  }
+  for (long long v = threadIdx.x + KEEP * 256; v < vecs; v += 256) fold(src[v]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = max(mx, (unsigned)__shfl_xor((int)mx, o));
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
+  auto widen = [](unsigned short b) { return BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); };
+  const float scale = widen((unsigned short)mx) / 127.0f;
+  if (threadIdx.x == 0) expanded_scale[j] = scale;
+  auto quantise = [&](const uint4 &v) {
+    const unsigned w[4] = {v.x, v.y, v.z, v.w};
+    unsigned q[2] = {0, 0};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // (a row of zeros has scale 0: the golden divides 0 by 0 there; it gets zeros)
+      const int lo = mx == 0 ? 0 : (int)rintf(widen((unsigned short)(w[i] & 0xFFFFu)) / scale);
+      const int hi = mx == 0 ? 0 : (int)rintf(widen((unsigned short)(w[i] >> 16)) / scale);
+      q[i >> 1] |= ((unsigned)(lo & 0xFF) | ((unsigned)(hi & 0xFF) << 8)) << (16 * (i & 1));
+    }
+    return make_uint2(q[0], q[1]);
+  };
+#pragma unroll
+  for (int u = 0; u < KEEP; ++u) {
+    const long long v = threadIdx.x + u * 256;
+    if (v < vecs) dst[v] = quantise(kept[u]);
+  }
+  for (long long v = threadIdx.x + KEEP * 256; v < vecs; v += 256) dst[v] = quantise(src[v]);
+}
+
 // float32 -> element type with round to nearest even, and back
 template <bool BF16>
 __device__ __forceinline__ unsigned short to_elem(float f) {
@@ -309,13 +369,17 @@ size_t msco_moe_init_routing_v2_workspace_bytes(int64_t num_rows, int64_t k, int
   return (size_t)(msco::route_blocks(n) * expert_num + n) * sizeof(int32_t);
 }
 
-int msco_moe_init_routing_v2(const void *x, const int32_t *expert_idx, void *expanded_x, int32_t *expanded_row_idx,
-                             int32_t *expert_tokens_count_or_cumsum, int32_t *expert_tokens_before_capacity,
-                             void *workspace, size_t workspace_bytes, int64_t num_rows, int64_t hidden, int64_t k,
-                             int64_t expert_num, int32_t elem_bytes, int32_t count_or_cumsum_flag, void *stream) {
+// quant_dtype: MSCO_DT_NONE copies rows of elem_bytes-wide elements; MSCO_DT_F16 / MSCO_DT_BF16 quantises rows of that
+// type to int8 and writes their scales
+static int route_and_gather(const void *x, const int32_t *expert_idx, void *expanded_x, float *expanded_scale,
+                            int32_t *expanded_row_idx, int32_t *expert_tokens_count_or_cumsum,
+                            int32_t *expert_tokens_before_capacity, void *workspace, size_t workspace_bytes, int64_t num_rows,
+                            int64_t hidden, int64_t k, int64_t expert_num, int32_t elem_bytes, int32_t quant_dtype,
+                            int32_t count_or_cumsum_flag, void *stream) {
   using namespace msco;
   if (num_rows < 0 || hidden <= 0 || k <= 0 || expert_num <= 0 || expert_num > kMaxExperts) return MSCO_ERR_SHAPE;
   if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) return MSCO_ERR_UNSUPPORTED;
+  if (quant_dtype != MSCO_DT_NONE && quant_dtype != MSCO_DT_F16 && quant_dtype != MSCO_DT_BF16) return MSCO_ERR_UNSUPPORTED;
   if ((hidden * elem_bytes) % 16 != 0) return MSCO_ERR_SHAPE;
   if (count_or_cumsum_flag < 0 || count_or_cumsum_flag > 2) return MSCO_ERR_INVALID_ARG;
   const long long n = num_rows * k;
@@ -327,6 +391,7 @@ int msco_moe_init_routing_v2(const void *x, const int32_t *expert_idx, void *exp
     return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
   }
   if (x == nullptr || expert_idx == nullptr || expanded_x == nullptr || expanded_row_idx == nullptr) return MSCO_ERR_INVALID_ARG;
+  if (quant_dtype != MSCO_DT_NONE && expanded_scale == nullptr) return MSCO_ERR_INVALID_ARG;
   if (count_or_cumsum_flag != 0 && expert_tokens_count_or_cumsum == nullptr) return MSCO_ERR_INVALID_ARG;
   if (workspace == nullptr || workspace_bytes < msco_moe_init_routing_v2_workspace_bytes(num_rows, k, expert_num))
     return MSCO_ERR_WORKSPACE;
@@ -344,9 +409,37 @@ int msco_moe_init_routing_v2(const void *x, const int32_t *expert_idx, void *exp
     hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(1024), (size_t)16 * expert_num * sizeof(int), s, expert_idx,
                        block_hist, expanded_row_idx, sorted_src, n, (int)expert_num);
   }
-  hipLaunchKernelGGL(route_gather_kernel, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned char *>(x), sorted_src,
-                     static_cast<unsigned char *>(expanded_x), (long long)hidden * elem_bytes, (int)k);
+  if (quant_dtype == MSCO_DT_NONE) {
+    hipLaunchKernelGGL(route_gather_kernel, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned char *>(x), sorted_src,
+                       static_cast<unsigned char *>(expanded_x), (long long)hidden * elem_bytes, (int)k);
+  } else if (quant_dtype == MSCO_DT_BF16) {
+    hipLaunchKernelGGL(route_gather_quant_kernel<true>, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned short *>(x),
+                       sorted_src, static_cast<signed char *>(expanded_x), expanded_scale, (long long)hidden, (int)k);
+  } else {
+    hipLaunchKernelGGL(route_gather_quant_kernel<false>, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned short *>(x),
+                       sorted_src, static_cast<signed char *>(expanded_x), expanded_scale, (long long)hidden, (int)k);
+  }
   return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
+}
+
+int msco_moe_init_routing_v2(const void *x, const int32_t *expert_idx, void *expanded_x, int32_t *expanded_row_idx,
+                             int32_t *expert_tokens_count_or_cumsum, int32_t *expert_tokens_before_capacity,
+                             void *workspace, size_t workspace_bytes, int64_t num_rows, int64_t hidden, int64_t k,
+                             int64_t expert_num, int32_t elem_bytes, int32_t count_or_cumsum_flag, void *stream) {
+  return route_and_gather(x, expert_idx, expanded_x, nullptr, expanded_row_idx, expert_tokens_count_or_cumsum,
+                          expert_tokens_before_capacity, workspace, workspace_bytes, num_rows, hidden, k, expert_num, elem_bytes,
+                          MSCO_DT_NONE, count_or_cumsum_flag, stream);
+}
+
+int msco_moe_init_routing_v2_quant(const void *x, const int32_t *expert_idx, int8_t *expanded_x, float *expanded_scale,
+                                   int32_t *expanded_row_idx, int32_t *expert_tokens_count_or_cumsum,
+                                   int32_t *expert_tokens_before_capacity, void *workspace, size_t workspace_bytes,
+                                   int64_t num_rows, int64_t hidden, int64_t k, int64_t expert_num, int32_t x_dtype,
+                                   int32_t count_or_cumsum_flag, void *stream) {
+  if (x_dtype != MSCO_DT_F16 && x_dtype != MSCO_DT_BF16) return MSCO_ERR_UNSUPPORTED;
+  return route_and_gather(x, expert_idx, expanded_x, expanded_scale, expanded_row_idx, expert_tokens_count_or_cumsum,
+                          expert_tokens_before_capacity, workspace, workspace_bytes, num_rows, hidden, k, expert_num, 2, x_dtype,
+                          count_or_cumsum_flag, stream);
 }
 
 int msco_moe_token_unpermute(const void *permuted_tokens, const int32_t *sorted_indices, const void *probs, void *out,

@@ -6,17 +6,22 @@ Restated from the reference's own goldens (read, not imported -- the test module
                             count / cumulative count :41-57); the op only accepts active_num = 0,
                             expert_capacity = 0, drop_pad_mode = 0 (ops/c_api/moe_init_routing_v2/moe_init_routing_v2.cc:107-109)
   * moe_token_unpermute     tests/st/test_custom_moe_token_unpermute.py:37-47
+  * dyn_quant               tests/st/test_grouped_matmul_w4.py:83-89 (per-row dynamic int8 quantisation of the
+                            activations in front of an int8-activation grouped matmul)
 
 Pins (tests/test_moe_routing.py): the routing restatement against an independent per-entry Python sort, against the
 permutation / gather invariants and against hand-written tiny cases; the un-permutation against scalar loops that
-round with an independent float16 / bfloat16 implementation (torch), against the K = 1 gather and the all-ones cases.
+round with an independent float16 / bfloat16 implementation (torch), against the K = 1 gather and the all-ones cases;
+dyn_quant against a per-element loop in Python floats with exact rational tie handling, and against what the
+formula fixes (the row maximum maps to +-127, scale * 127 gives the maximum back, |x - q * scale| <= scale / 2).
 No function here is "parity unpinned".
 """
 from __future__ import annotations
 
 import numpy as np
 
-__all__ = ["moe_init_routing_v2", "moe_init_routing_v2_by_loops", "moe_token_unpermute", "moe_token_unpermute_bf16"]
+__all__ = ["moe_init_routing_v2", "moe_init_routing_v2_by_loops", "moe_token_unpermute", "moe_token_unpermute_bf16",
+           "dyn_quant", "bf16_bits_to_f32"]
 
 
 def moe_init_routing_v2(x, expert_idx, expert_num: int, count_or_cumsum_flag: int = 1):
@@ -86,3 +91,24 @@ def moe_token_unpermute_bf16(permuted_bits, sorted_indices, probs_bits):
     for k in range(top_k):
         out = _bf16_round(out + _bf16_round(pr[:, k:k + 1] * pt[rows[:, k], :]))
     return (out.view(np.uint32) >> 16).astype(np.uint16)
+
+
+def bf16_bits_to_f32(bits):
+    """uint16 bfloat16 patterns -> float32 (exact)."""
+    return (np.asarray(bits).astype(np.uint32) << 16).view(np.float32)
+
+
+def dyn_quant(x):
+    """Per-row dynamic int8 quantisation, test_grouped_matmul_w4.py:83-89:
+        x_max = max |x| over the row (in x's type);  scale = float32(x_max) / 127;  q = int8(round(float32(x) / scale))
+    with numpy's round (half to even) and float32 divisions.  x: float16 array, or float32 array holding values that are
+    exact in the activation type (bfloat16 rows widened with bf16_bits_to_f32).  Returns (q int8 [rows, h], scale
+    float32 [rows]).  A row of zeros divides 0 by 0 in the golden; here it gets scale 0 and zeros."""
+    x = np.asarray(x)
+    x32 = x.astype(np.float32)
+    x_max = np.max(np.abs(x32), axis=-1, keepdims=True)                  # exact: a maximum rounds nothing
+    scale = x_max.astype(np.float32) / np.float32(127.0)
+    safe = np.where(scale == 0, np.float32(1.0), scale)
+    q = np.round(x32 / safe).astype(np.int8)
+    q[np.broadcast_to(scale == 0, q.shape)] = 0
+    return q, scale[..., 0]

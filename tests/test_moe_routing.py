@@ -13,6 +13,69 @@ from oracle import moe_oracle as M
 
 
 # ----------------------------------------------------------------------------------- oracle pins (CPU)
+def _f32_nearest_even(fr):
+    """The float32 nearest to a Fraction (ties to even), by integer arithmetic only."""
+    from fractions import Fraction
+    if fr == 0:
+        return 0.0
+    sign = -1 if fr < 0 else 1
+    fr = abs(fr)
+    e = 0
+    while fr >= 2 ** 24:
+        fr /= 2
+        e += 1
+    while fr < 2 ** 23:
+        fr *= 2
+        e -= 1
+    m = fr.numerator // fr.denominator
+    rest = fr - m
+    if rest > Fraction(1, 2) or (rest == Fraction(1, 2) and m % 2 == 1):
+        m += 1
+    return sign * float(m) * 2.0 ** e                       # exact in a double
+
+
+def _dyn_quant_by_loops(rows):
+    """test_grouped_matmul_w4.py:83-89 element by element: both divisions exactly, rounded to float32 once each; then
+    half-to-even to an integer."""
+    from fractions import Fraction
+    q = np.zeros(rows.shape, dtype=np.int8)
+    scale = np.zeros(rows.shape[0], dtype=np.float32)
+    for r in range(rows.shape[0]):
+        vals = [Fraction(float(v)) for v in rows[r]]
+        s = _f32_nearest_even(max(abs(v) for v in vals) / 127)
+        scale[r] = s
+        for h, v in enumerate(vals):
+            d = Fraction(_f32_nearest_even(v / Fraction(s)))
+            lo = d.numerator // d.denominator                # floor
+            frac = d - lo
+            q[r, h] = lo + (1 if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and lo % 2 == 1) else 0)
+    return q, scale
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_dyn_quant_oracle_against_exact_loops_and_what_the_formula_fixes(kind):
+    rng = np.random.default_rng(11)
+    if kind == "f16":
+        x = rng.uniform(-0.3, 0.3, (6, 40)).astype(np.float16)               # the reference test's distribution (:99)
+        x[1] *= 100
+    else:
+        x = M.bf16_bits_to_f32((rng.standard_normal((6, 40)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16))
+    x[2, 5] = 0
+    x[3] = np.abs(x[3]).max() * np.sign(x[3]) * np.where(np.arange(40) % 2 == 0, 0.5, 1.0)   # ties: half of the maximum -> 63.5
+    q, s = M.dyn_quant(x)
+    q2, s2 = _dyn_quant_by_loops(x.astype(np.float32))
+    assert np.array_equal(s.view(np.uint32), s2.view(np.uint32)) and np.array_equal(q, q2)
+    x32 = x.astype(np.float32)
+    amax = np.abs(x32).max(axis=1)
+    assert np.array_equal(np.abs(q).max(axis=1), np.full(6, 127))            # the row maximum maps to +-127
+    assert np.all(np.sign(q[np.arange(6), np.abs(x32).argmax(axis=1)]) == np.sign(x32[np.arange(6), np.abs(x32).argmax(axis=1)]))
+    assert np.allclose(s * 127, amax, rtol=2e-7)                              # scale * 127 gives the maximum back
+    assert np.all(np.abs(x32.astype(np.float64) - q.astype(np.float64) * s[:, None]) <= s[:, None] * 0.5000001)
+    assert set(np.unique(q[3])) <= {-127, -64, 64, 127}                       # 63.5 goes to the even neighbour
+    qz, sz = M.dyn_quant(np.zeros((2, 8), dtype=np.float16))                  # rows of zeros: scale 0, zeros
+    assert not qz.any() and not sz.any()
+
+
 def test_routing_oracle_tiny_case_by_hand():
     # 3 tokens, k = 2, 3 experts: flat expert ids [2, 0, 1, 2, 0, 0]; stable order of flat positions: 1, 4, 5 | 2 | 0, 3
     x = np.arange(12, dtype=np.float16).reshape(3, 4)
@@ -190,3 +253,58 @@ def test_token_unpermute_bf16_and_round_trip_with_routing():
     probs[:, 0] = 1
     back = _unpermute_gpu(ex.view(np.uint16), ridx, probs.view(np.uint16), cabi.DT_F16)
     assert np.array_equal(back, x.view(np.uint16))
+
+
+def _route_quant_gpu(x_bits, bf16, idx, e, flag):
+    n_rows, h = x_bits.shape
+    k = idx.shape[1]
+    dev = "cuda:0"
+    tx = torch.from_numpy(x_bits.view(np.int16)).to(dev)
+    ti = torch.from_numpy(idx).to(dev)
+    ex = torch.full((n_rows * k, h), 77, dtype=torch.int8, device=dev)
+    sc = torch.full((n_rows * k,), -1.0, dtype=torch.float32, device=dev)
+    ridx = torch.full((n_rows * k,), -5, dtype=torch.int32, device=dev)
+    tok = torch.full((e,), -5, dtype=torch.int32, device=dev)
+    wsb = cabi.moe_init_routing_v2_workspace_bytes(n_rows, k, e)
+    ws = torch.empty(max(wsb, 1), dtype=torch.uint8, device=dev)
+    for _ in range(2):
+        cabi.moe_init_routing_v2_quant(tx.data_ptr(), ti.data_ptr(), ex.data_ptr(), sc.data_ptr(), ridx.data_ptr(), tok.data_ptr(),
+                                       None, ws.data_ptr(), wsb, n_rows, h, k, e, cabi.DT_BF16 if bf16 else cabi.DT_F16, flag,
+                                       torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return ex.cpu().numpy(), sc.cpu().numpy(), ridx.cpu().numpy(), tok.cpu().numpy()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_rows,h,k,e,bf16", [(1, 8, 1, 1, False), (37, 1024, 2, 8, False), (300, 4096, 2, 8, True),
+                                              (64, 7168, 6, 64, False), (20, 10240, 3, 4, True), (9, 8200, 2, 3, False)])
+def test_routing_with_dynamic_quantisation_is_bit_exact(n_rows, h, k, e, bf16):
+    # the routing golden followed by the activation quantisation of the reference's int8-activation test
+    # (tests/st/test_grouped_matmul_w4.py:83-89,99), row by row; int8 rows and float32 scales bit for bit
+    rng = np.random.default_rng(n_rows + h)
+    x32 = rng.uniform(-0.3, 0.3, (n_rows, h)).astype(np.float32)
+    x32[::7] *= 37.0
+    if n_rows > 5:
+        x32[3] = 0.0                                                               # a row of zeros
+        x32[4, 1:] = 0.0                                                           # a single non-zero element
+    if bf16:
+        bits = (x32.view(np.uint32) >> 16).astype(np.uint16)
+        vals = M.bf16_bits_to_f32(bits)
+    else:
+        vals = x32.astype(np.float16)
+        bits = vals.view(np.uint16)
+    idx = rng.integers(0, e, (n_rows, k)).astype(np.int32)
+    ex, sc, ridx, tok = _route_quant_gpu(np.ascontiguousarray(bits), bf16, idx, e, 1)
+    ref_rows, ref_idx, ref_tok = M.moe_init_routing_v2(vals, idx, e, 1)
+    ref_q, ref_s = M.dyn_quant(ref_rows)
+    assert np.array_equal(ridx, ref_idx) and np.array_equal(tok, ref_tok)
+    assert np.array_equal(sc.view(np.uint32), ref_s.view(np.uint32))
+    assert np.array_equal(ex, ref_q)
+
+
+@pytest.mark.gpu
+def test_routing_with_dynamic_quantisation_rejects_what_it_cannot_take():
+    with pytest.raises(RuntimeError):                                               # float32 activations
+        cabi.moe_init_routing_v2_quant(1, 1, 1, 1, 1, None, None, 1, 0, 4, 64, 2, 8, cabi.DT_F32, 1)
+    with pytest.raises(RuntimeError):                                               # hidden not a multiple of 8
+        cabi.moe_init_routing_v2_quant(1, 1, 1, 1, 1, None, None, 1, 0, 4, 60, 2, 8, cabi.DT_F16, 1)
