@@ -222,6 +222,16 @@ def moe_neighbours(steps, warmup):
     out.append({"workload": f"moe_init_routing_v2: {rows} tokens x top-{k} of {e} experts, int8 rows of {h}", "launch_us": sec * 1e6,
                 "gbs": byts / sec / 1e9, "hbm_frac": byts / sec / 1e9 / PEAK_HBM_GBS, "bytes_per_launch": byts})
 
+    # the same routing on bfloat16 activations, quantised to int8 per token on the way (what c3's x and per-token scale
+    # come from when the layer's input is not quantised yet)
+    xb = torch.randn((rows, h), dtype=torch.bfloat16, device=dev, generator=g)
+    sc = torch.empty(rows * k, dtype=torch.float32, device=dev)
+    sec = timed(lambda: cabi.moe_init_routing_v2_quant(xb.data_ptr(), idx.data_ptr(), ex.data_ptr(), sc.data_ptr(), ridx.data_ptr(),
+                                                       tok.data_ptr(), None, ws.data_ptr(), wsb, rows, h, k, e, cabi.DT_BF16, 1, st))
+    byts = rows * h * 2 + rows * k * h + rows * k * 4 * 3 + e * 4      # x read once, int8 rows and scales written, indices in and out
+    out.append({"workload": f"moe_init_routing_v2_quant: {rows} tokens x top-{k} of {e} experts, bfloat16 rows of {h} -> int8",
+                "launch_us": sec * 1e6, "gbs": byts / sec / 1e9, "hbm_frac": byts / sec / 1e9 / PEAK_HBM_GBS, "bytes_per_launch": byts})
+
     # un-permutation: 4096 tokens x top-8, float16 rows of 7168 (the reference op's largest supported shape class)
     t, k, h = 4096, 8, 7168
     pt = torch.randn((t * k, h), dtype=torch.float16, device=dev, generator=g)

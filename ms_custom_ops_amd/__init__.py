@@ -19,6 +19,9 @@ and for the two MoE steps on either side of the grouped matmul:
                         expert_tokens_count_or_cumsum_flag, expert_tokens_before_capacity_flag)
     moe_token_unpermute(permuted_tokens, sorted_indices, probs, padded_mode=False, restore_shape=None)
 
+plus one fusion the reference has no operator for: moe_init_routing_quant(x, expert_idx, expert_num, flag), the routing
+step with the per-token int8 quantisation of the activations done on the way.
+
 Tensors are PyTorch-ROCm tensors on the GPU; PyTorch only provides device memory and the current
 stream.  The compiled operator layer (``ms_custom_ops_amd.ms_custom_ops``, pybind11) validates and
 plans, and the HIP backend behind the C ABI (``lib/libmsco_gmm.so``) does the work.  There is no
@@ -44,8 +47,8 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
         "ms_custom_ops_amd: the compiled operator module is missing; run `python ms_custom_ops_amd/build.py` "
         "(needs hipcc for gfx950 and g++). There is no fallback implementation.") from exc
 
-__all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "moe_init_routing_v2", "moe_token_unpermute",
-           "set_context", "get_context", "exec_mode",
+__all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "moe_init_routing_v2", "moe_init_routing_quant",
+           "moe_token_unpermute", "set_context", "get_context", "exec_mode",
            "GRAPH_MODE", "PYNATIVE_MODE", "dtype_to_type_id", "type_id_to_dtype", "plan_cache_stats", "trans_data"]
 
 GRAPH_MODE = 0
@@ -193,6 +196,22 @@ def moe_init_routing_v2(x, expert_idx, active_num, expert_capacity, expert_num, 
         outs = _C.moe_init_routing_v2(_wrap(x), _wrap(expert_idx), int(active_num), int(expert_capacity), int(expert_num),
                                       int(drop_pad_mode), int(expert_tokens_count_or_cumsum_flag),
                                       bool(expert_tokens_before_capacity_flag))
+    return tuple(o.owner for o in outs)
+
+
+def moe_init_routing_quant(x, expert_idx, expert_num, expert_tokens_count_or_cumsum_flag=1):
+    """moe_init_routing_v2's dropless routing with the activations quantised to int8 per token on the way, for an
+    int8-activation grouped matmul behind it.  The reference has no operator for the pair; the arithmetic per gathered row
+    is the dynamic quantisation its test applies to such activations (tests/st/test_grouped_matmul_w4.py:83-89):
+    scale = float32(max |row|) / 127, q = int8(round(float32(row) / scale)).
+    x float16 or bfloat16 [rows, hidden] (hidden a multiple of 8), expert_idx int32 [rows, k].
+    Returns (expanded_x int8 [rows*k, hidden], expanded_scale float32 [rows*k], expanded_row_idx, expert_tokens_count_or_cumsum):
+    x, per_token_scale and (flag 1) group_list of grouped_matmul_v4_cops."""
+    if _mode == GRAPH_MODE:
+        outs = _C._graph_run("moe_init_routing_quant", [_wrap(x), _wrap(expert_idx), int(expert_num),
+                                                        int(expert_tokens_count_or_cumsum_flag)])
+    else:
+        outs = _C.moe_init_routing_quant(_wrap(x), _wrap(expert_idx), int(expert_num), int(expert_tokens_count_or_cumsum_flag))
     return tuple(o.owner for o in outs)
 
 

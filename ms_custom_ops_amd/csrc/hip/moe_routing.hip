@@ -237,15 +237,26 @@ __global__ void __launch_bounds__(256) route_gather_quant_kernel(const unsigned 
   auto widen = [](unsigned short b) { return BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); };
   const float scale = widen((unsigned short)mx) / 127.0f;
   if (threadIdx.x == 0) expanded_scale[j] = scale;
+  // The golden rounds the correctly rounded quotient x / scale to an integer.  A correctly rounded division costs a
+  // dozen instructions per element; x * (1 / scale) is within 2^-22 * 128 of that quotient, so unless it lands within
+  // 1e-4 of a half-integer (then the division is done properly) both round to the same integer.
+  const float inv = 1.0f / scale;
+  auto to_int = [&](float f) {
+    const float r = f * inv;
+    const float n = rintf(r);
+    if (fabsf(r - n) > 0.4999f) return (int)rintf(f / scale);
+    return (int)n;
+  };
   auto quantise = [&](const uint4 &v) {
     const unsigned w[4] = {v.x, v.y, v.z, v.w};
     unsigned q[2] = {0, 0};
+    if (mx != 0) {   // (a row of zeros has scale 0: the golden divides 0 by 0 there; it gets zeros)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      // (a row of zeros has scale 0: the golden divides 0 by 0 there; it gets zeros)
-      const int lo = mx == 0 ? 0 : (int)rintf(widen((unsigned short)(w[i] & 0xFFFFu)) / scale);
-      const int hi = mx == 0 ? 0 : (int)rintf(widen((unsigned short)(w[i] >> 16)) / scale);
-      q[i >> 1] |= ((unsigned)(lo & 0xFF) | ((unsigned)(hi & 0xFF) << 8)) << (16 * (i & 1));
+      for (int i = 0; i < 4; ++i) {
+        const int lo = to_int(widen((unsigned short)(w[i] & 0xFFFFu)));
+        const int hi = to_int(widen((unsigned short)(w[i] >> 16)));
+        q[i >> 1] |= ((unsigned)(lo & 0xFF) | ((unsigned)(hi & 0xFF) << 8)) << (16 * (i & 1));
+      }
     }
     return make_uint2(q[0], q[1]);
   };

@@ -80,3 +80,43 @@ def test_moe_token_unpermute_unsupported_arguments(device, exec_mode):
             ms_custom_ops.moe_token_unpermute(*make(7168), padded_mode=True)
         with pytest.raises(RuntimeError, match="padded_mode"):
             ms_custom_ops.moe_token_unpermute(*make(7168), restore_shape=(16, 7168))
+
+
+@pytest.mark.parametrize("exec_mode", MODES)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_moe_init_routing_quant_feeds_the_grouped_matmul(device, exec_mode, dtype):
+    # routing + per-token int8 quantisation in one step, then the int8 grouped matmul on its three outputs: every
+    # stage bit for bit what the goldens give (routing: test_custom_moe_init_routing_v2.py:38-65; quantisation:
+    # test_grouped_matmul_w4.py:83-89; matmul: test_grouped_matmul_v4_cops.py:297-301)
+    from oracle import gmm_oracle as O
+    rows, hidden, k, e, n = 96, 1024, 2, 8, 256
+    rng = np.random.default_rng(5)
+    xt = torch.from_numpy(rng.uniform(-0.3, 0.3, (rows, hidden)).astype(np.float32)).to(dtype)
+    vals = xt.to(torch.float32).numpy() if dtype == torch.bfloat16 else xt.numpy()
+    idx = rng.integers(0, e, (rows, k)).astype(np.int32)
+    with ms_custom_ops.exec_mode(exec_mode):
+        q, scale, ridx, cum = ms_custom_ops.moe_init_routing_quant(xt.cuda(), _t(idx), e, 1)
+    ref_rows, ref_idx, ref_cum = M.moe_init_routing_v2(vals, idx, e, 1)
+    ref_q, ref_s = M.dyn_quant(ref_rows)
+    assert q.dtype == torch.int8 and q.shape == (rows * k, hidden) and scale.dtype == torch.float32 and scale.shape == (rows * k,)
+    assert np.array_equal(q.cpu().numpy(), ref_q) and np.array_equal(scale.cpu().numpy().view(np.uint32), ref_s.view(np.uint32))
+    assert np.array_equal(ridx.cpu().numpy(), ref_idx) and np.array_equal(cum.cpu().numpy(), ref_cum)
+    w = rng.integers(-127, 128, (e, hidden, n)).astype(np.int8)
+    ws = rng.uniform(1e-3, 1e-2, (e, n)).astype(np.float32)
+    with ms_custom_ops.exec_mode(exec_mode):
+        out = ms_custom_ops.grouped_matmul_v4_cops([q], [_t(w)], None, [_t(ws)], None, None, None, [scale], cum.to(torch.int64),
+                                                   None, None, None, split_item=3, group_type=0, group_list_type=0)[0]
+    ref = O.grouped_matmul_w8a8(ref_q, w, ref_cum.astype(np.int64), None, ws, ref_s, out_dtype="f16")
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+
+
+def test_moe_init_routing_quant_rejects_bad_arguments(device):
+    idx = torch.zeros(4, 2, dtype=torch.int32, device="cuda")
+    with pytest.raises(TypeError, match="Float16 or BFloat16"):
+        ms_custom_ops.moe_init_routing_quant(torch.zeros(4, 64, dtype=torch.float32, device="cuda"), idx, 8)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        ms_custom_ops.moe_init_routing_quant(torch.zeros(4, 60, dtype=torch.float16, device="cuda"), idx, 8)
+    with pytest.raises(ValueError, match="expert_num must be in"):
+        ms_custom_ops.moe_init_routing_quant(torch.zeros(4, 64, dtype=torch.float16, device="cuda"), idx, 0)
+    with pytest.raises(ValueError, match="same number of rows"):
+        ms_custom_ops.moe_init_routing_quant(torch.zeros(5, 64, dtype=torch.float16, device="cuda"), idx, 8)

@@ -287,6 +287,7 @@ def test_routing_with_dynamic_quantisation_is_bit_exact(n_rows, h, k, e, bf16):
     if n_rows > 5:
         x32[3] = 0.0                                                               # a row of zeros
         x32[4, 1:] = 0.0                                                           # a single non-zero element
+        x32[5] = np.where(np.arange(h) % 3 == 0, 2.0, np.where(np.arange(h) % 3 == 1, -1.0, 0.0078125))   # 63.5: exact ties
     if bf16:
         bits = (x32.view(np.uint32) >> 16).astype(np.uint16)
         vals = M.bf16_bits_to_f32(bits)
