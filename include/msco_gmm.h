@@ -148,6 +148,20 @@ MSCO_API int msco_gmm_destroy(msco_gmm_handle h);
 MSCO_API int msco_transpose_2d(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols,
                                int32_t elem_bytes, void *stream);
 
+/* Grouped A8W4 matmul -- the counterpart of internal_v2::CreateGroupedMatmulW4Op behind grouped_matmul_w4
+ * (ops/c_api/grouped_matmul_w4/grouped_matmul_w4.cc:50-88,186,218; golden tests/st/test_grouped_matmul_w4.py:100-113):
+ *   out[m, n] = x_scale[m] * sum_g weight_scale[e, g, n] * sum_{k in K group g} x[m, k] * w[e, n, k],   e = group of row m
+ * x int8 [m, k]; weight [e, n, k / 2] bytes, two signed 4-bit values per byte, k even in the low nibble
+ * (i8toi4, test_grouped_matmul_w4.py:115-118); group_list int32 [e] cumulative row ends; x_scale float32 [m];
+ * weight_scale float32 [e, k / group_size, n]; out float16 [m, n] (rows at or past group_list[e - 1] are not
+ * written).  k a multiple of 32 and of group_size, group_size a multiple of 32, k <= 8192.  The reference op also takes
+ * a float32 bias [e, n] that must hold 8 * sum_k dequantised w[e, k, n] (test :103-106): its kernel multiplies the
+ * nibbles unsigned and needs the term to compensate; this one multiplies them signed, so the argument does not exist
+ * here and the op layer above does not read it.  Nothing is allocated, everything is enqueued on the given stream. */
+MSCO_API int msco_gmm_a8w4(const int8_t *x, const void *weight, const int32_t *group_list, const float *x_scale,
+                           const float *weight_scale, void *out, int64_t m, int64_t k, int64_t n, int64_t e,
+                           int64_t group_size, void *stream);
+
 /* Weight prepack, once at load time -- the counterpart of the reference's trans_data ND -> FRACTAL_NZ step
  * (ops/c_api/trans_data/trans_data.cc:203-223, shape contract ops/c_api/trans_data/trans_data.md:45-99).
  * src is [e,k,n] int8 (or [e,n,k] when src_transposed); dst receives e * msco_packed_weight_bytes(k, n) bytes in the

@@ -31,7 +31,7 @@ WL_ROW_MAJOR, WL_PACKED = 0, 1
 
 EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco_gmm_plan_info", "msco_gmm_destroy",
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
-                    "msco_packed_weight_bytes", "msco_pack_weight",
+                    "msco_packed_weight_bytes", "msco_pack_weight", "msco_gmm_a8w4",
                     "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_init_routing_v2_quant",
                     "msco_moe_token_unpermute")
 
@@ -89,6 +89,8 @@ def load():
         lib.msco_moe_init_routing_v2.restype = ctypes.c_int
         lib.msco_moe_init_routing_v2.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_size_t] + [ctypes.c_int64] * 4 + \
                                                 [ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_gmm_a8w4.restype = ctypes.c_int
+        lib.msco_gmm_a8w4.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int64] * 5 + [ctypes.c_void_p]
         lib.msco_moe_init_routing_v2_quant.restype = ctypes.c_int
         lib.msco_moe_init_routing_v2_quant.argtypes = [ctypes.c_void_p] * 8 + [ctypes.c_size_t] + [ctypes.c_int64] * 4 + \
             [ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
@@ -123,6 +125,14 @@ def pack_weight(src: int, dst: int, e: int, k: int, n: int, src_transposed: bool
     layout that GmmOp(weight_layout=WL_PACKED) reads."""
     _check("msco_pack_weight", load().msco_pack_weight(ctypes.c_void_p(src), ctypes.c_void_p(dst), e, k, n,
                                                        int(bool(src_transposed)), ctypes.c_void_p(stream if stream else None)))
+
+
+def gmm_a8w4(x: int, weight: int, group_list: int, x_scale: int, weight_scale: int, out: int, m: int, k: int, n: int, e: int,
+             group_size: int, stream: Optional[int] = None):
+    """Raw-pointer call of msco_gmm_a8w4 (see include/msco_gmm.h)."""
+    vp = lambda v: ctypes.c_void_p(v if v else None)
+    _check("msco_gmm_a8w4", load().msco_gmm_a8w4(vp(x), vp(weight), vp(group_list), vp(x_scale), vp(weight_scale), vp(out),
+                                                 m, k, n, e, group_size, vp(stream)))
 
 
 def moe_init_routing_v2_workspace_bytes(num_rows: int, k: int, expert_num: int) -> int:

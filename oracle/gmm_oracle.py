@@ -17,6 +17,7 @@ its own system tests (the device kernels themselves are closed binaries):
 * dense goldens               tests/st/test_quant_batch_matmul.py:71-80,136-151,168-184,201-212
 * int64 dense scale format    tests/st/test_quant_batch_matmul.py:34-42  (trans_quant_param)
 * count-based comparator      tests/st/st_utils.py:23-49             (custom_compare)
+* A8W4 golden and nibble pack tests/st/test_grouped_matmul_w4.py:91-97,100-118
 
 How each function is pinned (tests/test_oracle_pins.py):
 
@@ -38,12 +39,17 @@ How each function is pinned (tests/test_oracle_pins.py):
 * ``a16w8_*``              float64 evaluation of x @ ((w + o) * s) on the exact
                            bf16 operand values; closed forms with constant scale.
 * ``decode_scale_int64``   round trip against the two wire formats above.
+* ``pack_int4`` / ``unpack_int4``   per-element loops, hand-written bytes, round trip.
+* ``golden_grouped_a8w4``  a float64 evaluation of the integer form
+                           x_scale * sum_g scale_g * (exact int32 sum over the K group), a brute-force loop on a tiny
+                           case, and the closed forms that constant scales give.
 """
 from __future__ import annotations
 
 import numpy as np
 
 __all__ = [
+    "pack_int4", "unpack_int4", "quant_int4_groups", "golden_grouped_a8w4", "grouped_a8w4_f64",
     "f32_to_bf16_bits", "bf16_bits_to_f32", "f32_to_f16", "int32_matmul_exact", "int32_matmul_bruteforce",
     "group_bounds", "grouped_int32_acc", "dequant_epilogue", "grouped_matmul_w8a8", "golden_np_qbmm",
     "golden_grouped_w8a8", "golden_v4_pertoken", "golden_v4_perchannel_bias", "golden_v4_a16w8",
@@ -404,3 +410,71 @@ def pack_weights(w):
     wp[:, :k, :n] = w
     # k = 64 b + 16 q + i, n = 16 a + c  ->  [e, a, b, q, c, i]
     return np.ascontiguousarray(wp.reshape(e, kb, 4, 16, ng, 16).transpose(0, 4, 1, 2, 5, 3)).reshape(e, -1)
+
+
+# ------------------------------------------------------------------------------------------ A8W4
+def pack_int4(w):
+    """int8 values in [-8, 7], last axis of even length -> bytes, two per byte, even index in the low nibble
+    (i8toi4, tests/st/test_grouped_matmul_w4.py:115-118)."""
+    u = ((np.asarray(w).astype(np.int16) + 16) % 16).astype(np.uint8)
+    return (u[..., 1::2] << 4) | u[..., ::2]
+
+
+def unpack_int4(packed):
+    """Inverse of pack_int4: bytes [..., k/2] -> int8 [..., k] in [-8, 7]."""
+    p = np.asarray(packed).astype(np.uint8)
+    out = np.empty(p.shape[:-1] + (p.shape[-1] * 2,), dtype=np.int8)
+    lo, hi = (p & 0x0F).astype(np.int8), (p >> 4).astype(np.int8)
+    out[..., ::2] = np.where(lo >= 8, lo - 16, lo)
+    out[..., 1::2] = np.where(hi >= 8, hi - 16, hi)
+    return out
+
+
+def quant_int4_groups(w_fp, group):
+    """The reference test's weight quantiser (quant, test_grouped_matmul_w4.py:91-97): float weights [e, k, n] -> int8
+    values in [-7, 7] [e, k, n] and float32 scales [e, k / group, 1, n] (max |w| over the K group / 7)."""
+    e, k, n = w_fp.shape
+    y = np.asarray(w_fp).reshape(e, k // group, group, n)
+    y_max = np.max(np.abs(y), keepdims=True, axis=-2)
+    scale = y_max.astype(np.float32) / 7.0
+    q = np.round(y.astype(np.float32) / scale).astype(np.int8).reshape(e, k, n)
+    return q, scale
+
+
+def golden_grouped_a8w4(x, w_packed, group_list, x_scale, w_scale, group):
+    """tests/st/test_grouped_matmul_w4.py:103-113 with the weights taken as the op gets them ([e, n, k/2] nibbles):
+    w_deq = int4 * scale per K group (float32); per expert matmul(x as float16, w_deq) * x_scale rows; float32 result
+    (the test compares the op's float16 output against it with custom_compare, limit 0.004)."""
+    x = np.asarray(x)
+    w = unpack_int4(w_packed).transpose(0, 2, 1)                        # [e, k, n]
+    e, k, n = w.shape
+    w_deq = (w.reshape(e, k // group, group, n).astype(np.float32) * np.asarray(w_scale, dtype=np.float32).reshape(e, k // group, 1, n))
+    w_deq = w_deq.reshape(e, k, n)
+    gl = [int(v) for v in np.asarray(group_list)]
+    out = np.zeros((x.shape[0], n), dtype=np.float32)
+    start = 0
+    for g in range(e):
+        end = gl[g]
+        if end > start:
+            out[start:end] = np.matmul(x[start:end].astype(np.float16), w_deq[g]) * np.asarray(x_scale, dtype=np.float32)[start:end, None]
+        start = max(start, end)
+    return out
+
+
+def grouped_a8w4_f64(x, w_packed, group_list, x_scale, w_scale, group):
+    """The same quantity from exact integers: x_scale * sum_g scale_g * (int sum over K group g), in float64."""
+    x = np.asarray(x).astype(np.int64)
+    w = unpack_int4(w_packed).transpose(0, 2, 1).astype(np.int64)
+    e, k, n = w.shape
+    sc = np.asarray(w_scale, dtype=np.float64).reshape(e, k // group, n)
+    gl = [int(v) for v in np.asarray(group_list)]
+    out = np.zeros((x.shape[0], n), dtype=np.float64)
+    start = 0
+    for g in range(e):
+        end = gl[g]
+        for kg in range(k // group):
+            if end > start:
+                part = x[start:end, kg * group:(kg + 1) * group] @ w[g, kg * group:(kg + 1) * group]
+                out[start:end] += part.astype(np.float64) * sc[g, kg][None, :]
+        start = max(start, end)
+    return out * np.asarray(x_scale, dtype=np.float64)[:, None]

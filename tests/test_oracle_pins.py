@@ -298,3 +298,44 @@ def test_pack_weights_follows_the_layout_definition_byte_by_byte():
                             kk, nn = 64 * b + 16 * (l // 16) + i, 16 * a + (l % 16)
                             want = w[g, kk, nn] if (kk < k and nn < n) else 0
                             assert blk[16 * l + i] == want
+
+
+# ------------------------------------------------------------------------------------------ A8W4
+def test_int4_packing_by_hand_loops_and_round_trip():
+    # -8 -> 0x8, -1 -> 0xF, 7 -> 0x7; even index in the low nibble (test_grouped_matmul_w4.py:115-118)
+    assert O.pack_int4(np.array([-8, 7, -1, 0, 3, -4], dtype=np.int8)).tolist() == [0x78, 0x0F, 0xC3]
+    rng = np.random.default_rng(0)
+    w = rng.integers(-8, 8, (3, 5, 16)).astype(np.int8)
+    p = O.pack_int4(w)
+    assert p.shape == (3, 5, 8) and p.dtype == np.uint8
+    for idx in np.ndindex(3, 5, 8):
+        lo, hi = int(w[idx[0], idx[1], 2 * idx[2]]), int(w[idx[0], idx[1], 2 * idx[2] + 1])
+        assert int(p[idx]) == ((hi & 0xF) << 4 | (lo & 0xF))
+    assert np.array_equal(O.unpack_int4(p), w)
+
+
+def test_a8w4_golden_against_integer_form_bruteforce_and_closed_forms():
+    rng = np.random.default_rng(1)
+    m, k, n, e, g = 9, 128, 16, 4, 32
+    x = rng.integers(-127, 128, (m, k)).astype(np.int8)
+    wq, ws = O.quant_int4_groups(rng.uniform(-0.3, 0.3, (e, k, n)).astype(np.float16), g)
+    assert np.abs(wq).max() == 7 and ws.shape == (e, k // g, 1, n)
+    wp = O.pack_int4(wq.transpose(0, 2, 1))                                   # [e, n, k/2], as the op takes it
+    xs = rng.uniform(1e-3, 1e-2, m).astype(np.float32)
+    gl = [2, 2, 7, 9]                                                         # one empty group
+    gold = O.golden_grouped_a8w4(x, wp, gl, xs, ws, g)
+    exact = O.grouped_a8w4_f64(x, wp, gl, xs, ws, g)
+    assert np.allclose(gold, exact, rtol=2e-5, atol=1e-7)
+    # brute force, one output at a time
+    grp_of = [0, 0, 2, 2, 2, 2, 2, 3, 3]
+    for (r, c) in [(0, 0), (3, 5), (8, 15)]:
+        acc = 0.0
+        for kk in range(k):
+            acc += float(x[r, kk]) * float(wq[grp_of[r], kk, c]) * float(ws[grp_of[r], kk // g, 0, c])
+        assert abs(acc * float(xs[r]) - exact[r, c]) <= 1e-9 * max(1.0, abs(exact[r, c]))
+    # constant scales: plain integer matmul times the constants; ones: column sums
+    ones = np.ones_like(ws)
+    got = O.golden_grouped_a8w4(x, wp, gl, np.full(m, 2.0, np.float32), ones * 0.5, g)
+    ref = np.concatenate([x[0:2].astype(np.int64) @ wq[0].astype(np.int64), x[2:7].astype(np.int64) @ wq[2].astype(np.int64),
+                          x[7:9].astype(np.int64) @ wq[3].astype(np.int64)])
+    assert np.array_equal(got, ref.astype(np.float32))
