@@ -232,6 +232,23 @@ def moe_neighbours(steps, warmup):
     out.append({"workload": f"moe_init_routing_v2_quant: {rows} tokens x top-{k} of {e} experts, bfloat16 rows of {h} -> int8",
                 "launch_us": sec * 1e6, "gbs": byts / sec / 1e9, "hbm_frac": byts / sec / 1e9 / PEAK_HBM_GBS, "bytes_per_launch": byts})
 
+    # grouped A8W4 at the reference test's shape: 32 rows routed to 256 experts, K = 7168, N = 256, K groups of 256
+    # (tests/st/test_grouped_matmul_w4.py:146-152).  Bytes: the int4 weights and scales of the experts that got rows.
+    m4, k4, n4, e4, g4 = 32, 7168, 256, 256, 256
+    x4 = torch.randint(-127, 128, (m4, k4), dtype=torch.int8, device=dev, generator=g)
+    w4 = torch.randint(0, 256, (e4, n4, k4 // 2), dtype=torch.uint8, device=dev, generator=g)
+    ws4 = torch.rand((e4, k4 // g4, n4), dtype=torch.float32, device=dev, generator=g) * 1e-2
+    xs4 = torch.rand(m4, dtype=torch.float32, device=dev, generator=g) * 1e-2
+    ends = torch.sort(torch.randint(1, m4 + 1, (e4 - 1,), device=dev, generator=g)).values.tolist() + [m4]
+    gl4 = torch.tensor(ends, dtype=torch.int32, device=dev)
+    o4 = torch.empty((m4, n4), dtype=torch.float16, device=dev)
+    sec = timed(lambda: cabi.gmm_a8w4(x4.data_ptr(), w4.data_ptr(), gl4.data_ptr(), xs4.data_ptr(), ws4.data_ptr(), o4.data_ptr(),
+                                      m4, k4, n4, e4, g4, st))
+    hit = len(set(ends))                                               # experts with at least one row
+    byts = hit * (n4 * k4 // 2 + (k4 // g4) * n4 * 4) + m4 * k4 + m4 * n4 * 2 + m4 * 4 + e4 * 4
+    out.append({"workload": f"grouped_matmul_w4: {m4} rows over {e4} experts ({hit} hit), K={k4}, N={n4}, K groups of {g4}",
+                "launch_us": sec * 1e6, "gbs": byts / sec / 1e9, "hbm_frac": byts / sec / 1e9 / PEAK_HBM_GBS, "bytes_per_launch": byts})
+
     # un-permutation: 4096 tokens x top-8, float16 rows of 7168 (the reference op's largest supported shape class)
     t, k, h = 4096, 8, 7168
     pt = torch.randn((t * k, h), dtype=torch.float16, device=dev, generator=g)

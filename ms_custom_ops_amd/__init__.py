@@ -12,6 +12,7 @@ Drop-in for the grouped / dense quantized matmul entries of ms_custom_ops
                            group_list_type=0, act_type=0, weight_format="ND", output_dtype=None)
     quant_batch_matmul(x1, x2, scale, offset=None, bias=None, pertoken_scale=None,
                        transpose_x1=False, transpose_x2=False, x2_format="ND", output_dtype=float16)
+    grouped_matmul_w4(x, weight, group_list, bias, x_scale, weight_scale)
 
 and for the two MoE steps on either side of the grouped matmul:
 
@@ -47,7 +48,7 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
         "ms_custom_ops_amd: the compiled operator module is missing; run `python ms_custom_ops_amd/build.py` "
         "(needs hipcc for gfx950 and g++). There is no fallback implementation.") from exc
 
-__all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "moe_init_routing_v2", "moe_init_routing_quant",
+__all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "grouped_matmul_w4", "quant_batch_matmul", "moe_init_routing_v2", "moe_init_routing_quant",
            "moe_token_unpermute", "set_context", "get_context", "exec_mode",
            "GRAPH_MODE", "PYNATIVE_MODE", "dtype_to_type_id", "type_id_to_dtype", "plan_cache_stats", "trans_data"]
 
@@ -182,6 +183,20 @@ def quant_batch_matmul(x1, x2, scale, offset=None, bias=None, pertoken_scale=Non
         return _C._graph_run("quant_batch_matmul", args)[0].owner
     return _C.quant_batch_matmul(_wrap(x1), _wrap(x2), _wrap(scale), _wrap(offset), _wrap(bias), _wrap(pertoken_scale),
                                  bool(transpose_x1), bool(transpose_x2), str(x2_format), od).owner
+
+
+def grouped_matmul_w4(x, weight, group_list, bias, x_scale, weight_scale):
+    """Grouped matmul of int8 activations with int4 weights (ops/c_api/grouped_matmul_w4/grouped_matmul_w4.cc:254-255;
+    golden tests/st/test_grouped_matmul_w4.py:100-113): out[m] = x_scale[m] * sum over K groups g of
+    weight_scale[e, g] * (x[m, K group g] @ w[e, K group g]) for the expert e of row m, float16 [m, n].
+    x int8 [m, k]; weight [e, n, k/2], two signed 4-bit values per byte (even k in the low nibble), as an int8 or uint8
+    tensor (torch has no 4-bit type); group_list int32 [e], cumulative; bias float32 [e, n] (the reference kernel's
+    compensation term 8 * column sums of the dequantised weight: checked, not read, the nibbles are multiplied signed
+    here); x_scale float32 [m]; weight_scale float32 [e, k/group_size, n]."""
+    args = [_wrap(x), _wrap(weight), _wrap(group_list), _wrap(bias), _wrap(x_scale), _wrap(weight_scale)]
+    if _mode == GRAPH_MODE:
+        return _C._graph_run("grouped_matmul_w4", args)[0].owner
+    return _C.grouped_matmul_w4(*args).owner
 
 
 def moe_init_routing_v2(x, expert_idx, active_num, expert_capacity, expert_num, drop_pad_mode,

@@ -6,10 +6,11 @@
 // (tests/st/test_grouped_matmul_w4.py:100-113; ops/c_api/grouped_matmul_w4/grouped_matmul_w4.cc:50-88.)  The
 // reference's workloads route 5 .. 32 rows to 256 experts: almost every group is empty or holds one row, so this is a
 // batch of matrix-vector products bound by the bytes of the weights of the experts that were hit.  Hence no MFMA:
-//   * one workgroup per (group, 64 columns); a workgroup whose group is empty leaves at once;
+//   * one workgroup per (group, 16 columns); a workgroup whose group is empty leaves at once;
 //   * the group's rows (eight at a time) sit in LDS, de-interleaved into even-k and odd-k bytes so that they line up
 //     with the low and the high nibbles of a weight word;
-//   * a wavefront walks one column at a time, lane L taking the 16-byte pieces L, L + 64, ... of the column (32
+//   * a wavefront owns four columns and requests all their weights at once (one memory round trip; they stay in
+//     registers for every block of rows), lane L holding the 16-byte pieces L, L + 64, ... of a column (32
 //     consecutive k, always inside one K group): nibbles are multiplied as u ^ 8 in [0, 15] with v_dot4_i32_i8 and
 //     8 * sum(x) of the piece is subtracted (u ^ 8 = s + 8 for the signed nibble s); the int32 sum of a piece is
 //     exact, is scaled by its K group's float32 scale and added up in float32; lanes are reduced with shuffles.
@@ -21,8 +22,10 @@ namespace msco {
 namespace {
 
 constexpr int W4_ROWS = 8;           // rows of a group held in LDS at a time
-constexpr int W4_COLS = 64;          // columns per workgroup (16 per wavefront)
+constexpr int W4_WAVE_COLS = 4;      // columns per wavefront, all in registers at once
+constexpr int W4_COLS = 4 * W4_WAVE_COLS;   // columns per workgroup
 constexpr int W4_MAX_K = 8192;
+constexpr int W4_LANE_PIECES = W4_MAX_K / 32 / 64;   // 16-byte pieces of a column per lane
 
 __device__ __forceinline__ int dot4(int a, int b, int c) { return __builtin_amdgcn_sdot4(a, b, c, false); }
 
@@ -40,6 +43,21 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
   const int pieces_per_group = group_size / 32;
   const unsigned char *wg = w + (long long)grp * n * (k / 2);
   const float *sg = w_scale + (long long)grp * k_groups * n;
+  const int col0 = blockIdx.x * W4_COLS + wave * W4_WAVE_COLS;
+
+  // this wavefront's columns: every piece and its scale requested at once (one memory round trip), nibbles as u ^ 8
+  uint4 wv[W4_WAVE_COLS][W4_LANE_PIECES];
+  float sc[W4_WAVE_COLS][W4_LANE_PIECES];
+#pragma unroll
+  for (int c = 0; c < W4_WAVE_COLS; ++c)
+#pragma unroll
+    for (int i = 0; i < W4_LANE_PIECES; ++i) {
+      const int p = lane + 64 * i, col = col0 + c;
+      const bool live = p < pieces && col < n;
+      wv[c][i] = live ? *(reinterpret_cast<const uint4 *>(wg + (long long)col * (k / 2)) + p) : make_uint4(0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u);
+      sc[c][i] = live ? sg[(long long)(p / pieces_per_group) * n + col] : 0.f;
+    }
+
   for (int r0 = g_start; r0 < g_end; r0 += W4_ROWS) {
     const int rows = min(W4_ROWS, g_end - r0);
     __syncthreads();   // the previous block of rows is no longer read
@@ -53,46 +71,41 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
       dst[0] = (int)e0; dst[1] = (int)e1; dst[4] = (int)o0; dst[5] = (int)o1;
     }
     __syncthreads();
-    for (int c = 0; c < W4_COLS / 4; ++c) {
-      const int col = blockIdx.x * W4_COLS + wave * (W4_COLS / 4) + c;
-      if (col >= n) break;   // wave-uniform
-      float acc[W4_ROWS];
+    for (int r = 0; r < rows; ++r) {
+      float acc[W4_WAVE_COLS];
 #pragma unroll
-      for (int r = 0; r < W4_ROWS; ++r) acc[r] = 0.f;
-      const uint4 *wc = reinterpret_cast<const uint4 *>(wg + (long long)col * (k / 2));
-      for (int p = lane; p < pieces; p += 64) {
-        const uint4 wv = *(wc + p);
-        const float s = sg[(long long)(p / pieces_per_group) * n + col];
-        const unsigned t[4] = {wv.x ^ 0x88888888u, wv.y ^ 0x88888888u, wv.z ^ 0x88888888u, wv.w ^ 0x88888888u};
-        int lo[4], hi[4];
+      for (int c = 0; c < W4_WAVE_COLS; ++c) acc[c] = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          lo[i] = (int)(t[i] & 0x0F0F0F0Fu);           // k = 8 i + 0, 2, 4, 6
-          hi[i] = (int)((t[i] >> 4) & 0x0F0F0F0Fu);    // k = 8 i + 1, 3, 5, 7
-        }
+      for (int i = 0; i < W4_LANE_PIECES; ++i) {
+        const int p = lane + 64 * i;
+        if (p < pieces) {
+          const int4 xe = *reinterpret_cast<const int4 *>(xs + (r * pieces + p) * 8);
+          const int4 xo = *reinterpret_cast<const int4 *>(xs + (r * pieces + p) * 8 + 4);
+          int sx = 0;
+          sx = dot4(xe.x, 0x01010101, sx); sx = dot4(xo.x, 0x01010101, sx); sx = dot4(xe.y, 0x01010101, sx);
+          sx = dot4(xo.y, 0x01010101, sx); sx = dot4(xe.z, 0x01010101, sx); sx = dot4(xo.z, 0x01010101, sx);
+          sx = dot4(xe.w, 0x01010101, sx); sx = dot4(xo.w, 0x01010101, sx);
 #pragma unroll
-        for (int r = 0; r < W4_ROWS; ++r) {
-          if (r < rows) {   // wave-uniform
-            const int4 xe = *reinterpret_cast<const int4 *>(xs + (r * pieces + p) * 8);
-            const int4 xo = *reinterpret_cast<const int4 *>(xs + (r * pieces + p) * 8 + 4);
-            int d = 0, sx = 0;
-            d = dot4(xe.x, lo[0], d); d = dot4(xo.x, hi[0], d); d = dot4(xe.y, lo[1], d); d = dot4(xo.y, hi[1], d);
-            d = dot4(xe.z, lo[2], d); d = dot4(xo.z, hi[2], d); d = dot4(xe.w, lo[3], d); d = dot4(xo.w, hi[3], d);
-            sx = dot4(xe.x, 0x01010101, sx); sx = dot4(xo.x, 0x01010101, sx); sx = dot4(xe.y, 0x01010101, sx);
-            sx = dot4(xo.y, 0x01010101, sx); sx = dot4(xe.z, 0x01010101, sx); sx = dot4(xo.z, 0x01010101, sx);
-            sx = dot4(xe.w, 0x01010101, sx); sx = dot4(xo.w, 0x01010101, sx);
-            acc[r] += (float)(d - 8 * sx) * s;
+          for (int c = 0; c < W4_WAVE_COLS; ++c) {
+            const unsigned t[4] = {wv[c][i].x ^ 0x88888888u, wv[c][i].y ^ 0x88888888u, wv[c][i].z ^ 0x88888888u, wv[c][i].w ^ 0x88888888u};
+            const int xev[4] = {xe.x, xe.y, xe.z, xe.w}, xov[4] = {xo.x, xo.y, xo.z, xo.w};
+            int d = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              d = dot4(xev[j], (int)(t[j] & 0x0F0F0F0Fu), d);           // k = 8 j + 0, 2, 4, 6
+              d = dot4(xov[j], (int)((t[j] >> 4) & 0x0F0F0F0Fu), d);    // k = 8 j + 1, 3, 5, 7
+            }
+            acc[c] += (float)(d - 8 * sx) * sc[c][i];
           }
         }
       }
+      const float xsr = x_scale[r0 + r];
 #pragma unroll
-      for (int r = 0; r < W4_ROWS; ++r) {
-        if (r < rows) {
-          float v = acc[r];
+      for (int c = 0; c < W4_WAVE_COLS; ++c) {
+        float v = acc[c];
 #pragma unroll
-          for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-          if (lane == 0) out[(long long)(r0 + r) * n + col] = f32_to_f16_rne(v * x_scale[r0 + r]);
-        }
+        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+        if (lane == 0 && col0 + c < n) out[(long long)(r0 + r) * n + col0 + c] = f32_to_f16_rne(v * xsr);
       }
     }
   }

@@ -78,3 +78,43 @@ def test_a8w4_rejects_bad_shapes():
         cabi.gmm_a8w4(1, 1, 1, 1, 1, 1, 4, 256, 16, 2, 96)        # k not a multiple of the group size
     with pytest.raises(RuntimeError):
         cabi.gmm_a8w4(1, 1, 1, 1, 1, 1, 4, 16384, 16, 2, 256)     # k beyond the supported range
+
+
+# ------------------------------------------------------------------------------- the Python entry, both modes
+@pytest.mark.parametrize("exec_mode", ["graph", "pynative"])
+@pytest.mark.parametrize("batch_size", [5, 17])
+def test_gmm_w4_swft_0(exec_mode, batch_size):
+    # the reference's level-0 case (tests/st/test_grouped_matmul_w4.py:146-158): m in {5, 17}, k = 7168, n = 256, 256 experts,
+    # with the bias the reference op requires (8 * column sums of the dequantised weight, :103-106)
+    import ms_custom_ops_amd as ms_custom_ops
+    e, k, n, g = 256, 7168, 256, 256
+    x, xs, wp, ws, gl = _case(batch_size, batch_size, k, n, e, g)
+    w_deq = (O.unpack_int4(wp).transpose(0, 2, 1).reshape(e, k // g, g, n).astype(np.float32) * ws.reshape(e, k // g, 1, n)).reshape(e, k, n)
+    bias = np.matmul(np.ones((e, 1, k), dtype=np.float16) * 8, w_deq).astype(np.float32).reshape(e, n)
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    mode = ms_custom_ops.GRAPH_MODE if exec_mode == "graph" else ms_custom_ops.PYNATIVE_MODE
+    with ms_custom_ops.exec_mode(mode):
+        out = ms_custom_ops.grouped_matmul_w4(t(x), t(wp.view(np.int8)), t(gl), t(bias), t(xs), t(ws))
+    assert out.dtype == torch.float16 and out.shape == (batch_size, n)
+    expect = O.golden_grouped_a8w4(x, wp, gl, xs, ws, g)
+    assert O.count_compare(out.cpu().numpy().astype(np.float32), expect, 0.004)
+
+
+def test_gmm_w4_rejects_what_the_reference_rejects():
+    import ms_custom_ops_amd as ms_custom_ops
+    z = lambda shape, dt: torch.zeros(shape, dtype=dt, device="cuda")
+    x, w, gl = z((4, 64), torch.int8), z((2, 16, 32), torch.uint8), z((2,), torch.int32)
+    b, xs, ws = z((2, 16), torch.float32), z((4,), torch.float32), z((2, 2, 16), torch.float32)
+    with pytest.raises(RuntimeError, match="input 'x' must be 2D"):
+        ms_custom_ops.grouped_matmul_w4(x[0], w, gl, b, xs, ws)
+    with pytest.raises(RuntimeError, match="must have the same dimension of 'k'"):
+        ms_custom_ops.grouped_matmul_w4(z((4, 96), torch.int8), w, gl, b, xs, ws)
+    with pytest.raises(RuntimeError, match="input 'x' must be int8"):
+        ms_custom_ops.grouped_matmul_w4(z((4, 64), torch.float16), w, gl, b, xs, ws)
+    with pytest.raises(RuntimeError, match="input 'bias' must be float32"):
+        ms_custom_ops.grouped_matmul_w4(x, w, gl, z((2, 16), torch.float16), xs, ws)
+    with pytest.raises(RuntimeError, match="input 'group_list' must be int32"):
+        ms_custom_ops.grouped_matmul_w4(x, w, z((2,), torch.int64), b, xs, ws)
+    with pytest.raises(ValueError, match="weight_scale must be"):
+        ms_custom_ops.grouped_matmul_w4(x, w, gl, b, xs, z((2, 2, 8), torch.float32))
+    assert ms_custom_ops.grouped_matmul_w4(x, w, gl, b, xs, ws).shape == (4, 16)

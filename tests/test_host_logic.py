@@ -181,7 +181,7 @@ def test_quant_batch_matmul_infer():
 
 # ------------------------------------------------------------------------------------- registration surface
 def test_registry_and_module_surface():
-    ops = ("grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "moe_init_routing_v2", "moe_init_routing_quant",
+    ops = ("grouped_matmul", "grouped_matmul_v4_cops", "grouped_matmul_w4", "quant_batch_matmul", "moe_init_routing_v2", "moe_init_routing_quant",
            "moe_token_unpermute")
     assert set(_C._registered_graph_ops()) == set(ops)
     for name in ops:
