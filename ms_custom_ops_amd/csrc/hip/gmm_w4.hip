@@ -6,8 +6,9 @@
 // (tests/st/test_grouped_matmul_w4.py:100-113; ops/c_api/grouped_matmul_w4/grouped_matmul_w4.cc:50-88.)  The
 // reference's workloads route 5 .. 32 rows to 256 experts: almost every group is empty or holds one row, so this is a
 // batch of matrix-vector products bound by the bytes of the weights of the experts that were hit.  Hence no MFMA:
-//   * one workgroup per (group, 16 columns); a workgroup whose group is empty leaves at once;
-//   * the group's rows (eight at a time) sit in LDS, de-interleaved into even-k and odd-k bytes so that they line up
+//   * one workgroup per (group that holds rows, 16 or more columns): the grid has min(E, M) group slots and a workgroup
+//     finds the group of its slot's rank with ballots over group_list; a short K lets several columns share a wavefront's lanes;
+//   * the group's rows (four at a time) sit in LDS, de-interleaved into even-k and odd-k bytes so that they line up
 //     with the low and the high nibbles of a weight word;
 //   * a wavefront owns four columns and requests all their weights at once (one memory round trip; they stay in
 //     registers for every block of rows), lane L holding the 16-byte pieces L, L + 64, ... of a column (32
@@ -21,9 +22,8 @@
 namespace msco {
 namespace {
 
-constexpr int W4_ROWS = 8;           // rows of a group held in LDS at a time
-constexpr int W4_WAVE_COLS = 4;      // columns per wavefront, all in registers at once
-constexpr int W4_COLS = 4 * W4_WAVE_COLS;   // columns per workgroup
+constexpr int W4_ROWS = 4;           // rows of a group held in LDS at a time (k bytes each: small, so that many workgroups fit a CU)
+constexpr int W4_WAVE_COLS = 4;      // columns per lane segment of a wavefront, all in registers at once
 constexpr int W4_MAX_K = 8192;
 constexpr int W4_LANE_PIECES = W4_MAX_K / 32 / 64;   // 16-byte pieces of a column per lane
 
@@ -32,18 +32,45 @@ __device__ __forceinline__ int dot4(int a, int b, int c) { return __builtin_amdg
 __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const unsigned char *w, const int *group_list,
                                                        const float *x_scale, const float *w_scale, unsigned short *out, int m,
                                                        int k, int n, int e, int group_size) {
-  __shared__ __align__(16) int xs[W4_ROWS * W4_MAX_K / 4];   // [row][piece of 32 k]: 4 words of even-k bytes, then 4 of odd-k bytes
-  const int grp = blockIdx.y;
-  const int g_start = grp == 0 ? 0 : min(max(group_list[grp - 1], 0), m);
-  const int g_end = min(max(group_list[grp], g_start), m);
-  if (g_end <= g_start) return;
+  extern __shared__ __align__(16) int xs[];   // min(W4_ROWS, m) rows: [row][piece of 32 k]: 4 words of even-k bytes, then 4 of odd-k bytes
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // blockIdx.y counts the groups that hold rows (at most min(e, m) of them): find the one with that rank, 64 groups
+  // per round of ballots, and leave if there are fewer
+  int grp = -1, g_start = 0, g_end = 0;
+  for (int g0 = 0, seen = 0; g0 < e && grp < 0; g0 += 256) {
+    int lo[4], hi[4];   // four rounds' worth of boundaries requested together: one memory round trip per 256 groups
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int g = g0 + 64 * u + lane;
+      lo[u] = g > 0 && g < e ? min(max(group_list[g - 1], 0), m) : 0;
+      hi[u] = g < e ? min(max(group_list[g], lo[u]), m) : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      unsigned long long holds = __ballot(hi[u] > lo[u]);
+      const int here = __popcll(holds);
+      if (grp < 0 && seen + here > (int)blockIdx.y) {
+        for (int skip = (int)blockIdx.y - seen; skip > 0; --skip) holds &= holds - 1;
+        const int src = __ffsll((long long)holds) - 1;
+        grp = g0 + 64 * u + src;
+        g_start = __shfl(lo[u], src);
+        g_end = __shfl(hi[u], src);
+      }
+      seen += here;
+    }
+  }
+  if (grp < 0) return;
   const int pieces = k / 32;
+  // a short K leaves lanes over: lanes_per_col lanes share a column, the wavefront works on 64 / lanes_per_col columns side by side
+  int lanes_per_col = 64;
+  while (lanes_per_col / 2 >= pieces) lanes_per_col /= 2;
+  const int side = 64 / lanes_per_col;
+  const int pl = lane % lanes_per_col, sub = lane / lanes_per_col;
   const int k_groups = k / group_size;
   const int pieces_per_group = group_size / 32;
   const unsigned char *wg = w + (long long)grp * n * (k / 2);
   const float *sg = w_scale + (long long)grp * k_groups * n;
-  const int col0 = blockIdx.x * W4_COLS + wave * W4_WAVE_COLS;
+  const int col0 = (blockIdx.x * 4 + wave) * W4_WAVE_COLS * side + sub;   // this lane's columns: col0 + c * side
 
   // this wavefront's columns: every piece and its scale requested at once (one memory round trip), nibbles as u ^ 8
   uint4 wv[W4_WAVE_COLS][W4_LANE_PIECES];
@@ -52,7 +79,7 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
   for (int c = 0; c < W4_WAVE_COLS; ++c)
 #pragma unroll
     for (int i = 0; i < W4_LANE_PIECES; ++i) {
-      const int p = lane + 64 * i, col = col0 + c;
+      const int p = pl + lanes_per_col * i, col = col0 + c * side;
       const bool live = p < pieces && col < n;
       wv[c][i] = live ? *(reinterpret_cast<const uint4 *>(wg + (long long)col * (k / 2)) + p) : make_uint4(0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u);
       sc[c][i] = live ? sg[(long long)(p / pieces_per_group) * n + col] : 0.f;
@@ -77,7 +104,7 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
       for (int c = 0; c < W4_WAVE_COLS; ++c) acc[c] = 0.f;
 #pragma unroll
       for (int i = 0; i < W4_LANE_PIECES; ++i) {
-        const int p = lane + 64 * i;
+        const int p = pl + lanes_per_col * i;
         if (p < pieces) {
           const int4 xe = *reinterpret_cast<const int4 *>(xs + (r * pieces + p) * 8);
           const int4 xo = *reinterpret_cast<const int4 *>(xs + (r * pieces + p) * 8 + 4);
@@ -104,8 +131,9 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
       for (int c = 0; c < W4_WAVE_COLS; ++c) {
         float v = acc[c];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-        if (lane == 0 && col0 + c < n) out[(long long)(r0 + r) * n + col0 + c] = f32_to_f16_rne(v * xsr);
+        for (int o = 32; o > 0; o >>= 1)
+          if (o < lanes_per_col) v += __shfl_xor(v, o);   // wave-uniform
+        if (pl == 0 && col0 + c * side < n) out[(long long)(r0 + r) * n + col0 + c * side] = f32_to_f16_rne(v * xsr);
       }
     }
   }
@@ -124,8 +152,12 @@ extern "C" int msco_gmm_a8w4(const int8_t *x, const void *weight, const int32_t 
   if (m == 0) return MSCO_OK;
   if (x == nullptr || weight == nullptr || group_list == nullptr || x_scale == nullptr || weight_scale == nullptr || out == nullptr)
     return MSCO_ERR_INVALID_ARG;
-  const dim3 grid((unsigned)((n + W4_COLS - 1) / W4_COLS), (unsigned)e);
-  hipLaunchKernelGGL(gmm_a8w4_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), x,
+  int lanes_per_col = 64;
+  while (lanes_per_col / 2 >= k / 32) lanes_per_col /= 2;
+  const long long wg_cols = 4ll * W4_WAVE_COLS * (64 / lanes_per_col);
+  const dim3 grid((unsigned)((n + wg_cols - 1) / wg_cols), (unsigned)(e < m ? e : m));
+  const size_t lds = (size_t)(m < W4_ROWS ? m : W4_ROWS) * (size_t)k;
+  hipLaunchKernelGGL(gmm_a8w4_kernel, grid, dim3(256), lds, static_cast<hipStream_t>(stream), x,
                      static_cast<const unsigned char *>(weight), group_list, x_scale, weight_scale,
                      static_cast<unsigned short *>(out), (int)m, (int)k, (int)n, (int)e, (int)group_size);
   return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
