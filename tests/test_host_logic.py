@@ -191,25 +191,28 @@ def test_registry_and_module_surface():
         assert token in header
 
 
-@pytest.mark.parametrize("op", ["grouped_matmul", "grouped_matmul_v4_cops", "quant_batch_matmul", "moe_init_routing_v2",
-                                "moe_token_unpermute"])
+@pytest.mark.parametrize("op", ["grouped_matmul", "grouped_matmul_v4_cops", "grouped_matmul_w4", "quant_batch_matmul",
+                                "moe_init_routing_v2", "moe_init_routing_quant", "moe_token_unpermute"])
 def test_yaml_prototype_agrees_with_pybind_signature(op):
     """The prototype and the pybind definition must agree on names, order and defaults
     (the reference's rule, docs/ops_develop_guide.md:378)."""
-    proto = yaml.safe_load(open(os.path.join(REPO, "ms_custom_ops_amd", "csrc", "ops", "c_api", op, op + "_op.yaml")))
-    names = list(proto[op]["args"].keys())
+    proto = yaml.safe_load(open(os.path.join(REPO, "ms_custom_ops_amd", "csrc", "ops", "c_api", "op_prototypes.yaml")))[op]
+    args = [a.split("=", 1) for a in proto["args"]]
+    names = [a[0] for a in args]
     doc = getattr(_C, op).__doc__
     sig = doc[doc.index("(") + 1:doc.index(") ->")]
     got = [a.split(":")[0].strip() for a in re.split(r",\s*(?=\w+:)", sig)]
     assert got == names
-    for name, spec in proto[op]["args"].items():
+    for a in args:
+        name = a[0]
         m = re.search(r"\b%s: [^=,]+? = ([^,]+?)(?:,|$)" % name, sig)
-        if "default" not in spec:
+        if len(a) == 1:
             assert m is None, name
             continue
-        want = str(spec["default"]).strip("'\"").replace("mstype.float16", "42")
+        want = a[1].strip("'\"").replace("mstype.float16", "42")
         have = m.group(1).strip().strip("'\"")
         assert have.lower() == want.lower(), (name, have, want)
+    assert len(proto["returns"]) >= 1
 
 
 def test_cpu_tensors_and_noncontiguous_inputs_are_rejected():
