@@ -58,3 +58,57 @@ def test_launch_is_graph_capturable_and_replays_match_eager(device, case):
         torch.cuda.synchronize()
         assert torch.equal(out, eager), (case, replay, "eager after replay")
     op.close()
+
+
+def test_moe_chain_is_graph_capturable(device):
+    """Quantising routing -> int8 grouped matmul on its outputs -> un-permutation, recorded as one graph: none of the
+    three allocates, clears memory with a memset node or synchronises, and the routing output feeds the matmul's
+    group_list on the device.  Every replay must reproduce the eager result bit for bit."""
+    rows, hidden, k, e, n = 256, 1024, 2, 8, 512
+    g = torch.Generator(device="cuda")
+    g.manual_seed(9)
+    x = torch.randn((rows, hidden), dtype=torch.bfloat16, device="cuda", generator=g)
+    idx = torch.argsort(torch.randn(rows, e, device="cuda", generator=g), dim=1)[:, :k].to(torch.int32).contiguous()
+    w = torch.randint(-127, 128, (e, hidden, n), dtype=torch.int8, device="cuda", generator=g)
+    wscale = torch.rand(e, n, device="cuda", generator=g) * 9e-3 + 1e-3
+    probs = torch.rand((rows, k), dtype=torch.bfloat16, device="cuda", generator=g)
+    xq = torch.empty((rows * k, hidden), dtype=torch.int8, device="cuda")
+    xs = torch.empty(rows * k, dtype=torch.float32, device="cuda")
+    ridx = torch.empty(rows * k, dtype=torch.int32, device="cuda")
+    cum = torch.empty(e, dtype=torch.int32, device="cuda")
+    y = torch.empty((rows * k, n), dtype=torch.int16, device="cuda")
+    out = torch.empty((rows, n), dtype=torch.int16, device="cuda")
+    rws_bytes = cabi.moe_init_routing_v2_workspace_bytes(rows, k, e)
+    rws = torch.empty(max(rws_bytes, 1), dtype=torch.uint8, device="cuda")
+    op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I32, scale_dtype=cabi.DT_F32,
+                    per_token_dtype=cabi.DT_F32)
+    ws_bytes = op.plan(rows * k, hidden, n, e)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device="cuda")
+
+    def chain(stream):
+        cabi.moe_init_routing_v2_quant(x.data_ptr(), idx.data_ptr(), xq.data_ptr(), xs.data_ptr(), ridx.data_ptr(), cum.data_ptr(), None,
+                                       rws.data_ptr(), rws_bytes, rows, hidden, k, e, cabi.DT_BF16, 1, stream)
+        op.launch([xq.data_ptr(), w.data_ptr(), None, wscale.data_ptr(), cum.data_ptr(), xs.data_ptr(), None, None], y.data_ptr(),
+                  ws.data_ptr(), ws_bytes, stream)
+        cabi.moe_token_unpermute(y.data_ptr(), ridx.data_ptr(), probs.data_ptr(), out.data_ptr(), rows, k, n, cabi.DT_BF16, stream)
+
+    chain(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    eager = out.clone()
+    assert eager.ne(0).any()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            chain(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for replay in range(3):
+        for t in (xq, y, out):
+            t.fill_(0)                         # eager work between replays
+        xs.fill_(0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), replay
+    op.close()
