@@ -146,11 +146,19 @@ __global__ void __launch_bounds__(1024) route_small_kernel(const int *expert_idx
   int *base = total + expert_num;
   for (int x = threadIdx.x; x < blocks * expert_num; x += 1024) first[x] = 0;
   __syncthreads();
+  // (all of a thread's ids are requested before the first is used: one memory round trip instead of one per block)
   int my_e = -1;
-  for (int b = 0; b < blocks; ++b) {
+  int ids[kSmallBlocks];
+#pragma unroll
+  for (int b = 0; b < kSmallBlocks; ++b) {
     const long long i = (long long)b * kRouteBlock + threadIdx.x;
-    if (i < n) {
-      const int e = clamp_expert(expert_idx[i], expert_num);
+    ids[b] = b < blocks && i < n ? expert_idx[i] : -1;
+  }
+#pragma unroll
+  for (int b = 0; b < kSmallBlocks; ++b) {
+    const long long i = (long long)b * kRouteBlock + threadIdx.x;
+    if (b < blocks && i < n) {
+      const int e = clamp_expert(ids[b], expert_num);
       atomicAdd(&first[b * expert_num + e], 1);
       if (b == (int)blockIdx.x) my_e = e;
     }
