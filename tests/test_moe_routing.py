@@ -237,6 +237,25 @@ def test_token_unpermute_matches_the_golden(token_num, hidden, top_k):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("token_num,hidden,top_k,bf16", [(1030, 7168, 8, False), (1500, 10240, 4, True), (1024, 2048, 2, False),
+                                                        (1100, 1032, 3, True), (1200, 40960, 1, False)])
+def test_token_unpermute_with_many_tokens(token_num, hidden, top_k, bf16):
+    # 1024 tokens and more: a workgroup takes four 2048-element pieces of the row together (3.5 pieces at 7168, a second
+    # workgroup with one piece at 10240, a run-time top_k, a row longer than the 16 workgroups of a token cover in one pass)
+    rng = np.random.default_rng(token_num)
+    si = rng.permutation(token_num * top_k).astype(np.int32)
+    if bf16:
+        pt = (rng.standard_normal((token_num * top_k, hidden)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        pr = (rng.standard_normal((token_num, top_k)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        assert np.array_equal(_unpermute_gpu(pt, si, pr, cabi.DT_BF16), M.moe_token_unpermute_bf16(pt, si, pr))
+    else:
+        pt = rng.standard_normal((token_num * top_k, hidden)).astype(np.float16)
+        pr = rng.standard_normal((token_num, top_k)).astype(np.float16)
+        got = _unpermute_gpu(pt.view(np.uint16), si, pr.view(np.uint16), cabi.DT_F16)
+        assert np.array_equal(got, M.moe_token_unpermute(pt, si, pr).view(np.uint16))
+
+
+@pytest.mark.gpu
 def test_token_unpermute_bf16_and_round_trip_with_routing():
     rng = np.random.default_rng(11)
     t, k, h = 257, 4, 1024
