@@ -211,3 +211,26 @@ def test_weight_only_generic_kernel_on_packed_weights(device):
     assert "generic" in info
     got = to_f(bits).astype(np.float64)
     assert (np.abs(got[:last] - exact[:last]) <= 2.0 ** -7 * np.abs(exact[:last]) + 1e-5 * mag[:last]).all(), info
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_persistent_tile_kernel_random_shapes_both_layouts(device, seed):
+    # a seeded sweep over K (every slab count from 4 up, whole and with 16..112-byte tails, i.e. every mix of the
+    # steady-state and the general K-loop body), N with and without a tail, group counts and ragged group lists with
+    # empty groups, partial m-tiles of at most and more than 128 rows; packed weights and [E,N,K], bit for bit
+    from gpu_utils import run_w8a8
+    rng = np.random.default_rng(1000 + seed)
+    k = int(rng.integers(4, 18)) * 128 + int(rng.choice([0, 0, 16, 48, 64, 112]))
+    n = int(rng.integers(1, 5)) * 256 - int(rng.choice([0, 0, 16, 240]))
+    e = int(rng.choice([1, 2, 3, 5, 8]))
+    m = int(rng.integers(200, 1400))
+    cuts = np.sort(rng.integers(0, m + 1, e - 1)) if e > 1 else np.array([], dtype=np.int64)
+    gl = [int(v) for v in cuts] + [m - int(rng.choice([0, 0, 7]))]
+    gl = list(np.maximum.accumulate(gl))
+    x, w, bias, scale, pt = _inputs(seed, m, k, n, e)
+    info = _check(x, w, gl, bias, scale, pt, override=cabi.OV_TILE_256_W4)
+    assert "tile_256x256x128_w4" in info and "layout=packed" in info, info
+    ref = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt)
+    bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", transpose_b=True, override=cabi.OV_TILE_256_W4, launches=2)   # stores [E,N,K]
+    assert "tile_256x256x128_w4" in info, info
+    assert np.array_equal(bits[:gl[-1]], ref[:gl[-1]]), info
