@@ -71,6 +71,22 @@ def test_a8w4_ragged_groups_row_blocks_and_tails(m, k, n, e, g, gl):
     _check(_run(*case, g), *case, g)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_a8w4_random_small_shapes(seed):
+    # a seeded sweep: K from 32 to 1024 (1 to 32 pieces of 32 per column: every lane-sharing factor), K groups of 32 to
+    # 256, any N, 1 to 40 experts with empty ones, up to 60 rows (groups of more than four rows take several row blocks)
+    rng = np.random.default_rng(500 + seed)
+    g = int(rng.choice([32, 64, 128, 256]))
+    k = g * int(rng.integers(1, 1024 // g + 1))
+    n = int(rng.integers(1, 90))
+    e = int(rng.integers(1, 41))
+    m = int(rng.integers(1, 61))
+    gl = sorted(int(v) for v in rng.integers(0, m + 1, e - 1)) + [m - int(rng.choice([0, 0, 1])) if m > 1 else m]
+    gl = [int(v) for v in np.maximum.accumulate(gl)]
+    case = _case(seed, m, k, n, e, g, gl)
+    _check(_run(*case, g), *case, g)
+
+
 def test_a8w4_rejects_bad_shapes():
     with pytest.raises(RuntimeError):
         cabi.gmm_a8w4(1, 1, 1, 1, 1, 1, 4, 100, 16, 2, 32)        # k not a multiple of 32
