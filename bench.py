@@ -2,7 +2,7 @@
 """Benchmark of the grouped W8A8 matmul path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout packed|nk|kn] [--no-sweep] [--no-cpu]
-    python bench.py --probe c3|c2_m16|...|copy|moe [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs)
+    python bench.py --probe c3|c2_m16|...|copy|moe|mfma [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs)
 
 A step is one pass of the hot path over one batch of synthetic input (inputs resident in HBM before
 the timed region).  The headline workload is the Mixtral-shaped MoE configuration (E=8, top-2 over
@@ -17,6 +17,7 @@ Prints ONE JSON line.  Besides the contract keys it carries
   cpu_baseline  the numpy restatement of the reference golden timed on this box's host cores,
   sweep         the other configurations (dense decode / prefill sweep, skewed MoE, weight-only
                 decode) as TOPS and GB/s with their roofline fractions, per weight layout.
+`mfma_pipe` (and `--probe mfma`) is a yardstick: a loop of nothing but the int8 MFMA instruction on random and on zero operands.
 --probe runs a few untimed launches of one workload (or, for `copy`, of a plain device-to-device copy
 of COPY_BYTES bytes, the reference a counter reading is scaled by) so that a profiler sees nothing else.
 """
@@ -36,6 +37,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 ROTATE_BYTES = 768e6      # HBM-bound cases rotate over weight copies totalling more than the 256 MB Infinity Cache
 LAYOUT_TEXT = {"nk": "prepacked once to [E,N,K]", "kn": "[E,K,N] as generated",
                "packed": "prepacked once to the blocked layout"}
+WARM_MIN_LAUNCHES, WARM_MIN_MS, WARM_MAX_MS, WARM_TOLERANCE = 40, 30.0, 1500.0, 0.01
 COPY_BYTES = 1 << 29      # --probe copy: one launch reads and writes this many bytes
 TRAFFIC_FILE = os.path.join(REPO, "ms_custom_ops_amd", "measured_traffic.json")
 
@@ -45,7 +47,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=40,
-                    help="untimed steps; the GPU clock needs a few tens of launches to settle")
+                    help="untimed steps, a floor: warm-up goes on until the launch period is stable (see DeviceProblem.time)")
     ap.add_argument("--workload", default="c3")
     ap.add_argument("--layout", default="packed", choices=["kn", "nk", "packed"],
                     help="weight storage the op sees: packed=the blocked layout of msco_pack_weight (prepacked once, the default), "
@@ -128,23 +130,53 @@ class DeviceProblem:
         self.op.launch(ins, self.out.data_ptr(), self.ws.data_ptr(), self.ws_bytes, self.stream)
 
     def time(self, steps, warmup):
-        """Returns (wall seconds of `steps` steps, mean per-launch seconds: one pair of HIP events on the launch stream
-        around the `steps` back-to-back launches, so the figure is the launch-to-launch period of a running stream and
-        agrees with a profiler's kernel durations)."""
+        """Returns (wall seconds of `steps` steps, mean per-launch seconds, details).  The per-launch figure comes from
+        one pair of HIP events on the launch stream around the `steps` back-to-back launches, so it is the
+        launch-to-launch period of a running stream and agrees with a profiler's kernel durations.
+
+        `warmup` is a floor.  The shader clock takes tens of launches to settle under this load, so the untimed phase
+        goes on (in batches of ten launches, each timed with events) until at least WARM_MIN_LAUNCHES launches and
+        WARM_MIN_MS of device time have passed and two batches in a row agree within WARM_TOLERANCE, or WARM_MAX_MS is
+        used up.  `details` records the warm-up launches actually made and the period of the first and the last
+        quarter of the timed steps, so a figure taken while the clock still moved shows."""
         torch = self.torch
+        ev = lambda: torch.cuda.Event(enable_timing=True)
         for _ in range(warmup):
             self.step()
         torch.cuda.synchronize()
-        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        done, spent_ms, prev, stable = warmup, 0.0, None, False
+        while spent_ms < WARM_MAX_MS:
+            a, b = ev(), ev()
+            a.record()
+            for _ in range(10):
+                self.step()
+            b.record()
+            torch.cuda.synchronize()
+            batch = a.elapsed_time(b)
+            done += 10
+            spent_ms += batch
+            stable = prev is not None and abs(batch - prev) <= WARM_TOLERANCE * prev
+            prev = batch
+            if stable and done >= WARM_MIN_LAUNCHES and spent_ms >= WARM_MIN_MS:
+                break
+        marks = sorted({0, steps // 4, steps - steps // 4, steps})
+        events = {}
         t0 = time.perf_counter()
-        first.record()
-        for _ in range(steps):
-            self.step()
-        last.record()
+        for i in range(steps + 1):
+            if i in marks:
+                events[i] = ev()
+                events[i].record()
+            if i < steps:
+                self.step()
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
-        per_launch = first.elapsed_time(last) / steps * 1e-3
-        return wall, per_launch
+        per_launch = events[0].elapsed_time(events[steps]) / steps * 1e-3
+        details = {"warmup_launches": done, "warmup_settled": bool(stable)}
+        if steps >= 4:
+            q = steps // 4
+            details["first_quarter_us"] = events[0].elapsed_time(events[q]) / q * 1e3
+            details["last_quarter_us"] = events[steps - q].elapsed_time(events[steps]) / q * 1e3
+        return wall, per_launch, details
 
 
 def rates(wl, seconds):
@@ -267,6 +299,35 @@ def moe_neighbours(steps, warmup):
     return out
 
 
+def mfma_pipe_probe(iters=20000, launches=12):
+    """Rate of a loop of nothing but v_mfma_i32_32x32x32_i8 (msco_probe_mfma: 256 workgroups, one wavefront per SIMD, no
+    memory traffic) on uniformly random int8 operands, the distribution of the workloads, and on zeros: what the matrix
+    pipe sustains at the clock the chip holds under each.  Every figure is the mean over the last half of the launches
+    (one pair of events around them), after the first half has let the clock settle."""
+    import torch
+    from ms_custom_ops_amd import cabi
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    sink = torch.empty(cabi.PROBE_MFMA_WORKGROUPS * 256, dtype=torch.int32, device=dev)
+    ops = cabi.PROBE_MFMA_WORKGROUPS * 4 * iters * 16 * 65536.0
+    out = {"ops_per_launch": ops, "iters": iters}
+    for name, operands in (("random_int8", torch.randint(-127, 128, (cabi.PROBE_MFMA_OPERAND_BYTES,), dtype=torch.int8, device=dev, generator=g)),
+                           ("zeros", torch.zeros(cabi.PROBE_MFMA_OPERAND_BYTES, dtype=torch.int8, device=dev))):
+        for _ in range(launches // 2):
+            cabi.probe_mfma(operands.data_ptr(), sink.data_ptr(), iters, st)
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(launches - launches // 2):
+            cabi.probe_mfma(operands.data_ptr(), sink.data_ptr(), iters, st)
+        b.record()
+        torch.cuda.synchronize()
+        sec = a.elapsed_time(b) * 1e-3 / (launches - launches // 2)
+        out[name] = {"launch_us": sec * 1e6, "tops": ops / sec / 1e12, "int8_frac": ops / sec / 1e12 / PEAK_INT8_TOPS}
+    return out
+
+
 def measured_traffic(workload, layout, kernel):
     """HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs (scaled by
     the same counters' reading for a copy of known size); None when no measurement of this kernel is on file."""
@@ -290,6 +351,9 @@ def probe(args):
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"probe": "copy", "bytes_read": COPY_BYTES, "bytes_written": COPY_BYTES, "launches": args.steps}))
+        return
+    if args.probe == "mfma":
+        print(json.dumps({"probe": "mfma", "mfma_pipe": mfma_pipe_probe()}))
         return
     if args.probe == "moe":
         print(json.dumps({"probe": "moe", "moe_neighbours": moe_neighbours(args.steps, 5)}))
@@ -320,7 +384,7 @@ def main():
         return
     wl = workloads.make(args.workload)
     prob = DeviceProblem(wl, args.layout)
-    wall, per_launch = prob.time(args.steps, args.warmup)
+    wall, per_launch, timing = prob.time(args.steps, args.warmup)
     work, _, _ = rates(wl, per_launch)
     step_s = wall / args.steps
     tops_wall = work["ops"] / step_s / 1e12
@@ -328,7 +392,7 @@ def main():
     plan = prob.op.plan_info()
     mfma_bound = (work["ops"] / work["bytes"]) > (PEAK_INT8_TOPS * 1e12) / (PEAK_HBM_GBS * 1e9)
     if mfma_bound:
-        roof = {"bound": "mfma", "achieved": tops_kernel, "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
+        roof = {"bound": "mfma", "achieved": tops_kernel, "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                 "frac": tops_kernel / PEAK_INT8_TOPS, "traffic": None}
     else:
         gbs = work["bytes"] / per_launch / 1e9
@@ -336,6 +400,8 @@ def main():
                 "traffic": None}
     roof["kernel"] = plan.split("kernel=")[1].split(" ")[0]
     roof["traffic"] = measured_traffic(wl.name, args.layout, roof["kernel"])
+    roof["traffic_source"] = None if roof["traffic"] is None else \
+        "stored: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs summarised under profiles/ (not re-measured in this run)"
     roof["launch_us"] = per_launch * 1e6
     roof["ops_per_launch"] = work["ops"]
     roof["bytes_per_launch"] = work["bytes"]
@@ -348,7 +414,7 @@ def main():
         "config": {"workload": f"{wl.name}: grouped W8A8, E={wl.e}, rows={work['rows']}, K={wl.k}, N={wl.n}, "
                                f"weights {LAYOUT_TEXT[args.layout]}, "
                                "routing top-2 of softmax(N(0,1))",
-                   "plan": plan, "prepack_ms": prob.prepack_ms},
+                   "plan": plan, "prepack_ms": prob.prepack_ms, "timing": timing},
         "hbm_gbs": work["bytes"] / step_s / 1e9, "hbm_frac": work["bytes"] / step_s / 1e9 / PEAK_HBM_GBS,
         "int8_frac": tops_wall / PEAK_INT8_TOPS,
         "roofline": roof,
@@ -369,7 +435,7 @@ def main():
             hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5", "c3_decode")
             copies = max(1, int(np.ceil(ROTATE_BYTES / w_bytes))) if hbm_bound_guess else 1
             p2 = DeviceProblem(w2, layout, copies)
-            _, sec = p2.time(max(20, min(200, args.steps)), args.warmup)
+            _, sec, _ = p2.time(max(20, min(200, args.steps)), args.warmup)
             wk, tops, gbs = rates(w2, sec)
             sweep.append({"workload": name, "layout": layout, "launch_us": sec * 1e6, "tops": tops,
                           "int8_frac": tops / PEAK_INT8_TOPS, "gbs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS,
@@ -378,6 +444,7 @@ def main():
             torch.cuda.empty_cache()
         result["sweep"] = sweep
         result["moe_neighbours"] = moe_neighbours(max(20, min(100, args.steps)), 10)
+        result["mfma_pipe"] = mfma_pipe_probe()
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(wl)

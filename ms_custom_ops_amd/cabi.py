@@ -33,7 +33,8 @@ EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
                     "msco_packed_weight_bytes", "msco_pack_weight", "msco_gmm_a8w4",
                     "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_init_routing_v2_quant",
-                    "msco_moe_token_unpermute")
+                    "msco_moe_token_unpermute", "msco_probe_mfma")
+PROBE_MFMA_WORKGROUPS, PROBE_MFMA_OPERAND_BYTES = 256, 8 * 256 * 16
 
 
 class GmmDesc(ctypes.Structure):
@@ -96,6 +97,8 @@ def load():
             [ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
         lib.msco_moe_token_unpermute.restype = ctypes.c_int
         lib.msco_moe_token_unpermute.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int64] * 3 + [ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_probe_mfma.restype = ctypes.c_int
+        lib.msco_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
         _lib = lib
     return _lib
 
@@ -133,6 +136,13 @@ def gmm_a8w4(x: int, weight: int, group_list: int, x_scale: int, weight_scale: i
     vp = lambda v: ctypes.c_void_p(v if v else None)
     _check("msco_gmm_a8w4", load().msco_gmm_a8w4(vp(x), vp(weight), vp(group_list), vp(x_scale), vp(weight_scale), vp(out),
                                                  m, k, n, e, group_size, vp(stream)))
+
+
+def probe_mfma(operands: int, sink: int, iters: int, stream: Optional[int] = None):
+    """Raw-pointer call of msco_probe_mfma (see include/msco_gmm.h); PROBE_MFMA_WORKGROUPS * 4 * iters * 16 * 65536 int8
+    operations per launch."""
+    vp = lambda v: ctypes.c_void_p(v if v else None)
+    _check("msco_probe_mfma", load().msco_probe_mfma(vp(operands), vp(sink), iters, vp(stream)))
 
 
 def moe_init_routing_v2_workspace_bytes(num_rows: int, k: int, expert_num: int) -> int:

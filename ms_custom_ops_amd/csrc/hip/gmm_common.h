@@ -214,6 +214,18 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_over(const void *base, 
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
 }
 
+// ---- split-K hand-off ------------------------------------------------------------------------------
+// Called by every thread of a workgroup after it has written its share of a partial tile with agent-scope stores
+// and before one thread bumps the tile's arrival counter.  A workgroup-scope release fence does not wait for the
+// outstanding vector stores of the other wavefronts, so every wavefront drains its own stores (vmcnt == 0: each
+// store has been acknowledged at the scope its cache bits name) before it enters the barrier; the thread that
+// bumps the counter behind the barrier therefore does so after all the workgroup's partials are visible to the agent.
+__device__ __forceinline__ void publish_partials_and_sync() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __syncthreads();
+}
+
 // ---- byte shuffles -----------------------------------------------------------------------------
 // v_perm_b32: result byte i = byte sel[i] of the 8-byte value {hi:lo} (0..3 -> lo, 4..7 -> hi).
 __device__ __forceinline__ unsigned perm(unsigned hi, unsigned lo, unsigned sel) {

@@ -171,8 +171,7 @@ __global__ void __launch_bounds__(AW_THREADS, 4) gmm_a16w8_skinny_kernel(const G
                            __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    publish_partials_and_sync();
     if (tid == 0) s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != (unsigned)(p.split_k - 1)) return;

@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(SK_THREADS, NK ? 3 : 4) gmm_w8a8_skinny_kernel
     // ---- cross-workgroup reduction through the workspace --------------------------------------
     // Partial tiles and the arrival counter are exchanged with agent-scope atomic accesses: they
     // bypass the per-XCD L2 for this data only, so no cache-wide write-back / invalidate fence is
-    // needed.  The stores are complete (vmcnt == 0) before the counter is bumped.  A tile is kept in
+    // needed.  Every wavefront waits for its own stores (vmcnt == 0) before the barrier that precedes the counter bump.  A tile is kept in
     // the threads' own fragment order: slice s, 64-bit word e of thread t at ((s * 8 + e) * 256 + t).
     const long long tile = ((long long)grp * p.max_chunks + mc) * p.n_strips + strip;
     i64 *base = reinterpret_cast<i64 *>(p.partial) + tile * p.split_k * (SK_TILE_INTS / 2);
@@ -140,8 +140,7 @@ __global__ void __launch_bounds__(SK_THREADS, NK ? 3 : 4) gmm_w8a8_skinny_kernel
         __hip_atomic_store(mine + e * SK_THREADS, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    publish_partials_and_sync();
     if (tid == 0) s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != (unsigned)(p.split_k - 1)) return;
@@ -372,8 +371,7 @@ __global__ void __launch_bounds__(W16_THREADS) gmm_w8a8_skinny16_kernel(const Gm
         __hip_atomic_store(mine + e * W16_REDUCERS, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    publish_partials_and_sync();
     if (tid == 0) s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != (unsigned)(p.split_k - 1)) return;

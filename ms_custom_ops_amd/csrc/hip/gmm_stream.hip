@@ -182,8 +182,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
         __hip_atomic_store(mine + e * ST_THREADS, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    publish_partials_and_sync();
     if (tid == 0) *s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*s_ticket != (unsigned)(p.split_k - 1)) return;
@@ -409,8 +408,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_streamm_kernel(const G
         const i64 word = (i64)(((unsigned long long)(unsigned)v[j][2 * hf + 1] << 32) | (unsigned)v[j][2 * hf]);
         __hip_atomic_store(mine + (j * 2 + hf) * ST_THREADS, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    publish_partials_and_sync();
     if (tid == 0) *s_ticket = __hip_atomic_fetch_add(&p.counters[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*s_ticket != (unsigned)(p.split_k - 1)) return;
@@ -651,8 +649,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
         __hip_atomic_store(mine + 2048 + 2 * lane + 1, pack(xs[2], xs[3]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    publish_partials_and_sync();
     if (tid == 0) *s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (*s_ticket != (unsigned)(p.split_k - 1)) return;

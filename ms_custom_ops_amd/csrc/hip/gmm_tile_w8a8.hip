@@ -456,8 +456,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
           const i64 word = (i64)(((unsigned long long)(unsigned)acc[f][i][r + 1] << 32) | (unsigned)acc[f][i][r]);
           __hip_atomic_store(mine + ((f * FM + i) * 8 + r / 2) * NT, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
+    publish_partials_and_sync();
     if (tid == 0) s_ticket = __hip_atomic_fetch_add(&p.counters[lid], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != (unsigned)(split - 1)) return;
@@ -647,7 +646,8 @@ const char *tile_cfg_name(int tile_cfg) {
 size_t tile_count_bound(int tile_cfg, int64_t m, int64_t n, int64_t e) {
   int bm, bn;
   tile_cfg_dims(tile_cfg, &bm, &bn);
-  return (size_t)(((m + bm - 1) / bm + e) * ((n + bn - 1) / bn));
+  // every group that holds rows adds at most one partial m-tile, and at most min(e, m) groups hold rows
+  return (size_t)(((m + bm - 1) / bm + (e < m ? e : m)) * ((n + bn - 1) / bn));
 }
 
 size_t tile_workspace_bytes(int tile_cfg, int64_t m, int64_t n, int64_t e, int split_k) {

@@ -37,13 +37,21 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
   // blockIdx.y counts the groups that hold rows (at most min(e, m) of them): find the one with that rank, 64 groups
   // per round of ballots, and leave if there are fewer
   int grp = -1, g_start = 0, g_end = 0;
-  for (int g0 = 0, seen = 0; g0 < e && grp < 0; g0 += 256) {
+  for (int g0 = 0, seen = 0, carry = 0; g0 < e && grp < 0; g0 += 256) {
     int lo[4], hi[4];   // four rounds' worth of boundaries requested together: one memory round trip per 256 groups
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int g = g0 + 64 * u + lane;
-      lo[u] = g > 0 && g < e ? min(max(group_list[g - 1], 0), m) : 0;
-      hi[u] = g < e ? min(max(group_list[g], lo[u]), m) : 0;
+      hi[u] = g < e ? min(max(group_list[g], 0), m) : 0;
+    }
+    // row end of a group = running maximum of the list clamped into [0, m] (a list that is not monotonic can then
+    // never make two groups overlap); `carry` is the end of the last group of the round before
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      hi[u] = max(carry, wave_scan_max(hi[u], lane));
+      const int prev = __shfl_up(hi[u], 1);
+      lo[u] = lane == 0 ? carry : prev;
+      carry = wave_bcast(hi[u], 63);
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {

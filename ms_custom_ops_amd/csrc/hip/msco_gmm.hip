@@ -33,6 +33,7 @@ constexpr int kMaxSplitK = 8;             // keeps the last arriver's reduction 
 constexpr int kNumCUs = 256;
 constexpr int kTileTargetWorkgroups = 256;   // tile kernels with a K split: aim for this many workgroups (one per CU)
 constexpr int kTileSplitMaxTiles = 128;      // ... and only split below this many tiles (measured: beyond it the partial-tile exchange costs more than it hides)
+constexpr size_t kTileSplitMaxWorkspace = (size_t)128 << 20;   // bytes of split-K partial tiles a plan may ask the caller for
 constexpr int kTileMinSlabs = 4;               // 64-byte K slabs every slice keeps at least
 
 int env_int(const char *name, int fallback) {
@@ -184,6 +185,9 @@ void choose_plan(msco_gmm_op *op) {
       want = std::max(1, std::min(std::min(want, kMaxSplitK), cap));
       const int forced_split = env_int("MSCO_TILE_SPLIT_K", 0);
       if (forced_split > 0) want = std::min(forced_split, cap);
+      // the partial tiles of a K split are sized for the worst group_list (one partial m-tile per group): with many
+      // groups that bound dwarfs the problem, so the split is halved until the workspace fits under the cap
+      while (want > 1 && tile_workspace_bytes(op->tile_cfg, m, n, e, want) > kTileSplitMaxWorkspace) want /= 2;
       op->split_k = want;
       op->workspace_bytes = tile_workspace_bytes(op->tile_cfg, m, n, e, op->split_k);
     }
@@ -347,6 +351,13 @@ int msco_gmm_plan(msco_gmm_handle h, int64_t m, int64_t k, int64_t n, int64_t e,
         return MSCO_ERR_DEVICE;
       }
       h->counters_cap = need;
+    } else if (h->counters != nullptr) {
+      // the counters reset themselves at the end of a launch; one that was abandoned half-way (a failed launch, a
+      // destroyed stream) may have left tickets behind, so a new plan starts from zero again
+      if (hipMemset(h->counters, 0, h->counters_cap * sizeof(unsigned)) != hipSuccess) {
+        (void)hipGetLastError();
+        return MSCO_ERR_DEVICE;
+      }
     }
   }
   h->planned = true;

@@ -134,3 +134,17 @@ def test_gmm_w4_rejects_what_the_reference_rejects():
     with pytest.raises(ValueError, match="weight_scale must be"):
         ms_custom_ops.grouped_matmul_w4(x, w, gl, b, xs, z((2, 2, 8), torch.float32))
     assert ms_custom_ops.grouped_matmul_w4(x, w, gl, b, xs, ws).shape == (4, 16)
+
+
+def test_a8w4_malformed_group_list_is_clamped_like_the_other_kernels():
+    # a list that is not monotonic or runs past m: the row end of a group is the running maximum clamped into [0, m],
+    # so groups never overlap and the result is that of the repaired list
+    m, k, n, e, g = 12, 256, 48, 4, 64
+    bad = [5, 3, 8, 100]
+    good = [5, 5, 8, 12]
+    case_bad = _case(11, m, k, n, e, g, bad)
+    case_good = _case(11, m, k, n, e, g, good)
+    a = _run(*case_bad, g)
+    b = _run(*case_good, g)
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+    _check(b, *case_good, g)
