@@ -133,6 +133,16 @@ MSCO_API int msco_gmm_plan(msco_gmm_handle h, int64_t m, int64_t k, int64_t n, i
 MSCO_API int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, void *workspace,
                     size_t workspace_bytes, void *stream);
 
+/* The same launch for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The split-K partial tiles that
+ * msco_gmm_launch keeps in the caller's workspace go to a fixed array of MSCO_GMM_STATIC_WORKSPACE_BYTES bytes inside
+ * the library instead (every GPU the library runs on holds it until the process ends); a plan whose workspace is
+ * larger is refused with MSCO_ERR_WORKSPACE and a message on stderr.  Nothing is allocated or freed.  All calls on one
+ * GPU share the array: two calls that overlap in time on one GPU (different streams, or different handles on
+ * different streams) race; calls on one stream are ordered and safe. */
+#define MSCO_GMM_STATIC_WORKSPACE_BYTES (32u << 20)
+MSCO_API int msco_gmm_launch_static(msco_gmm_handle h, const void *const *inputs, void *out, void *stream);
+
 /* Human-readable description of the current plan (kernel family, tile, grid, split) -- the
  * counterpart of the reference's INTERNAL_PRINT_TILING switch.  Returns the number of characters
  * that the full text needs (excluding the terminating NUL). */

@@ -33,7 +33,8 @@ EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
                     "msco_packed_weight_bytes", "msco_pack_weight", "msco_gmm_a8w4",
                     "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_init_routing_v2_quant",
-                    "msco_moe_token_unpermute", "msco_probe_mfma")
+                    "msco_moe_token_unpermute", "msco_probe_mfma", "msco_gmm_launch_static")
+STATIC_WORKSPACE_BYTES = 32 << 20
 PROBE_MFMA_WORKGROUPS, PROBE_MFMA_OPERAND_BYTES = 256, 8 * 256 * 16
 
 
@@ -97,6 +98,8 @@ def load():
             [ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
         lib.msco_moe_token_unpermute.restype = ctypes.c_int
         lib.msco_moe_token_unpermute.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int64] * 3 + [ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_gmm_launch_static.restype = ctypes.c_int
+        lib.msco_gmm_launch_static.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_void_p]
         lib.msco_probe_mfma.restype = ctypes.c_int
         lib.msco_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
         _lib = lib
@@ -217,6 +220,15 @@ class GmmOp:
         _check("msco_gmm_launch", load().msco_gmm_launch(self._h, arr, ctypes.c_void_p(out),
                                                          ctypes.c_void_p(workspace if workspace else None),
                                                          workspace_bytes, ctypes.c_void_p(stream if stream else None)))
+
+    def launch_static(self, inputs: Sequence[Optional[int]], out: int, stream: Optional[int] = None):
+        """msco_gmm_launch_static: the launch that takes its split-K workspace from the library's fixed device array."""
+        arr = (ctypes.c_void_p * IN_COUNT)()
+        for i in range(IN_COUNT):
+            v = inputs[i] if i < len(inputs) else None
+            arr[i] = ctypes.c_void_p(v if v else None)
+        _check("msco_gmm_launch_static", load().msco_gmm_launch_static(self._h, arr, ctypes.c_void_p(out),
+                                                                       ctypes.c_void_p(stream if stream else None)))
 
     def close(self):
         if self._h:

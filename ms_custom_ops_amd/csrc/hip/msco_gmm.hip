@@ -434,6 +434,54 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
 }
 
+// ---- launch without a caller workspace ----------------------------------------------------------------------------
+// The split-K partial tiles go to a fixed device array instead of a caller buffer.  Host code never passes the array's
+// name to a kernel or a runtime call (on the host it is a stand-in, not a device address): the address on each device
+// is looked up once with hipGetSymbolAddress, with that device current, and kept.
+namespace {
+static __device__ __align__(256) unsigned char scratch[MSCO_GMM_STATIC_WORKSPACE_BYTES];
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+// the current device's copy of `scratch`; nullptr (and *status set) on failure
+void *scratch_of_current_device(int *status) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    *status = MSCO_ERR_DEVICE;
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+      (void)hipGetLastError();
+      *status = MSCO_ERR_DEVICE;
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+}  // namespace
+
+int msco_gmm_launch_static(msco_gmm_handle h, const void *const *inputs, void *out, void *stream) {
+  if (h == nullptr || inputs == nullptr) return MSCO_ERR_INVALID_ARG;
+  if (!h->planned) return MSCO_ERR_NOT_PLANNED;
+  if (h->workspace_bytes > (size_t)MSCO_GMM_STATIC_WORKSPACE_BYTES) {
+    std::fprintf(stderr, "msco_gmm_launch_static: the plan needs %zu bytes of workspace, the static one holds %zu\n",
+                 h->workspace_bytes, (size_t)MSCO_GMM_STATIC_WORKSPACE_BYTES);
+    return MSCO_ERR_WORKSPACE;
+  }
+  int status = MSCO_OK;
+  void *ws = scratch_of_current_device(&status);
+  if (ws == nullptr) return status;
+  // nothing in the array has to start at zero: every K slice writes its whole partial tile before it takes a ticket,
+  // and the tickets live in the handle
+  return msco_gmm_launch(h, inputs, out, ws, (size_t)MSCO_GMM_STATIC_WORKSPACE_BYTES, stream);
+}
+
 int msco_transpose_2d(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int32_t elem_bytes,
                       void *stream) {
   if (batch < 0 || rows < 0 || cols < 0 || batch > 65535) return MSCO_ERR_SHAPE;
