@@ -61,7 +61,7 @@ def parse():
 class DeviceProblem:
     """One workload resident on the GPU plus a planned backend operator."""
 
-    def __init__(self, wl, layout="kn", copies=1):
+    def __init__(self, wl, layout="kn", copies=1, zero_operands=False, act_type=0):
         import torch
         from ms_custom_ops_amd import cabi
         self.torch, self.cabi, self.wl = torch, cabi, wl
@@ -71,6 +71,9 @@ class DeviceProblem:
         t = lambda a: None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(dev)
         self.x = t(wl.x.view(np.int16)) if self.a16 else t(wl.x)
         w0 = t(wl.w)
+        if zero_operands:   # same shapes, routing and kernel, operands that toggle nothing: a timing yardstick only
+            self.x.zero_()
+            w0.zero_()
         self.prepack_ms = None
         if nk:
             # one-time prepack [E,K,N] -> [E,N,K] through the backend's own transpose entry point
@@ -112,7 +115,7 @@ class DeviceProblem:
             self.op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,
                                  scale_dtype=cabi.DT_F32, per_token_dtype=cabi.DT_F32,
                                  bias_dtype=cabi.DT_I32 if self.bias is not None else cabi.DT_NONE,
-                                 transpose_b=int(nk),
+                                 transpose_b=int(nk), act_type=act_type,
                                  weight_layout=cabi.WL_PACKED if layout == "packed" else cabi.WL_ROW_MAJOR)
         self.ws_bytes = self.op.plan(wl.m, wl.k, wl.n, wl.e)
         self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
@@ -445,6 +448,22 @@ def main():
         result["sweep"] = sweep
         result["moe_neighbours"] = moe_neighbours(max(20, min(100, args.steps)), 10)
         result["mfma_pipe"] = mfma_pipe_probe()
+        # the headline kernel once more on all-zero x and weights: same instruction stream and memory traffic, but the
+        # matrix pipe toggles nothing, so the chip holds a higher clock; the gap to the figure above is what the
+        # operand distribution costs, the gap to the peak is what the kernel's own stalls and padding cost
+        pz = DeviceProblem(wl, args.layout, zero_operands=True)
+        _, secz, _ = pz.time(max(20, min(100, args.steps)), args.warmup)
+        result["zero_operand_check"] = {"workload": wl.name, "layout": args.layout, "launch_us": secz * 1e6,
+                                        "tops": work["ops"] / secz / 1e12, "int8_frac": work["ops"] / secz / 1e12 / PEAK_INT8_TOPS}
+        del pz
+        torch.cuda.empty_cache()
+        # and with an activation fused into the epilogue (act_type 5, silu)
+        pa = DeviceProblem(wl, args.layout, act_type=5)
+        _, seca, _ = pa.time(max(20, min(100, args.steps)), args.warmup)
+        result["fused_activation"] = {"workload": wl.name, "layout": args.layout, "act_type": 5, "launch_us": seca * 1e6,
+                                      "tops": work["ops"] / seca / 1e12, "int8_frac": work["ops"] / seca / 1e12 / PEAK_INT8_TOPS}
+        del pa
+        torch.cuda.empty_cache()
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(wl)

@@ -81,6 +81,24 @@ enum {
   MSCO_WL_PACKED = 1           /* e * msco_packed_weight_bytes(k, n) bytes written by msco_pack_weight */
 };
 
+/* Activation fused into the epilogue: the act_type argument that the reference forwards unchanged to
+ * aclnnGroupedMatmulV4 (ops/c_api/grouped_matmul_v4_cops/grouped_matmul_v4_cops.cc:96,112,363; the reference defines no
+ * values and holds no golden for it, so the values are those of CANN's GMMActType and the functions their textbook
+ * forms).  Applied to the float32 result of the dequant epilogue (or of the weight-only matmul), before the cast to
+ * bf16 / f16; not available with int32 output.
+ *   RELU       max(v, 0)
+ *   GELU_TANH  v * sigmoid(2 * sqrt(2 / pi) * (v + 0.044715 v^3))      (= 0.5 v (1 + tanh(...)))
+ *   FAST_GELU  v * sigmoid(1.702 v)
+ *   SILU       v * sigmoid(v) */
+enum {
+  MSCO_ACT_NONE = 0,
+  MSCO_ACT_RELU = 1,
+  MSCO_ACT_GELU_TANH = 2,
+  MSCO_ACT_GELU_ERF = 3,       /* listed by CANN as unsupported; refused here too */
+  MSCO_ACT_FAST_GELU = 4,
+  MSCO_ACT_SILU = 5
+};
+
 /* Positional inputs of msco_gmm_launch.  Slots 0..6 follow the order the reference passes to its
  * kernel object (grouped_matmul.cc:201-207,301-307); slot 7 is the V4 antiquant offset
  * (grouped_matmul_v4_cops.cc:94-97). */
@@ -115,7 +133,8 @@ typedef struct msco_gmm_desc {
   int32_t scale_is_scalar;   /* 1: scale holds a single element broadcast over N */
   int32_t kernel_override;   /* 0 auto; else force a kernel family (see msco_gmm_plan_info), for tests */
   int32_t weight_layout;     /* MSCO_WL_ROW_MAJOR: as transpose_b says; MSCO_WL_PACKED: written by msco_pack_weight */
-  int32_t reserved[4];
+  int32_t act_type;          /* msco_act: activation applied to the dequantised float32 value before the output cast */
+  int32_t reserved[3];
 } msco_gmm_desc;
 
 typedef struct msco_gmm_op *msco_gmm_handle;

@@ -26,6 +26,9 @@ IN_COUNT = 8
 # msco_gmm_desc.kernel_override
 OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC, OV_TILE_256_W4 = range(7)
 
+# msco_gmm_desc.act_type
+ACT_NONE, ACT_RELU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_FAST_GELU, ACT_SILU = range(6)
+
 # msco_gmm_desc.weight_layout
 WL_ROW_MAJOR, WL_PACKED = 0, 1
 
@@ -42,7 +45,7 @@ class GmmDesc(ctypes.Structure):
     _fields_ = [(name, ctypes.c_int32) for name in (
         "abi_version", "x_dtype", "weight_dtype", "out_dtype", "group_list_dtype", "group_list_type", "bias_dtype",
         "scale_dtype", "per_token_dtype", "antiquant_dtype", "has_antiquant_offset", "transpose_b", "scale_per_group",
-        "scale_is_scalar", "kernel_override", "weight_layout")] + [("reserved", ctypes.c_int32 * 4)]
+        "scale_is_scalar", "kernel_override", "weight_layout", "act_type")] + [("reserved", ctypes.c_int32 * 3)]
 
 
 class BackendError(RuntimeError):

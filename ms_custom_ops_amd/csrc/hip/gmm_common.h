@@ -49,6 +49,7 @@ struct GmmParams {
   int n_strips;             // ceil(N / kSkinnyCols)
   int max_chunks;           // ceil(M / kSkinnyRows): 16-row chunks a group can have (skinny W8A8 kernel)
   int strip_groups;         // packed-layout kernels: 16-column groups per strip (1..16); n_strips counts these strips
+  int act_type;             // ACT_*: activation on the float32 result before the output cast (never with int32 output)
 };
 
 // ---- group_list --------------------------------------------------------------------------------
@@ -188,7 +189,46 @@ __device__ __forceinline__ float dequant(int acc_plus_bias, float scale, float p
   return f;
 }
 
+// Activation on the dequantised value (msco_act in include/msco_gmm.h).  The three smooth ones are v * sigmoid(t(v));
+// written as v / (1 + exp(-t)) there is no cancellation anywhere on the real line (exp(-t) = inf gives -0 for very
+// negative v, where the true value underflows).  Fast exponential and reciprocal: a few float32 ulps, far below the
+// rounding of the 16-bit output.
+enum : int { ACT_NONE = 0, ACT_RELU = 1, ACT_GELU_TANH = 2, ACT_GELU_ERF = 3, ACT_FAST_GELU = 4, ACT_SILU = 5 };
+__device__ __forceinline__ float activate(float v, int act) {
+  if (act == ACT_RELU) return v < 0.0f ? 0.0f : v;
+  float t = v;
+  if (act == ACT_FAST_GELU) t = 1.702f * v;
+  if (act == ACT_GELU_TANH) t = 1.5957691216057308f * (v + 0.044715f * v * v * v);
+  return __fdividef(v, 1.0f + __expf(-t));
+}
+
+// float32 result -> 16-bit output pattern (bf16 or f16 as the plan says), activation first
+__device__ __forceinline__ unsigned short half_out(const GmmParams &p, float f) {
+  if (p.act_type != ACT_NONE) f = activate(f, p.act_type);
+  return p.out_dtype == DT_BF16 ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+}
+
+// The same without branches, for epilogues whose instruction schedule must not split into paths: the activation as
+// two wave-uniform coefficients of t(v) = v (c1 + c3 v^2) and a flag for the one that is not smooth.
+struct ActCoeffs {
+  float c1, c3;
+  bool relu;
+};
+__device__ __forceinline__ ActCoeffs act_coeffs(int act) {
+  ActCoeffs c;
+  c.relu = act == ACT_RELU;
+  c.c1 = act == ACT_FAST_GELU ? 1.702f : act == ACT_GELU_TANH ? 1.5957691216057308f : 1.0f;
+  c.c3 = act == ACT_GELU_TANH ? 1.5957691216057308f * 0.044715f : 0.0f;
+  return c;
+}
+__device__ __forceinline__ float activate(float v, const ActCoeffs &c) {
+  const float t = v * (c.c1 + c.c3 * v * v);
+  const float smooth = __fdividef(v, 1.0f + __expf(-t));
+  return c.relu ? (v < 0.0f ? 0.0f : v) : smooth;
+}
+
 __device__ __forceinline__ void store_out(const GmmParams &p, long long idx, int acc_plus_bias, float f) {
+  if (p.act_type != ACT_NONE) f = activate(f, p.act_type);
   if (p.out_dtype == DT_BF16) {
     reinterpret_cast<unsigned short *>(p.out)[idx] = f32_to_bf16_rne(f);
   } else if (p.out_dtype == DT_F16) {

@@ -79,7 +79,7 @@ __global__ void __launch_bounds__(256) gmm_a16w8_generic_kernel(const GmmParams 
   const float s = p.aq_scale ? load_half_like(p.aq_scale, (long long)g * p.n + n, p.x_dtype) : 1.0f;
   const float o = p.aq_offset ? load_half_like(p.aq_offset, (long long)g * p.n + n, p.x_dtype) : 0.0f;
   const float f = (acc + o * xsum) * s;
-  out[idx] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+  out[idx] = half_out(p, f);
 }
 
 // Batched 2-D transpose through a padded LDS tile: src [batch, rows, cols] -> dst [batch, cols, rows].

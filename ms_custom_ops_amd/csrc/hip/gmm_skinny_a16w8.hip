@@ -225,7 +225,7 @@ __global__ void __launch_bounds__(AW_THREADS, 4) gmm_a16w8_skinny_kernel(const G
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float f = fmaf(o - 128.0f, xs[r], v[e][r]) * s;
-        tile_out[4 * h + r][cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+        tile_out[4 * h + r][cl] = half_out(p, f);
       }
     }
   }

@@ -196,7 +196,7 @@ __global__ void __launch_bounds__(SK_THREADS, NK ? 3 : 4) gmm_w8a8_skinny_kernel
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float f = dequant(v[e][r] + bias, sc, pt[r]);
-          tile_out[4 * h + r][cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+          tile_out[4 * h + r][cl] = half_out(p, f);
         }
       }
     }
@@ -414,7 +414,7 @@ __global__ void __launch_bounds__(W16_THREADS) gmm_w8a8_skinny16_kernel(const Gm
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float f = dequant(v[r] + ep_bias, ep_scale, ep_pt[r]);
-        tile_out[4 * h + r][ep_cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+        tile_out[4 * h + r][ep_cl] = half_out(p, f);
       }
     }
   }

@@ -235,7 +235,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float f = dequant(v[e][r] + bias, sc, pt[r]);
-          tile_out[4 * h + r][cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+          tile_out[4 * h + r][cl] = half_out(p, f);
         }
       }
     }
@@ -451,7 +451,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_streamm_kernel(const G
             reinterpret_cast<int *>(p.out)[(long long)(m0 + row) * p.n + n] = v[j][r] + bias;
           } else {
             const float f32 = dequant(v[j][r] + bias, sc, p.per_token ? p.per_token[m0 + row] : 1.0f);
-            tile_out[row][cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f32) : f32_to_f16_rne(f32);
+            tile_out[row][cl] = half_out(p, f32);
           }
         }
       }
@@ -702,7 +702,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float f = fmaf(o - 128.0f, xs[r], v[e][r]) * s;
-        tile_out[4 * h + r][cl] = (p.out_dtype == DT_BF16) ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+        tile_out[4 * h + r][cl] = half_out(p, f);
       }
     }
   }

@@ -159,7 +159,8 @@ __device__ __forceinline__ T4Tile t4_locate(const int *meta_end, const int *meta
 // blocks; staging quad (u, wave) is block 4 u + wave = (column group 2 u + wave / 2, K block wave % 2) and goes to LDS as
 // it is, so only the global offsets and the weight fragment addresses differ: MFMA row r of a 32-row block is column
 // t4_col_of_q(r), K quarter q is K block q / 2, 16-byte chunks 2 (q % 2) + hh.
-template <int MODE, bool PK>
+// ACT: an activation (p.act_type) follows the dequantisation; a template flag so that the plain epilogue stays as it is.
+template <int MODE, bool PK, bool ACT>
 __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const GmmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -590,7 +591,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
             }
         }
       };
-      auto compute = [&](auto u_c) {
+      auto compute = [&](auto u_c) __attribute__((always_inline)) {
         constexpr int U = decltype(u_c)::value, PIECE = U / T4_F, I = U % T4_F;
         const float pt = tb_pt[32 * I + e_l32];
 #pragma unroll
@@ -618,6 +619,17 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
               float v[8];
 #pragma unroll
               for (int j = 0; j < 8; ++j) v[j] = dequant(a8[j], __uint_as_float(sraw[ff][s2][j]), pt);
+              if constexpr (ACT) {
+                // one value after the other (the empty asm statements keep their order): eight exponentials in flight at
+                // once would need registers that this kernel does not have
+                const ActCoeffs ac = act_coeffs(p.act_type);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                  asm volatile("" : "+v"(v[j]));
+                  v[j] = activate(v[j], ac);
+                  asm volatile("" : "+v"(v[j]));
+                }
+              }
               uint4 r;
               if constexpr (MODE == 0) {
                 r.x = pack_bf16x2(v[0], v[1]); r.y = pack_bf16x2(v[2], v[3]);
@@ -679,9 +691,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   }
 }
 
-template <int MODE, bool PK>
+template <int MODE, bool PK, bool ACT>
 static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t stream) {
-  auto kern = gmm_w8a8_tile4_nk_kernel<MODE, PK>;
+  auto kern = gmm_w8a8_tile4_nk_kernel<MODE, PK, ACT>;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -702,10 +714,16 @@ hipError_t launch_tile4_w8a8_nk(const GmmParams &p, bool packed, hipStream_t str
   long long grid = ((total_ub + kNumXcd - 1) / kNumXcd) * kNumXcd;
   if (grid > T4_MAX_WGS) grid = T4_MAX_WGS;
   if (grid <= 0) return hipSuccess;
+  const bool act = p.act_type != ACT_NONE;
+  const unsigned g = (unsigned)grid;
   switch (p.out_dtype) {
-    case DT_BF16: return packed ? t4_launch<0, true>(p, (unsigned)grid, stream) : t4_launch<0, false>(p, (unsigned)grid, stream);
-    case DT_F16: return packed ? t4_launch<1, true>(p, (unsigned)grid, stream) : t4_launch<1, false>(p, (unsigned)grid, stream);
-    case DT_I32: return packed ? t4_launch<2, true>(p, (unsigned)grid, stream) : t4_launch<2, false>(p, (unsigned)grid, stream);
+    case DT_BF16:
+      if (act) return packed ? t4_launch<0, true, true>(p, g, stream) : t4_launch<0, false, true>(p, g, stream);
+      return packed ? t4_launch<0, true, false>(p, g, stream) : t4_launch<0, false, false>(p, g, stream);
+    case DT_F16:
+      if (act) return packed ? t4_launch<1, true, true>(p, g, stream) : t4_launch<1, false, true>(p, g, stream);
+      return packed ? t4_launch<1, true, false>(p, g, stream) : t4_launch<1, false, false>(p, g, stream);
+    case DT_I32: return packed ? t4_launch<2, true, false>(p, g, stream) : t4_launch<2, false, false>(p, g, stream);
     default: return hipErrorInvalidValue;
   }
 }

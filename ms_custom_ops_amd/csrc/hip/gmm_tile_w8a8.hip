@@ -538,6 +538,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
             float v[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) v[j] = dequant(acc[f][i][8 * s2 + j] + bi[j], sc[j], pt[i]);
+            if (p.act_type != ACT_NONE) {
+#pragma unroll
+              for (int j = 0; j < 8; ++j) v[j] = activate(v[j], p.act_type);
+            }
             uint4 q;
             if (p.out_dtype == DT_BF16) {
               q.x = pack_bf16x2(v[0], v[1]); q.y = pack_bf16x2(v[2], v[3]);

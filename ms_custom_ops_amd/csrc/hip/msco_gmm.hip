@@ -79,6 +79,9 @@ int check_desc(const msco_gmm_desc &d) {
   if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
   if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_256_W4) return MSCO_ERR_INVALID_ARG;
   if (d.weight_layout != MSCO_WL_ROW_MAJOR && d.weight_layout != MSCO_WL_PACKED) return MSCO_ERR_INVALID_ARG;
+  if (d.act_type < MSCO_ACT_NONE || d.act_type > MSCO_ACT_SILU) return MSCO_ERR_INVALID_ARG;
+  if (d.act_type == MSCO_ACT_GELU_ERF) return MSCO_ERR_UNSUPPORTED;
+  if (d.act_type != MSCO_ACT_NONE && d.out_dtype == MSCO_DT_I32) return MSCO_ERR_UNSUPPORTED;
   if (is_w8a8(d)) {
     if (d.out_dtype != MSCO_DT_BF16 && d.out_dtype != MSCO_DT_F16 && d.out_dtype != MSCO_DT_I32)
       return MSCO_ERR_UNSUPPORTED;
@@ -417,6 +420,7 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   p.n_strips = h->n_strips;
   p.max_chunks = h->max_chunks;
   p.strip_groups = h->strip_groups;
+  p.act_type = d.act_type;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t err = hipSuccess;

@@ -12,8 +12,9 @@
 //     (bf16/f16 x, int8 weight, antiquant scale and offset [E,N]);
 //   * group_type -1 (independent x[i] @ weight[i]) is one dense launch per pair.
 // Not implemented on this backend and refused with a message: float x float matmuls, int4 weights,
-// uint64 scales with int8 output, `offset`, the activation inputs, act_type != 0, FRACTAL_NZ weights,
-// group_type 1.
+// uint64 scales with int8 output, `offset`, the activation inputs, group_type 1.  act_type selects an activation
+// fused into the epilogue (0 none, 1 relu, 2 gelu_tanh, 4 fast_gelu, 5 silu: the values of CANN's GMMActType, which the
+// reference passes through without naming them).
 #include <optional>
 #include <string>
 #include <vector>
@@ -43,9 +44,15 @@ void CheckV4Support(const V4Args &a) {
     MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", weight_format must be 'ND' or 'FRACTAL_NZ', but got '"
                      << a.weight_format << "'.";
   }
-  if (a.act_type != 0 || !a.activation_input.empty() || !a.activation_quant_scale.empty() ||
-      !a.activation_quant_offset.empty()) {
-    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", fused activation is not implemented by the HIP backend.";
+  // act_type goes to the backend as the reference hands it to aclnnGroupedMatmulV4 (grouped_matmul_v4_cops.cc:96,363):
+  // 0 none, 1 relu, 2 gelu (tanh form), 4 fast gelu, 5 silu; 3 (gelu, erf form) is the value CANN itself lists as unsupported
+  if (a.act_type < MSCO_ACT_NONE || a.act_type > MSCO_ACT_SILU || a.act_type == MSCO_ACT_GELU_ERF) {
+    MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", act_type must be 0 (none), 1 (relu), 2 (gelu_tanh), "
+                       << "4 (fast_gelu) or 5 (silu), but got " << a.act_type;
+  }
+  if (!a.activation_input.empty() || !a.activation_quant_scale.empty() || !a.activation_quant_offset.empty()) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName
+                     << ", 'activation_input', 'activation_quant_scale' and 'activation_quant_offset' are not implemented by the HIP backend.";
   }
   if (!a.offset.empty()) {
     MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", 'offset' is not implemented by the HIP backend.";
@@ -72,7 +79,7 @@ void CheckV4Support(const V4Args &a) {
 void LaunchOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias, const ms::Tensor &scale,
                const ms::Tensor &aq_scale, const ms::Tensor &aq_offset, const ms::Tensor &per_token,
                const ms::Tensor &group_list, int64_t group_list_type, const ms::Tensor &out, int64_t m, int64_t k,
-               int64_t n, int64_t e, bool packed, void *stream) {
+               int64_t n, int64_t e, bool packed, int64_t act_type, void *stream) {
   const std::string op_name = "GroupedMatmulV4";
   const TypeId xt = x.data_type();
   msco_gmm_desc d{};
@@ -84,6 +91,11 @@ void LaunchOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias,
   d.group_list_type = static_cast<int32_t>(group_list_type);
   d.scale_per_group = 1;
   d.weight_layout = packed ? MSCO_WL_PACKED : MSCO_WL_ROW_MAJOR;
+  if (act_type != MSCO_ACT_NONE && out.data_type() == kNumberTypeInt32) {
+    MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", act_type " << act_type
+                       << " needs a floating-point output (give 'scale'), but the output is Int32.";
+  }
+  d.act_type = static_cast<int32_t>(act_type);
   const void *addrs[MSCO_IN_COUNT] = {nullptr};
   addrs[MSCO_IN_X] = x.GetDataPtr();
   addrs[MSCO_IN_WEIGHT] = w.GetDataPtr();
@@ -177,7 +189,7 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
                          << " elements, but got " << a.group_list.data_type() << " " << a.group_list.shape();
     }
     LaunchOne(x, w, At(a.bias, 0), At(a.scale, 0), At(a.antiquant_scale, 0), At(a.antiquant_offset, 0),
-              At(a.per_token_scale, 0), a.group_list, a.group_list_type, outputs.at(0), m, k, n, e, packed, stream);
+              At(a.per_token_scale, 0), a.group_list, a.group_list_type, outputs.at(0), m, k, n, e, packed, a.act_type, stream);
     return;
   }
   if (a.group_type != kGroupTypeMultiOutput) {
@@ -202,7 +214,7 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
     }
     const int64_t rows = k > 0 ? x.numel() / k : 0;
     LaunchOne(x, w, At(a.bias, i), At(a.scale, i), At(a.antiquant_scale, i), At(a.antiquant_offset, i),
-              At(a.per_token_scale, i), ms::Tensor(), 0, outputs.at(i), rows, k, n, 1, packed, stream);
+              At(a.per_token_scale, i), ms::Tensor(), 0, outputs.at(i), rows, k, n, 1, packed, a.act_type, stream);
   }
 }
 }  // namespace

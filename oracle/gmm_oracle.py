@@ -18,6 +18,10 @@ its own system tests (the device kernels themselves are closed binaries):
 * int64 dense scale format    tests/st/test_quant_batch_matmul.py:34-42  (trans_quant_param)
 * count-based comparator      tests/st/st_utils.py:23-49             (custom_compare)
 * A8W4 golden and nibble pack tests/st/test_grouped_matmul_w4.py:91-97,100-118
+* fused activation            PARITY UNPINNED BY THE REFERENCE: act_type is passed through to aclnnGroupedMatmulV4
+                              (ops/c_api/grouped_matmul_v4_cops/grouped_matmul_v4_cops.cc:96,112,363) without values, a
+                              description or a golden (grouped_matmul_v4_cops_doc.md:26 is one line); ``activation``
+                              takes the values of CANN's GMMActType and the functions' textbook forms.
 
 How each function is pinned (tests/test_oracle_pins.py):
 
@@ -39,6 +43,9 @@ How each function is pinned (tests/test_oracle_pins.py):
 * ``a16w8_*``              float64 evaluation of x @ ((w + o) * s) on the exact
                            bf16 operand values; closed forms with constant scale.
 * ``decode_scale_int64``   round trip against the two wire formats above.
+* ``activation``           what the mathematics fixes: torch's relu / silu / gelu(approximate="tanh") in float64,
+                           the tanh form of the gelu against the sigmoid form used here, CANN's published fast-gelu
+                           expression against x * sigmoid(1.702 x), silu(x) - silu(-x) = x, limits at +-40.
 * ``pack_int4`` / ``unpack_int4``   per-element loops, hand-written bytes, round trip.
 * ``golden_grouped_a8w4``  a float64 evaluation of the integer form
                            x_scale * sum_g scale_g * (exact int32 sum over the K group), a brute-force loop on a tiny
@@ -54,8 +61,12 @@ __all__ = [
     "group_bounds", "grouped_int32_acc", "dequant_epilogue", "grouped_matmul_w8a8", "golden_np_qbmm",
     "golden_grouped_w8a8", "golden_v4_pertoken", "golden_v4_perchannel_bias", "golden_v4_a16w8",
     "quant_batch_matmul_oracle", "a16w8_grouped_f64", "encode_scale_int64", "encode_scale_int64_qbmm", "pack_weights",
-    "decode_scale_int64", "random_group_list", "count_compare", "bf16_ulp_check",
+    "decode_scale_int64", "random_group_list", "count_compare", "bf16_ulp_check", "activation",
+    "ACT_NONE", "ACT_RELU", "ACT_GELU_TANH", "ACT_GELU_ERF", "ACT_FAST_GELU", "ACT_SILU",
 ]
+
+# act_type values (CANN's GMMActType; 3, the erf form of the gelu, is the one CANN lists as unsupported)
+ACT_NONE, ACT_RELU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_FAST_GELU, ACT_SILU = range(6)
 
 # K-chunk for the exact accumulator: 127*127*1024 = 16 516 096 < 2**24, so every
 # partial sum inside one chunk is an integer that float32 represents exactly.
@@ -205,6 +216,26 @@ def dequant_epilogue(acc, bias=None, scale=None, per_token=None, out_dtype: str 
     if out_dtype == "bf16":
         return f32_to_bf16_bits(f)
     raise ValueError(out_dtype)
+
+
+def activation(v, act_type: int) -> np.ndarray:
+    """Activation of the dequantised float32 values, evaluated in float64 (the caller rounds to the output type).
+    relu max(v, 0); gelu_tanh v * sigmoid(2 sqrt(2/pi) (v + 0.044715 v^3)); fast_gelu v * sigmoid(1.702 v);
+    silu v * sigmoid(v).  sigmoid(t) is taken as exp(-logaddexp(0, -t)), which neither overflows nor cancels."""
+    v = np.asarray(v, dtype=np.float32).astype(np.float64)
+    if act_type == ACT_NONE:
+        return v
+    if act_type == ACT_RELU:
+        return np.where(v < 0, 0.0, v)
+    if act_type == ACT_GELU_TANH:
+        t = 2.0 * np.sqrt(2.0 / np.pi) * (v + 0.044715 * v ** 3)
+    elif act_type == ACT_FAST_GELU:
+        t = 1.702 * v
+    elif act_type == ACT_SILU:
+        t = v
+    else:
+        raise ValueError(f"act_type {act_type} is not supported")
+    return v * np.exp(-np.logaddexp(0.0, -t))
 
 
 def _rows_of(param, starts, ends, m):

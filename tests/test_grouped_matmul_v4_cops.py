@@ -179,8 +179,6 @@ def test_v4_errors(device):
         f([x], [w], group_list=gl, split_item=3, group_type=0, weight_format="FRACTAL_NZ")
     with pytest.raises(RuntimeError, match="weight_format must be 'ND' or 'FRACTAL_NZ'"):
         f([x], [w], group_list=gl, split_item=3, group_type=0, weight_format="NC1HWC0")
-    with pytest.raises(RuntimeError, match="fused activation is not implemented"):
-        f([x], [w], group_list=gl, split_item=3, group_type=0, act_type=1)
     with pytest.raises(RuntimeError, match="quantized paths only"):
         f([x.bfloat16()], [w.bfloat16()], group_list=gl, split_item=3, group_type=0)
     with pytest.raises(ValueError, match="group_type 0 needs 'group_list'"):

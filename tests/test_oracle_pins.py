@@ -339,3 +339,33 @@ def test_a8w4_golden_against_integer_form_bruteforce_and_closed_forms():
     ref = np.concatenate([x[0:2].astype(np.int64) @ wq[0].astype(np.int64), x[2:7].astype(np.int64) @ wq[2].astype(np.int64),
                           x[7:9].astype(np.int64) @ wq[3].astype(np.int64)])
     assert np.array_equal(got, ref.astype(np.float32))
+
+
+# ---------------------------------------------------------------- fused activation (no golden in the reference)
+def test_activation_against_torch_other_formulations_and_identities():
+    rng = np.random.default_rng(5)
+    v = np.concatenate([rng.uniform(-60, 60, 4000), rng.uniform(-3, 3, 4000), [0.0, -0.0, 40.0, -40.0, 1e-6, -1e-6]]).astype(np.float32)
+    t = torch.from_numpy(v).double()
+    close = lambda a, b: np.allclose(a, b, rtol=1e-12, atol=1e-300)
+    # library routines in float64
+    assert np.array_equal(O.activation(v, O.ACT_NONE), v.astype(np.float64))
+    assert np.array_equal(O.activation(v, O.ACT_RELU), torch.relu(t).numpy())
+    assert close(O.activation(v, O.ACT_SILU), torch.nn.functional.silu(t).numpy())
+    # (torch's tanh form cancels for very negative arguments where the sigmoid form does not: compare where it is accurate)
+    mid = np.abs(v) < 4
+    assert np.allclose(O.activation(v, O.ACT_GELU_TANH)[mid], torch.nn.functional.gelu(t, approximate="tanh").numpy()[mid], rtol=1e-9, atol=0)
+    # the textbook tanh form against the sigmoid form used by the oracle
+    x = v.astype(np.float64)
+    tanh_form = 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x ** 3)))
+    assert np.allclose(O.activation(v, O.ACT_GELU_TANH)[mid], tanh_form[mid], rtol=1e-9, atol=0)
+    # CANN's published fast-gelu expression x / (1 + exp(-1.702 |x|)) * exp(0.851 (x - |x|)) is x * sigmoid(1.702 x)
+    cann = x / (1.0 + np.exp(-1.702 * np.abs(x))) * np.exp(0.851 * (x - np.abs(x)))
+    assert close(O.activation(v, O.ACT_FAST_GELU), cann)
+    # identities and limits: x * sigmoid(t(x)) with an odd t gives f(x) - f(-x) = x; f(40) = 40 and f(-40) = -0 to double precision
+    for act in (O.ACT_SILU, O.ACT_FAST_GELU, O.ACT_GELU_TANH):
+        f = lambda a: O.activation(np.asarray(a, dtype=np.float32), act)
+        assert np.allclose(f(v) - f(-v), x, rtol=1e-12, atol=1e-12)
+        assert abs(f([40.0])[0] - 40.0) < 1e-12 and abs(f([-40.0])[0]) < 1e-12
+        assert f([0.0])[0] == 0.0
+    with pytest.raises(ValueError):
+        O.activation(v, O.ACT_GELU_ERF)
