@@ -2,7 +2,7 @@
 """Benchmark of the grouped W8A8 matmul path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout packed|nk|kn] [--no-sweep] [--no-cpu]
-    python bench.py --probe c3|c2_m16|...|copy|moe|mfma [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs)
+    python bench.py --probe c3|c2_m16|...|copy|moe|mfma|read [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs)
 
 A step is one pass of the hot path over one batch of synthetic input (inputs resident in HBM before
 the timed region).  The headline workload is the Mixtral-shaped MoE configuration (E=8, top-2 over
@@ -331,6 +331,45 @@ def mfma_pipe_probe(iters=20000, launches=12):
     return out
 
 
+def read_floor(sizes=(45.09e6, 469.8e6), steps=60):
+    """Duration of one launch that only reads a buffer of the given size front to back (msco_probe_read), the floor under
+    a single-launch decode kernel whose weights have that size.  Successive launches read successive windows of a
+    buffer larger than the 256 MB memory-side cache, so every launch streams from HBM.  The best of a few workgroup
+    counts is reported."""
+    import torch
+    from ms_custom_ops_amd import cabi
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    out = []
+    for size in sizes:
+        size = int(size) // 4096 * 4096
+        windows = max(3, int(np.ceil(ROTATE_BYTES / size)) + 1)
+        buf = torch.randint(-127, 128, (windows * size,), dtype=torch.int8, device=dev)
+        best = None
+        for wgs in (256, 344, 512, 1024, 2048):
+            sink = torch.empty(wgs * 256, dtype=torch.int32, device=dev)
+            turn = [0]
+            def one():
+                turn[0] += 1
+                cabi.probe_read(buf.data_ptr() + (turn[0] % windows) * size, size, sink.data_ptr(), wgs, st)
+            for _ in range(10):
+                one()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(steps):
+                one()
+            b.record()
+            torch.cuda.synchronize()
+            sec = a.elapsed_time(b) / steps * 1e-3
+            if best is None or sec < best[0]:
+                best = (sec, wgs)
+        out.append({"bytes": size, "launch_us": best[0] * 1e6, "workgroups": best[1], "gbs": size / best[0] / 1e9,
+                    "hbm_frac": size / best[0] / 1e9 / PEAK_HBM_GBS})
+        del buf
+        torch.cuda.empty_cache()
+    return out
+
+
 def measured_traffic(workload, layout, kernel):
     """HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs (scaled by
     the same counters' reading for a copy of known size); None when no measurement of this kernel is on file."""
@@ -354,6 +393,9 @@ def probe(args):
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"probe": "copy", "bytes_read": COPY_BYTES, "bytes_written": COPY_BYTES, "launches": args.steps}))
+        return
+    if args.probe == "read":
+        print(json.dumps({"probe": "read", "read_floor": read_floor()}))
         return
     if args.probe == "mfma":
         print(json.dumps({"probe": "mfma", "mfma_pipe": mfma_pipe_probe()}))
@@ -448,6 +490,7 @@ def main():
         result["sweep"] = sweep
         result["moe_neighbours"] = moe_neighbours(max(20, min(100, args.steps)), 10)
         result["mfma_pipe"] = mfma_pipe_probe()
+        result["read_floor"] = read_floor()
         # the headline kernel once more on all-zero x and weights: same instruction stream and memory traffic, but the
         # matrix pipe toggles nothing, so the chip holds a higher clock; the gap to the figure above is what the
         # operand distribution costs, the gap to the peak is what the kernel's own stalls and padding cost

@@ -134,7 +134,8 @@ typedef struct msco_gmm_desc {
   int32_t kernel_override;   /* 0 auto; else force a kernel family (see msco_gmm_plan_info), for tests */
   int32_t weight_layout;     /* MSCO_WL_ROW_MAJOR: as transpose_b says; MSCO_WL_PACKED: written by msco_pack_weight */
   int32_t act_type;          /* msco_act: activation applied to the dequantised float32 value before the output cast */
-  int32_t reserved[3];
+  int32_t force_split_k;     /* 0 auto; else the K split across workgroups of the kernels that have one, for tests */
+  int32_t reserved[2];
 } msco_gmm_desc;
 
 typedef struct msco_gmm_op *msco_gmm_handle;
@@ -208,6 +209,12 @@ MSCO_API int msco_pack_weight(const void *src, void *dst, int64_t e, int64_t k, 
 #define MSCO_PROBE_MFMA_WORKGROUPS 256
 #define MSCO_PROBE_MFMA_OPERAND_BYTES (8 * 256 * 16)
 MSCO_API int msco_probe_mfma(const void *operands, void *sink, int32_t iters, void *stream);
+
+/* Measurement aid with no counterpart in the reference: one launch that only reads `bytes` bytes (rounded down to a
+ * multiple of 4096) front to back with `workgroups` workgroups of 256 threads, each taking one contiguous share in the
+ * access pattern of the packed-layout decode kernels.  Its duration is the floor under any single-launch decode kernel
+ * whose weights have that size.  `sink` receives workgroups * 256 int32 values of no meaning. */
+MSCO_API int msco_probe_read(const void *src, size_t bytes, void *sink, int32_t workgroups, void *stream);
 
 /* Static text for a status code. */
 MSCO_API const char *msco_status_string(int status);

@@ -36,7 +36,7 @@ EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
                     "msco_packed_weight_bytes", "msco_pack_weight", "msco_gmm_a8w4",
                     "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_init_routing_v2_quant",
-                    "msco_moe_token_unpermute", "msco_probe_mfma", "msco_gmm_launch_static")
+                    "msco_moe_token_unpermute", "msco_probe_mfma", "msco_probe_read", "msco_gmm_launch_static")
 STATIC_WORKSPACE_BYTES = 32 << 20
 PROBE_MFMA_WORKGROUPS, PROBE_MFMA_OPERAND_BYTES = 256, 8 * 256 * 16
 
@@ -45,7 +45,7 @@ class GmmDesc(ctypes.Structure):
     _fields_ = [(name, ctypes.c_int32) for name in (
         "abi_version", "x_dtype", "weight_dtype", "out_dtype", "group_list_dtype", "group_list_type", "bias_dtype",
         "scale_dtype", "per_token_dtype", "antiquant_dtype", "has_antiquant_offset", "transpose_b", "scale_per_group",
-        "scale_is_scalar", "kernel_override", "weight_layout", "act_type")] + [("reserved", ctypes.c_int32 * 3)]
+        "scale_is_scalar", "kernel_override", "weight_layout", "act_type", "force_split_k")] + [("reserved", ctypes.c_int32 * 2)]
 
 
 class BackendError(RuntimeError):
@@ -103,6 +103,8 @@ def load():
         lib.msco_moe_token_unpermute.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int64] * 3 + [ctypes.c_int32, ctypes.c_void_p]
         lib.msco_gmm_launch_static.restype = ctypes.c_int
         lib.msco_gmm_launch_static.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_void_p]
+        lib.msco_probe_read.restype = ctypes.c_int
+        lib.msco_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
         lib.msco_probe_mfma.restype = ctypes.c_int
         lib.msco_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
         _lib = lib
@@ -149,6 +151,12 @@ def probe_mfma(operands: int, sink: int, iters: int, stream: Optional[int] = Non
     operations per launch."""
     vp = lambda v: ctypes.c_void_p(v if v else None)
     _check("msco_probe_mfma", load().msco_probe_mfma(vp(operands), vp(sink), iters, vp(stream)))
+
+
+def probe_read(src: int, nbytes: int, sink: int, workgroups: int, stream: Optional[int] = None):
+    """Raw-pointer call of msco_probe_read (see include/msco_gmm.h)."""
+    vp = lambda v: ctypes.c_void_p(v if v else None)
+    _check("msco_probe_read", load().msco_probe_read(vp(src), nbytes, vp(sink), workgroups, vp(stream)))
 
 
 def moe_init_routing_v2_workspace_bytes(num_rows: int, k: int, expert_num: int) -> int:

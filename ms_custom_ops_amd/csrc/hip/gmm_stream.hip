@@ -90,7 +90,10 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
   extern __shared__ __align__(16) unsigned char st_smem[];
   v4i(*red)[ST_GROUPS][64] = reinterpret_cast<v4i(*)[ST_GROUPS][64]>(st_smem);   // [wave][column group][lane]
   unsigned *s_ticket = reinterpret_cast<unsigned *>(st_smem + ST_LDS - 16);
-  constexpr int D = NB < 8 ? NB : 8;   // loads in flight per wave
+#ifndef MSCO_STREAM_DEPTH
+#define MSCO_STREAM_DEPTH 8
+#endif
+  constexpr int D = NB < MSCO_STREAM_DEPTH ? NB : MSCO_STREAM_DEPTH;   // loads in flight per wave
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -138,6 +141,21 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
     constexpr int J = decltype(j_c)::value;
     if constexpr (J < D) issue(0, j_c, j_c);
   });
+  // epilogue operands of this thread's outputs (column groups wave + 4 e, rows 4 h .. 4 h + 3), requested behind the
+  // first weight loads so that they are in registers long before the stream ends: a memory round trip after the
+  // reduction is as long as a tenth of the whole kernel on a 45 MB weight set
+  const bool rows_ok = 4 * h < chunk_rows;  // at least one of the lane's 4 rows is part of the chunk
+  int ep_bias[4];
+  float ep_scale[4], pt[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int n = n0 + 16 * (wave + 4 * e) + c16;
+    const bool live = wave + 4 * e < cg_count && n < p.n && rows_ok;
+    ep_bias[e] = live ? load_bias(p, grp, n) : 0;
+    ep_scale[e] = (live && p.out_dtype != DT_I32) ? load_scale(p, grp, n) : 1.0f;
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) pt[r] = (p.per_token && 4 * h + r < chunk_rows) ? p.per_token[m0 + 4 * h + r] : 1.0f;
   for (int cg = 0; cg < cg_count; ++cg) {
     v4i a0 = v4i{0, 0, 0, 0}, a1 = v4i{0, 0, 0, 0};
     static_for<NB>([&](auto j_c) {
@@ -166,7 +184,6 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
     }
     v[e] = s;
   }
-  const bool rows_ok = 4 * h < chunk_rows;  // at least one of the lane's 4 rows is part of the chunk
 
   if (p.split_k > 1) {
     // cross-workgroup reduction through the workspace with agent-scope relaxed atomics (no cache-wide
@@ -214,9 +231,6 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
   }
 
   // ---- epilogue: v[e] = rows 4h..4h+3 of column 16 (wave + 4 e) + c ---------------------------------------
-  float pt[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) pt[r] = (p.per_token && 4 * h + r < chunk_rows) ? p.per_token[m0 + 4 * h + r] : 1.0f;
   unsigned short(*tile_out)[ST_COLS + 8] = reinterpret_cast<unsigned short(*)[ST_COLS + 8]>(st_smem);
   __syncthreads();  // every wave is done reading red[]
 #pragma unroll
@@ -224,14 +238,14 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
     const int cl = 16 * (wave + 4 * e) + c16;  // column inside the strip
     const int n = n0 + cl;
     if (wave + 4 * e < cg_count && n < p.n && rows_ok) {
-      const int bias = load_bias(p, grp, n);
+      const int bias = ep_bias[e];
       if (p.out_dtype == DT_I32) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)
           if (4 * h + r < chunk_rows)
             reinterpret_cast<int *>(p.out)[(long long)(m0 + 4 * h + r) * p.n + n] = v[e][r] + bias;
       } else {
-        const float sc = load_scale(p, grp, n);
+        const float sc = ep_scale[e];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const float f = dequant(v[e][r] + bias, sc, pt[r]);

@@ -30,7 +30,7 @@ constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-st
 constexpr int64_t kSkinnyMaxChunkSlots = 1024;   // (group, 16-row chunk) slots up to which many small groups take the decode kernels
 constexpr int kTargetWorkgroups = 512;  // skinny kernels with a K split: aim for this many workgroups (2 per CU)
 constexpr int kMaxSplitK = 8;             // keeps the last arriver's reduction to two rounds of loads
-constexpr int kNumCUs = 256;
+constexpr int kDefaultCUs = 256;   // MI355X; the plan uses the count the device reports
 constexpr int kTileTargetWorkgroups = 256;   // tile kernels with a K split: aim for this many workgroups (one per CU)
 constexpr int kTileSplitMaxTiles = 128;      // ... and only split below this many tiles (measured: beyond it the partial-tile exchange costs more than it hides)
 constexpr size_t kTileSplitMaxWorkspace = (size_t)128 << 20;   // bytes of split-K partial tiles a plan may ask the caller for
@@ -40,6 +40,21 @@ int env_int(const char *name, int fallback) {
   const char *v = std::getenv(name);
   return (v && *v) ? std::atoi(v) : fallback;
 }
+
+// Debug switches, read from the environment once per process (the first plan); planning itself reads no environment.
+struct Tuning {
+  int print_plan, tile_cfg, tile_target_wgs, tile_split_k, stream_max_slots, skinny_wide16, stream_min_wgs, stream_groups,
+      skinny_target_wgs, skinny_split_k;
+};
+const Tuning &tuning() {
+  static const Tuning t = {env_int("MSCO_PRINT_PLAN", 0),        env_int("MSCO_TILE_CFG", -1),
+                           env_int("MSCO_TILE_TARGET_WGS", 0),   env_int("MSCO_TILE_SPLIT_K", 0),
+                           env_int("MSCO_STREAM_MAX_SLOTS", 0),  env_int("MSCO_SKINNY_WIDE16", -1),
+                           env_int("MSCO_STREAM_MIN_WGS", 0),    env_int("MSCO_STREAM_GROUPS", 0),
+                           env_int("MSCO_SKINNY_TARGET_WGS", 0), env_int("MSCO_SKINNY_SPLIT_K", 0)};
+  return t;
+}
+int or_default(int v, int fallback) { return v > 0 ? v : fallback; }
 
 }  // namespace
 
@@ -59,6 +74,7 @@ struct msco_gmm_op {
   size_t workspace_bytes = 0;
   unsigned *counters = nullptr;
   size_t counters_cap = 0;
+  int num_cus = kDefaultCUs;   // compute units of the device that was current at create time
   std::string info;
   std::mutex mu;
 };
@@ -79,6 +95,7 @@ int check_desc(const msco_gmm_desc &d) {
   if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
   if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_256_W4) return MSCO_ERR_INVALID_ARG;
   if (d.weight_layout != MSCO_WL_ROW_MAJOR && d.weight_layout != MSCO_WL_PACKED) return MSCO_ERR_INVALID_ARG;
+  if (d.force_split_k < 0) return MSCO_ERR_INVALID_ARG;
   if (d.act_type < MSCO_ACT_NONE || d.act_type > MSCO_ACT_SILU) return MSCO_ERR_INVALID_ARG;
   if (d.act_type == MSCO_ACT_GELU_ERF) return MSCO_ERR_UNSUPPORTED;
   if (d.act_type != MSCO_ACT_NONE && d.out_dtype == MSCO_DT_I32) return MSCO_ERR_UNSUPPORTED;
@@ -112,6 +129,7 @@ int pow2_at_least(int v) {
 
 void choose_plan(msco_gmm_op *op) {
   const msco_gmm_desc &d = op->desc;
+  const int num_cus = op->num_cus;
   const int64_t m = op->m, k = op->k, n = op->n, e = op->e;
   const bool aligned = (k % 16 == 0) && (n % 16 == 0) && k >= 16 && n >= 16;
   op->split_k = 1;
@@ -174,7 +192,7 @@ void choose_plan(msco_gmm_op *op) {
   if ((family == FAM_TILE || family == FAM_SKINNY) && !(aligned && fits32)) family = FAM_GENERIC;
   if (family == FAM_TILE && !is_w8a8(d)) family = FAM_SKINNY;
   if (family == FAM_TILE) {
-    const int forced = env_int("MSCO_TILE_CFG", -1);
+    const int forced = tuning().tile_cfg;
     if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO) op->tile_cfg = forced;
     // Few tiles (M of a few hundred rows): split K across workgroups until about kTileTargetWorkgroups of them
     // stream operands; every slice keeps at least kTileMinSlabs 64-byte K slabs.  Small tile shapes only.
@@ -182,11 +200,11 @@ void choose_plan(msco_gmm_op *op) {
       int bm, bn;
       tile_cfg_dims(op->tile_cfg, &bm, &bn);
       const int64_t t = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
-      const int target = env_int("MSCO_TILE_TARGET_WGS", kTileTargetWorkgroups);
+      const int target = or_default(tuning().tile_target_wgs, kTileTargetWorkgroups);
       int want = t <= kTileSplitMaxTiles ? (int)((target + t / 2) / std::max<int64_t>(t, 1)) : 1;
       const int cap = (int)std::max<int64_t>(1, ((k + 63) / 64) / kTileMinSlabs);
       want = std::max(1, std::min(std::min(want, kMaxSplitK), cap));
-      const int forced_split = env_int("MSCO_TILE_SPLIT_K", 0);
+      const int forced_split = d.force_split_k > 0 ? d.force_split_k : tuning().tile_split_k;
       if (forced_split > 0) want = std::min(forced_split, cap);
       // the partial tiles of a K split are sized for the worst group_list (one partial m-tile per group): with many
       // groups that bound dwarfs the problem, so the split is halved until the workspace fits under the cap
@@ -201,7 +219,7 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t rows = e == 1 ? m : (m + e - 1) / e;
     op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
     // fewer, larger chunks when the (group, chunk) grid would be mostly empty slots
-    while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > env_int("MSCO_STREAM_MAX_SLOTS", (int)kSkinnyMaxChunkSlots))
+    while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch = op->stream_tch == 1 ? 2 : op->stream_tch * 2;
   }
   if (family == FAM_SKINNY) {
@@ -216,8 +234,8 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t active = std::max<int64_t>(
       1, std::min<int64_t>(e * op->max_chunks, std::min<int64_t>(m, e) + m / (kSkinnyRows * op->stream_tch)));
     const int64_t tiles128 = ((n + 127) / 128) * active;
-    int wide16 = is_w8a8(d) && tiles128 <= kNumCUs && !is_packed(d);
-    const int forced_variant = env_int("MSCO_SKINNY_WIDE16", -1);
+    int wide16 = is_w8a8(d) && tiles128 <= num_cus && !is_packed(d);
+    const int forced_variant = tuning().skinny_wide16;
     if (forced_variant >= 0 && is_w8a8(d)) wide16 = forced_variant != 0;
     op->skinny_wide16 = wide16;
     int want, cap;
@@ -238,9 +256,9 @@ void choose_plan(msco_gmm_op *op) {
       const int slice_blocks = is_w8a8(d) ? 128 : 64;
       const int floor_split = (int)((k_blocks + slice_blocks - 1) / slice_blocks);
       int groups = 16;
-      const int min_wgs = env_int("MSCO_STREAM_MIN_WGS", kNumCUs);
+      const int min_wgs = or_default(tuning().stream_min_wgs, num_cus);
       while (groups > 1 && ((col_groups + groups - 1) / groups) * active * floor_split < min_wgs) groups /= 2;
-      const int forced_groups = env_int("MSCO_STREAM_GROUPS", 0);
+      const int forced_groups = tuning().stream_groups;
       if (forced_groups >= 1 && forced_groups <= 16) groups = forced_groups;
       op->strip_groups = groups;
       op->n_strips = (int)((col_groups + groups - 1) / groups);
@@ -252,19 +270,19 @@ void choose_plan(msco_gmm_op *op) {
       cap = kMaxSplitK * 64;
     } else if (wide16) {
       // at most one 16-wave workgroup per CU, every wave keeps at least one block
-      want = (int)(kNumCUs / std::max<int64_t>(tiles128, 1));
+      want = (int)(num_cus / std::max<int64_t>(tiles128, 1));
       cap = std::max<int>(1, (int)(d.transpose_b ? (k + 63) / 64 : (k + 31) / 32) / 16);
       want = std::min(want, 8);
     } else {
       // K is split across workgroups until about kTargetWorkgroups of them stream weights
       const int64_t base = (int64_t)op->n_strips * active;
-      const int target = env_int("MSCO_SKINNY_TARGET_WGS", kTargetWorkgroups);
+      const int target = or_default(tuning().skinny_target_wgs, 2 * num_cus);
       want = (int)((target + base / 2) / base);
       cap = std::max<int>(1, (int)(d.transpose_b ? (k + 63) / 64 : (k + 31) / 32) / 4);
       want = std::min(want, kMaxSplitK);
     }
     want = std::max(1, std::min(want, cap));
-    const int forced = env_int("MSCO_SKINNY_SPLIT_K", 0);
+    const int forced = d.force_split_k > 0 ? d.force_split_k : tuning().skinny_split_k;
     if (forced > 0) want = std::min(forced, cap);
     if (is_packed(d) && op->stream_tch == 1) {   // also under a forced split
       const int slice_blocks = is_w8a8(d) ? 128 : 64;
@@ -326,6 +344,13 @@ int msco_gmm_create(const msco_gmm_desc *desc, msco_gmm_handle *out_handle) {
   msco_gmm_op *op = new (std::nothrow) msco_gmm_op();
   if (op == nullptr) return MSCO_ERR_DEVICE;
   op->desc = *desc;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+      cus > 0) {
+    op->num_cus = cus;
+  } else {
+    (void)hipGetLastError();   // no device yet: planning falls back to the MI355X count, launch reports the error
+  }
   *out_handle = op;
   return MSCO_OK;
 }
@@ -365,7 +390,7 @@ int msco_gmm_plan(msco_gmm_handle h, int64_t m, int64_t k, int64_t n, int64_t e,
   }
   h->planned = true;
   if (workspace_bytes) *workspace_bytes = h->workspace_bytes;
-  if (env_int("MSCO_PRINT_PLAN", 0)) std::fprintf(stderr, "%s\n", h->info.c_str());
+  if (tuning().print_plan) std::fprintf(stderr, "%s\n", h->info.c_str());
   return MSCO_OK;
 }
 

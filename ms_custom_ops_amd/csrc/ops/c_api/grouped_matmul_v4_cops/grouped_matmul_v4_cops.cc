@@ -75,14 +75,26 @@ void CheckV4Support(const V4Args &a) {
   }
 }
 
+// One backend launch: descriptor, problem size, positional device addresses and the output.
+struct OneLaunch {
+  msco_gmm_desc desc{};
+  GmmProblem problem{};
+  const void *addrs[MSCO_IN_COUNT] = {nullptr};
+  void *out{nullptr};
+};
+const char *const kBackendOpName = "GroupedMatmulV4";
+
 // One launch: x [M,K], weight [E,K,N], optional per-group rows of bias / scale / antiquant.
-void LaunchOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias, const ms::Tensor &scale,
-               const ms::Tensor &aq_scale, const ms::Tensor &aq_offset, const ms::Tensor &per_token,
-               const ms::Tensor &group_list, int64_t group_list_type, const ms::Tensor &out, int64_t m, int64_t k,
-               int64_t n, int64_t e, bool packed, int64_t act_type, void *stream) {
-  const std::string op_name = "GroupedMatmulV4";
+OneLaunch BuildOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias, const ms::Tensor &scale,
+                   const ms::Tensor &aq_scale, const ms::Tensor &aq_offset, const ms::Tensor &per_token,
+                   const ms::Tensor &group_list, int64_t group_list_type, const ms::Tensor &out, int64_t m, int64_t k,
+                   int64_t n, int64_t e, bool packed, int64_t act_type) {
   const TypeId xt = x.data_type();
-  msco_gmm_desc d{};
+  OneLaunch one;
+  one.problem = GmmProblem{m, k, n, e};
+  one.out = out.GetDataPtr();
+  msco_gmm_desc &d = one.desc;
+  const void **addrs = one.addrs;
   d.abi_version = MSCO_GMM_ABI_VERSION;
   d.x_dtype = ToBackendDtype(xt);
   d.weight_dtype = MSCO_DT_I8;
@@ -96,7 +108,6 @@ void LaunchOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias,
                        << " needs a floating-point output (give 'scale'), but the output is Int32.";
   }
   d.act_type = static_cast<int32_t>(act_type);
-  const void *addrs[MSCO_IN_COUNT] = {nullptr};
   addrs[MSCO_IN_X] = x.GetDataPtr();
   addrs[MSCO_IN_WEIGHT] = w.GetDataPtr();
   addrs[MSCO_IN_GROUP_LIST] = group_list.is_defined() ? group_list.GetDataPtr() : nullptr;
@@ -146,16 +157,12 @@ void LaunchOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &bias,
     addrs[MSCO_IN_ANTIQUANT_SCALE] = aq_scale.GetDataPtr();
     addrs[MSCO_IN_ANTIQUANT_OFFSET] = aq_offset.is_defined() ? aq_offset.GetDataPtr() : nullptr;
   }
-  auto plan = GmmPlanCache::GetInstance().GetOrCreate(op_name, d, GmmProblem{m, k, n, e}, stream);
-  ms::Tensor workspace;
-  if (plan->workspace_bytes > 0) {
-    workspace = AllocateTensor(kNumberTypeInt8, ShapeVector{static_cast<int64_t>(plan->workspace_bytes)});
-  }
-  LaunchPlan(op_name, plan, addrs, out.GetDataPtr(), workspace.is_defined() ? workspace.GetDataPtr() : nullptr,
-             plan->workspace_bytes, stream);
+  return one;
 }
 
-void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
+// The backend launches a call consists of, in order: one for group_type 0, one per (x[i], weight[i]) pair for -1.
+std::vector<OneLaunch> BuildLaunches(const V4Args &a, const TensorVec &outputs) {
+  std::vector<OneLaunch> launches;
   CheckV4Support(a);
   TensorVec all = a.x;
   for (const auto *v : {&a.weight, &a.bias, &a.scale, &a.antiquant_scale, &a.antiquant_offset, &a.per_token_scale}) {
@@ -164,7 +171,6 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
   all.push_back(a.group_list);
   CheckContiguous("GroupedMatmulV4", all, true);
   CheckContiguous("GroupedMatmulV4", outputs, false);
-  void *stream = CurrentStream();
 
   if (a.group_type == kGroupTypeSingleOutput) {
     const auto &x = a.x[0];
@@ -188,9 +194,10 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", 'group_list' must be Int64 with E = " << e
                          << " elements, but got " << a.group_list.data_type() << " " << a.group_list.shape();
     }
-    LaunchOne(x, w, At(a.bias, 0), At(a.scale, 0), At(a.antiquant_scale, 0), At(a.antiquant_offset, 0),
-              At(a.per_token_scale, 0), a.group_list, a.group_list_type, outputs.at(0), m, k, n, e, packed, a.act_type, stream);
-    return;
+    launches.push_back(BuildOne(x, w, At(a.bias, 0), At(a.scale, 0), At(a.antiquant_scale, 0), At(a.antiquant_offset, 0),
+                                At(a.per_token_scale, 0), a.group_list, a.group_list_type, outputs.at(0), m, k, n, e, packed,
+                                a.act_type));
+    return launches;
   }
   if (a.group_type != kGroupTypeMultiOutput) {
     MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", group_type " << a.group_type
@@ -213,9 +220,47 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
                          << "but got " << k << " and " << wk;
     }
     const int64_t rows = k > 0 ? x.numel() / k : 0;
-    LaunchOne(x, w, At(a.bias, i), At(a.scale, i), At(a.antiquant_scale, i), At(a.antiquant_offset, i),
-              At(a.per_token_scale, i), ms::Tensor(), 0, outputs.at(i), rows, k, n, 1, packed, a.act_type, stream);
+    launches.push_back(BuildOne(x, w, At(a.bias, i), At(a.scale, i), At(a.antiquant_scale, i), At(a.antiquant_offset, i),
+                                At(a.per_token_scale, i), ms::Tensor(), 0, outputs.at(i), rows, k, n, 1, packed, a.act_type));
   }
+  return launches;
+}
+
+// Pynative: plan (cached), take the workspace from the framework's allocator, launch.
+void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
+  void *stream = CurrentStream();
+  for (const OneLaunch &one : BuildLaunches(a, outputs)) {
+    auto plan = GmmPlanCache::GetInstance().GetOrCreate(kBackendOpName, one.desc, one.problem, stream);
+    ms::Tensor workspace;
+    if (plan->workspace_bytes > 0) {
+      workspace = AllocateTensor(kNumberTypeInt8, ShapeVector{static_cast<int64_t>(plan->workspace_bytes)});
+    }
+    LaunchPlan(kBackendOpName, plan, one.addrs, one.out, workspace.is_defined() ? workspace.GetDataPtr() : nullptr,
+               plan->workspace_bytes, stream);
+  }
+}
+
+V4Args ArgsFromGraphInputs(const KernelTensorList &inputs) {
+  V4Args args;
+  auto list = [&](size_t i) { return inputs[i].IsNone() ? TensorVec() : inputs[i].sequence; };
+  args.x = list(kXIndex);
+  args.weight = list(kWeightIndex);
+  args.bias = list(kBiasIndex);
+  args.scale = list(kScaleIndex);
+  args.offset = list(kOffsetIndex);
+  args.antiquant_scale = list(kAntiquantScaleIndex);
+  args.antiquant_offset = list(kAntiquantOffsetIndex);
+  args.per_token_scale = list(kPerTokenScaleIndex);
+  args.group_list = inputs[kGroupListIndex].tensor;
+  args.activation_input = list(kActivationInputIndex);
+  args.activation_quant_scale = list(kActivationInputIndex + 1);
+  args.activation_quant_offset = list(kActivationInputIndex + 2);
+  args.split_item = inputs[kSplitItemIndex].GetValueWithCheck<int64_t>();
+  args.group_type = inputs[kGroupTypeIndex].GetValueWithCheck<int64_t>();
+  args.group_list_type = inputs[kGroupListTypeIndex].GetValueWithCheck<int64_t>();
+  args.act_type = inputs[kActTypeIndex].GetValueWithCheck<int64_t>();
+  args.weight_format = inputs[kWeightFormatIndex].GetValueWithCheck<std::string>();
+  return args;
 }
 }  // namespace
 
@@ -224,43 +269,41 @@ void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
 // =============================================================================
 class GroupedMatmulV4CopsHip : public KernelMod {
  public:
-  // Resize = the reference's GetWorkSpaceInfo: recover the lists and the trailing scalars
-  // (grouped_matmul_v4_cops.cc:101-137).  Inputs arrive as twelve list slots followed by the scalars.
-  std::vector<size_t> Resize(const KernelTensorList &inputs, const std::vector<ms::Tensor> &) override {
+  // Resize = the reference's GetWorkSpaceInfo (grouped_matmul_v4_cops.cc:101-137): recover the lists and the trailing
+  // scalars (the inputs arrive as twelve list slots followed by the scalars), plan every backend launch of the call and
+  // return one workspace size per launch.  Only shapes, dtypes and scalars are kept: Launch reads the tensors it is
+  // given, as the reference's does (:85-96).
+  std::vector<size_t> Resize(const KernelTensorList &inputs, const std::vector<ms::Tensor> &outputs) override {
     group_info_ = FetchGroupInfo(inputs);
     start_idxs_ = ComputeStartIdxsFromGroupInfo(group_info_);
-    args_ = V4Args();
-    auto list = [&](size_t i) { return inputs[i].IsNone() ? TensorVec() : inputs[i].sequence; };
-    args_.x = list(kXIndex);
-    args_.weight = list(kWeightIndex);
-    args_.bias = list(kBiasIndex);
-    args_.scale = list(kScaleIndex);
-    args_.offset = list(kOffsetIndex);
-    args_.antiquant_scale = list(kAntiquantScaleIndex);
-    args_.antiquant_offset = list(kAntiquantOffsetIndex);
-    args_.per_token_scale = list(kPerTokenScaleIndex);
-    args_.group_list = inputs[kGroupListIndex].tensor;
-    args_.activation_input = list(kActivationInputIndex);
-    args_.activation_quant_scale = list(kActivationInputIndex + 1);
-    args_.activation_quant_offset = list(kActivationInputIndex + 2);
-    args_.split_item = inputs[kSplitItemIndex].GetValueWithCheck<int64_t>();
-    args_.group_type = inputs[kGroupTypeIndex].GetValueWithCheck<int64_t>();
-    args_.group_list_type = inputs[kGroupListTypeIndex].GetValueWithCheck<int64_t>();
-    args_.act_type = inputs[kActTypeIndex].GetValueWithCheck<int64_t>();
-    args_.weight_format = inputs[kWeightFormatIndex].GetValueWithCheck<std::string>();
-    return {};
+    std::vector<size_t> sizes;
+    void *stream = CurrentStream();
+    for (const OneLaunch &one : BuildLaunches(ArgsFromGraphInputs(inputs), outputs)) {
+      sizes.push_back(GmmPlanCache::GetInstance().GetOrCreate(kBackendOpName, one.desc, one.problem, stream)->workspace_bytes);
+    }
+    return sizes;
   }
 
-  bool Launch(const KernelTensorList &, const std::vector<ms::Tensor> &, const std::vector<ms::Tensor> &outputs,
-              void *) override {
-    RunGroupedMatmulV4(args_, outputs);
+  bool Launch(const KernelTensorList &inputs, const std::vector<ms::Tensor> &workspace, const std::vector<ms::Tensor> &outputs,
+              void *stream) override {
+    const std::vector<OneLaunch> launches = BuildLaunches(ArgsFromGraphInputs(inputs), outputs);
+    for (size_t i = 0; i < launches.size(); ++i) {
+      // the plan of the stream this launch goes to (a cache hit unless the stream changed since Resize)
+      auto plan = GmmPlanCache::GetInstance().GetOrCreate(kBackendOpName, launches[i].desc, launches[i].problem, stream);
+      const bool have = i < workspace.size() && workspace[i].is_defined();
+      if (plan->workspace_bytes > 0 && (!have || workspace[i].nbytes() < plan->workspace_bytes)) {
+        MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", Launch got no workspace of " << plan->workspace_bytes
+                         << " bytes for launch " << i << ": Resize must run when shapes change.";
+      }
+      LaunchPlan(kBackendOpName, plan, launches[i].addrs, launches[i].out, have ? workspace[i].GetDataPtr() : nullptr,
+                 have ? workspace[i].nbytes() : 0, stream);
+    }
     return true;
   }
 
   const std::vector<int64_t> &start_idxs() const { return start_idxs_; }
 
  private:
-  V4Args args_;
   std::vector<int64_t> group_info_{};
   std::vector<int64_t> start_idxs_{};
 };

@@ -104,7 +104,8 @@ class CustomGroupedMatmulW4 : public KernelMod {
  public:
   std::vector<size_t> Resize(const KernelTensorList &, const std::vector<ms::Tensor> &) override { return {}; }
   bool Launch(const KernelTensorList &inputs, const std::vector<ms::Tensor> &, const std::vector<ms::Tensor> &outputs,
-              void *) override {
+              void *stream) override {
+    LaunchStreamScope on_launch_stream(stream);   // the routine below enqueues on CurrentStream()
     RunGroupedMatmulW4(inputs[0].tensor, inputs[1].tensor, inputs[2].tensor, inputs[3].tensor, inputs[4].tensor,
                        inputs[5].tensor, outputs[0]);
     return true;

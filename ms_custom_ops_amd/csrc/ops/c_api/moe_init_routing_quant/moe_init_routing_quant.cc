@@ -100,7 +100,8 @@ class MoeInitRoutingQuantHip : public KernelMod {
  public:
   std::vector<size_t> Resize(const KernelTensorList &, const std::vector<ms::Tensor> &) override { return {}; }
   bool Launch(const KernelTensorList &inputs, const std::vector<ms::Tensor> &, const std::vector<ms::Tensor> &outputs,
-              void *) override {
+              void *stream) override {
+    LaunchStreamScope on_launch_stream(stream);   // the routine below enqueues on CurrentStream()
     RunMoeInitRoutingQuant(inputs[0].tensor, inputs[1].tensor, inputs[2].GetValueWithCheck<int64_t>(),
                            inputs[3].GetValueWithCheck<int64_t>(), outputs);
     return true;

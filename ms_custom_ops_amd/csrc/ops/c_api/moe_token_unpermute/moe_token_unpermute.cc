@@ -87,7 +87,8 @@ class MoeTokenUnpermuteHip : public KernelMod {
  public:
   std::vector<size_t> Resize(const KernelTensorList &, const std::vector<ms::Tensor> &) override { return {}; }
   bool Launch(const KernelTensorList &inputs, const std::vector<ms::Tensor> &, const std::vector<ms::Tensor> &outputs,
-              void *) override {
+              void *stream) override {
+    LaunchStreamScope on_launch_stream(stream);   // the routine below enqueues on CurrentStream()
     const bool padded = inputs.size() > 3 && !inputs[3].IsNone() && inputs[3].GetValueWithCheck<bool>();
     const bool restore = inputs.size() > 4 && !inputs[4].IsNone();
     RunMoeTokenUnpermute(inputs[0].tensor, inputs[1].tensor, inputs[2].tensor, padded, restore, outputs.at(0));

@@ -209,7 +209,8 @@ class QuantBatchMatmulCustomHip : public KernelMod {
     return {};  // workspace is requested from the framework inside the launch routine
   }
   bool Launch(const KernelTensorList &inputs, const std::vector<ms::Tensor> &, const std::vector<ms::Tensor> &outputs,
-              void *) override {
+              void *stream) override {
+    LaunchStreamScope on_launch_stream(stream);   // the routine below enqueues on CurrentStream()
     RunQuantBatchMatmul(inputs[kQbmmInputX1].tensor, inputs[kQbmmInputX2].tensor, inputs[kQbmmInputScale].tensor,
                         inputs[kQbmmInputOffset].tensor, inputs[kQbmmInputBias].tensor,
                         inputs[kQbmmInputPertokenScaleOptional].tensor, transpose_x1_, transpose_x2_, x2_format_,

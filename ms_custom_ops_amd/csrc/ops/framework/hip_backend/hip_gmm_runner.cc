@@ -128,15 +128,21 @@ std::vector<size_t> HipGmmKernelMod::Resize(const KernelTensorList &inputs, cons
   const TensorList backend_inputs = GetBackendInputs(inputs);
   CheckContiguous(kernel_name_, backend_inputs, true);
   CheckContiguous(kernel_name_, outputs, false);
-  const msco_gmm_desc desc = CreateKernel(inputs, backend_inputs, outputs);
-  const GmmProblem problem = GetProblem(inputs, backend_inputs, outputs);
-  plan_ = GmmPlanCache::GetInstance().GetOrCreate(kernel_name_, desc, problem, CurrentStream());
+  desc_ = CreateKernel(inputs, backend_inputs, outputs);
+  problem_ = GetProblem(inputs, backend_inputs, outputs);
+  plan_stream_ = CurrentStream();
+  plan_ = GmmPlanCache::GetInstance().GetOrCreate(kernel_name_, desc_, problem_, plan_stream_);
   return plan_->workspace_bytes ? std::vector<size_t>{plan_->workspace_bytes} : std::vector<size_t>{};
 }
 
 bool HipGmmKernelMod::Launch(const KernelTensorList &inputs, const std::vector<ms::Tensor> &workspace,
                              const std::vector<ms::Tensor> &outputs, void *stream) {
   if (plan_ == nullptr) MS_LOG_EXCEPTION << "For " << kernel_name_ << ", Launch called before Resize.";
+  if (stream != plan_stream_) {
+    // a kernel object keeps cross-workgroup reduction state and serves one stream: take the one of this stream
+    plan_ = GmmPlanCache::GetInstance().GetOrCreate(kernel_name_, desc_, problem_, stream);
+    plan_stream_ = stream;
+  }
   const TensorList backend_inputs = GetBackendInputs(inputs);
   const void *addrs[MSCO_IN_COUNT] = {nullptr};
   for (size_t i = 0; i < backend_inputs.size() && i < MSCO_IN_COUNT; ++i) {

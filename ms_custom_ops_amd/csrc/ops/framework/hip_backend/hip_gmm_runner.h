@@ -106,6 +106,9 @@ class HipGmmKernelMod : public KernelMod {
                                 const std::vector<ms::Tensor> &outputs) = 0;
   std::string kernel_name_;
   GmmPlanPtr plan_;
+  void *plan_stream_{nullptr};   // the stream plan_ belongs to (kernel objects are per stream)
+  msco_gmm_desc desc_{};         // what Resize planned for: Launch fetches the plan of its own stream with these
+  GmmProblem problem_{};
 };
 }  // namespace ms_custom_ops
 #endif  // MS_CUSTOM_OPS_HIP_GMM_RUNNER_H_

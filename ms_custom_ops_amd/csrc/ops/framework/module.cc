@@ -3,6 +3,10 @@
 // a registered op through infer -> KernelMod::Init -> Resize -> Launch.
 #include "ops/framework/module.h"
 
+#include <map>
+#include <mutex>
+#include <sstream>
+
 #include "ops/framework/hip_backend/hip_gmm_runner.h"
 
 namespace py = pybind11;
@@ -18,7 +22,22 @@ ms::Tensor AllocateTensor(TypeId type, const ShapeVector &shape) {
   return hooks.allocate(static_cast<int>(type), shape).cast<ms::Tensor>();
 }
 
+namespace {
+thread_local bool t_launch_stream_active = false;
+thread_local void *t_launch_stream = nullptr;
+}  // namespace
+
+LaunchStreamScope::LaunchStreamScope(void *stream) : prev_active_(t_launch_stream_active), prev_stream_(t_launch_stream) {
+  t_launch_stream_active = true;
+  t_launch_stream = stream;
+}
+LaunchStreamScope::~LaunchStreamScope() {
+  t_launch_stream_active = prev_active_;
+  t_launch_stream = prev_stream_;
+}
+
 void *CurrentStream() {
+  if (t_launch_stream_active) return t_launch_stream;
   auto &hooks = FrameworkHooks::Get();
   if (hooks.current_stream.is_none() || !hooks.current_stream) return nullptr;
   py::gil_scoped_acquire gil;
@@ -47,6 +66,51 @@ KernelTensor ToKernelTensor(const py::handle &obj) {
   return kt;
 }
 
+// What Resize depends on: kind, dtype and shape of every input and the values of the scalar attributes.
+std::string InputSignature(const KernelTensorList &inputs) {
+  std::ostringstream os;
+  auto tensor = [&](const ms::Tensor &t) {
+    os << (t.is_contiguous() ? 't' : 's') << static_cast<int>(t.data_type()) << '[';
+    for (int64_t d : t.shape()) os << d << ',';
+    os << ']';
+  };
+  for (const auto &in : inputs) {
+    if (in.IsNone()) {
+      os << "N;";
+    } else if (in.IsSequence()) {
+      os << 'L';
+      for (const auto &t : in.sequence) tensor(t);
+      os << ';';
+    } else if (in.tensor.is_defined()) {
+      tensor(in.tensor);
+      os << ';';
+    } else if (std::holds_alternative<bool>(in.value)) {
+      os << 'b' << std::get<bool>(in.value) << ';';
+    } else if (std::holds_alternative<int64_t>(in.value)) {
+      os << 'i' << std::get<int64_t>(in.value) << ';';
+    } else if (std::holds_alternative<std::string>(in.value)) {
+      os << 's' << std::get<std::string>(in.value) << ';';
+    } else {
+      os << "?;";
+    }
+  }
+  return os.str();
+}
+
+// One kernel module per operator, as a graph holds one per node: Init ran once, Resize runs again only when the
+// input signature changes (docs/ops_develop_guide.md:193-197).
+struct GraphNode {
+  std::shared_ptr<KernelMod> kernel;
+  std::string signature;
+  std::vector<size_t> workspace_sizes;
+  size_t inits{0}, resizes{0}, launches{0};
+};
+std::mutex g_nodes_mu;
+std::map<std::string, GraphNode> &GraphNodes() {
+  static auto *nodes = new std::map<std::string, GraphNode>();   // leaked: kernel modules may hold device state
+  return *nodes;
+}
+
 // Graph-mode execution of one registered op: the reference's compile-time infer plus the kernel
 // module life cycle (Init once per instance, Resize on new shapes, Launch).
 std::vector<ms::Tensor> GraphRun(const std::string &name, const py::list &args) {
@@ -60,9 +124,31 @@ std::vector<ms::Tensor> GraphRun(const std::string &name, const py::list &args) 
   if (shapes.size() != types.size()) MS_LOG_EXCEPTION << "For " << name << ", infer returned mismatching outputs.";
   std::vector<ms::Tensor> outputs;
   for (size_t i = 0; i < shapes.size(); ++i) outputs.push_back(AllocateTensor(types[i], shapes[i]));
-  auto kernel = reg->kernel_mod();
-  if (!kernel->Init(inputs, outputs)) MS_LOG_EXCEPTION << "For " << name << ", KernelMod::Init failed.";
-  const std::vector<size_t> ws_sizes = kernel->Resize(inputs, outputs);
+  std::shared_ptr<KernelMod> kernel;
+  std::vector<size_t> ws_sizes;
+  {
+    std::lock_guard<std::mutex> lock(g_nodes_mu);
+    GraphNode &node = GraphNodes()[name];
+    if (node.kernel == nullptr) {
+      node.kernel = reg->kernel_mod();
+      if (!node.kernel->Init(inputs, outputs)) {
+        node.kernel = nullptr;
+        MS_LOG_EXCEPTION << "For " << name << ", KernelMod::Init failed.";
+      }
+      ++node.inits;
+      node.signature.clear();
+    }
+    const std::string signature = InputSignature(inputs);
+    if (node.resizes == 0 || signature != node.signature) {
+      node.signature.clear();                       // stays empty if Resize throws: the next call plans again
+      node.workspace_sizes = node.kernel->Resize(inputs, outputs);
+      node.signature = signature;
+      ++node.resizes;
+    }
+    ++node.launches;
+    kernel = node.kernel;
+    ws_sizes = node.workspace_sizes;
+  }
   std::vector<ms::Tensor> workspace;
   for (size_t sz : ws_sizes) workspace.push_back(AllocateTensor(kNumberTypeInt8, ShapeVector{static_cast<int64_t>(sz)}));
   if (!kernel->Launch(inputs, workspace, outputs, CurrentStream())) {
@@ -111,6 +197,13 @@ PYBIND11_MODULE(MS_EXTENSION_NAME, m) {
     auto &c = ms_custom_ops::GmmPlanCache::GetInstance();
     return py::make_tuple(c.hits(), c.misses(), c.size());
   });
+  m.def("_graph_node_stats", [](const std::string &name) -> py::tuple {
+    std::lock_guard<std::mutex> lock(ms_custom_ops::g_nodes_mu);
+    auto &nodes = ms_custom_ops::GraphNodes();
+    auto it = nodes.find(name);
+    if (it == nodes.end()) return py::make_tuple(0, 0, 0);
+    return py::make_tuple(it->second.inits, it->second.resizes, it->second.launches);
+  }, "(Init, Resize, Launch) calls of an operator's graph-mode kernel module so far");
   m.def("_plan_cache_clear", []() { ms_custom_ops::GmmPlanCache::GetInstance().Clear(); });
   m.def("_backend_abi_version", []() { return msco_gmm_abi_version(); });
 

@@ -90,7 +90,20 @@ struct FrameworkHooks {
 };
 
 ms::Tensor AllocateTensor(TypeId type, const ShapeVector &shape);
+// The stream operator code enqueues on: the host framework's current stream, or -- inside a graph-mode
+// KernelMod::Launch -- the stream that Launch was given (LaunchStreamScope).
 void *CurrentStream();
+class LaunchStreamScope {
+ public:
+  explicit LaunchStreamScope(void *stream);
+  ~LaunchStreamScope();
+  LaunchStreamScope(const LaunchStreamScope &) = delete;
+  LaunchStreamScope &operator=(const LaunchStreamScope &) = delete;
+
+ private:
+  bool prev_active_;
+  void *prev_stream_;
+};
 
 class GilReleaseWithCheck {
  public:

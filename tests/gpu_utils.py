@@ -29,7 +29,7 @@ def pack_on_device(tw, e, k, n, src_transposed=False):
 
 def run_w8a8(x, w, group_list, bias=None, scale=None, per_token=None, *, out="bf16", transpose_b=False, override=0,
              group_list_type=0, gl_dtype=np.int64, scale_dtype=cabi.DT_F32, scale_per_group=1, scale_is_scalar=0,
-             launches=1, poison=True, packed=False, act_type=0):
+             launches=1, poison=True, packed=False, act_type=0, force_split_k=0):
     """x int8 [M,K]; w int8 [E,K,N] in logical layout (transposed here when transpose_b; with `packed` that row-major
     tensor is then packed on the device and the op reads the packed layout).  Returns (numpy output, plan info)."""
     m, k = x.shape
@@ -50,7 +50,7 @@ def run_w8a8(x, w, group_list, bias=None, scale=None, per_token=None, *, out="bf
                     per_token_dtype=cabi.DT_F32 if tp is not None else cabi.DT_NONE,
                     transpose_b=0 if packed else int(transpose_b), weight_layout=cabi.WL_PACKED if packed else cabi.WL_ROW_MAJOR,
                     scale_per_group=scale_per_group, scale_is_scalar=scale_is_scalar, kernel_override=override,
-                    act_type=act_type)
+                    act_type=act_type, force_split_k=force_split_k)
     ws = op.plan(m, k, n, e)
     tws = torch.empty(max(ws, 1), dtype=torch.uint8, device="cuda:0")
     fill = -7777 if raw else 0x7FC0  # poison: a value no correct run produces (bf16/f16 NaN pattern)

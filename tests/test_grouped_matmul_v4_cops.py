@@ -190,3 +190,27 @@ def test_v4_errors(device):
           group_type=0)
     with pytest.raises(TypeError):
         f(x, [w], group_list=gl)
+
+
+def test_graph_kernel_module_inits_once_resizes_on_new_shapes_and_reads_fresh_tensors(device):
+    """The graph-mode life cycle of the reference (docs/ops_develop_guide.md:193-197): Init once per node, Resize only
+    when shapes, dtypes or attributes change, Launch on the tensors of the call (not on those seen by Resize)."""
+    rng = np.random.default_rng(21)
+    stats = lambda: ms_custom_ops._C._graph_node_stats("grouped_matmul_v4_cops")
+    def run(m, seed):
+        r = np.random.default_rng(seed)
+        x = r.integers(-127, 128, (m, 64), dtype=np.int8)
+        w = r.integers(-127, 128, (8, 64, 128), dtype=np.int8)
+        counts = np.full(8, m // 8, dtype=np.int64)
+        with ms_custom_ops.exec_mode(ms_custom_ops.GRAPH_MODE):
+            out = ms_custom_ops.grouped_matmul_v4_cops([_t(x)], [_t(w)], group_list=_t(counts), split_item=3, group_type=0,
+                                                       group_list_type=1)[0]
+        assert np.array_equal(out.cpu().numpy(), O.grouped_matmul_w8a8(x, w, counts, group_list_type=1, out_dtype="i32"))
+    run(32, 1)
+    inits0, resizes0, launches0 = stats()
+    run(32, 2)          # same signature, other tensors (other device addresses, other values)
+    run(32, 3)
+    assert stats() == (inits0, resizes0, launches0 + 2)
+    run(64, 4)          # new shape: planned again, same kernel module
+    assert stats() == (inits0, resizes0 + 1, launches0 + 3)
+    assert inits0 == 1

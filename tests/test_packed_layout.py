@@ -20,18 +20,18 @@ def _inputs(seed, m, k, n, e):
     return x, w, bias, scale, pt
 
 
-def _check(x, w, gl, bias, scale, pt, *, src_transposed=False, override=cabi.OV_AUTO, group_list_type=0):
+def _check(x, w, gl, bias, scale, pt, *, src_transposed=False, override=cabi.OV_AUTO, group_list_type=0, split=0):
     from gpu_utils import run_w8a8
     _, ends = O.group_bounds(gl, group_list_type)
     last = int(ends[-1])
     ref_acc = O.grouped_matmul_w8a8(x, w, gl, bias, group_list_type=group_list_type, out_dtype="i32")
     ref_bits = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt, group_list_type=group_list_type)
     acc, info = run_w8a8(x, w, gl, bias, out="i32", transpose_b=src_transposed, override=override, packed=True,
-                         group_list_type=group_list_type, launches=2)
+                         group_list_type=group_list_type, launches=2, force_split_k=split)
     assert np.array_equal(acc[:last], ref_acc[:last]), info
     assert (acc[last:] == -7777).all(), info                       # rows past the last boundary stay untouched
     bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", transpose_b=src_transposed, override=override, packed=True,
-                          group_list_type=group_list_type, launches=2)
+                          group_list_type=group_list_type, launches=2, force_split_k=split)
     assert np.array_equal(bits[:last], ref_bits[:last]), info
     return info
 
@@ -67,10 +67,9 @@ def test_streaming_decode_kernel_is_bit_exact(device, m, k, n, e, gl):
 
 
 @pytest.mark.parametrize("split", [2, 3, 8])
-def test_streaming_decode_with_forced_k_split(device, split, monkeypatch):
-    monkeypatch.setenv("MSCO_SKINNY_SPLIT_K", str(split))
+def test_streaming_decode_with_forced_k_split(device, split):
     x, w, bias, scale, pt = _inputs(12, 21, 2048, 528, 2)
-    info = _check(x, w, [10, 21], bias, scale, pt, src_transposed=True)
+    info = _check(x, w, [10, 21], bias, scale, pt, src_transposed=True, split=split)
     assert f"split_k={split} " in info
 
 
@@ -102,10 +101,9 @@ def test_multi_row_streaming_kernel_is_bit_exact(device, m, k, n, e, gl):
     (128, 2048, 512, 1, [128], 0),                                  # few tiles: K split across workgroups
     (200, 720, 144, 2, [90, 200], 2),                               # forced K split, K not a multiple of 64
 ])
-def test_eight_wave_and_small_tile_kernels_on_packed_weights(device, monkeypatch, family, override, m, k, n, e, gl, split):
-    monkeypatch.setenv("MSCO_TILE_SPLIT_K", str(split))
+def test_eight_wave_and_small_tile_kernels_on_packed_weights(device, family, override, m, k, n, e, gl, split):
     x, w, bias, scale, pt = _inputs(19, m, k, n, e)
-    info = _check(x, w, gl, bias, scale, pt, override=override)
+    info = _check(x, w, gl, bias, scale, pt, override=override, split=split)
     assert f"tile_{family}" in info and "layout=packed" in info
 
 
