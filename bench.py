@@ -54,6 +54,7 @@ def parse():
                          "nk=[E,N,K] (prepacked once by a transpose), kn=[E,K,N] as generated")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--zero-operands", action="store_true", help="with --probe <workload>: all-zero x and weights (same kernel, nothing toggles)")
     ap.add_argument("--probe", default=None, help="workload name, `copy` or `moe` (the routing / un-permutation pair): launches only, for counter collection")
     return ap.parse_args()
 
@@ -61,7 +62,7 @@ def parse():
 class DeviceProblem:
     """One workload resident on the GPU plus a planned backend operator."""
 
-    def __init__(self, wl, layout="kn", copies=1, zero_operands=False, act_type=0):
+    def __init__(self, wl, layout="kn", copies=1, zero_operands=False, act_type=0, force_split_k=0):
         import torch
         from ms_custom_ops_amd import cabi
         self.torch, self.cabi, self.wl = torch, cabi, wl
@@ -115,7 +116,7 @@ class DeviceProblem:
             self.op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,
                                  scale_dtype=cabi.DT_F32, per_token_dtype=cabi.DT_F32,
                                  bias_dtype=cabi.DT_I32 if self.bias is not None else cabi.DT_NONE,
-                                 transpose_b=int(nk), act_type=act_type,
+                                 transpose_b=int(nk), act_type=act_type, force_split_k=force_split_k,
                                  weight_layout=cabi.WL_PACKED if layout == "packed" else cabi.WL_ROW_MAJOR)
         self.ws_bytes = self.op.plan(wl.m, wl.k, wl.n, wl.e)
         self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
@@ -404,11 +405,11 @@ def probe(args):
         print(json.dumps({"probe": "moe", "moe_neighbours": moe_neighbours(args.steps, 5)}))
         return
     wl = workloads.make(args.probe)
-    prob = DeviceProblem(wl, args.layout)
+    prob = DeviceProblem(wl, args.layout, zero_operands=args.zero_operands)
     for _ in range(args.steps):
         prob.step()
     torch.cuda.synchronize()
-    print(json.dumps({"probe": args.probe, "plan": prob.op.plan_info(), "launches": args.steps}))
+    print(json.dumps({"probe": args.probe, "zero_operands": args.zero_operands, "plan": prob.op.plan_info(), "launches": args.steps}))
 
 
 def main():
