@@ -1,7 +1,10 @@
 // MoE routing (stable counting sort of (token, k) entries by expert + activation gather) and weighted
 // un-permutation for gfx950.  Both are HBM-bound row copies around a small integer problem:
 //
-//   init_routing   (steps 1-3 are one launch for up to 16 blocks, every block repeating the small steps 1 and 2 for itself)
+//   init_routing   up to 16384 entries, plain row copy: ONE launch (route_fused_kernel): every workgroup counts all expert
+//                  ids itself, places its own 32 entries and copies their rows.  Otherwise (more entries, or the
+//                  quantising gather) the steps below; 1-3 are one launch for up to 16 blocks, every block repeating
+//                  the small steps 1 and 2 for itself
 //                  1. per block of 1024 entries: histogram of the expert ids (LDS atomics)
 //                  2. one workgroup: per expert, exclusive scan over the blocks, then over the experts;
 //                     writes the count / cumulative-count output
@@ -196,6 +199,164 @@ __global__ void __launch_bounds__(1024) route_small_kernel(const int *expert_idx
   rank_block(chunk_first, first + blockIdx.x * expert_num, i, my_e >= 0, my_e, expanded_row_idx, sorted_src, expert_num);
 }
 
+// ---- per-row dynamic int8 quantisation (tests/st/test_grouped_matmul_w4.py:83-89), shared by the gather kernels ----
+//   scale = float32(max |x[t, :]|) / 127,   q[h] = int8(rint(float32(x[t, h]) / scale))
+// |x| is ordered like its bit pattern without the sign, so the maximum is taken on 15-bit integers and converted once.
+template <bool BF16>
+__device__ __forceinline__ float rq_widen(unsigned short b) { return BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); }
+__device__ __forceinline__ void rq_fold(unsigned &mx, const uint4 &v) {
+  const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    mx = max(mx, w[i] & 0x7FFFu);
+    mx = max(mx, (w[i] >> 16) & 0x7FFFu);
+  }
+}
+// The golden rounds the correctly rounded quotient x / scale to an integer.  A correctly rounded division costs a
+// dozen instructions per element; x * (1 / scale) is within 2^-22 * 128 of that quotient, so unless it lands within
+// 1e-4 of a half-integer (then the division is done properly) both round to the same integer.
+__device__ __forceinline__ int rq_to_int(float f, float scale, float inv) {
+  const float r = f * inv;
+  const float n = rintf(r);
+  if (fabsf(r - n) > 0.4999f) return (int)rintf(f / scale);
+  return (int)n;
+}
+// eight elements -> eight int8; `nonzero`: the row's maximum is not zero (a row of zeros has scale 0: the golden divides
+// 0 by 0 there; it gets zeros)
+template <bool BF16>
+__device__ __forceinline__ uint2 rq_quantise(const uint4 &v, float scale, float inv, bool nonzero) {
+  const unsigned w[4] = {v.x, v.y, v.z, v.w};
+  unsigned q[2] = {0, 0};
+  if (nonzero) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int lo = rq_to_int(rq_widen<BF16>((unsigned short)(w[i] & 0xFFFFu)), scale, inv);
+      const int hi = rq_to_int(rq_widen<BF16>((unsigned short)(w[i] >> 16)), scale, inv);
+      q[i >> 1] |= ((unsigned)(lo & 0xFF) | ((unsigned)(hi & 0xFF) << 8)) << (16 * (i & 1));
+    }
+  }
+  return make_uint2(q[0], q[1]);
+}
+
+// Routing in ONE launch for up to kFusedMaxEntries entries: every workgroup owns kFusedRows consecutive entries (its
+// slice), finds their output rows by itself and copies their rows.  For that it counts, over ALL entries, how many carry
+// each expert id (total) and how many of those lie before its slice (before): the output row of entry i with id e is
+//     (entries with a smaller id) + (entries with id e before the slice) + (entries with id e inside the slice before i),
+// which is the position a stable sort gives it.  The counting is redundant across workgroups (a few thousand LDS
+// atomics each, on `rep` interleaved copies of the tables so that the lanes of a wavefront rarely meet on one address),
+// but nothing waits for another workgroup, so the sort, the index outputs and the row copy need no second launch.
+#ifndef MSCO_FUSED_ROWS
+#define MSCO_FUSED_ROWS 32
+#endif
+constexpr int kFusedRows = MSCO_FUSED_ROWS;   // 16, 32 or 64: one to four rows per wavefront
+constexpr int kFusedThreads = 1024;   // sixteen wavefronts: the counting is a chain of dependent LDS atomics per wavefront, four per SIMD overlap them
+constexpr int kFusedIdsPerThread = 16;
+constexpr long long kFusedMaxEntries = (long long)kFusedThreads * kFusedIdsPerThread;   // 16384
+__global__ void __launch_bounds__(kFusedThreads) route_fused_kernel(const unsigned char *x, const int *expert_idx,
+                                                                    unsigned char *expanded_x,
+                                                                    int *expanded_row_idx, int *count_or_cumsum,
+                                                                    int *before_capacity, long long n, int expert_num, int flag,
+                                                                    long long row_bytes, int k, int rep) {
+  extern __shared__ int lds[];   // total[rep][expert_num], before[rep][expert_num], base[expert_num], wave_sum[16], dest[kFusedRows]
+  int *total = lds;
+  int *before = total + rep * expert_num;
+  int *base = before + rep * expert_num;
+  int *wave_sum = base + expert_num;
+  int *dest = wave_sum + 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const long long start = (long long)blockIdx.x * kFusedRows;
+  for (int i = tid; i < 2 * rep * expert_num; i += kFusedThreads) lds[i] = 0;
+  // all of a thread's ids are requested before the first is used: entries 4 (tid + 1024 j) .. + 3 (ids past n read as 0,
+  // by the range check of the buffer load, and are skipped by their index; only the vector offset is range-checked)
+  const __amdgpu_buffer_rsrc_t rs_ids = buffer_over(expert_idx, n * 4);
+  v4i ids[kFusedIdsPerThread / 4];
+  static_for<kFusedIdsPerThread / 4>([&](auto j_c) {
+    constexpr int J = decltype(j_c)::value;
+    ids[J] = __builtin_amdgcn_raw_buffer_load_b128(rs_ids, (unsigned)(16 * (tid + kFusedThreads * J)), 0, 0);
+  });
+  __syncthreads();
+  const int copy = (lane & (rep - 1)) * expert_num;   // rep is a power of two
+  static_for<kFusedIdsPerThread / 4>([&](auto j_c) {
+    constexpr int J = decltype(j_c)::value;
+    const long long i0 = 4ll * (tid + kFusedThreads * J);
+    static_for<4>([&](auto u_c) {
+      constexpr int U = decltype(u_c)::value;
+      if (i0 + U < n) {
+        const int e = clamp_expert(ids[J][U], expert_num);
+        atomicAdd(&total[copy + e], 1);
+        if (i0 + U < start) atomicAdd(&before[copy + e], 1);
+      }
+    });
+  });
+  __syncthreads();
+  // fold the copies; exclusive scan of the totals over the experts (one expert per thread)
+  int tsum = 0, bsum = 0;
+  if (tid < expert_num) {
+    for (int r = 0; r < rep; ++r) {
+      tsum += total[r * expert_num + tid];
+      bsum += before[r * expert_num + tid];
+    }
+    before[tid] = bsum;   // copy 0 now holds the folded value (a thread touches only its own expert)
+  }
+  const int incl = wave_scan_add(tsum, lane);
+  if (lane == 63) wave_sum[wave] = incl;
+  __syncthreads();
+  int offset = incl - tsum;
+  for (int w = 0; w < wave; ++w) offset += wave_sum[w];
+  if (tid < expert_num) {
+    base[tid] = offset;
+    if (blockIdx.x == 0) {
+      if (count_or_cumsum != nullptr && flag == 1) count_or_cumsum[tid] = offset + tsum;
+      if (count_or_cumsum != nullptr && flag == 2) count_or_cumsum[tid] = tsum;
+      if (before_capacity != nullptr) before_capacity[tid] = 0;
+    }
+  }
+  __syncthreads();
+  // the slice's entries, one per lane of wavefront 0: rank among equal ids inside the slice by ballots
+  if (wave == 0) {
+    const long long i = start + lane;
+    const bool live = lane < kFusedRows && i < n;
+    const int e = live ? clamp_expert(expert_idx[i], expert_num) : -1;
+    unsigned long long todo = __ballot(live);
+    int rank = 0;
+    while (todo) {
+      const int leader = __ffsll((long long)todo) - 1;
+      const int e0 = __shfl(e, leader);
+      const unsigned long long same = __ballot(e == e0) & todo;
+      if (e == e0) rank = __popcll(same & ((1ull << lane) - 1ull));
+      todo &= ~same;
+    }
+    if (live) {
+      const int d = base[e] + before[e] + rank;
+      dest[lane] = d;
+      expanded_row_idx[i] = d;
+    }
+  }
+  __syncthreads();
+  // copy the rows: wavefront w takes the slice's rows w, w + 16, ...; a lane's vectors of all of them in flight together
+  const long long vecs = row_bytes / 16;
+  constexpr int RPW = kFusedRows / 16;   // rows per wavefront
+  for (long long v0 = 0; v0 < vecs; v0 += 64 * 4) {
+    uint4 buf[RPW][4];
+    static_for<4 * RPW>([&](auto q_c) {
+      constexpr int RR = decltype(q_c)::value / 4, C = decltype(q_c)::value % 4;
+      const long long i = start + wave + 16 * RR;
+      const uint4 *src = reinterpret_cast<const uint4 *>(x + (i < n ? i / k : 0) * row_bytes);
+      const long long v = v0 + lane + 64 * C;
+      buf[RR][C] = (i < n && v < vecs) ? src[v] : make_uint4(0, 0, 0, 0);
+    });
+    static_for<4 * RPW>([&](auto q_c) {
+      constexpr int RR = decltype(q_c)::value / 4, C = decltype(q_c)::value % 4;
+      const long long i = start + wave + 16 * RR;
+      const long long v = v0 + lane + 64 * C;
+      if (i < n && v < vecs) {
+        uint4 *dst = reinterpret_cast<uint4 *>(expanded_x + (long long)dest[wave + 16 * RR] * row_bytes);
+        dst[v] = buf[RR][C];   // kept cacheable: the matmul reads it next
+      }
+    });
+  }
+}
+
 __global__ void __launch_bounds__(256) route_gather_kernel(const unsigned char *x, const int *sorted_src, unsigned char *expanded_x,
                                                            long long row_bytes, int k) {
   const long long j = blockIdx.x;
@@ -222,14 +383,7 @@ __global__ void __launch_bounds__(256) route_gather_quant_kernel(const unsigned 
   constexpr int KEEP = 4;
   uint4 kept[KEEP];
   unsigned mx = 0;
-  auto fold = [&](const uint4 &v) {
-    const unsigned w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      mx = max(mx, w[i] & 0x7FFFu);
-      mx = max(mx, (w[i] >> 16) & 0x7FFFu);
-    }
-  };
+  auto fold = [&](const uint4 &v) { rq_fold(mx, v); };
 #pragma unroll
   for (int u = 0; u < KEEP; ++u) {
     const long long v = threadIdx.x + u * 256;
@@ -242,32 +396,10 @@ __global__ void __launch_bounds__(256) route_gather_quant_kernel(const unsigned 
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = mx;
   __syncthreads();
   mx = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
-  auto widen = [](unsigned short b) { return BF16 ? bf16_bits_to_f32(b) : f16_bits_to_f32(b); };
-  const float scale = widen((unsigned short)mx) / 127.0f;
+  const float scale = rq_widen<BF16>((unsigned short)mx) / 127.0f;
   if (threadIdx.x == 0) expanded_scale[j] = scale;
-  // The golden rounds the correctly rounded quotient x / scale to an integer.  A correctly rounded division costs a
-  // dozen instructions per element; x * (1 / scale) is within 2^-22 * 128 of that quotient, so unless it lands within
-  // 1e-4 of a half-integer (then the division is done properly) both round to the same integer.
   const float inv = 1.0f / scale;
-  auto to_int = [&](float f) {
-    const float r = f * inv;
-    const float n = rintf(r);
-    if (fabsf(r - n) > 0.4999f) return (int)rintf(f / scale);
-    return (int)n;
-  };
-  auto quantise = [&](const uint4 &v) {
-    const unsigned w[4] = {v.x, v.y, v.z, v.w};
-    unsigned q[2] = {0, 0};
-    if (mx != 0) {   // (a row of zeros has scale 0: the golden divides 0 by 0 there; it gets zeros)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int lo = to_int(widen((unsigned short)(w[i] & 0xFFFFu)));
-        const int hi = to_int(widen((unsigned short)(w[i] >> 16)));
-        q[i >> 1] |= ((unsigned)(lo & 0xFF) | ((unsigned)(hi & 0xFF) << 8)) << (16 * (i & 1));
-      }
-    }
-    return make_uint2(q[0], q[1]);
-  };
+  auto quantise = [&](const uint4 &v) { return rq_quantise<BF16>(v, scale, inv, mx != 0); };
 #pragma unroll
   for (int u = 0; u < KEEP; ++u) {
     const long long v = threadIdx.x + u * 256;
@@ -428,6 +560,19 @@ static int route_and_gather(const void *x, const int32_t *expert_idx, void *expa
   if (count_or_cumsum_flag != 0 && expert_tokens_count_or_cumsum == nullptr) return MSCO_ERR_INVALID_ARG;
   if (workspace == nullptr || workspace_bytes < msco_moe_init_routing_v2_workspace_bytes(num_rows, k, expert_num))
     return MSCO_ERR_WORKSPACE;
+  if (quant_dtype == MSCO_DT_NONE && n <= kFusedMaxEntries) {
+    // small problems: the sort and the row copy in one launch, no workspace traffic.  (The quantising gather stays a
+    // launch of its own: it is bound by its arithmetic, and one workgroup per row overlaps that better -- fused the
+    // same way it measured 27.5 us against 24.4 us.)
+    int rep = 8;
+    while (rep > 1 && rep * expert_num > 512) rep /= 2;
+    const size_t lds_bytes = (size_t)(2 * rep * expert_num + expert_num + 16 + kFusedRows) * sizeof(int);
+    hipLaunchKernelGGL(route_fused_kernel, dim3((unsigned)((n + kFusedRows - 1) / kFusedRows)), dim3(kFusedThreads), lds_bytes, s,
+                       static_cast<const unsigned char *>(x), expert_idx, static_cast<unsigned char *>(expanded_x), expanded_row_idx,
+                       expert_tokens_count_or_cumsum, expert_tokens_before_capacity, n, (int)expert_num, (int)count_or_cumsum_flag,
+                       (long long)hidden * elem_bytes, (int)k, rep);
+    return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
+  }
   const long long blocks = route_blocks(n);
   int *block_hist = static_cast<int *>(workspace);
   int *sorted_src = block_hist + blocks * expert_num;

@@ -172,7 +172,11 @@ def _route_gpu(x, idx, e, flag):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("n_rows,h,k,e,flag", [(1, 1024, 1, 1, 1), (10, 2048, 8, 8, 1), (1001, 1024, 2, 8, 2),
-                                              (513, 1024, 6, 64, 1), (300, 7168, 4, 256, 1)])
+                                              (513, 1024, 6, 64, 1), (300, 7168, 4, 256, 1),
+                                              (40, 256, 8, 1024, 1),       # the most experts (one copy of the count tables)
+                                              (2048, 64, 8, 8, 1),         # 16384 entries: the largest single-launch problem
+                                              (3000, 256, 6, 64, 2),       # 18000 entries: histogram, scan, ranking and gather launches
+                                              (17000, 32, 1, 128, 1)])     # 17 blocks of 1024 entries
 def test_init_routing_matches_the_golden(n_rows, h, k, e, flag):
     np.random.seed(0)                                                             # the reference test's stream (:102-104)
     x = np.random.uniform(-1, 1, size=(n_rows, h)).astype(np.float16)
@@ -296,7 +300,8 @@ def _route_quant_gpu(x_bits, bf16, idx, e, flag):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("n_rows,h,k,e,bf16", [(1, 8, 1, 1, False), (37, 1024, 2, 8, False), (300, 4096, 2, 8, True),
-                                              (64, 7168, 6, 64, False), (20, 10240, 3, 4, True), (9, 8200, 2, 3, False)])
+                                              (64, 7168, 6, 64, False), (20, 10240, 3, 4, True), (9, 8200, 2, 3, False),
+                                              (2100, 512, 8, 8, True)])    # 16800 entries: the separate launches
 def test_routing_with_dynamic_quantisation_is_bit_exact(n_rows, h, k, e, bf16):
     # the routing golden followed by the activation quantisation of the reference's int8-activation test
     # (tests/st/test_grouped_matmul_w4.py:83-89,99), row by row; int8 rows and float32 scales bit for bit
