@@ -371,6 +371,35 @@ def read_floor(sizes=(45.09e6, 469.8e6), steps=60):
     return out
 
 
+def library_reference(wl, steps=20):
+    """The vendor library on the same operands, for scale: torch._int_mm (hipBLASLt) on ONE dense int8 matmul with the
+    headline's M, K and N (all rows against one expert's weights; int32 out, no grouping, no epilogue), weights [K,N] as
+    generated and [N,K] (passed as a transposed view).  Reported, not used."""
+    import torch
+    out = {}
+    try:
+        dev = torch.device("cuda:0")
+        x = torch.from_numpy(np.ascontiguousarray(wl.x)).to(dev)
+        w_kn = torch.from_numpy(np.ascontiguousarray(wl.w[0])).to(dev)
+        w_nk = w_kn.t().contiguous()
+        ops = 2.0 * wl.x.shape[0] * wl.k * wl.n
+        for name, b in (("kn", w_kn), ("nk", w_nk.t())):
+            for _ in range(10):
+                torch._int_mm(x, b)
+            first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            first.record()
+            for _ in range(steps):
+                torch._int_mm(x, b)
+            last.record()
+            torch.cuda.synchronize()
+            sec = first.elapsed_time(last) / steps * 1e-3
+            out[name] = {"launch_us": sec * 1e6, "tops": ops / sec / 1e12, "int8_frac": ops / sec / 1e12 / PEAK_INT8_TOPS}
+        out["what"] = f"torch._int_mm, dense [{wl.x.shape[0]},{wl.k}] x [{wl.k},{wl.n}] int8 -> int32"
+    except Exception as exc:   # not every build of torch carries the routine
+        out["error"] = repr(exc)
+    return out
+
+
 def measured_traffic(workload, layout, kernel):
     """HBM bytes per launch of the dominant kernel from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs (scaled by
     the same counters' reading for a copy of known size); None when no measurement of this kernel is on file."""
@@ -492,6 +521,7 @@ def main():
         result["moe_neighbours"] = moe_neighbours(max(20, min(100, args.steps)), 10)
         result["mfma_pipe"] = mfma_pipe_probe()
         result["read_floor"] = read_floor()
+        result["library_reference"] = library_reference(wl)
         # the headline kernel once more on all-zero x and weights: same instruction stream and memory traffic, but the
         # matrix pipe toggles nothing, so the chip holds a higher clock; the gap to the figure above is what the
         # operand distribution costs, the gap to the peak is what the kernel's own stalls and padding cost
