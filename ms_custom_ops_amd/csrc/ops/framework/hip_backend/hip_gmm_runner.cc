@@ -150,7 +150,8 @@ bool HipGmmKernelMod::Launch(const KernelTensorList &inputs, const std::vector<m
   }
   void *ws = workspace.empty() ? nullptr : workspace[0].GetDataPtr();
   const size_t ws_bytes = workspace.empty() ? 0 : workspace[0].nbytes();
-  LaunchPlan(kernel_name_, plan_, addrs, outputs.at(0).GetDataPtr(), ws, ws_bytes, stream);
+  const GmmPlanPtr plan = plan_;   // the launch drops the GIL: another thread's Resize may replace plan_ meanwhile
+  LaunchPlan(kernel_name_, plan, addrs, outputs.at(0).GetDataPtr(), ws, ws_bytes, stream);
   return true;
 }
 }  // namespace ms_custom_ops
