@@ -122,11 +122,22 @@ def _wrap_list(ts):
     return [_wrap(t) for t in ts]
 
 
+_CUDA = torch.device("cuda")
+
+
 def _allocate(type_id: int, shape: Sequence[int]):
-    return _wrap(torch.empty(tuple(shape), dtype=type_id_to_dtype(type_id), device="cuda"))
+    # (called once or twice per operator call from the C++ layer: kept free of argument checks and string parsing)
+    t = torch.empty(tuple(shape), dtype=_DTYPES[type_id], device=_CUDA)
+    return _C.Tensor(t.data_ptr(), type_id, list(shape), list(t.stride()), t)
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def _current_stream() -> int:
+    # the raw getter skips the construction of a torch.cuda.Stream object (a few microseconds per operator call)
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
