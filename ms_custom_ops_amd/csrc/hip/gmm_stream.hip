@@ -85,7 +85,11 @@ size_t packed_weight_bytes(int64_t k, int64_t n) { return (size_t)packed_group_b
 
 // ---- W8A8 ----------------------------------------------------------------------------------------------
 // NB = K blocks a wave meets per column group (the slice has at most 4 NB blocks); 4, 8, 16 or 32.
-template <int NB>
+// XLDS: the chunk's x rows reach the waves through LDS.  Read straight from memory, a wave's fragment load touches 16
+// rows x 64 bytes = 16 half lines, twice the line requests of a weight load of the same size, and the request rate of
+// the load path is what bounds these kernels; staged, the workgroup reads every x line once with whole-line requests
+// (four rows x 256 contiguous bytes per wave instruction) and the waves pick their fragments out of LDS.
+template <int NB, bool XLDS>
 __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const GmmParams p) {
   extern __shared__ __align__(16) unsigned char st_smem[];
   v4i(*red)[ST_GROUPS][64] = reinterpret_cast<v4i(*)[ST_GROUPS][64]>(st_smem);   // [wave][column group][lane]
@@ -118,16 +122,32 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
 
   // the wave's blocks kb_begin + wave + 4 j: x fragments (zero past the slice or past K, which also cancels
   // whatever a masked weight load returns) and byte offsets inside a column group
-  const int8_t *xrow = reinterpret_cast<const int8_t *>(p.x) + (long long)min(m0 + c16, g_end - 1) * p.k;
   v4i xf[NB];
   unsigned voff[NB];
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     const int kb = kb_begin + wave + ST_WAVES * j;
-    const int k0 = kb * 64 + 16 * h;   // K % 16 == 0: 16 K bytes all inside or all outside
-    const bool ok = kb < kb_end && k0 < p.k;
-    xf[j] = ok ? *reinterpret_cast<const v4i *>(xrow + k0) : v4i{0, 0, 0, 0};
     voff[j] = kb < kb_end ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob;
+  }
+  v4i xtmp[XLDS ? NB : 1];
+  const int st_row = tid >> 4, st_col = tid & 15;                      // staging: 16 threads per row, 256 bytes per pass
+  const int slice_bytes = (kb_end - kb_begin) * 64, x_pitch = slice_bytes + 64;   // the pad spreads the 16 rows of a fragment read over all banks
+  if constexpr (XLDS) {
+    const int8_t *srow = reinterpret_cast<const int8_t *>(p.x) + (long long)min(m0 + st_row, g_end - 1) * p.k + kb_begin * 64;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int off = (st_col + 16 * j) * 16;
+      xtmp[j] = (off < slice_bytes && kb_begin * 64 + off < p.k) ? *reinterpret_cast<const v4i *>(srow + off) : v4i{0, 0, 0, 0};
+    }
+  } else {
+    const int8_t *xrow = reinterpret_cast<const int8_t *>(p.x) + (long long)min(m0 + c16, g_end - 1) * p.k;
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int kb = kb_begin + wave + ST_WAVES * j;
+      const int k0 = kb * 64 + 16 * h;   // K % 16 == 0: 16 K bytes all inside or all outside
+      const bool ok = kb < kb_end && k0 < p.k;
+      xf[j] = ok ? *reinterpret_cast<const v4i *>(xrow + k0) : v4i{0, 0, 0, 0};
+    }
   }
 
   v4i ring[D];
@@ -141,6 +161,23 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
     constexpr int J = decltype(j_c)::value;
     if constexpr (J < D) issue(0, j_c, j_c);
   });
+  if constexpr (XLDS) {
+    // (the x rows were requested before the weights, so waiting for them does not wait for the weight stream; the
+    // staging area is the reduction area of the end of the kernel: the second barrier keeps a wave that is already
+    // parking its first partial tile from overwriting fragments another wave has not read yet)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int off = (st_col + 16 * j) * 16;
+      if (off < slice_bytes) *reinterpret_cast<v4i *>(st_smem + st_row * x_pitch + off) = xtmp[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int kb_rel = wave + ST_WAVES * j;
+      xf[j] = kb_rel * 64 < slice_bytes ? *reinterpret_cast<const v4i *>(st_smem + c16 * x_pitch + kb_rel * 64 + 16 * h) : v4i{0, 0, 0, 0};
+    }
+    __syncthreads();
+  }
   // epilogue operands of this thread's outputs (column groups wave + 4 e, rows 4 h .. 4 h + 3), requested behind the
   // first weight loads so that they are in registers long before the stream ends: a memory round trip after the
   // reduction is as long as a tenth of the whole kernel on a 45 MB weight set
@@ -275,17 +312,19 @@ int stream_blocks_per_wave(int64_t k, int split_k) {
   return (int)((per_split + ST_WAVES - 1) / ST_WAVES);
 }
 
-template <int NB>
+template <int NB, bool XLDS>
 static hipError_t stream_launch_w8a8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
-  auto kern = gmm_w8a8_stream_kernel<NB>;
+  auto kern = gmm_w8a8_stream_kernel<NB, XLDS>;
+  // the x staging area (16 rows of at most 4 NB blocks of 64 bytes, 64 bytes of padding per row) shares the LDS of the
+  // reduction area
+  constexpr size_t lds = XLDS ? (ST_LDS > (size_t)16 * (4 * NB * 64 + 64) + 16 ? ST_LDS : (size_t)16 * (4 * NB * 64 + 64) + 16) : ST_LDS;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)ST_LDS);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(ST_THREADS), ST_LDS, stream, p);
+  hipLaunchKernelGGL(kern, grid, dim3(ST_THREADS), lds, stream, p);
   return hipGetLastError();
 }
 
@@ -294,10 +333,15 @@ hipError_t launch_stream_w8a8(const GmmParams &p, hipStream_t stream) {
   const int nb = stream_blocks_per_wave(p.k, p.split_k);
   if (nb > 32 || p.strip_groups < 1 || p.strip_groups > ST_GROUPS) return hipErrorInvalidValue;   // the plan splits K until a slice has at most 128 blocks
   const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
-  if (nb > 16) return stream_launch_w8a8<32>(p, grid, stream);
-  if (nb > 8) return stream_launch_w8a8<16>(p, grid, stream);
-  if (nb > 4) return stream_launch_w8a8<8>(p, grid, stream);
-  return stream_launch_w8a8<4>(p, grid, stream);
+  if (nb > 16) return stream_launch_w8a8<32, false>(p, grid, stream);   // (a 128-block slice of 16 rows would need 128 KiB of LDS)
+  if (p.x_via_lds) {
+    if (nb > 8) return stream_launch_w8a8<16, true>(p, grid, stream);
+    if (nb > 4) return stream_launch_w8a8<8, true>(p, grid, stream);
+    return stream_launch_w8a8<4, true>(p, grid, stream);
+  }
+  if (nb > 8) return stream_launch_w8a8<16, false>(p, grid, stream);
+  if (nb > 4) return stream_launch_w8a8<8, false>(p, grid, stream);
+  return stream_launch_w8a8<4, false>(p, grid, stream);
 }
 
 // ---- W8A8, more than 16 rows per group (packed weights) -----------------------------------------------------

@@ -446,6 +446,9 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   p.max_chunks = h->max_chunks;
   p.strip_groups = h->strip_groups;
   p.act_type = d.act_type;
+  // rows a 16-row chunk is expected to hold (shapes only): measured on the dense 45 MB decode, 16 rows 13.1 -> 12.35 us with
+  // the x rows staged through LDS, one row 11.85 -> 12.2 us, four rows per chunk (8 experts x 32 rows) 70.1 -> 70.4 us
+  p.x_via_lds = (h->e > 0 ? (h->m + h->e - 1) / h->e : h->m) >= 8;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t err = hipSuccess;
