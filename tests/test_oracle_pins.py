@@ -369,3 +369,55 @@ def test_activation_against_torch_other_formulations_and_identities():
         assert f([0.0])[0] == 0.0
     with pytest.raises(ValueError):
         O.activation(v, O.ACT_GELU_ERF)
+
+
+# ---------------------------------------------------------------- the two helpers that only had shape checks
+def test_quant_int4_groups_element_by_element_and_by_what_the_formula_fixes():
+    """quant (tests/st/test_grouped_matmul_w4.py:91-97): per (expert, K group, column) scale = max|y| / 7 in float32 and
+    q = round(y / scale) -- restated with scalar loops in exact rational arithmetic, plus the properties the formula
+    fixes: the group's largest magnitude maps to +-7 with its sign, 7 * scale returns it, |y - q * scale| <= scale / 2."""
+    from fractions import Fraction
+    rng = np.random.default_rng(8)
+    e, k, n, g = 2, 64, 5, 32
+    y = rng.uniform(-0.3, 0.3, (e, k, n)).astype(np.float16)
+    q, s = O.quant_int4_groups(y, g)
+    assert q.shape == (e, k, n) and s.shape == (e, k // g, 1, n) and s.dtype == np.float32 and q.dtype == np.int8
+    for ee in range(e):
+        for kg in range(k // g):
+            for c in range(n):
+                col = [Fraction(float(v)) for v in y[ee, kg * g:(kg + 1) * g, c]]
+                big = max(abs(v) for v in col)
+                scale = np.float32(float(big)) / np.float32(7.0)          # the golden divides float32 by float32
+                assert s[ee, kg, 0, c] == scale
+                for j, v in enumerate(col):
+                    quot = np.float32(np.float32(float(v)) / scale)       # float32 quotient, as numpy computes it
+                    want = int(np.round(quot))                            # half to even
+                    assert q[ee, kg * g + j, c] == want
+                    assert abs(float(v) - want * float(scale)) <= float(scale) / 2 * (1 + 1e-6)
+                top = int(np.argmax([abs(v) for v in col]))
+                assert abs(int(q[ee, kg * g + top, c])) == 7 and np.sign(q[ee, kg * g + top, c]) == np.sign(float(col[top]))
+                assert abs(7 * float(scale) - float(big)) <= 1e-6 * float(big)
+
+
+def test_count_compare_counts_like_the_reference_comparator():
+    """custom_compare (tests/st/st_utils.py:23-49): at most int(size * limit) elements may have a relative error above
+    limit -- on hand-built cases either side of the count and of the error threshold."""
+    expect = np.ones(1000, dtype=np.float32)
+    out = expect.copy()
+    assert O.count_compare(out, expect, 0.004)
+    out[:4] = 1.0 + 0.0041                       # 4 elements just above the limit: int(1000 * 0.004) = 4 are allowed
+    assert O.count_compare(out, expect, 0.004)
+    out[4] = 1.0 + 0.0041                        # the fifth is one too many
+    assert not O.count_compare(out, expect, 0.004)
+    out[:5] = 1.0 + 0.0039                       # below the error threshold nothing counts
+    assert O.count_compare(out, expect, 0.004)
+    out[:] = 2.0                                 # bfloat16's limit: 0.03 of the elements, 0.03 relative
+    assert not O.count_compare(out, expect, 0.03)
+    out[:] = 1.0
+    out[:30] = 1.05
+    assert O.count_compare(out, expect, 0.03)
+    out[30] = 1.05
+    assert not O.count_compare(out, expect, 0.03)
+    # relative to the expected value, sign and scale free
+    assert O.count_compare(np.array([-100.3]), np.array([-100.0]), 0.004)
+    assert not O.count_compare(np.array([-100.5] * 1000), np.array([-100.0] * 1000), 0.004)
