@@ -1,16 +1,18 @@
 // MoE routing (stable counting sort of (token, k) entries by expert + activation gather) and weighted
 // un-permutation for gfx950.  Both are HBM-bound row copies around a small integer problem:
 //
-//   init_routing   up to 16384 entries, plain row copy: ONE launch (route_fused_kernel): every workgroup counts all expert
-//                  ids itself, places its own 32 entries and copies their rows.  Otherwise (more entries, or the
-//                  quantising gather) the steps below; 1-3 are one launch for up to 16 blocks, every block repeating
-//                  the small steps 1 and 2 for itself
+//   init_routing   up to 16384 entries: ONE launch (route_fused_kernel): every workgroup counts all expert ids itself,
+//                  places its own 32 entries and moves their rows (plain copy, or per-row dynamic int8 quantisation);
+//                  a wavefront owns consecutive entries, so the k entries of a token cost one read (and one
+//                  quantisation) of its row.  More entries take the steps below; 1-3 are one launch for up to 16
+//                  blocks, every block repeating the small steps 1 and 2 for itself
 //                  1. per block of 1024 entries: histogram of the expert ids (LDS atomics)
 //                  2. one workgroup: per expert, exclusive scan over the blocks, then over the experts;
 //                     writes the count / cumulative-count output
 //                  3. per block, sixteen wavefronts rank 64 consecutive entries each among equal expert ids with
 //                     ballots; a prefix over the sixteen chunks keeps the flat order, so the sort is stable
-//                  4. one workgroup per output row copies x[token] with 16-byte loads and stores
+//                  4. plain copy: one workgroup per output row copies x[token] with 16-byte loads and stores;
+//                     quantising: one wavefront per token quantises its row once and writes it to its k rows
 //   unpermute      one workgroup per token: 16 bytes of every selected row per lane, the running sum kept
 //                  in the element type and rounded exactly where the golden rounds it
 #include "msco_moe.h"
@@ -213,29 +215,159 @@ __device__ __forceinline__ void rq_fold(unsigned &mx, const uint4 &v) {
   }
 }
 // The golden rounds the correctly rounded quotient x / scale to an integer.  A correctly rounded division costs a
-// dozen instructions per element; x * (1 / scale) is within 2^-22 * 128 of that quotient, so unless it lands within
-// 1e-4 of a half-integer (then the division is done properly) both round to the same integer.
-__device__ __forceinline__ int rq_to_int(float f, float scale, float inv) {
-  const float r = f * inv;
-  const float n = rintf(r);
-  if (fabsf(r - n) > 0.4999f) return (int)rintf(f / scale);
-  return (int)n;
-}
+// dozen instructions per element.  r = x * (1 / scale) differs from that quotient by at most 1.5 * 2^-23 * 127.5 < 2.3e-5
+// (two roundings here, one there), so unless r lies within kRqMargin = 5e-5 of a half-integer both round to the same
+// integer.  Adding 1.5 * 2^23 rounds r to that integer (nearest, ties to even, like rint) in the low mantissa bits: its
+// low byte is the int8.  Elements too close to a half-integer (1e-4 of them) are done again with the division.
 // eight elements -> eight int8; `nonzero`: the row's maximum is not zero (a row of zeros has scale 0: the golden divides
 // 0 by 0 there; it gets zeros)
+constexpr float kRqMargin = 5e-5f;
 template <bool BF16>
 __device__ __forceinline__ uint2 rq_quantise(const uint4 &v, float scale, float inv, bool nonzero) {
+  constexpr float kRound = 12582912.0f;   // 1.5 * 2^23
   const unsigned w[4] = {v.x, v.y, v.z, v.w};
-  unsigned q[2] = {0, 0};
-  if (nonzero) {
+  float f[8], d[8];
+  unsigned b[8];
+  float worst = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int lo = rq_to_int(rq_widen<BF16>((unsigned short)(w[i] & 0xFFFFu)), scale, inv);
-      const int hi = rq_to_int(rq_widen<BF16>((unsigned short)(w[i] >> 16)), scale, inv);
-      q[i >> 1] |= ((unsigned)(lo & 0xFF) | ((unsigned)(hi & 0xFF) << 8)) << (16 * (i & 1));
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = BF16 ? __uint_as_float(w[i] << 16) : f16_bits_to_f32((unsigned short)(w[i] & 0xFFFFu));
+    f[2 * i + 1] = BF16 ? __uint_as_float(w[i] & 0xFFFF0000u) : f16_bits_to_f32((unsigned short)(w[i] >> 16));
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e += 2) {
+    const float r0 = f[e] * inv, r1 = f[e + 1] * inv;
+    const float t0 = r0 + kRound, t1 = r1 + kRound;
+    b[e] = __float_as_uint(t0);
+    b[e + 1] = __float_as_uint(t1);
+    d[e] = r0 - (t0 - kRound);
+    d[e + 1] = r1 - (t1 - kRound);
+    worst = fmaxf(fmaxf(fabsf(d[e]), fabsf(d[e + 1])), worst);
+  }
+  if (!(worst <= 0.5f - kRqMargin)) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      if (!(fabsf(d[e]) <= 0.5f - kRqMargin)) b[e] = (unsigned)(int)rintf(f[e] / scale);
     }
   }
-  return make_uint2(q[0], q[1]);
+  // bytes 0 of b[0..3] and of b[4..7] side by side (v_perm_b32: selector 0-3 picks a byte of the second operand, 4-7 of the first)
+  unsigned q[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const unsigned p01 = __builtin_amdgcn_perm(b[4 * h + 1], b[4 * h], 0x0c0c0400u);
+    const unsigned p23 = __builtin_amdgcn_perm(b[4 * h + 3], b[4 * h + 2], 0x0c0c0400u);
+    q[h] = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+  }
+  return nonzero ? make_uint2(q[0], q[1]) : make_uint2(0, 0);
+}
+
+// ---- one wavefront moves one source row to `copies` destination rows ----
+// The k entries of a token are neighbours in the flat entry order, so a wavefront that owns consecutive entries reads
+// (and quantises) a token's row once and writes it k times: half the loads and half the arithmetic at top-2.
+
+// Rows are read and written through buffer descriptors over exactly one row (the row's address is the same for the whole
+// wavefront: callers derive it from a wavefront index made scalar with readfirstlane): what lies past the row's end
+// reads as zeros and is not written, so no lane ever branches around a load (a conditional load costs a full
+// `s_waitcnt vmcnt(0)` where its value meets the zero of the other path).
+typedef unsigned rq_v4u __attribute__((ext_vector_type(4)));
+typedef unsigned rq_v2u __attribute__((ext_vector_type(2)));
+typedef int rq_v2i __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 row_load16(__amdgpu_buffer_rsrc_t rs, long long byte_offset) {
+  const unsigned off = byte_offset > 0x7FFFFFFFll ? 0x7FFFFFFFu : (unsigned)byte_offset;   // (past any row: zeros)
+  const rq_v4u v = __builtin_bit_cast(rq_v4u, __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void row_store16(__amdgpu_buffer_rsrc_t rs, long long byte_offset, const uint4 &v) {
+  const unsigned off = byte_offset > 0x7FFFFFFFll ? 0x7FFFFFFFu : (unsigned)byte_offset;
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, rq_v4u{v.x, v.y, v.z, v.w}), rs, off, 0, 0);
+}
+__device__ __forceinline__ void row_store8(__amdgpu_buffer_rsrc_t rs, long long byte_offset, const uint2 &v) {
+  const unsigned off = byte_offset > 0x7FFFFFFFll ? 0x7FFFFFFFu : (unsigned)byte_offset;
+  __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(rq_v2i, rq_v2u{v.x, v.y}), rs, off, 0, 0);
+}
+
+// the first KV vectors per lane of a row (lane + 64 u), requested together; zeros past the row's end
+template <int KV>
+__device__ __forceinline__ void wave_load_row(uint4 (&kept)[KV], __amdgpu_buffer_rsrc_t src, int lane, long long first_byte = 0) {
+  static_for<KV>([&](auto u_c) {
+    constexpr int U = decltype(u_c)::value;
+    kept[U] = row_load16(src, first_byte + 16ll * (lane + 64 * U));
+  });
+}
+
+// `first`: what wave_load_row brought of this row; dest_row(j): the j-th destination row
+template <int KV, typename DestFn>
+__device__ __forceinline__ void wave_copy_row(const uint4 (&first)[KV], __amdgpu_buffer_rsrc_t src, int lane, int copies,
+                                              DestFn dest_row, unsigned char *expanded_x, long long row_bytes) {
+  for (int j = 0; j < copies; ++j) {
+    const __amdgpu_buffer_rsrc_t dst = buffer_over(expanded_x + (long long)dest_row(j) * row_bytes, row_bytes);
+    static_for<KV>([&](auto u_c) {
+      constexpr int U = decltype(u_c)::value;
+      row_store16(dst, 16ll * (lane + 64 * U), first[U]);   // kept cacheable: the matmul reads it next
+    });
+  }
+  for (long long b0 = 1024ll * KV; b0 < row_bytes; b0 += 1024ll * KV) {
+    uint4 buf[KV];
+    wave_load_row(buf, src, lane, b0);
+    for (int j = 0; j < copies; ++j) {
+      const __amdgpu_buffer_rsrc_t dst = buffer_over(expanded_x + (long long)dest_row(j) * row_bytes, row_bytes);
+      static_for<KV>([&](auto u_c) {
+        constexpr int U = decltype(u_c)::value;
+        row_store16(dst, b0 + 16ll * (lane + 64 * U), buf[U]);
+      });
+    }
+  }
+}
+
+// The same with the per-row dynamic int8 quantisation on the way: the row's maximum needs no LDS (one wavefront holds
+// the whole row); a lane keeps KEEP vectors of the row in registers (64 lanes x KEEP x 16 bytes in one pass), what lies
+// beyond is read again for the division (L2 hits).  Zeros past the row's end change neither the maximum nor anything
+// that is stored.
+template <bool BF16, int KEEP, typename DestFn>
+__device__ __forceinline__ void wave_quantise_row(const uint4 (&kept)[KEEP], __amdgpu_buffer_rsrc_t src, int lane, int copies,
+                                                  DestFn dest_row, signed char *expanded_x, float *expanded_scale,
+                                                  long long hidden) {
+  const long long row_bytes = 2 * hidden;
+  unsigned mx = 0;
+  static_for<KEEP>([&](auto u_c) { rq_fold(mx, kept[decltype(u_c)::value]); });
+  for (long long b = 1024ll * KEEP; b < row_bytes; b += 1024) rq_fold(mx, row_load16(src, b + 16 * lane));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = max(mx, (unsigned)__shfl_xor((int)mx, o));
+  const float scale = rq_widen<BF16>((unsigned short)mx) / 127.0f;
+  const float inv = 1.0f / scale;
+  if (lane == 0) {
+    for (int j = 0; j < copies; ++j) expanded_scale[dest_row(j)] = scale;
+  }
+  // two vectors at a time, to every copy (the quantised row never exists as a whole in registers).  A lane's eight
+  // bytes and its neighbour's are consecutive in the row: the even lane of a pair takes both lanes' bytes of the first
+  // vector and the odd lane both of the second, so that every lane stores 16 bytes (rows of a multiple of 16 bytes).
+  const bool wide = (hidden & 15) == 0;
+  const long long pair_byte = 512 * (lane & 1) + 16 * (lane >> 1);
+  static_for<KEEP / 2>([&](auto p_c) {
+    constexpr int P = decltype(p_c)::value;
+    const uint2 qa = rq_quantise<BF16>(kept[2 * P], scale, inv, mx != 0);
+    const uint2 qb = rq_quantise<BF16>(kept[2 * P + 1], scale, inv, mx != 0);
+    if (wide) {
+      const bool odd = lane & 1;
+      const unsigned sx = odd ? qa.x : qb.x, sy = odd ? qa.y : qb.y;
+      const unsigned rx = (unsigned)__builtin_amdgcn_update_dpp(0, (int)sx, 0xB1, 0xF, 0xF, true);   // quad_perm [1,0,3,2]
+      const unsigned ry = (unsigned)__builtin_amdgcn_update_dpp(0, (int)sy, 0xB1, 0xF, 0xF, true);
+      const uint4 out = odd ? make_uint4(rx, ry, qb.x, qb.y) : make_uint4(qa.x, qa.y, rx, ry);
+      for (int j = 0; j < copies; ++j)
+        row_store16(buffer_over(expanded_x + (long long)dest_row(j) * hidden, hidden), 1024ll * P + pair_byte, out);
+    } else {
+      for (int j = 0; j < copies; ++j) {
+        const __amdgpu_buffer_rsrc_t dst = buffer_over(expanded_x + (long long)dest_row(j) * hidden, hidden);
+        row_store8(dst, 8ll * (lane + 128 * P), qa);
+        row_store8(dst, 8ll * (lane + 128 * P + 64), qb);
+      }
+    }
+  });
+  for (long long b = 1024ll * KEEP; b < row_bytes; b += 1024) {
+    const uint2 q = rq_quantise<BF16>(row_load16(src, b + 16 * lane), scale, inv, mx != 0);
+    for (int j = 0; j < copies; ++j)
+      row_store8(buffer_over(expanded_x + (long long)dest_row(j) * hidden, hidden), (b >> 1) + 8 * lane, q);
+  }
 }
 
 // Routing in ONE launch for up to kFusedMaxEntries entries: every workgroup owns kFusedRows consecutive entries (its
@@ -252,8 +384,10 @@ constexpr int kFusedRows = MSCO_FUSED_ROWS;   // 16, 32 or 64: one to four rows 
 constexpr int kFusedThreads = 1024;   // sixteen wavefronts: the counting is a chain of dependent LDS atomics per wavefront, four per SIMD overlap them
 constexpr int kFusedIdsPerThread = 16;
 constexpr long long kFusedMaxEntries = (long long)kFusedThreads * kFusedIdsPerThread;   // 16384
+// QUANT: 0 copies rows of row_bytes bytes; 1 / 2 quantise float16 / bfloat16 rows to int8 and write their scales.
+template <int QUANT>
 __global__ void __launch_bounds__(kFusedThreads) route_fused_kernel(const unsigned char *x, const int *expert_idx,
-                                                                    unsigned char *expanded_x,
+                                                                    unsigned char *expanded_x, float *expanded_scale,
                                                                     int *expanded_row_idx, int *count_or_cumsum,
                                                                     int *before_capacity, long long n, int expert_num, int flag,
                                                                     long long row_bytes, int k, int rep) {
@@ -263,8 +397,11 @@ __global__ void __launch_bounds__(kFusedThreads) route_fused_kernel(const unsign
   int *base = before + rep * expert_num;
   int *wave_sum = base + expert_num;
   int *dest = wave_sum + 16;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const long long start = (long long)blockIdx.x * kFusedRows;
+  constexpr int RPW = kFusedRows / 16;   // consecutive entries per wavefront
+  constexpr int KV = 8;                  // vectors of a row per lane and pass
+  const long long entry0 = start + RPW * wave;
   for (int i = tid; i < 2 * rep * expert_num; i += kFusedThreads) lds[i] = 0;
   // all of a thread's ids are requested before the first is used: entries 4 (tid + 1024 j) .. + 3 (ids past n read as 0,
   // by the range check of the buffer load, and are skipped by their index; only the vector offset is range-checked)
@@ -274,6 +411,20 @@ __global__ void __launch_bounds__(kFusedThreads) route_fused_kernel(const unsign
     constexpr int J = decltype(j_c)::value;
     ids[J] = __builtin_amdgcn_raw_buffer_load_b128(rs_ids, (unsigned)(16 * (tid + kFusedThreads * J)), 0, 0);
   });
+  // the slice's own ids for the ranking by wavefront 0, requested now: a load issued where they are needed would put a
+  // memory round trip between two barriers (other lanes ask beyond the list and get zeros)
+  const int slice_id = __builtin_amdgcn_raw_buffer_load_b32(
+      rs_ids, wave == 0 && lane < kFusedRows && start + lane < n ? (unsigned)(4 * (start + lane)) : 0xFFFFFFFCu, 0, 0);
+  // The plain copy requests the row of the wavefront's first entry right behind the ids (loads return in order: the
+  // counting must not wait for it): where it comes from is known from the entry's index alone (token = entry / k), only
+  // where it goes has to wait for the counting below.  (Measured: 0.4 us less for the copy at 8192 entries of 4 KiB; the
+  // quantising variant is 0.7 us slower with it.)
+  constexpr bool kPreload = QUANT == 0;
+  uint4 row0[KV];
+  if constexpr (kPreload) {
+    wave_load_row(row0, buffer_over(x + (long long)(entry0 < n ? (unsigned)entry0 / (unsigned)k : 0u) * row_bytes, entry0 < n ? row_bytes : 0),
+                  lane);
+  }
   __syncthreads();
   const int copy = (lane & (rep - 1)) * expert_num;   // rep is a power of two
   static_for<kFusedIdsPerThread / 4>([&](auto j_c) {
@@ -316,7 +467,7 @@ __global__ void __launch_bounds__(kFusedThreads) route_fused_kernel(const unsign
   if (wave == 0) {
     const long long i = start + lane;
     const bool live = lane < kFusedRows && i < n;
-    const int e = live ? clamp_expert(expert_idx[i], expert_num) : -1;
+    const int e = live ? clamp_expert(slice_id, expert_num) : -1;
     unsigned long long todo = __ballot(live);
     int rank = 0;
     while (todo) {
@@ -333,27 +484,25 @@ __global__ void __launch_bounds__(kFusedThreads) route_fused_kernel(const unsign
     }
   }
   __syncthreads();
-  // copy the rows: wavefront w takes the slice's rows w, w + 16, ...; a lane's vectors of all of them in flight together
-  const long long vecs = row_bytes / 16;
-  constexpr int RPW = kFusedRows / 16;   // rows per wavefront
-  for (long long v0 = 0; v0 < vecs; v0 += 64 * 4) {
-    uint4 buf[RPW][4];
-    static_for<4 * RPW>([&](auto q_c) {
-      constexpr int RR = decltype(q_c)::value / 4, C = decltype(q_c)::value % 4;
-      const long long i = start + wave + 16 * RR;
-      const uint4 *src = reinterpret_cast<const uint4 *>(x + (i < n ? i / k : 0) * row_bytes);
-      const long long v = v0 + lane + 64 * C;
-      buf[RR][C] = (i < n && v < vecs) ? src[v] : make_uint4(0, 0, 0, 0);
-    });
-    static_for<4 * RPW>([&](auto q_c) {
-      constexpr int RR = decltype(q_c)::value / 4, C = decltype(q_c)::value % 4;
-      const long long i = start + wave + 16 * RR;
-      const long long v = v0 + lane + 64 * C;
-      if (i < n && v < vecs) {
-        uint4 *dst = reinterpret_cast<uint4 *>(expanded_x + (long long)dest[wave + 16 * RR] * row_bytes);
-        dst[v] = buf[RR][C];   // kept cacheable: the matmul reads it next
-      }
-    });
+  // move the rows: wavefront w takes the slice's entries RPW w .. RPW w + RPW - 1; neighbours of one token share a pass
+  int r = 0;
+  while (r < RPW) {
+    const long long i = entry0 + r;
+    if (i >= n) break;
+    const unsigned token = (unsigned)i / (unsigned)k;   // (entries fit 31 bits: 32-bit divisions)
+    int copies = 1;
+    while (r + copies < RPW && i + copies < n && (unsigned)(i + copies) / (unsigned)k == token) ++copies;
+    const int first = RPW * wave + r;
+    auto dest_row = [&](int j) { return __builtin_amdgcn_readfirstlane(dest[first + j]); };
+    const __amdgpu_buffer_rsrc_t src = buffer_over(x + (long long)token * row_bytes, row_bytes);
+    if (r != 0 || !kPreload) wave_load_row(row0, src, lane);
+    if constexpr (QUANT == 0) {
+      wave_copy_row(row0, src, lane, copies, dest_row, expanded_x, row_bytes);
+    } else {
+      wave_quantise_row<QUANT == 2>(row0, src, lane, copies, dest_row, reinterpret_cast<signed char *>(expanded_x),
+                                    expanded_scale, row_bytes / 2);
+    }
+    r += copies;
   }
 }
 
@@ -366,46 +515,21 @@ __global__ void __launch_bounds__(256) route_gather_kernel(const unsigned char *
   for (long long v = threadIdx.x; v < row_bytes / 16; v += 256) dst[v] = src[v];   // kept cacheable: the matmul reads it next
 }
 
-// The gather with per-row dynamic int8 quantisation on the way (tests/st/test_grouped_matmul_w4.py:83-89):
-//   scale = float32(max |x[t, :]|) / 127,   q[h] = int8(rint(float32(x[t, h]) / scale))
-// One workgroup per output row, 16 bytes (8 elements) per lane and step.  Up to four steps a lane keeps its elements
-// in registers between the maximum and the division; longer rows are read again (they are L2 hits).  |x| is ordered
-// like its bit pattern without the sign, so the maximum is taken on 15-bit integers and converted once.
+// Per-row dynamic int8 quantisation on the way to the sorted rows, for problems beyond the single launch: one wavefront
+// per token quantises its row once and writes it to the k rows expanded_row_idx names for it.
 template <bool BF16>
-__global__ void __launch_bounds__(256) route_gather_quant_kernel(const unsigned short *x, const int *sorted_src, signed char *expanded_x,
-                                                                 float *expanded_scale, long long hidden, int k) {
-  __shared__ unsigned wave_max[4];
-  const long long j = blockIdx.x;
-  const long long token = sorted_src[j] / k;
-  const uint4 *src = reinterpret_cast<const uint4 *>(x + token * hidden);
-  uint2 *dst = reinterpret_cast<uint2 *>(expanded_x + j * hidden);
-  const long long vecs = hidden / 8;
-  constexpr int KEEP = 4;
-  uint4 kept[KEEP];
-  unsigned mx = 0;
-  auto fold = [&](const uint4 &v) { rq_fold(mx, v); };
-#pragma unroll
-  for (int u = 0; u < KEEP; ++u) {
-    const long long v = threadIdx.x + u * 256;
-    kept[u] = v < vecs ? src[v] : make_uint4(0, 0, 0, 0);
-    fold(kept[u]);
-  }
-  for (long long v = threadIdx.x + KEEP * 256; v < vecs; v += 256) fold(src[v]);
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) mx = max(mx, (unsigned)__shfl_xor((int)mx, o));
-  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = mx;
-  __syncthreads();
-  mx = max(max(wave_max[0], wave_max[1]), max(wave_max[2], wave_max[3]));
-  const float scale = rq_widen<BF16>((unsigned short)mx) / 127.0f;
-  if (threadIdx.x == 0) expanded_scale[j] = scale;
-  const float inv = 1.0f / scale;
-  auto quantise = [&](const uint4 &v) { return rq_quantise<BF16>(v, scale, inv, mx != 0); };
-#pragma unroll
-  for (int u = 0; u < KEEP; ++u) {
-    const long long v = threadIdx.x + u * 256;
-    if (v < vecs) dst[v] = quantise(kept[u]);
-  }
-  for (long long v = threadIdx.x + KEEP * 256; v < vecs; v += 256) dst[v] = quantise(src[v]);
+__global__ void __launch_bounds__(256) route_scatter_quant_kernel(const unsigned short *x, const int *expanded_row_idx,
+                                                                  signed char *expanded_x, float *expanded_scale,
+                                                                  long long num_rows, long long hidden, int k) {
+  const int lane = threadIdx.x & 63;
+  const long long token = (long long)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (token >= num_rows) return;
+  const int *dests = expanded_row_idx + token * k;
+  const __amdgpu_buffer_rsrc_t src = buffer_over(x + token * hidden, 2 * hidden);
+  uint4 kept[16];
+  wave_load_row(kept, src, lane);
+  wave_quantise_row<BF16>(kept, src, lane, k, [&](int j) { return __builtin_amdgcn_readfirstlane(dests[j]); }, expanded_x,
+                          expanded_scale, hidden);
 }
 
 // float32 -> element type with round to nearest even, and back
@@ -560,17 +684,21 @@ static int route_and_gather(const void *x, const int32_t *expert_idx, void *expa
   if (count_or_cumsum_flag != 0 && expert_tokens_count_or_cumsum == nullptr) return MSCO_ERR_INVALID_ARG;
   if (workspace == nullptr || workspace_bytes < msco_moe_init_routing_v2_workspace_bytes(num_rows, k, expert_num))
     return MSCO_ERR_WORKSPACE;
-  if (quant_dtype == MSCO_DT_NONE && n <= kFusedMaxEntries) {
-    // small problems: the sort and the row copy in one launch, no workspace traffic.  (The quantising gather stays a
-    // launch of its own: it is bound by its arithmetic, and one workgroup per row overlaps that better -- fused the
-    // same way it measured 27.5 us against 24.4 us.)
+  if (n <= kFusedMaxEntries) {
+    // small problems: the sort and the row movement in one launch, no workspace traffic
     int rep = 8;
     while (rep > 1 && rep * expert_num > 512) rep /= 2;
     const size_t lds_bytes = (size_t)(2 * rep * expert_num + expert_num + 16 + kFusedRows) * sizeof(int);
-    hipLaunchKernelGGL(route_fused_kernel, dim3((unsigned)((n + kFusedRows - 1) / kFusedRows)), dim3(kFusedThreads), lds_bytes, s,
-                       static_cast<const unsigned char *>(x), expert_idx, static_cast<unsigned char *>(expanded_x), expanded_row_idx,
-                       expert_tokens_count_or_cumsum, expert_tokens_before_capacity, n, (int)expert_num, (int)count_or_cumsum_flag,
-                       (long long)hidden * elem_bytes, (int)k, rep);
+    const dim3 grid((unsigned)((n + kFusedRows - 1) / kFusedRows)), block(kFusedThreads);
+#define MSCO_ROUTE_FUSED(Q)                                                                                                  \
+    hipLaunchKernelGGL(route_fused_kernel<Q>, grid, block, lds_bytes, s, static_cast<const unsigned char *>(x), expert_idx,   \
+                       static_cast<unsigned char *>(expanded_x), expanded_scale, expanded_row_idx,                            \
+                       expert_tokens_count_or_cumsum, expert_tokens_before_capacity, n, (int)expert_num,                      \
+                       (int)count_or_cumsum_flag, (long long)hidden * (quant_dtype == MSCO_DT_NONE ? elem_bytes : 2), (int)k, rep)
+    if (quant_dtype == MSCO_DT_NONE) MSCO_ROUTE_FUSED(0);
+    else if (quant_dtype == MSCO_DT_F16) MSCO_ROUTE_FUSED(1);
+    else MSCO_ROUTE_FUSED(2);
+#undef MSCO_ROUTE_FUSED
     return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
   }
   const long long blocks = route_blocks(n);
@@ -590,12 +718,17 @@ static int route_and_gather(const void *x, const int32_t *expert_idx, void *expa
   if (quant_dtype == MSCO_DT_NONE) {
     hipLaunchKernelGGL(route_gather_kernel, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned char *>(x), sorted_src,
                        static_cast<unsigned char *>(expanded_x), (long long)hidden * elem_bytes, (int)k);
-  } else if (quant_dtype == MSCO_DT_BF16) {
-    hipLaunchKernelGGL(route_gather_quant_kernel<true>, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned short *>(x),
-                       sorted_src, static_cast<signed char *>(expanded_x), expanded_scale, (long long)hidden, (int)k);
   } else {
-    hipLaunchKernelGGL(route_gather_quant_kernel<false>, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned short *>(x),
-                       sorted_src, static_cast<signed char *>(expanded_x), expanded_scale, (long long)hidden, (int)k);
+    const dim3 grid((unsigned)((num_rows + 3) / 4)), block(256);
+    if (quant_dtype == MSCO_DT_BF16) {
+      hipLaunchKernelGGL(route_scatter_quant_kernel<true>, grid, block, 0, s, static_cast<const unsigned short *>(x),
+                         expanded_row_idx, static_cast<signed char *>(expanded_x), expanded_scale, (long long)num_rows,
+                         (long long)hidden, (int)k);
+    } else {
+      hipLaunchKernelGGL(route_scatter_quant_kernel<false>, grid, block, 0, s, static_cast<const unsigned short *>(x),
+                         expanded_row_idx, static_cast<signed char *>(expanded_x), expanded_scale, (long long)num_rows,
+                         (long long)hidden, (int)k);
+    }
   }
   return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
 }

@@ -301,7 +301,9 @@ def _route_quant_gpu(x_bits, bf16, idx, e, flag):
 @pytest.mark.gpu
 @pytest.mark.parametrize("n_rows,h,k,e,bf16", [(1, 8, 1, 1, False), (37, 1024, 2, 8, False), (300, 4096, 2, 8, True),
                                               (64, 7168, 6, 64, False), (20, 10240, 3, 4, True), (9, 8200, 2, 3, False),
-                                              (2100, 512, 8, 8, True)])    # 16800 entries: the separate launches
+                                              (2100, 512, 8, 8, True),     # 16800 entries: the separate launches
+                                              (2100, 8200, 8, 8, False),   # ... with rows longer than a lane keeps in registers
+                                              (16500, 64, 1, 8, True), (33, 4104, 1, 5, False)])   # one entry per token
 def test_routing_with_dynamic_quantisation_is_bit_exact(n_rows, h, k, e, bf16):
     # the routing golden followed by the activation quantisation of the reference's int8-activation test
     # (tests/st/test_grouped_matmul_w4.py:83-89,99), row by row; int8 rows and float32 scales bit for bit
