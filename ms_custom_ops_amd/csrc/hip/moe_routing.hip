@@ -4,15 +4,13 @@
 //   init_routing   up to 16384 entries: ONE launch (route_fused_kernel): every workgroup counts all expert ids itself,
 //                  places its own 32 entries and moves their rows (plain copy, or per-row dynamic int8 quantisation);
 //                  a wavefront owns consecutive entries, so the k entries of a token cost one read (and one
-//                  quantisation) of its row.  More entries take the steps below; 1-3 are one launch for up to 16
-//                  blocks, every block repeating the small steps 1 and 2 for itself
+//                  quantisation) of its row.  More entries take four launches:
 //                  1. per block of 1024 entries: histogram of the expert ids (LDS atomics)
-//                  2. one workgroup: per expert, exclusive scan over the blocks, then over the experts;
-//                     writes the count / cumulative-count output
-//                  3. per block, sixteen wavefronts rank 64 consecutive entries each among equal expert ids with
-//                     ballots; a prefix over the sixteen chunks keeps the flat order, so the sort is stable
-//                  4. plain copy: one workgroup per output row copies x[token] with 16-byte loads and stores;
-//                     quantising: one wavefront per token quantises its row once and writes it to its k rows
+//                  2. one workgroup: per expert, exclusive scan over the blocks (runs of blocks in parallel), then over
+//                     the experts; writes the count / cumulative-count output
+//                  3. per block, sixteen wavefronts rank 64 consecutive entries each among equal expert ids (one ballot
+//                     per bit of the id); a prefix over the sixteen chunks keeps the flat order, so the sort is stable
+//                  4. one wavefront per token moves (or quantises) its row once and writes it to its k rows
 //   unpermute      one workgroup per token: 16 bytes of every selected row per lane, the running sum kept
 //                  in the element type and rounded exactly where the golden rounds it
 #include "msco_moe.h"
@@ -56,36 +54,67 @@ __global__ void __launch_bounds__(256) route_hist_kernel(const int *expert_idx, 
   for (int e = threadIdx.x; e < expert_num; e += 256) block_hist[(long long)blockIdx.x * expert_num + e] = hist[e];
 }
 
-// block_hist[b][e] becomes the first output position of block b's entries of expert e
-__global__ void __launch_bounds__(1024) route_scan_kernel(int *block_hist, int *count_or_cumsum, int *before_capacity,
-                                                          int blocks, int expert_num, int flag) {
-  __shared__ int total[kMaxExperts];
-  __shared__ int base[kMaxExperts];
-  const int e = threadIdx.x;
-  int running = 0;
-  if (e < expert_num) {
-    for (int b = 0; b < blocks; ++b) {
-      const int v = block_hist[(long long)b * expert_num + e];
-      block_hist[(long long)b * expert_num + e] = running;
-      running += v;
-    }
-    total[e] = running;
+// The lanes of the wavefront that carry the same id as this one, among the live lanes: one ballot per bit of the id
+// (ids below 2^bits), whatever the number of distinct ids in the wavefront.
+__device__ __forceinline__ unsigned long long wave_match(int e, bool live, int bits) {
+  unsigned long long same = __ballot(live);
+  for (int k = 0; k < bits; ++k) {
+    const bool bit = (e >> k) & 1;
+    const unsigned long long b = __ballot(bit);
+    same &= bit ? b : ~b;
   }
+  return same;
+}
+__device__ __forceinline__ int id_bits(int expert_num) { return expert_num > 1 ? 32 - __clz(expert_num - 1) : 0; }
+
+// block_hist[b][e] becomes the first position of block b's entries of expert e among the entries of that expert;
+// expert_base[e] the number of entries of smaller experts (the ranking adds the two).  One workgroup: thread (g, e) owns
+// expert e in the g-th of G = 1024 / expert_num runs of consecutive blocks, sums its run, the runs of an expert are
+// scanned in LDS, and the thread walks its run again writing the running positions -- loads in batches of eight ahead of
+// their stores (in place: a load behind a store would wait for it).
+__global__ void __launch_bounds__(1024) route_scan_kernel(int *block_hist, int *expert_base, int *count_or_cumsum,
+                                                          int *before_capacity, int blocks, int expert_num, int flag) {
+  __shared__ int part[1024];
+  __shared__ int wave_sum[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int groups = 1024 / expert_num;                 // expert_num <= 1024
+  const int e = tid % expert_num, g = tid / expert_num;
+  const int per = (blocks + groups - 1) / groups;
+  const int b_lo = min(blocks, g * per), b_hi = g < groups ? min(blocks, b_lo + per) : b_lo;
+  int sum = 0;
+#pragma unroll 8
+  for (int b = b_lo; b < b_hi; ++b) sum += block_hist[(long long)b * expert_num + e];
+  part[tid] = sum;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int acc = 0;
-    for (int j = 0; j < expert_num; ++j) {
-      base[j] = acc;
-      acc += total[j];
+  int total = 0;
+  if (tid < expert_num) {
+    for (int r = 0; r < groups; ++r) {
+      const int v = part[r * expert_num + tid];
+      part[r * expert_num + tid] = total;
+      total += v;
     }
   }
+  const int incl = wave_scan_add(total, lane);
+  if (lane == 63) wave_sum[wave] = incl;
   __syncthreads();
-  if (e < expert_num) {
-    const int b0 = base[e];
-    for (int b = 0; b < blocks; ++b) block_hist[(long long)b * expert_num + e] += b0;
-    if (count_or_cumsum != nullptr && flag == 1) count_or_cumsum[e] = b0 + total[e];
-    if (count_or_cumsum != nullptr && flag == 2) count_or_cumsum[e] = total[e];
-    if (before_capacity != nullptr) before_capacity[e] = 0;
+  if (tid < expert_num) {
+    int base = incl - total;
+    for (int w = 0; w < wave; ++w) base += wave_sum[w];
+    if (expert_base != nullptr) expert_base[tid] = base;
+    if (count_or_cumsum != nullptr && flag == 1) count_or_cumsum[tid] = base + total;
+    if (count_or_cumsum != nullptr && flag == 2) count_or_cumsum[tid] = total;
+    if (before_capacity != nullptr) before_capacity[tid] = 0;
+  }
+  int running = part[tid];
+  for (int b0 = b_lo; b0 < b_hi; b0 += 8) {
+    int v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = b0 + u < b_hi ? block_hist[(long long)(b0 + u) * expert_num + e] : 0;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (b0 + u < b_hi) block_hist[(long long)(b0 + u) * expert_num + e] = running;
+      running += v[u];
+    }
   }
 }
 
@@ -93,25 +122,19 @@ __global__ void __launch_bounds__(1024) route_scan_kernel(int *block_hist, int *
 // equal expert ids with ballots (one round per distinct id in the chunk) and leaves the chunk's per-expert counts
 // in LDS; a prefix over the sixteen chunks turns the counts into first positions; rank + first position is the
 // output row.  Chunks, and positions inside a chunk, are taken in flat order, so the sort is stable.
-// (block_first: this block's row of first positions, in global memory or in LDS; e: the entry's expert id, -1 for none)
-__device__ __forceinline__ void rank_block(int *chunk_first, const int *block_first, long long i, bool live, int e,
-                                           int *expanded_row_idx, int *sorted_src, int expert_num) {
+// (block_first: this block's row of first positions, in global memory or in LDS; expert_base: what to add to them per
+// expert, or null; e: the entry's expert id, -1 for none)
+__device__ __forceinline__ void rank_block(int *chunk_first, const int *block_first, const int *expert_base, long long i,
+                                           bool live, int e, int *expanded_row_idx, int expert_num) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int *mine = chunk_first + wave * expert_num;
   for (int x = lane; x < expert_num; x += 64) mine[x] = 0;
-  unsigned long long todo = __ballot(live);
-  int rank = 0;
-  while (todo) {
-    const int leader = __ffsll((long long)todo) - 1;
-    const int e0 = __shfl(e, leader);
-    const unsigned long long same = __ballot(e == e0) & todo;
-    if (e == e0) rank = __popcll(same & ((1ull << lane) - 1ull));
-    if (lane == leader) mine[e0] = __popcll(same);      // after the zero fill above: one wavefront's LDS operations stay in order
-    todo &= ~same;
-  }
+  const unsigned long long same = wave_match(e, live, id_bits(expert_num));
+  const int rank = __popcll(same & ((1ull << lane) - 1ull));
+  if (live && rank == 0) mine[e] = __popcll(same);      // after the zero fill above: one wavefront's LDS operations stay in order
   __syncthreads();
   for (int x = threadIdx.x; x < expert_num; x += 1024) {
-    int running = block_first[x];
+    int running = block_first[x] + (expert_base != nullptr ? expert_base[x] : 0);
 #pragma unroll
     for (int w = 0; w < 16; ++w) {
       const int c = chunk_first[w * expert_num + x];
@@ -120,85 +143,16 @@ __device__ __forceinline__ void rank_block(int *chunk_first, const int *block_fi
     }
   }
   __syncthreads();
-  if (live) {
-    const int dest = mine[e] + rank;
-    expanded_row_idx[i] = dest;
-    sorted_src[dest] = (int)i;
-  }
+  if (live) expanded_row_idx[i] = mine[e] + rank;
 }
 
-__global__ void __launch_bounds__(1024) route_rank_kernel(const int *expert_idx, const int *block_first, int *expanded_row_idx,
-                                                          int *sorted_src, long long n, int expert_num) {
+__global__ void __launch_bounds__(1024) route_rank_kernel(const int *expert_idx, const int *block_first, const int *expert_base,
+                                                          int *expanded_row_idx, long long n, int expert_num) {
   extern __shared__ int chunk_first[];   // [16][expert_num]
   const long long i = (long long)blockIdx.x * kRouteBlock + threadIdx.x;
   const bool live = i < n;
   const int e = live ? clamp_expert(expert_idx[i], expert_num) : -1;
-  rank_block(chunk_first, block_first + (long long)blockIdx.x * expert_num, i, live, e, expanded_row_idx, sorted_src, expert_num);
-}
-
-// Histogram, scan and ranking in one launch for problems of at most kSmallBlocks blocks: every block histograms all
-// entries itself (a few thousand LDS atomics) instead of waiting for the other blocks, then ranks its own 1024.  At
-// this size the three launches above cost more in launch gaps than in work.
-constexpr int kSmallBlocks = 16;
-__global__ void __launch_bounds__(1024) route_small_kernel(const int *expert_idx, int *count_or_cumsum, int *before_capacity,
-                                                           int *expanded_row_idx, int *sorted_src, long long n, int expert_num,
-                                                           int flag) {
-  extern __shared__ int lds[];   // first[blocks][expert_num], chunk_first[16][expert_num], total[expert_num], base[expert_num]
-  const int blocks = gridDim.x;
-  int *first = lds;
-  int *chunk_first = first + blocks * expert_num;
-  int *total = chunk_first + 16 * expert_num;
-  int *base = total + expert_num;
-  for (int x = threadIdx.x; x < blocks * expert_num; x += 1024) first[x] = 0;
-  __syncthreads();
-  // (all of a thread's ids are requested before the first is used: one memory round trip instead of one per block)
-  int my_e = -1;
-  int ids[kSmallBlocks];
-#pragma unroll
-  for (int b = 0; b < kSmallBlocks; ++b) {
-    const long long i = (long long)b * kRouteBlock + threadIdx.x;
-    ids[b] = b < blocks && i < n ? expert_idx[i] : -1;
-  }
-#pragma unroll
-  for (int b = 0; b < kSmallBlocks; ++b) {
-    const long long i = (long long)b * kRouteBlock + threadIdx.x;
-    if (b < blocks && i < n) {
-      const int e = clamp_expert(ids[b], expert_num);
-      atomicAdd(&first[b * expert_num + e], 1);
-      if (b == (int)blockIdx.x) my_e = e;
-    }
-  }
-  __syncthreads();
-  const int e = threadIdx.x;
-  if (e < expert_num) {
-    int running = 0;
-    for (int b = 0; b < blocks; ++b) {
-      const int v = first[b * expert_num + e];
-      first[b * expert_num + e] = running;
-      running += v;
-    }
-    total[e] = running;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int acc = 0;
-    for (int j = 0; j < expert_num; ++j) {
-      base[j] = acc;
-      acc += total[j];
-    }
-  }
-  __syncthreads();
-  if (e < expert_num) {
-    first[blockIdx.x * expert_num + e] += base[e];
-    if (blockIdx.x == 0) {
-      if (count_or_cumsum != nullptr && flag == 1) count_or_cumsum[e] = base[e] + total[e];
-      if (count_or_cumsum != nullptr && flag == 2) count_or_cumsum[e] = total[e];
-      if (before_capacity != nullptr) before_capacity[e] = 0;
-    }
-  }
-  __syncthreads();
-  const long long i = (long long)blockIdx.x * kRouteBlock + threadIdx.x;
-  rank_block(chunk_first, first + blockIdx.x * expert_num, i, my_e >= 0, my_e, expanded_row_idx, sorted_src, expert_num);
+  rank_block(chunk_first, block_first + (long long)blockIdx.x * expert_num, expert_base, i, live, e, expanded_row_idx, expert_num);
 }
 
 // ---- per-row dynamic int8 quantisation (tests/st/test_grouped_matmul_w4.py:83-89), shared by the gather kernels ----
@@ -468,15 +422,7 @@ __global__ void __launch_bounds__(kFusedThreads) route_fused_kernel(const unsign
     const long long i = start + lane;
     const bool live = lane < kFusedRows && i < n;
     const int e = live ? clamp_expert(slice_id, expert_num) : -1;
-    unsigned long long todo = __ballot(live);
-    int rank = 0;
-    while (todo) {
-      const int leader = __ffsll((long long)todo) - 1;
-      const int e0 = __shfl(e, leader);
-      const unsigned long long same = __ballot(e == e0) & todo;
-      if (e == e0) rank = __popcll(same & ((1ull << lane) - 1ull));
-      todo &= ~same;
-    }
+    const int rank = __popcll(wave_match(e, live, id_bits(expert_num)) & ((1ull << lane) - 1ull));
     if (live) {
       const int d = base[e] + before[e] + rank;
       dest[lane] = d;
@@ -506,13 +452,19 @@ __global__ void __launch_bounds__(kFusedThreads) route_fused_kernel(const unsign
   }
 }
 
-__global__ void __launch_bounds__(256) route_gather_kernel(const unsigned char *x, const int *sorted_src, unsigned char *expanded_x,
-                                                           long long row_bytes, int k) {
-  const long long j = blockIdx.x;
-  const long long token = sorted_src[j] / k;
-  const uint4 *src = reinterpret_cast<const uint4 *>(x + token * row_bytes);
-  uint4 *dst = reinterpret_cast<uint4 *>(expanded_x + j * row_bytes);
-  for (long long v = threadIdx.x; v < row_bytes / 16; v += 256) dst[v] = src[v];   // kept cacheable: the matmul reads it next
+// The row movement behind the sort for problems beyond the single launch: one wavefront per token reads its row once and
+// writes it to the k rows expanded_row_idx names for it.
+__global__ void __launch_bounds__(256) route_scatter_kernel(const unsigned char *x, const int *expanded_row_idx,
+                                                            unsigned char *expanded_x, long long num_rows, long long row_bytes,
+                                                            int k) {
+  const int lane = threadIdx.x & 63;
+  const long long token = (long long)blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (token >= num_rows) return;
+  const int *dests = expanded_row_idx + token * k;
+  const __amdgpu_buffer_rsrc_t src = buffer_over(x + token * row_bytes, row_bytes);
+  uint4 first[8];
+  wave_load_row(first, src, lane);
+  wave_copy_row(first, src, lane, k, [&](int j) { return __builtin_amdgcn_readfirstlane(dests[j]); }, expanded_x, row_bytes);
 }
 
 // Per-row dynamic int8 quantisation on the way to the sorted rows, for problems beyond the single launch: one wavefront
@@ -654,8 +606,8 @@ extern "C" {
 size_t msco_moe_init_routing_v2_workspace_bytes(int64_t num_rows, int64_t k, int64_t expert_num) {
   if (num_rows <= 0 || k <= 0 || expert_num <= 0) return 0;
   const long long n = num_rows * k;
-  // per-block expert histograms / first positions, then the source entry of every output row
-  return (size_t)(msco::route_blocks(n) * expert_num + n) * sizeof(int32_t);
+  // per-block expert histograms / first positions, then the first position of every expert
+  return (size_t)(msco::route_blocks(n) + 1) * expert_num * sizeof(int32_t);
 }
 
 // quant_dtype: MSCO_DT_NONE copies rows of elem_bytes-wide elements; MSCO_DT_F16 / MSCO_DT_BF16 quantises rows of that
@@ -675,8 +627,8 @@ static int route_and_gather(const void *x, const int32_t *expert_idx, void *expa
   if (n > 0x7FFFFFFFll) return MSCO_ERR_SHAPE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (n == 0) {   // no entries: the count outputs are all zero (the scan kernel over zero blocks writes just that)
-    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, static_cast<int *>(nullptr), expert_tokens_count_or_cumsum,
-                       expert_tokens_before_capacity, 0, (int)expert_num, (int)count_or_cumsum_flag);
+    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, static_cast<int *>(nullptr), static_cast<int *>(nullptr),
+                       expert_tokens_count_or_cumsum, expert_tokens_before_capacity, 0, (int)expert_num, (int)count_or_cumsum_flag);
     return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
   }
   if (x == nullptr || expert_idx == nullptr || expanded_x == nullptr || expanded_row_idx == nullptr) return MSCO_ERR_INVALID_ARG;
@@ -703,21 +655,16 @@ static int route_and_gather(const void *x, const int32_t *expert_idx, void *expa
   }
   const long long blocks = route_blocks(n);
   int *block_hist = static_cast<int *>(workspace);
-  int *sorted_src = block_hist + blocks * expert_num;
-  const size_t small_lds = (size_t)(blocks + 16 + 2) * expert_num * sizeof(int);
-  if (blocks <= kSmallBlocks && small_lds <= 64 * 1024) {
-    hipLaunchKernelGGL(route_small_kernel, dim3((unsigned)blocks), dim3(1024), small_lds, s, expert_idx, expert_tokens_count_or_cumsum,
-                       expert_tokens_before_capacity, expanded_row_idx, sorted_src, n, (int)expert_num, (int)count_or_cumsum_flag);
-  } else {
-    hipLaunchKernelGGL(route_hist_kernel, dim3((unsigned)blocks), dim3(256), 0, s, expert_idx, block_hist, n, (int)expert_num);
-    hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, block_hist, expert_tokens_count_or_cumsum,
-                       expert_tokens_before_capacity, (int)blocks, (int)expert_num, (int)count_or_cumsum_flag);
-    hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(1024), (size_t)16 * expert_num * sizeof(int), s, expert_idx,
-                       block_hist, expanded_row_idx, sorted_src, n, (int)expert_num);
-  }
+  int *expert_base = block_hist + blocks * expert_num;
+  hipLaunchKernelGGL(route_hist_kernel, dim3((unsigned)blocks), dim3(256), 0, s, expert_idx, block_hist, n, (int)expert_num);
+  hipLaunchKernelGGL(route_scan_kernel, dim3(1), dim3(1024), 0, s, block_hist, expert_base, expert_tokens_count_or_cumsum,
+                     expert_tokens_before_capacity, (int)blocks, (int)expert_num, (int)count_or_cumsum_flag);
+  hipLaunchKernelGGL(route_rank_kernel, dim3((unsigned)blocks), dim3(1024), (size_t)16 * expert_num * sizeof(int), s, expert_idx,
+                     block_hist, expert_base, expanded_row_idx, n, (int)expert_num);
   if (quant_dtype == MSCO_DT_NONE) {
-    hipLaunchKernelGGL(route_gather_kernel, dim3((unsigned)n), dim3(256), 0, s, static_cast<const unsigned char *>(x), sorted_src,
-                       static_cast<unsigned char *>(expanded_x), (long long)hidden * elem_bytes, (int)k);
+    hipLaunchKernelGGL(route_scatter_kernel, dim3((unsigned)((num_rows + 3) / 4)), dim3(256), 0, s, static_cast<const unsigned char *>(x),
+                       expanded_row_idx, static_cast<unsigned char *>(expanded_x), (long long)num_rows, (long long)hidden * elem_bytes,
+                       (int)k);
   } else {
     const dim3 grid((unsigned)((num_rows + 3) / 4)), block(256);
     if (quant_dtype == MSCO_DT_BF16) {

@@ -175,8 +175,13 @@ def _route_gpu(x, idx, e, flag):
                                               (513, 1024, 6, 64, 1), (300, 7168, 4, 256, 1),
                                               (40, 256, 8, 1024, 1),       # the most experts (one copy of the count tables)
                                               (2048, 64, 8, 8, 1),         # 16384 entries: the largest single-launch problem
-                                              (3000, 256, 6, 64, 2),       # 18000 entries: histogram, scan, ranking and gather launches
-                                              (17000, 32, 1, 128, 1)])     # 17 blocks of 1024 entries
+                                              (3000, 256, 6, 64, 2),       # 18000 entries: histogram, scan, ranking and row launches
+                                              (17000, 32, 1, 128, 1),      # 17 blocks of 1024 entries
+                                              (8192, 64, 6, 64, 1),        # 48 blocks in 16 runs of 3 per expert
+                                              (25000, 16, 2, 1024, 1),     # the most experts: one run of 49 blocks per expert
+                                              (20000, 16, 3, 3, 2),        # 341 runs for 59 blocks: most runs are empty
+                                              (70000, 8, 1, 1, 1),         # one expert
+                                              (9000, 2064, 2, 7, 1)])      # rows of more than one pass (8 KiB) of the row movement
 def test_init_routing_matches_the_golden(n_rows, h, k, e, flag):
     np.random.seed(0)                                                             # the reference test's stream (:102-104)
     x = np.random.uniform(-1, 1, size=(n_rows, h)).astype(np.float16)
