@@ -141,7 +141,7 @@ def test_c_abi_exports_the_moe_entry_points_and_rejects_bad_shapes():
     lib = cabi.load()
     for name in ("msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_token_unpermute"):
         assert hasattr(lib, name)
-    assert cabi.moe_init_routing_v2_workspace_bytes(4096, 2, 8) == (8 * 8 + 8192) * 4
+    assert cabi.moe_init_routing_v2_workspace_bytes(4096, 2, 8) == (8 + 1) * 8 * 4    # (blocks of 1024 entries + 1) x experts ints
     # argument checks happen before anything touches a device
     with pytest.raises(cabi.BackendError):
         cabi.moe_token_unpermute(1, 1, 1, 1, 4, 8, 1001, cabi.DT_F16)        # hidden not a multiple of 8
