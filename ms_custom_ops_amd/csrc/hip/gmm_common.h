@@ -209,25 +209,6 @@ __device__ __forceinline__ unsigned short half_out(const GmmParams &p, float f) 
   return p.out_dtype == DT_BF16 ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
 }
 
-// The same without branches, for epilogues whose instruction schedule must not split into paths: the activation as
-// two wave-uniform coefficients of t(v) = v (c1 + c3 v^2) and a flag for the one that is not smooth.
-struct ActCoeffs {
-  float c1, c3;
-  bool relu;
-};
-__device__ __forceinline__ ActCoeffs act_coeffs(int act) {
-  ActCoeffs c;
-  c.relu = act == ACT_RELU;
-  c.c1 = act == ACT_FAST_GELU ? 1.702f : act == ACT_GELU_TANH ? 1.5957691216057308f : 1.0f;
-  c.c3 = act == ACT_GELU_TANH ? 1.5957691216057308f * 0.044715f : 0.0f;
-  return c;
-}
-__device__ __forceinline__ float activate(float v, const ActCoeffs &c) {
-  const float t = v * (c.c1 + c.c3 * v * v);
-  const float smooth = __fdividef(v, 1.0f + __expf(-t));
-  return c.relu ? (v < 0.0f ? 0.0f : v) : smooth;
-}
-
 __device__ __forceinline__ void store_out(const GmmParams &p, long long idx, int acc_plus_bias, float f) {
   if (p.act_type != ACT_NONE) f = activate(f, p.act_type);
   if (p.out_dtype == DT_BF16) {

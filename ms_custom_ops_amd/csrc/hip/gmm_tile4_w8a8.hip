@@ -159,8 +159,11 @@ __device__ __forceinline__ T4Tile t4_locate(const int *meta_end, const int *meta
 // blocks; staging quad (u, wave) is block 4 u + wave = (column group 2 u + wave / 2, K block wave % 2) and goes to LDS as
 // it is, so only the global offsets and the weight fragment addresses differ: MFMA row r of a 32-row block is column
 // t4_col_of_q(r), K quarter q is K block q / 2, 16-byte chunks 2 (q % 2) + hh.
-// ACT: an activation (p.act_type) follows the dequantisation; a template flag so that the plain epilogue stays as it is.
-template <int MODE, bool PK, bool ACT>
+// ACT: an activation (p.act_type) follows the dequantisation; a template parameter so that the plain epilogue stays as it
+// is (0).  The epilogue is bound by instruction issue, so the common forms get code of their own: 3 relu (one
+// instruction per value), 2 v * sigmoid(c v) with a uniform c (silu, fast gelu: five instructions, two of them
+// transcendental), 1 the tanh form of gelu (three more for its cubic).
+template <int MODE, bool PK, int ACT>
 __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const GmmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
 
@@ -619,14 +622,23 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
               float v[8];
 #pragma unroll
               for (int j = 0; j < 8; ++j) v[j] = dequant(a8[j], __uint_as_float(sraw[ff][s2][j]), pt);
-              if constexpr (ACT) {
+              if constexpr (ACT != 0) {
                 // one value after the other (the empty asm statements keep their order): eight exponentials in flight at
                 // once would need registers that this kernel does not have
-                const ActCoeffs ac = act_coeffs(p.act_type);
+                // v * sigmoid(t) = v / (1 + 2^(-t log2 e)); t = c v (silu: c = 1, fast gelu: 1.702) or, for the tanh form of
+                // gelu, t = v (c1 + c3 v^2) with c1 = 2 sqrt(2 / pi), c3 = 0.044715 c1
+                const float slu_k = (p.act_type == ACT_FAST_GELU ? -1.702f : -1.0f) * 1.4426950408889634f;
+                constexpr float gelu_k1 = -1.5957691216057308f * 1.4426950408889634f, gelu_k3 = gelu_k1 * 0.044715f;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                   asm volatile("" : "+v"(v[j]));
-                  v[j] = activate(v[j], ac);
+                  if constexpr (ACT == 3) {
+                    v[j] = v[j] < 0.0f ? 0.0f : v[j];
+                  } else if constexpr (ACT == 2) {
+                    v[j] = v[j] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v[j] * slu_k));
+                  } else {
+                    v[j] = v[j] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v[j] * __builtin_fmaf(v[j] * v[j], gelu_k3, gelu_k1)));
+                  }
                   asm volatile("" : "+v"(v[j]));
                 }
               }
@@ -691,7 +703,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   }
 }
 
-template <int MODE, bool PK, bool ACT>
+template <int MODE, bool PK, int ACT>
 static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t stream) {
   auto kern = gmm_w8a8_tile4_nk_kernel<MODE, PK, ACT>;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
@@ -714,18 +726,20 @@ hipError_t launch_tile4_w8a8_nk(const GmmParams &p, bool packed, hipStream_t str
   long long grid = ((total_ub + kNumXcd - 1) / kNumXcd) * kNumXcd;
   if (grid > T4_MAX_WGS) grid = T4_MAX_WGS;
   if (grid <= 0) return hipSuccess;
-  const bool act = p.act_type != ACT_NONE;
+  const int act = p.act_type == ACT_NONE ? 0 : p.act_type == ACT_RELU ? 3 : (p.act_type == ACT_SILU || p.act_type == ACT_FAST_GELU) ? 2 : 1;
   const unsigned g = (unsigned)grid;
+#define MSCO_T4_BY_ACT(MODE, PK)                                   \
+  (act == 0   ? t4_launch<MODE, PK, 0>(p, g, stream)               \
+   : act == 1 ? t4_launch<MODE, PK, 1>(p, g, stream)               \
+   : act == 2 ? t4_launch<MODE, PK, 2>(p, g, stream)               \
+              : t4_launch<MODE, PK, 3>(p, g, stream))
   switch (p.out_dtype) {
-    case DT_BF16:
-      if (act) return packed ? t4_launch<0, true, true>(p, g, stream) : t4_launch<0, false, true>(p, g, stream);
-      return packed ? t4_launch<0, true, false>(p, g, stream) : t4_launch<0, false, false>(p, g, stream);
-    case DT_F16:
-      if (act) return packed ? t4_launch<1, true, true>(p, g, stream) : t4_launch<1, false, true>(p, g, stream);
-      return packed ? t4_launch<1, true, false>(p, g, stream) : t4_launch<1, false, false>(p, g, stream);
-    case DT_I32: return packed ? t4_launch<2, true, false>(p, g, stream) : t4_launch<2, false, false>(p, g, stream);
+    case DT_BF16: return packed ? MSCO_T4_BY_ACT(0, true) : MSCO_T4_BY_ACT(0, false);
+    case DT_F16: return packed ? MSCO_T4_BY_ACT(1, true) : MSCO_T4_BY_ACT(1, false);
+    case DT_I32: return packed ? t4_launch<2, true, 0>(p, g, stream) : t4_launch<2, false, 0>(p, g, stream);
     default: return hipErrorInvalidValue;
   }
+#undef MSCO_T4_BY_ACT
 }
 
 }  // namespace msco
