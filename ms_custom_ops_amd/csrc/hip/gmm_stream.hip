@@ -623,22 +623,22 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
   const int kb_begin = ks * per_split;
   const int kb_end = min(k_blocks, kb_begin + per_split);
 
-  const unsigned short *xrow = reinterpret_cast<const unsigned short *>(p.x) + (long long)min(m0 + c16, g_end - 1) * p.k;
-  const unsigned ones = BF16 ? 0x3F803F80u : 0x3C003C00u;
-  const v4i ones_frag = v4i{(int)ones, (int)ones, (int)ones, (int)ones};
+  // x fragments of the wave's blocks, through a descriptor over the chunk's rows (zeros past the slice or past K): all
+  // requested before anything waits -- a load under a condition would be waited for on the spot (vmcnt(0)), one
+  // memory round trip per fragment before the first weight is asked for
+  const __amdgpu_buffer_rsrc_t rx = buffer_over(reinterpret_cast<const unsigned short *>(p.x) + (long long)m0 * p.k,
+                                                2ll * chunk_rows * p.k);
+  const unsigned x_row_byte = 2u * (unsigned)min(c16, chunk_rows - 1) * (unsigned)p.k;
   v4i xf[NB][2];
   unsigned voff[NB];
-  v4f rs = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int j = 0; j < NB; ++j) {
     const int kb = kb_begin + wave + ST_WAVES * j;
     const int k0 = kb * 64 + 16 * h;   // K % 16 == 0: the 16 K positions are all inside or all outside
     const bool ok = kb < kb_end && k0 < p.k;
-    xf[j][0] = ok ? *reinterpret_cast<const v4i *>(xrow + k0) : v4i{0, 0, 0, 0};
-    xf[j][1] = ok ? *reinterpret_cast<const v4i *>(xrow + k0 + 8) : v4i{0, 0, 0, 0};
+    xf[j][0] = __builtin_amdgcn_raw_buffer_load_b128(rx, ok ? x_row_byte + 2u * (unsigned)k0 : kBufferOob, 0, 0);
+    xf[j][1] = __builtin_amdgcn_raw_buffer_load_b128(rx, ok ? x_row_byte + 2u * (unsigned)k0 + 16u : kBufferOob, 0, 0);
     voff[j] = kb < kb_end ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob;
-    rs = sa_mfma<BF16>(xf[j][0], ones_frag, rs);
-    rs = sa_mfma<BF16>(xf[j][1], ones_frag, rs);
   }
 
   v4i ring[D];
@@ -652,6 +652,22 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
     constexpr int J = decltype(j_c)::value;
     if constexpr (J < D) issue(0, j_c, j_c);
   });
+  // antiquant scale and offset of this thread's output columns (column groups wave + 4 e), requested behind the first
+  // weight loads (16-bit elements: the word that holds them, branch-free; decoded in the epilogue)
+  const bool rows_ok = 4 * h < chunk_rows;
+  unsigned sc_word[4], of_word[4];
+  {
+    const __amdgpu_buffer_rsrc_t rs_sc = buffer_over(p.aq_scale, p.aq_scale ? 2ll * p.e * p.n : 0);
+    const __amdgpu_buffer_rsrc_t rs_of = buffer_over(p.aq_offset, p.aq_offset ? 2ll * p.e * p.n : 0);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int n = n0 + 16 * (wave + 4 * e) + c16;
+      const bool live = wave + 4 * e < cg_count && n < p.n && rows_ok;
+      const unsigned byte = 2u * (unsigned)((long long)grp * p.n + n);
+      sc_word[e] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_sc, live ? (byte & ~3u) : kBufferOob, 0, 0);
+      of_word[e] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_of, live ? (byte & ~3u) : kBufferOob, 0, 0);
+    }
+  }
   for (int cg = 0; cg < cg_count; ++cg) {
     v4f a0 = v4f{0.f, 0.f, 0.f, 0.f}, a1 = v4f{0.f, 0.f, 0.f, 0.f};
     static_for<NB>([&](auto j_c) {
@@ -664,8 +680,20 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
       a1 = sa_mfma<BF16>(xf[J][1], sa_frag<BF16>(d2, d3), a1);
       if constexpr (J + D < NB) issue(cg, std::integral_constant<int, J + D>{}, std::integral_constant<int, SLOT>{});
       else issue(cg + 1, std::integral_constant<int, J + D - NB>{}, std::integral_constant<int, SLOT>{});
+      // the refill stays behind the step that freed its slot: left to itself the scheduler gathers the next column
+      // group's loads at the end of the loop body, and the wave's load queue runs empty once per column group
+      __builtin_amdgcn_sched_barrier(0);
     });
     red[wave][cg][lane] = a0 + a1;
+  }
+  // row sums of x over the wave's K blocks (for the offset term), by the matrix pipe against a fragment of ones
+  const unsigned ones = BF16 ? 0x3F803F80u : 0x3C003C00u;
+  const v4i ones_frag = v4i{(int)ones, (int)ones, (int)ones, (int)ones};
+  v4f rs = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < NB; ++j) {
+    rs = sa_mfma<BF16>(xf[j][0], ones_frag, rs);
+    rs = sa_mfma<BF16>(xf[j][1], ones_frag, rs);
   }
   red_rs[wave][lane] = rs;
   __syncthreads();
@@ -686,7 +714,6 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
   v4f xs = red_rs[0][lane];
 #pragma unroll
   for (int w = 1; w < ST_WAVES; ++w) xs += red_rs[w][lane];
-  const bool rows_ok = 4 * h < chunk_rows;
 
   if (p.split_k > 1) {
     // float32 partials through the workspace, added in slice order by the last arriver.  Slice s: word e (0..7) of
@@ -748,15 +775,14 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
   // ---- epilogue: v[e] = rows 4h..4h+3 of column 16 (wave + 4 e) + c --------------------------------------------
   unsigned short(*tile_out)[ST_COLS + 8] = reinterpret_cast<unsigned short(*)[ST_COLS + 8]>(st_smem);
   __syncthreads();   // every wave is done reading red[]
-  const unsigned short *sc = reinterpret_cast<const unsigned short *>(p.aq_scale);
-  const unsigned short *of = reinterpret_cast<const unsigned short *>(p.aq_offset);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int cl = 16 * (wave + 4 * e) + c16;
     const int n = n0 + cl;
     if (wave + 4 * e < cg_count && n < p.n && rows_ok) {
-      const float s = sc ? sa_half_like<BF16>(sc[(long long)grp * p.n + n]) : 1.0f;
-      const float o = of ? sa_half_like<BF16>(of[(long long)grp * p.n + n]) : 0.0f;
+      const bool upper = ((long long)grp * p.n + n) & 1;   // which half of its word the element is
+      const float s = p.aq_scale ? sa_half_like<BF16>((unsigned short)(upper ? sc_word[e] >> 16 : sc_word[e])) : 1.0f;
+      const float o = p.aq_offset ? sa_half_like<BF16>((unsigned short)(upper ? of_word[e] >> 16 : of_word[e])) : 0.0f;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float f = fmaf(o - 128.0f, xs[r], v[e][r]) * s;

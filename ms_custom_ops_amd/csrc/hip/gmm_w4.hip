@@ -23,7 +23,10 @@ namespace msco {
 namespace {
 
 constexpr int W4_ROWS = 4;           // rows of a group held in LDS at a time (k bytes each: small, so that many workgroups fit a CU)
-constexpr int W4_WAVE_COLS = 4;      // columns per lane segment of a wavefront, all in registers at once
+#ifndef MSCO_W4_WAVE_COLS
+#define MSCO_W4_WAVE_COLS 4
+#endif
+constexpr int W4_WAVE_COLS = MSCO_W4_WAVE_COLS;      // columns per lane segment of a wavefront, all in registers at once
 constexpr int W4_MAX_K = 8192;
 constexpr int W4_LANE_PIECES = W4_MAX_K / 32 / 64;   // 16-byte pieces of a column per lane
 
@@ -37,13 +40,16 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
   // blockIdx.y counts the groups that hold rows (at most min(e, m) of them): find the one with that rank, 64 groups
   // per round of ballots, and leave if there are fewer
   int grp = -1, g_start = 0, g_end = 0;
+  const __amdgpu_buffer_rsrc_t rs_list = buffer_over(group_list, 4ll * e);
   for (int g0 = 0, seen = 0, carry = 0; g0 < e && grp < 0; g0 += 256) {
-    int lo[4], hi[4];   // four rounds' worth of boundaries requested together: one memory round trip per 256 groups
+    // four rounds' worth of boundaries requested together: one memory round trip per 256 groups.  Through a buffer
+    // descriptor over the list (entries past its end read as 0): a load under `g < e ? ... : 0` is a branch, and the
+    // compiler waits for every such load (vmcnt(0)) where its value meets the 0 of the other path.
+    int lo[4], hi[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int g = g0 + 64 * u + lane;
-      hi[u] = g < e ? min(max(group_list[g], 0), m) : 0;
-    }
+    for (int u = 0; u < 4; ++u) hi[u] = __builtin_amdgcn_raw_buffer_load_b32(rs_list, 4u * (unsigned)(g0 + 64 * u + lane), 0, 0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) hi[u] = min(max(hi[u], 0), m);
     // row end of a group = running maximum of the list clamped into [0, m] (a list that is not monotonic can then
     // never make two groups overlap); `carry` is the end of the last group of the round before
 #pragma unroll
@@ -78,32 +84,69 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
   const int pieces_per_group = group_size / 32;
   const unsigned char *wg = w + (long long)grp * n * (k / 2);
   const float *sg = w_scale + (long long)grp * k_groups * n;
-  const int col0 = (blockIdx.x * 4 + wave) * W4_WAVE_COLS * side + sub;   // this lane's columns: col0 + c * side
+  const int wg_cols = 4 * W4_WAVE_COLS * side;          // columns of this workgroup
+  const int col_base = blockIdx.x * wg_cols;
+  const int col0 = col_base + wave * W4_WAVE_COLS * side + sub;   // this lane's columns: col0 + c * side
 
-  // this wavefront's columns: every piece and its scale requested at once (one memory round trip), nibbles as u ^ 8
+  // this wavefront's columns: every piece and its scale requested at once (one memory round trip), nibbles as u ^ 8.
+  // Branch-free, through buffer descriptors over this workgroup's columns of the group's weights and scales: what a
+  // lane has no use for (a piece past K, a column past N) is asked at an offset beyond the descriptor and reads as 0.
+  const int cols_here = min(wg_cols, n - col_base);
+  const __amdgpu_buffer_rsrc_t rs_w = buffer_over(wg + (long long)col_base * (k / 2), (long long)cols_here * (k / 2));
+  const __amdgpu_buffer_rsrc_t rs_s = buffer_over(sg + col_base, 4ll * ((long long)(k_groups - 1) * n + cols_here));
+  // (Staging the scales through LDS with coalesced requests measured slower, 12.4 against 11.4 us: the per-lane form
+  // below repeats cache lines, but it needs no barrier between the scales and the first dot product.)
   uint4 wv[W4_WAVE_COLS][W4_LANE_PIECES];
   float sc[W4_WAVE_COLS][W4_LANE_PIECES];
 #pragma unroll
   for (int c = 0; c < W4_WAVE_COLS; ++c)
 #pragma unroll
     for (int i = 0; i < W4_LANE_PIECES; ++i) {
-      const int p = pl + lanes_per_col * i, col = col0 + c * side;
-      const bool live = p < pieces && col < n;
-      wv[c][i] = live ? *(reinterpret_cast<const uint4 *>(wg + (long long)col * (k / 2)) + p) : make_uint4(0x88888888u, 0x88888888u, 0x88888888u, 0x88888888u);
-      sc[c][i] = live ? sg[(long long)(p / pieces_per_group) * n + col] : 0.f;
+      const int p = pl + lanes_per_col * i, cl = col0 + c * side - col_base;   // column inside the workgroup
+      const bool live = p < pieces && cl < cols_here;
+      const v4i raw = __builtin_amdgcn_raw_buffer_load_b128(rs_w, live ? (unsigned)(cl * (k / 2) + p * 16) : 0xFFFFFFF0u, 0, 0);
+      wv[c][i] = make_uint4((unsigned)raw[0], (unsigned)raw[1], (unsigned)raw[2], (unsigned)raw[3]);
+      sc[c][i] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(
+          rs_s, live ? 4u * (unsigned)((p / pieces_per_group) * n + cl) : 0xFFFFFFFCu, 0, 0));
     }
+
+  // A block of up to W4_ROWS rows of the group is rows * k consecutive bytes of x: thread t holds the 16-byte pieces
+  // t, t + 256, ... of them (requested through a descriptor over just these bytes, so nothing branches), together with
+  // the rows' activation scales.  The first block is requested right behind the weights -- loads return in order, so
+  // it costs no round trip of its own -- and before anything waits for the weights.
+  constexpr int W4_X_VECS = W4_ROWS * (W4_MAX_K / 16) / 256;   // 16-byte pieces of a block per thread
+  uint4 xr[W4_X_VECS];
+  float xsr[W4_ROWS];
+  const __amdgpu_buffer_rsrc_t rs_xs = buffer_over(x_scale, 4ll * m);
+  auto request_rows = [&](int r0, int rows) {
+    const __amdgpu_buffer_rsrc_t rs_x = buffer_over(x + (long long)r0 * k, (long long)rows * k);
+#pragma unroll
+    for (int u = 0; u < W4_X_VECS; ++u) {
+      const v4i raw = __builtin_amdgcn_raw_buffer_load_b128(rs_x, 16u * (unsigned)(threadIdx.x + 256 * u), 0, 0);
+      xr[u] = make_uint4((unsigned)raw[0], (unsigned)raw[1], (unsigned)raw[2], (unsigned)raw[3]);
+    }
+#pragma unroll
+    for (int r = 0; r < W4_ROWS; ++r)
+      xsr[r] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_xs, r < rows ? 4u * (unsigned)(r0 + r) : 0xFFFFFFFCu, 0, 0));
+  };
+  request_rows(g_start, min(W4_ROWS, g_end - g_start));
 
   for (int r0 = g_start; r0 < g_end; r0 += W4_ROWS) {
     const int rows = min(W4_ROWS, g_end - r0);
+    if (r0 != g_start) request_rows(r0, rows);
     __syncthreads();   // the previous block of rows is no longer read
-    for (int idx = threadIdx.x; idx < rows * pieces * 2; idx += 256) {
+#pragma unroll
+    for (int u = 0; u < W4_X_VECS; ++u) {
       // 16 bytes (k0 .. k15 of a half piece) -> two words of even-k bytes and two of odd-k bytes
-      const int r = idx / (pieces * 2), h = idx - r * pieces * 2;
-      const uint4 v = *reinterpret_cast<const uint4 *>(x + (long long)(r0 + r) * k + h * 16);
-      const unsigned e0 = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u), o0 = __builtin_amdgcn_perm(v.y, v.x, 0x07050301u);
-      const unsigned e1 = __builtin_amdgcn_perm(v.w, v.z, 0x06040200u), o1 = __builtin_amdgcn_perm(v.w, v.z, 0x07050301u);
-      int *dst = xs + (r * pieces + (h >> 1)) * 8 + (h & 1) * 2;
-      dst[0] = (int)e0; dst[1] = (int)e1; dst[4] = (int)o0; dst[5] = (int)o1;
+      const int idx = threadIdx.x + 256 * u;
+      if (idx < rows * pieces * 2) {
+        const uint4 v = xr[u];
+        const int r = idx / (pieces * 2), h = idx - r * pieces * 2;
+        const unsigned e0 = __builtin_amdgcn_perm(v.y, v.x, 0x06040200u), o0 = __builtin_amdgcn_perm(v.y, v.x, 0x07050301u);
+        const unsigned e1 = __builtin_amdgcn_perm(v.w, v.z, 0x06040200u), o1 = __builtin_amdgcn_perm(v.w, v.z, 0x07050301u);
+        int *dst = xs + (r * pieces + (h >> 1)) * 8 + (h & 1) * 2;
+        dst[0] = (int)e0; dst[1] = (int)e1; dst[4] = (int)o0; dst[5] = (int)o1;
+      }
     }
     __syncthreads();
     for (int r = 0; r < rows; ++r) {
@@ -134,14 +177,16 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
           }
         }
       }
-      const float xsr = x_scale[r0 + r];
+      float xs_r = xsr[0];   // (selected, not indexed: the array stays in registers)
+#pragma unroll
+      for (int q = 1; q < W4_ROWS; ++q) xs_r = r == q ? xsr[q] : xs_r;
 #pragma unroll
       for (int c = 0; c < W4_WAVE_COLS; ++c) {
         float v = acc[c];
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1)
           if (o < lanes_per_col) v += __shfl_xor(v, o);   // wave-uniform
-        if (pl == 0 && col0 + c * side < n) out[(long long)(r0 + r) * n + col0 + c * side] = f32_to_f16_rne(v * xsr);
+        if (pl == 0 && col0 + c * side < n) out[(long long)(r0 + r) * n + col0 + c * side] = f32_to_f16_rne(v * xs_r);
       }
     }
   }
