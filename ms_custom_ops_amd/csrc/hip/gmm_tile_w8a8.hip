@@ -38,7 +38,10 @@ constexpr int BK = 64;        // bytes of K per slab = one MFMA K step
 constexpr int KN_STAGES = 2;  // LDS stages of the transposed [K,N] weight slab
 constexpr int KN_RING = 3;    // [K,N] weight slabs in flight in registers
 
-__device__ __forceinline__ int swz64(int r) { return (r >> 2) & 3; }
+// rows of BKT bytes in LDS: 16-byte chunk c of row r sits at position c ^ swz<BKT>(r), so that the 16 lanes of a
+// fragment read (16 consecutive rows, one logical chunk) cover all 16 slots of a 256-byte LDS cycle
+template <int BKT>
+__device__ __forceinline__ int swz(int r) { return BKT == 64 ? (r >> 2) & 3 : (r >> 1) & 7; }
 
 // MFMA output row q (0..31) of a 32 x 32 block <-> weight column inside the block.  Lane half hh holds
 // rows q = 8 g + 4 hh + t (g = 0..3, t = 0..3); mapping them to columns 16 (g/2) + 8 hh + 4 (g%2) + t
@@ -108,9 +111,16 @@ __device__ __forceinline__ void wait_vmcnt() {
 // w[k = 64 b + 16 (l / 16) + i][n = 16 a + l % 16]).  A 64-byte K slab of the tile is then one block per column group:
 // the LDS-direct load of a block copies it as it lies, and a weight fragment is read at block (column / 16), chunk
 // 2 kk + hh, row (column % 16) -- conflict free without a swizzle.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES, bool PK = false>
+// KS = 32-byte MFMA K steps per slab (packed weights only for KS = 4): a slab is BKT = 32 KS bytes of K.  With 128-byte
+// slabs every x row piece is a whole cache line (64-byte pieces are half lines, and the load path is bound by line
+// requests), a column group contributes two consecutive 1 KiB blocks, and there is one barrier per 4 K steps.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES, bool PK = false, int KS = 2>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel(const GmmParams p) {
   static_assert(!PK || NK, "packed weights use the LDS-direct weight path");
+  static_assert(KS == 2 || (KS == 4 && NK), "128-byte slabs are built for K-major weights");
+  constexpr int BKT = 32 * KS;                      // bytes of K per slab
+  constexpr int ROWS_PER_LOAD = 1024 / BKT;         // x rows one wave instruction (1 KiB) brings
+  constexpr int KB_PER_SLAB = BKT / 64;             // packed 1 KiB blocks of a column group per slab
   constexpr int NSTAGE = STAGES;
   constexpr int AHEAD = STAGES - 1;                 // slabs requested ahead of the one being multiplied
   static_assert(NK || STAGES == 4, "the [K,N] register ring is three slabs deep");
@@ -118,16 +128,16 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   constexpr int NT = NW * 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   constexpr int FM = WTM / 32, FN = WTN / 32;     // 32 x 32 MFMA blocks per wave
-  constexpr int A_LD = BM / 16 / NW;                // 16-row blocks (1 KiB of LDS) of the x slab per wave
-  constexpr int B_LD = BN / 16 / NW;                // same for an [N,K] weight slab
-  constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK;
+  constexpr int A_LD = BM / ROWS_PER_LOAD / NW;     // 1 KiB pieces (16 or 8 rows) of the x slab per wave
+  constexpr int B_LD = BN * BKT / 1024 / NW;        // same for an [N,K] weight slab
+  constexpr int A_STAGE = BM * BKT, B_STAGE = BN * BKT;
   constexpr int PANEL = 8;                          // m-tiles that share a streamed weight panel
   constexpr unsigned OOB = 0x80000000u;             // buffer offset that always reads zero
   constexpr int VM_PER_SLAB = A_LD + (NK ? B_LD : 8);   // vector-memory loads a wave issues per slab
   // [K,N] weight slab: 8 K-chunks of 8 rows x BN/4 column groups -> one 8(k) x 4(n)-byte block per thread
   static_assert(NK || NT == 2 * BN, "one [K,N] block per thread");
   static_assert(FM >= 1 && FN >= 1 && A_LD >= 1 && B_LD >= 1, "tile shape");
-  static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "row blocks per wave");
+  static_assert(BM % (ROWS_PER_LOAD * NW) == 0 && BN % (16 * NW) == 0, "row blocks per wave");
 
   // LDS: operand ring, reused by the epilogue staging; behind both, the tile's epilogue operands
   constexpr int LOOP_LDS = NSTAGE * A_STAGE + (NK ? NSTAGE : KN_STAGES) * B_STAGE;
@@ -135,7 +145,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   constexpr int PARAM_OFF = LOOP_LDS > EPI_LDS ? LOOP_LDS : EPI_LDS;
   static_assert(BM <= 256 && BN <= 256, "epilogue operand table holds 256 entries");
   extern __shared__ __align__(16) unsigned char smem[];
-  unsigned char *lds_a = smem;                      // [NSTAGE][BM * BK], rows of 64 B, chunk c at c ^ swz64(row)
+  unsigned char *lds_a = smem;                      // [NSTAGE][BM * BKT], rows of BKT bytes, chunk c at c ^ swz<BKT>(row)
   unsigned char *lds_b = smem + NSTAGE * A_STAGE;   // [N,K]: [NSTAGE][BN * BK] like x; [K,N]: [KN_STAGES][4][BN][16]
 
   const int tid = threadIdx.x;
@@ -157,7 +167,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   }
   // K split across workgroups (small problems): the slices of one tile sit next to each other in the
   // grid, on the same XCD
-  const int split = p.split_k > 1 ? p.split_k : 1;
+  constexpr bool CAN_SPLIT = BM * BN <= 128 * 128;   // the plan splits K for the small tile shapes only
+  const int split = (CAN_SPLIT && p.split_k > 1) ? p.split_k : 1;
   const int per_xcd = (total + kNumXcd - 1) / kNumXcd;
   const int slot = blockIdx.x / kNumXcd;
   const int local = slot / split, ks = slot - local * split;
@@ -192,7 +203,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
 
   const int m0 = g_start + mt * BM;
   const int n0 = nt * BN;
-  const int k_slabs_all = (p.k + BK - 1) / BK;
+  const int k_slabs_all = (p.k + BKT - 1) / BKT;
   const int per_slice = (k_slabs_all + split - 1) / split;
   const int k_first = ks * per_slice;                                   // first slab of this workgroup's K slice
   const int k_slabs = max(0, min(k_slabs_all, k_first + per_slice) - k_first);
@@ -229,43 +240,55 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   // Only the per-lane offset is range-checked by the buffer unit, so everything that can run past
   // the tensor (rows, columns, the K tail) lives in the per-lane offset; the scalar offset carries
   // just the slab position inside a row.
-  const int d_row = lane >> 2;
-  const int d_c = (lane & 3) ^ (lane >> 4);
+  // (general form: lane L writes row L / (BKT/16) of its 1 KiB piece, position L % (BKT/16), which holds logical
+  // chunk position ^ swz<BKT>(row); with 128-byte rows the swizzle depends on the piece, so offsets are per piece)
+  constexpr int CHUNKS = BKT / 16;
+  const int d_row = lane / CHUNKS;
   unsigned a_voff[A_LD];
+  int a_chunk[A_LD];                                 // logical chunk of this lane in piece u (for the K tail)
 #pragma unroll
-  for (int u = 0; u < A_LD; ++u) a_voff[u] = (unsigned)((wave * A_LD + u) * 16 + d_row) * (unsigned)p.k + d_c * 16;
+  for (int u = 0; u < A_LD; ++u) {
+    const int row = (wave * A_LD + u) * ROWS_PER_LOAD + d_row;
+    a_chunk[u] = (lane % CHUNKS) ^ swz<BKT>(row);
+    a_voff[u] = (unsigned)row * (unsigned)p.k + a_chunk[u] * 16;
+  }
   // [N,K] weights: LDS row rho = 32 * block + q feeds MFMA row q of that block and holds weight
   // column 32 * block + col_of_q(q) of the tile.
   unsigned b_voff[NK ? B_LD : 1];
+  int b_chunk[NK ? B_LD : 1];                        // row-major weights: logical chunk of this lane in piece u
   if constexpr (NK) {
 #pragma unroll
     for (int u = 0; u < B_LD; ++u) {
       const int blk = wave * B_LD + u;
-      const int rho = blk * 16 + d_row;
-      if constexpr (PK) b_voff[u] = (unsigned)(blk * pk_blocks * 1024 + lane * 16);   // column group blk of the tile
-      else b_voff[u] = (unsigned)((rho & ~31) + col_of_q(rho & 31)) * (unsigned)p.k + d_c * 16;
+      const int rho = blk * ROWS_PER_LOAD + d_row;
+      b_chunk[u] = (lane % CHUNKS) ^ swz<BKT>(rho);
+      if constexpr (PK) b_voff[u] = (unsigned)((blk / KB_PER_SLAB) * pk_blocks * 1024 + lane * 16);   // piece blk: column group blk / KB_PER_SLAB of the tile
+      else b_voff[u] = (unsigned)((rho & ~31) + col_of_q(rho & 31)) * (unsigned)p.k + b_chunk[u] * 16;
     }
   }
   auto issue_direct = [&](int kt) {
     const int stage = kt % NSTAGE;
-    const unsigned kbase = (k_first + kt) * BK;
+    const unsigned kbase = (k_first + kt) * BKT;
     // K tail, and whole slabs past K (requested by the last steps of the branch-free loop): read as zero
-    const unsigned kill = (kbase + d_c * 16 >= (unsigned)p.k) ? OOB : 0u;
 #pragma unroll
     for (int u = 0; u < A_LD; ++u) {
       const int blk = wave * A_LD + u;
-      buffer_load_lds_b128(rx, lds_a + stage * A_STAGE + blk * 1024, a_voff[u] | kill, kbase);
+      const unsigned kill_a = (kbase + a_chunk[u] * 16 >= (unsigned)p.k) ? OOB : 0u;
+      buffer_load_lds_b128(rx, lds_a + stage * A_STAGE + blk * 1024, a_voff[u] | kill_a, kbase);
     }
     if constexpr (NK) {
 #pragma unroll
       for (int u = 0; u < B_LD; ++u) {
         const int blk = wave * B_LD + u;
         if constexpr (PK) {
-          // K block k_first + kt of the column group; blocks past K do not exist (the last one is zero padded)
-          const unsigned kill_w = (k_first + kt >= pk_blocks) ? OOB : 0u;
-          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, (k_first + kt) * 1024);
+          // K block (k_first + kt) KB_PER_SLAB + blk % KB_PER_SLAB of the column group; blocks past K do not exist
+          // (the last one is zero padded)
+          const int kblock = (k_first + kt) * KB_PER_SLAB + blk % KB_PER_SLAB;
+          const unsigned kill_w = (kblock >= pk_blocks) ? OOB : 0u;
+          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, kblock * 1024);
         } else {
-          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill, kbase);
+          const unsigned kill_b = (kbase + b_chunk[u] * 16 >= (unsigned)p.k) ? OOB : 0u;
+          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase);
         }
       }
     }
@@ -310,17 +333,19 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   auto read_x = [&](int kt, int i, int kk) -> v4i {
     const unsigned char *a = lds_a + (kt % NSTAGE) * A_STAGE;
     const int row = wave_m * WTM + 32 * i + l32;
-    return *reinterpret_cast<const v4i *>(a + row * BK + (((2 * kk + hh) ^ swz64(row)) << 4));
+    return *reinterpret_cast<const v4i *>(a + row * BKT + (((2 * kk + hh) ^ swz<BKT>(row)) << 4));
   };
   auto read_w = [&](int kt, int f, int kk) -> v4i {
     const int rho = wave_n * WTN + 32 * f + l32;
     if constexpr (PK) {
       const unsigned char *b = lds_b + (kt % NSTAGE) * B_STAGE;
       const int col = wave_n * WTN + 32 * f + col_of_q(l32);   // MFMA row l32 of block f is this column of the tile
-      return *reinterpret_cast<const v4i *>(b + (col >> 4) * 1024 + (2 * kk + hh) * 256 + (col & 15) * 16);
+      // chunk 2 kk + hh of the slab: block (2 kk + hh) / 4 of the column group's blocks in this slab, chunk % 4 inside it
+      return *reinterpret_cast<const v4i *>(b + ((col >> 4) * KB_PER_SLAB + ((2 * kk + hh) >> 2)) * 1024 +
+                                            ((2 * kk + hh) & 3) * 256 + (col & 15) * 16);
     } else if constexpr (NK) {
       const unsigned char *b = lds_b + (kt % NSTAGE) * B_STAGE;
-      return *reinterpret_cast<const v4i *>(b + rho * BK + (((2 * kk + hh) ^ swz64(rho)) << 4));
+      return *reinterpret_cast<const v4i *>(b + rho * BKT + (((2 * kk + hh) ^ swz<BKT>(rho)) << 4));
     } else {
       // 16 K bytes of chunk c = 2 kk + hh: planes 2 c and 2 c + 1, 8 bytes each.  Read with
       // hand-written ds_read_b64: the compiler makes every LDS read it knows about wait for all
@@ -371,13 +396,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     constexpr int SLOT = decltype(ring_slot)::value;          // == kt % KN_RING, compile-time for register indexing
     issue_direct(kt + AHEAD);
     load_kn(kt + 3, SLOT);                                    // (kt + 3) % 3 == kt % 3: that slot was emptied last step
-    v4i xf[2][FM], wf[2][FN];
+    v4i xf[KS][FM], wf[KS][FN];
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
+    for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
       for (int f = 0; f < FN; ++f) wf[kk][f] = read_w(kt, f, kk);
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
+    for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
       for (int i = 0; i < FM; ++i) xf[kk][i] = read_x(kt, i, kk);
     if constexpr (!NK) {
@@ -395,7 +420,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
       __builtin_amdgcn_s_setprio(2);
     }
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk)
+    for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
       for (int f = 0; f < FN; ++f)
 #pragma unroll
@@ -440,7 +465,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   // workgroup), takes a ticket on the tile's counter, and all but the last one leave.  int32 addition
   // is associative, so the result does not depend on the arrival order.  Agent-scope relaxed atomics
   // keep the exchange in L2 without cache-wide fences; the counter resets itself for the next launch.
-  if (split > 1) {
+  if constexpr (CAN_SPLIT) if (split > 1) {
     __shared__ unsigned s_ticket;
     constexpr int TILE_INTS = BM * BN;
     constexpr int WORDS = FN * FM * 8;   // 64-bit words per thread: accumulator registers (r, r + 1) travel together
@@ -461,6 +486,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     __syncthreads();
     if (s_ticket != (unsigned)(split - 1)) return;
     if (tid == 0) __hip_atomic_store(&p.counters[lid], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // (two slices per round trip measured slower: 15.7 against 15.1 us on the M = 128 dense case)
     for (int s = 0; s < split; ++s) {
       if (s == ks) continue;
       const i64 *other = base + (long long)s * (TILE_INTS / 2) + tid;
@@ -584,12 +610,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
 }
 
 // ---- host launcher ---------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4, bool PK = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4, bool PK = false, int KS = 2>
 static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
-  const size_t loop_lds = (size_t)STAGES * BM * BK + (size_t)(NK ? STAGES : KN_STAGES) * BN * BK;
+  constexpr int BKT = 32 * KS;
+  const size_t loop_lds = (size_t)STAGES * BM * BKT + (size_t)(NK ? STAGES : KN_STAGES) * BN * BKT;
   const size_t epi_lds = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * 144;   // epilogue staging, 144-byte row pitch
   const size_t lds = (loop_lds > epi_lds ? loop_lds : epi_lds) + 3 * 1024;   // + epilogue operand table
-  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES, PK>;
+  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES, PK, KS>;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -606,11 +633,19 @@ static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// The small tile shapes on K-major weights (row-major [E,N,K] or packed) run 128-byte K slabs through a 4-stage ring
+// (measured against 64-byte slabs on M = 256, K = 4096, N = 11008 packed: 26.0 against 28.8 us; 3 / 2 stages 26.7 / 34.1)
+#ifndef MSCO_SMALL_TILE_KS
+#define MSCO_SMALL_TILE_KS 4
+#endif
+#ifndef MSCO_SMALL_TILE_STAGES
+#define MSCO_SMALL_TILE_STAGES 4
+#endif
 hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool packed, hipStream_t stream) {
   if (packed) {
     switch (tile_cfg) {
-      case TILE_128x128: return launch_cfg<128, 128, 2, 2, true, 4, true>(p, stream);
-      case TILE_64x128: return launch_cfg<64, 128, 2, 2, true, 4, true>(p, stream);
+      case TILE_128x128: return launch_cfg<128, 128, 2, 2, true, MSCO_SMALL_TILE_KS == 4 ? MSCO_SMALL_TILE_STAGES : 4, true, MSCO_SMALL_TILE_KS>(p, stream);
+      case TILE_64x128: return launch_cfg<64, 128, 2, 2, true, MSCO_SMALL_TILE_KS == 4 ? MSCO_SMALL_TILE_STAGES : 4, true, MSCO_SMALL_TILE_KS>(p, stream);
       case TILE_256x256_W4:
         if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, true, stream);
         return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
@@ -622,9 +657,11 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
     case TILE_256x256:
       return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     case TILE_128x128:
-      return nk ? launch_cfg<128, 128, 2, 2, true>(p, stream) : launch_cfg<128, 128, 2, 2, false>(p, stream);
+      return nk ? launch_cfg<128, 128, 2, 2, true, MSCO_SMALL_TILE_KS == 4 ? MSCO_SMALL_TILE_STAGES : 4, false, MSCO_SMALL_TILE_KS>(p, stream)
+                : launch_cfg<128, 128, 2, 2, false>(p, stream);
     case TILE_64x128:
-      return nk ? launch_cfg<64, 128, 2, 2, true>(p, stream) : launch_cfg<64, 128, 2, 2, false>(p, stream);
+      return nk ? launch_cfg<64, 128, 2, 2, true, MSCO_SMALL_TILE_KS == 4 ? MSCO_SMALL_TILE_STAGES : 4, false, MSCO_SMALL_TILE_KS>(p, stream)
+                : launch_cfg<64, 128, 2, 2, false>(p, stream);
     case TILE_128x256:   // two 4-wave workgroups per CU; [N,K] weights only
       return nk ? launch_cfg<128, 256, 1, 4, true, 3>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     case TILE_256x256_W4:   // needs [N,K] weights, at least four 128-byte K slabs per tile, a group table that fits in LDS
@@ -638,8 +675,8 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
 const char *tile_cfg_name(int tile_cfg) {
   switch (tile_cfg) {
     case TILE_256x256: return "256x256x64";
-    case TILE_128x128: return "128x128x64";
-    case TILE_64x128: return "64x128x64";
+    case TILE_128x128: return "128x128";   // 128-byte K slabs on K-major weights, 64-byte on [E,K,N]
+    case TILE_64x128: return "64x128";
     case TILE_128x256: return "128x256x64";
     case TILE_256x256_W4: return "256x256x128_w4";
     default: return "?";
