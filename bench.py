@@ -62,7 +62,7 @@ def parse():
 class DeviceProblem:
     """One workload resident on the GPU plus a planned backend operator."""
 
-    def __init__(self, wl, layout="kn", copies=1, zero_operands=False, act_type=0, force_split_k=0):
+    def __init__(self, wl, layout="kn", copies=1, zero_operands=False, act_type=0, force_split_k=0, kernel_override=0):
         import torch
         from ms_custom_ops_amd import cabi
         self.torch, self.cabi, self.wl = torch, cabi, wl
@@ -116,7 +116,7 @@ class DeviceProblem:
             self.op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,
                                  scale_dtype=cabi.DT_F32, per_token_dtype=cabi.DT_F32,
                                  bias_dtype=cabi.DT_I32 if self.bias is not None else cabi.DT_NONE,
-                                 transpose_b=int(nk), act_type=act_type, force_split_k=force_split_k,
+                                 transpose_b=int(nk), act_type=act_type, force_split_k=force_split_k, kernel_override=kernel_override,
                                  weight_layout=cabi.WL_PACKED if layout == "packed" else cabi.WL_ROW_MAJOR)
         self.ws_bytes = self.op.plan(wl.m, wl.k, wl.n, wl.e)
         self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)

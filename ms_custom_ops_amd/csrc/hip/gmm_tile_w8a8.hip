@@ -634,18 +634,20 @@ static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
 }
 
 // The small tile shapes on K-major weights (row-major [E,N,K] or packed) run 128-byte K slabs through a 4-stage ring
-// (measured against 64-byte slabs on M = 256, K = 4096, N = 11008 packed: 26.0 against 28.8 us; 3 / 2 stages 26.7 / 34.1)
-#ifndef MSCO_SMALL_TILE_KS
-#define MSCO_SMALL_TILE_KS 4
-#endif
-#ifndef MSCO_SMALL_TILE_STAGES
-#define MSCO_SMALL_TILE_STAGES 4
-#endif
+// when the plan says so (GmmParams::wide_k_slabs: the workgroups fit one round; measured against 64-byte slabs on M = 256,
+// K = 4096, N = 11008 packed: 26.0 against 28.8 us; 3 / 2 stages 26.7 / 34.1)
+template <int BM, int BN>
+static hipError_t launch_small(const GmmParams &p, bool nk, bool packed, hipStream_t stream) {
+  if (packed) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, true, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, true, 4, true>(p, stream);
+  if (nk) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, false, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, true>(p, stream);
+  return launch_cfg<BM, BN, 2, 2, false>(p, stream);
+}
+
 hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool packed, hipStream_t stream) {
+  if (tile_cfg == TILE_128x128) return launch_small<128, 128>(p, nk, packed, stream);
+  if (tile_cfg == TILE_64x128) return launch_small<64, 128>(p, nk, packed, stream);
   if (packed) {
     switch (tile_cfg) {
-      case TILE_128x128: return launch_cfg<128, 128, 2, 2, true, MSCO_SMALL_TILE_KS == 4 ? MSCO_SMALL_TILE_STAGES : 4, true, MSCO_SMALL_TILE_KS>(p, stream);
-      case TILE_64x128: return launch_cfg<64, 128, 2, 2, true, MSCO_SMALL_TILE_KS == 4 ? MSCO_SMALL_TILE_STAGES : 4, true, MSCO_SMALL_TILE_KS>(p, stream);
       case TILE_256x256_W4:
         if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, true, stream);
         return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
@@ -656,12 +658,6 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
   switch (tile_cfg) {
     case TILE_256x256:
       return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
-    case TILE_128x128:
-      return nk ? launch_cfg<128, 128, 2, 2, true, MSCO_SMALL_TILE_KS == 4 ? MSCO_SMALL_TILE_STAGES : 4, false, MSCO_SMALL_TILE_KS>(p, stream)
-                : launch_cfg<128, 128, 2, 2, false>(p, stream);
-    case TILE_64x128:
-      return nk ? launch_cfg<64, 128, 2, 2, true, MSCO_SMALL_TILE_KS == 4 ? MSCO_SMALL_TILE_STAGES : 4, false, MSCO_SMALL_TILE_KS>(p, stream)
-                : launch_cfg<64, 128, 2, 2, false>(p, stream);
     case TILE_128x256:   // two 4-wave workgroups per CU; [N,K] weights only
       return nk ? launch_cfg<128, 256, 1, 4, true, 3>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     case TILE_256x256_W4:   // needs [N,K] weights, at least four 128-byte K slabs per tile, a group table that fits in LDS

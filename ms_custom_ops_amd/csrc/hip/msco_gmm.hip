@@ -71,6 +71,7 @@ struct msco_gmm_op {
   int n_strips = 0;
   int strip_groups = 16;
   int stream_tch = 1;        // packed W8A8: 16-row fragments per chunk (1: gmm_w8a8_stream_kernel, 2/4/8: the multi-row kernel)
+  int wide_k_slabs = 0;      // small tile kernels on K-major weights: 128-byte K slabs
   size_t workspace_bytes = 0;
   unsigned *counters = nullptr;
   size_t counters_cap = 0;
@@ -139,6 +140,7 @@ void choose_plan(msco_gmm_op *op) {
   op->n_strips = (int)((n + kSkinnyCols - 1) / kSkinnyCols);
   op->workspace_bytes = 0;
   op->tile_cfg = TILE_256x256;
+  op->wide_k_slabs = 0;
 
   int family;
   // packed weights are K-contiguous per column like [E,N,K]: the same tile kernels read them
@@ -149,13 +151,13 @@ void choose_plan(msco_gmm_op *op) {
     family = FAM_GENERIC;
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
-  } else if (is_packed(d) ? (m <= kSkinnyMaxRows || many_small_groups)
-                          : ((m <= kSkinnyMaxRows && !(e == 1 && m > 2 * kSkinnyRows)) || many_small_groups)) {
+  } else if ((m <= kSkinnyMaxRows && !(e == 1 && m > (k_major ? 1 : 2) * kSkinnyRows)) || many_small_groups) {
     // decode: few rows in total, or groups of about one 16-row chunk each (the weights stream once per chunk).  The
     // grid enumerates every (group, chunk) a malformed-to-the-limit group_list could fill; beyond a thousand slots
-    // the empty workgroups cost more than the tile kernel's partial tiles.  On row-major weights a single group of
-    // more than two 16-row chunks would stream the weights once per chunk and takes the small tile instead; on packed
-    // weights the multi-row streaming kernel covers up to 64 rows in one pass.
+    // the empty workgroups cost more than the tile kernel's partial tiles.  A single group of more than one 16-row
+    // chunk (two on [E,K,N] weights) takes the small tile kernel with a K split instead (measured on packed weights,
+    // K = 4096, N = 11008: 32 / 48 / 64 rows 17.1 / 17.5 / 18.0 us against 18.7 / 24.4 / 26.3 us of the multi-row
+    // streaming kernel, which stays for several groups of a few dozen rows each).
     family = FAM_SKINNY;
   } else {
     family = FAM_TILE;
@@ -200,10 +202,28 @@ void choose_plan(msco_gmm_op *op) {
       int bm, bn;
       tile_cfg_dims(op->tile_cfg, &bm, &bn);
       const int64_t t = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
-      const int target = or_default(tuning().tile_target_wgs, kTileTargetWorkgroups);
-      int want = t <= kTileSplitMaxTiles ? (int)((target + t / 2) / std::max<int64_t>(t, 1)) : 1;
+      // t tiles x s slices run in ceil(t s / CUs) rounds (the operand ring takes most of a CU's LDS: one workgroup per
+      // CU).  In units of one 64-byte K slab of a tile (0.2 us): a round costs its slabs plus 10 (prologue, epilogue),
+      // a split adds 8 per slice for 64 x 128 tiles and 12 for 128 x 128 (its partial tile out and in, one round trip of
+      // the last arriver), less 2.  The cheapest s wins, the smaller one on a tie.  Fitted to M = 128, K = N = 4096
+      // (64 tiles; s = 1 / 2 / 3 / 4 / 6: 18.7 / 15.2 / 14.5 / 15.3 / 21.3 us) and M = 64, K = 4096, N = 11008 (86 tiles;
+      // s = 1 / 2 / 3: 20.9 / 18.0 / 24.3 us, the third slice starting a second round).
+      const int cus = or_default(tuning().tile_target_wgs, num_cus > 0 ? num_cus : kTileTargetWorkgroups);
       const int cap = (int)std::max<int64_t>(1, ((k + 63) / 64) / kTileMinSlabs);
-      want = std::max(1, std::min(std::min(want, kMaxSplitK), cap));
+      auto split_cost = [&](int sl) {
+        const int64_t slabs = ((k + 63) / 64 + sl - 1) / sl;
+        const int64_t rounds = (t * sl + cus - 1) / cus;
+        const int64_t exchange = sl > 1 ? (int64_t)(4 + bm * bn / 2048) * sl - 2 : 0;
+        return rounds * (slabs + 10 + exchange);
+      };
+      int want = 1;
+      if (t <= kTileSplitMaxTiles && k_major) {
+        for (int sl = 2; sl <= std::min(kMaxSplitK, cap); ++sl)
+          if (split_cost(sl) < split_cost(want)) want = sl;
+      } else if (t <= kTileSplitMaxTiles) {
+        // [E,K,N] weights (64-byte slabs, two workgroups per CU, register-transposed weights): about one workgroup per CU
+        want = std::max(1, std::min(std::min((int)((cus + t / 2) / std::max<int64_t>(t, 1)), kMaxSplitK), cap));
+      }
       const int forced_split = d.force_split_k > 0 ? d.force_split_k : tuning().tile_split_k;
       if (forced_split > 0) want = std::min(forced_split, cap);
       // the partial tiles of a K split are sized for the worst group_list (one partial m-tile per group): with many
@@ -211,6 +231,10 @@ void choose_plan(msco_gmm_op *op) {
       while (want > 1 && tile_workspace_bytes(op->tile_cfg, m, n, e, want) > kTileSplitMaxWorkspace) want /= 2;
       op->split_k = want;
       op->workspace_bytes = tile_workspace_bytes(op->tile_cfg, m, n, e, op->split_k);
+      // 128-byte K slabs (a 4-stage ring of them takes most of a CU's LDS: one workgroup per CU) when the workgroups
+      // run in one round; more tiles than CUs keep 64-byte slabs and two workgroups per CU (M = 512, N = 11008: 344
+      // tiles, 46.8 us against 50.1 us)
+      op->wide_k_slabs = k_major && t * want <= (num_cus > 0 ? num_cus : kTileTargetWorkgroups);
     }
   }
   op->stream_tch = 1;
@@ -449,6 +473,7 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   // rows a 16-row chunk is expected to hold (shapes only): measured on the dense 45 MB decode, 16 rows 13.1 -> 12.35 us with
   // the x rows staged through LDS, one row 11.85 -> 12.2 us, four rows per chunk (8 experts x 32 rows) 70.1 -> 70.4 us
   p.x_via_lds = (h->e > 0 ? (h->m + h->e - 1) / h->e : h->m) >= 8;
+  p.wide_k_slabs = h->wide_k_slabs;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t err = hipSuccess;

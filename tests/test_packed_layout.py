@@ -86,12 +86,22 @@ def test_counts_and_rows_past_the_last_boundary(device):
     (300, 720, 144, 2, [100, 300]),                             # chunks of 128 rows, K not a multiple of 64
     (500, 512, 64, 8, [0, 40, 40, 200, 210, 350, 480, 490]),    # ragged groups, empty groups, rows past the last boundary
     (1000, 256, 1040, 4, [250, 500, 750, 1000]),                # several chunks per group, 17 strips
+    (60, 1024, 160, 3, [25, 25, 60]),                           # a few dozen rows in several groups: planned by itself
 ])
 def test_multi_row_streaming_kernel_is_bit_exact(device, m, k, n, e, gl):
-    """Planned by itself up to 64 rows; forced here for the larger cases (which the plan gives to the tile kernels)."""
+    """Planned by itself for up to 64 rows in several groups; forced here for the other cases (one group of more than
+    16 rows, or more rows, go to the tile kernels)."""
     x, w, bias, scale, pt = _inputs(16, m, k, n, e)
-    info = _check(x, w, gl, bias, scale, pt, src_transposed=(e == 8), override=cabi.OV_AUTO if m <= 64 else cabi.OV_SKINNY)
+    auto = m <= 64 and e > 1
+    info = _check(x, w, gl, bias, scale, pt, src_transposed=(e == 8), override=cabi.OV_AUTO if auto else cabi.OV_SKINNY)
     assert "w8a8_stream_rows" in info and "layout=packed" in info
+
+
+@pytest.mark.parametrize("m,k,n", [(17, 512, 80), (32, 4096, 1408), (48, 1024, 128), (64, 2048, 272)])
+def test_one_group_of_17_to_64_rows_takes_the_small_tile_with_a_k_split(device, m, k, n):
+    x, w, bias, scale, pt = _inputs(26, m, k, n, 1)
+    info = _check(x, w, [m], bias, scale, pt)
+    assert "w8a8_tile_64x128" in info and "layout=packed" in info, info
 
 
 @pytest.mark.parametrize("family,override", [("64x128", cabi.OV_TILE_64), ("128x128", cabi.OV_TILE_128), ("256x256x64", cabi.OV_TILE_256)])
