@@ -44,14 +44,15 @@ int env_int(const char *name, int fallback) {
 // Debug switches, read from the environment once per process (the first plan); planning itself reads no environment.
 struct Tuning {
   int print_plan, tile_cfg, tile_target_wgs, tile_split_k, stream_max_slots, skinny_wide16, stream_min_wgs, stream_groups,
-      skinny_target_wgs, skinny_split_k;
+      skinny_target_wgs, skinny_split_k, tile_wide_k, stream_tch;
 };
 const Tuning &tuning() {
   static const Tuning t = {env_int("MSCO_PRINT_PLAN", 0),        env_int("MSCO_TILE_CFG", -1),
                            env_int("MSCO_TILE_TARGET_WGS", 0),   env_int("MSCO_TILE_SPLIT_K", 0),
                            env_int("MSCO_STREAM_MAX_SLOTS", 0),  env_int("MSCO_SKINNY_WIDE16", -1),
                            env_int("MSCO_STREAM_MIN_WGS", 0),    env_int("MSCO_STREAM_GROUPS", 0),
-                           env_int("MSCO_SKINNY_TARGET_WGS", 0), env_int("MSCO_SKINNY_SPLIT_K", 0)};
+                           env_int("MSCO_SKINNY_TARGET_WGS", 0), env_int("MSCO_SKINNY_SPLIT_K", 0),
+                           env_int("MSCO_TILE_WIDE_K", -1),      env_int("MSCO_STREAM_TCH", 0)};
   return t;
 }
 int or_default(int v, int fallback) { return v > 0 ? v : fallback; }
@@ -145,7 +146,11 @@ void choose_plan(msco_gmm_op *op) {
   int family;
   // packed weights are K-contiguous per column like [E,N,K]: the same tile kernels read them
   const bool k_major = d.transpose_b != 0 || is_packed(d);
-  const bool many_small_groups = e > 1 && (m + e - 1) / e <= kSkinnyRows &&
+  // (row-major [E,N,K] weights have 16-row chunks only: a group that overflows its chunk streams its weights twice, so
+  // 1.5 x the average has to fit -- 128 rows over 8 experts: 111 us with 64 x 128 tiles against 140 us)
+  const int64_t avg_rows = (m + (e > 0 ? e : 1) - 1) / (e > 0 ? e : 1);
+  const bool nk_row_major = d.transpose_b != 0 && !is_packed(d);
+  const bool many_small_groups = e > 1 && (nk_row_major ? avg_rows + avg_rows / 2 : avg_rows) <= kSkinnyRows &&
                                  e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots;
   if (!aligned) {
     family = FAM_GENERIC;
@@ -164,7 +169,19 @@ void choose_plan(msco_gmm_op *op) {
     // tile shape from shapes only: average rows per group and how many tiles fill 256 CUs
     const int64_t rows_per_group = m / (e > 0 ? e : 1);
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    if (rows_per_group >= 192 && tiles(256, 256) >= 256) {
+    // several groups on K-major weights, a few dozen to a few hundred rows each: the launch is bound by the weight
+    // stream (every group's matrix is read once per m-tile of the group), so the m-tile should hold a whole group --
+    // real routings are uneven, hence 1.5 x the average -- as long as there are tiles for most CUs.  Measured (E = 8,
+    // K = 4096, N = 14336, packed; 64 x 128 / 128 x 128 / 256 x 256 tiles): 64 rows per group 112 / 97 / 100 us, 128 rows per
+    // group 162 / 150 / 109 us, 32 rows per group 87.5 us with the first.
+    auto group_tiles = [&](int bm, int bn) { return e * ((rows_per_group + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    const int64_t cover = rows_per_group + rows_per_group / 2;
+    const int64_t busy = (num_cus > 0 ? num_cus : kTileTargetWorkgroups) * 3 / 4;
+    if (e > 1 && k_major && cover > 128 && cover <= 384 && k >= 512 && e <= 1024 && group_tiles(256, 256) >= busy) {
+      op->tile_cfg = TILE_256x256_W4;
+    } else if (e > 1 && k_major && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
+      op->tile_cfg = TILE_128x128;
+    } else if (rows_per_group >= 192 && tiles(256, 256) >= 256) {
       // K-major weights take the persistent four-wave kernel when a tile has at least four 128-byte K slabs
       op->tile_cfg = (k_major && k >= 512 && e <= 1024) ? TILE_256x256_W4 : TILE_256x256;
     } else if (rows_per_group >= 96 && tiles(128, 128) >= 256) {
@@ -235,16 +252,21 @@ void choose_plan(msco_gmm_op *op) {
       // run in one round; more tiles than CUs keep 64-byte slabs and two workgroups per CU (M = 512, N = 11008: 344
       // tiles, 46.8 us against 50.1 us)
       op->wide_k_slabs = k_major && t * want <= (num_cus > 0 ? num_cus : kTileTargetWorkgroups);
+      if (tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;
     }
   }
   op->stream_tch = 1;
   if (family == FAM_SKINNY && is_packed(d) && is_w8a8(d)) {
     // rows a group is expected to hold (shapes only): 16-row chunks up to 16 rows, else chunks of 32 / 64 / 128 rows
-    const int64_t rows = e == 1 ? m : (m + e - 1) / e;
+    // (several groups: 1.5 x the average, real routings are uneven and a group that overflows its chunk streams its
+    // weights twice -- 128 rows over 8 experts: 90.5 us with 32-row chunks against 105 us with 16-row chunks)
+    const int64_t avg = (m + e - 1) / e;
+    const int64_t rows = e == 1 ? m : avg + avg / 2;
     op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
     // fewer, larger chunks when the (group, chunk) grid would be mostly empty slots
     while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch = op->stream_tch == 1 ? 2 : op->stream_tch * 2;
+    if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8) op->stream_tch = tuning().stream_tch;
   }
   if (family == FAM_SKINNY) {
     // grid.y enumerates (group, chunk of 16 * stream_tch rows)

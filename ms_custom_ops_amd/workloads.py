@@ -110,8 +110,8 @@ def make(name: str, *, scale_down: int = 1) -> Workload:
         logits = np.random.randn(t, e)
         gl, _, _ = route_topk(logits, top_k, e)
         return Workload(name, "w8a8", m, k, n, e, x, w, s, pt, None, None, gl)
-    if name == "c3_decode":
-        t, e, top_k = 16, 8, 2
+    if name == "c3_decode" or name.startswith("c3_t"):   # c3_t<T>: the MoE layer of c3 with T tokens (c3_decode = c3_t16)
+        t, e, top_k = (16 if name == "c3_decode" else int(name[4:])), 8, 2
         k, n = 4096 // sd, 14336 // sd
         m = t * top_k
         x = _int8((m, k)); w = _int8((e, k, n)); s = _scale((e, n)); pt = _scale((m,))
