@@ -504,10 +504,13 @@ def main():
                              ("c4", "packed"), ("c4", "nk"), ("c4", "kn"), ("c1", "packed"), ("c2_m256", "packed"),
                              ("c1", "nk"), ("c1", "kn"), ("c2_m256", "nk"), ("c2_m256", "kn"), ("c2_m16", "nk"),
                              ("c2_m16", "kn"), ("c2_m16", "packed"), ("c2_m1", "kn"), ("c2_m1", "packed"), ("c5", "kn"),
-                             ("c5", "packed"), ("c3_decode", "kn"), ("c3_decode", "packed")]:
+                             ("c5", "packed"), ("c3_decode", "kn"), ("c3_decode", "packed"),
+                             # the headline MoE layer at serving batch sizes (T tokens, top-2 of 8): bound by the 470 MB of weights
+                             ("c3_t64", "packed"), ("c3_t128", "packed"), ("c3_t256", "packed"), ("c3_t512", "packed"),
+                             ("c3_t1024", "packed")]:
             w2 = workloads.make(name)
             w_bytes = w2.w.nbytes
-            hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5", "c3_decode")
+            hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5", "c3_decode") or name.startswith("c3_t")
             copies = max(1, int(np.ceil(ROTATE_BYTES / w_bytes))) if hbm_bound_guess else 1
             p2 = DeviceProblem(w2, layout, copies)
             _, sec, _ = p2.time(max(20, min(200, args.steps)), args.warmup)
