@@ -651,7 +651,9 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
       case TILE_256x256_W4:
         if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, true, stream);
         return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
-      case TILE_256x256: case TILE_128x256: return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
+      case TILE_128x256:   // four waves side by side, 128 x 64 each
+        return p.wide_k_slabs ? launch_cfg<128, 256, 1, 4, true, 3, true, 4>(p, stream) : launch_cfg<128, 256, 1, 4, true, 3, true>(p, stream);
+      case TILE_256x256: return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
       default: return hipErrorInvalidValue;
     }
   }

@@ -173,14 +173,15 @@ void choose_plan(msco_gmm_op *op) {
     // stream (every group's matrix is read once per m-tile of the group), so the m-tile should hold a whole group --
     // real routings are uneven, hence 1.5 x the average -- as long as there are tiles for most CUs.  Measured (E = 8,
     // K = 4096, N = 14336, packed; 64 x 128 / 128 x 128 / 256 x 256 tiles): 64 rows per group 112 / 97 / 100 us, 128 rows per
-    // group 162 / 150 / 109 us, 32 rows per group 87.5 us with the first.
+    // group 162 / 150 / 109 us (136 us with 128 x 256), 32 rows per group 87.5 us with the first.
     auto group_tiles = [&](int bm, int bn) { return e * ((rows_per_group + bm - 1) / bm) * ((n + bn - 1) / bn); };
     const int64_t cover = rows_per_group + rows_per_group / 2;
     const int64_t busy = (num_cus > 0 ? num_cus : kTileTargetWorkgroups) * 3 / 4;
     if (e > 1 && k_major && cover > 128 && cover <= 384 && k >= 512 && e <= 1024 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
     } else if (e > 1 && k_major && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
-      op->tile_cfg = TILE_128x128;
+      // (128 x 256 tiles re-read x half as often: 64 / 96 rows per group 93 / 99 us against 100 / 111 us)
+      op->tile_cfg = group_tiles(128, 256) >= busy ? TILE_128x256 : TILE_128x128;
     } else if (rows_per_group >= 192 && tiles(256, 256) >= 256) {
       // K-major weights take the persistent four-wave kernel when a tile has at least four 128-byte K slabs
       op->tile_cfg = (k_major && k >= 512 && e <= 1024) ? TILE_256x256_W4 : TILE_256x256;
@@ -254,6 +255,7 @@ void choose_plan(msco_gmm_op *op) {
       op->wide_k_slabs = k_major && t * want <= (num_cus > 0 ? num_cus : kTileTargetWorkgroups);
       if (tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;
     }
+    if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
   }
   op->stream_tch = 1;
   if (family == FAM_SKINNY && is_packed(d) && is_w8a8(d)) {

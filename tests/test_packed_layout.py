@@ -97,6 +97,14 @@ def test_multi_row_streaming_kernel_is_bit_exact(device, m, k, n, e, gl):
     assert "w8a8_stream_rows" in info and "layout=packed" in info
 
 
+def test_groups_of_about_a_hundred_rows_take_128_row_tiles_over_256_columns(device):
+    # several groups whose 1.5-fold average size fits a 128-row m-tile, enough columns for three quarters of the CUs: one
+    # group longer than the tile (140 rows: two m-tiles), one short (40), a tail of 60
+    x, w, bias, scale, pt = _inputs(27, 320, 1024, 12288, 4)
+    info = _check(x, w, [40, 180, 260, 320], bias, scale, pt)
+    assert "w8a8_tile_128x256" in info and "layout=packed" in info, info
+
+
 @pytest.mark.parametrize("m,k,n", [(17, 512, 80), (32, 4096, 1408), (48, 1024, 128), (64, 2048, 272)])
 def test_one_group_of_17_to_64_rows_takes_the_small_tile_with_a_k_split(device, m, k, n):
     x, w, bias, scale, pt = _inputs(26, m, k, n, 1)
