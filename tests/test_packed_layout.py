@@ -250,3 +250,27 @@ def test_persistent_tile_kernel_random_shapes_both_layouts(device, seed):
     bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", transpose_b=True, override=cabi.OV_TILE_256_W4, launches=2)   # stores [E,N,K]
     assert "tile_256x256x128_w4" in info, info
     assert np.array_equal(bits[:gl[-1]], ref[:gl[-1]]), info
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_whatever_the_plan_picks_is_bit_exact_on_every_layout(device, seed):
+    # a seeded sweep over the shapes where the plan changes its mind: one group or several, a handful to several hundred
+    # rows per group (16- and 32-row streaming chunks, 64 / 128 / 256-row tiles, K splits), K with and without 64- and
+    # 128-byte tails, narrow and wide N; packed weights, [E,N,K] and [E,K,N], every one against the oracle bit for bit
+    from gpu_utils import run_w8a8
+    rng = np.random.default_rng(5000 + seed)
+    wide = seed >= 16   # the last seeds: enough columns that several groups of 70 .. 260 rows get 128- and 256-row tiles
+    e = int(rng.choice([4, 8])) if wide else int(rng.choice([1, 1, 2, 4, 8, 12]))
+    per_group = int(rng.choice([70, 100, 150, 260])) if wide else int(rng.choice([6, 14, 20, 40, 70, 100, 150, 260]))
+    m = max(1, int(per_group * e * rng.uniform(0.8, 1.2)))
+    k = int(rng.integers(8, 12) if wide else rng.integers(2, 40)) * 64 + int(rng.choice([0, 0, 16, 32, 48]))
+    n = int(rng.choice([6144, 12288 - 16])) if wide else int(rng.choice([48, 128, 272, 1024, 1408, 3072]))
+    cuts = np.sort(rng.integers(0, m + 1, e - 1)) if e > 1 else np.array([], dtype=np.int64)
+    gl = list(np.maximum.accumulate([int(v) for v in cuts] + [m - int(rng.choice([0, 0, 3]))]))
+    x, w, bias, scale, pt = _inputs(100 + seed, m, k, n, e)
+    ref = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt)
+    infos = []
+    for kwargs in ({"packed": True}, {"transpose_b": True}, {}):
+        bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", launches=2, **kwargs)
+        infos.append(info)
+        assert np.array_equal(bits[:gl[-1]], ref[:gl[-1]]), (m, k, n, e, gl, info)
