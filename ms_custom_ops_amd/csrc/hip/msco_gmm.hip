@@ -182,6 +182,15 @@ void choose_plan(msco_gmm_op *op) {
     } else if (e > 1 && k_major && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
       // (128 x 256 tiles re-read x half as often: 64 / 96 rows per group 93 / 99 us against 100 / 111 us)
       op->tile_cfg = group_tiles(128, 256) >= busy ? TILE_128x256 : TILE_128x128;
+    } else if (e == 1 && k_major && k >= 512 && tiles(256, 256) >= busy * 2 / 3 && tiles(128, 256) > busy * 4 / 3) {
+      // one group, K-major weights, a few hundred to a thousand rows: the persistent kernel already on half of the CUs
+      // when 128 x 256 tiles would no longer run in one round (N = 11008: M = 768 / 1024: 47 / 52 us against 63 / 68 us
+      // with 128 x 128 tiles) ...
+      op->tile_cfg = TILE_256x256_W4;
+    } else if (e == 1 && k_major && tiles(128, 256) >= busy * 4 / 5 && tiles(128, 256) <= busy * 4 / 3) {
+      // ... and 128 x 256 tiles while they do and fill most of the chip (M = 448 .. 640: 40 - 42 us against 45 - 47 us;
+      // M = 384, 129 tiles: 41 us against 35 us with 128 x 128)
+      op->tile_cfg = TILE_128x256;
     } else if (rows_per_group >= 192 && tiles(256, 256) >= 256) {
       // K-major weights take the persistent four-wave kernel when a tile has at least four 128-byte K slabs
       op->tile_cfg = (k_major && k >= 512 && e <= 1024) ? TILE_256x256_W4 : TILE_256x256;
