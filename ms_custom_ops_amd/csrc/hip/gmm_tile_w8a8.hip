@@ -486,23 +486,33 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     __syncthreads();
     if (s_ticket != (unsigned)(split - 1)) return;
     if (tid == 0) __hip_atomic_store(&p.counters[lid], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // (two slices per round trip measured slower: 15.7 against 15.1 us on the M = 128 dense case)
-    for (int s = 0; s < split; ++s) {
-      if (s == ks) continue;
-      const i64 *other = base + (long long)s * (TILE_INTS / 2) + tid;
-      // all loads of a slice are issued before the first add: one memory round trip per slice, not one per word
-      i64 t[WORDS];
+    // the other slices, two per memory round trip (the j-th other slice is j, or j + 1 from this one's index on); an
+    // odd one out is read alone
+    const int others = split - 1;
+    for (int j0 = 0; j0 < others; j0 += 2) {
+      const bool two = j0 + 1 < others;
+      const int sa = j0 < ks ? j0 : j0 + 1, sb = two ? (j0 + 1 < ks ? j0 + 1 : j0 + 2) : sa;
+      const i64 *oa = base + (long long)sa * (TILE_INTS / 2) + tid, *ob = base + (long long)sb * (TILE_INTS / 2) + tid;
+      i64 ta[WORDS], tb[WORDS];
 #pragma unroll
-      for (int u = 0; u < WORDS; ++u) t[u] = __hip_atomic_load(other + u * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int u = 0; u < WORDS; ++u) ta[u] = __hip_atomic_load(oa + u * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (two) {
+#pragma unroll
+        for (int u = 0; u < WORDS; ++u) tb[u] = __hip_atomic_load(ob + u * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      } else {
+#pragma unroll
+        for (int u = 0; u < WORDS; ++u) tb[u] = 0;
+      }
 #pragma unroll
       for (int f = 0; f < FN; ++f)
 #pragma unroll
         for (int i = 0; i < FM; ++i)
 #pragma unroll
           for (int r = 0; r < 16; r += 2) {
-            const unsigned long long w = (unsigned long long)t[(f * FM + i) * 8 + r / 2];
-            acc[f][i][r] += (int)(unsigned)w;
-            acc[f][i][r + 1] += (int)(unsigned)(w >> 32);
+            const unsigned long long wa = (unsigned long long)ta[(f * FM + i) * 8 + r / 2];
+            const unsigned long long wb = (unsigned long long)tb[(f * FM + i) * 8 + r / 2];
+            acc[f][i][r] += (int)(unsigned)wa + (int)(unsigned)wb;
+            acc[f][i][r + 1] += (int)(unsigned)(wa >> 32) + (int)(unsigned)(wb >> 32);
           }
     }
   }
