@@ -57,15 +57,17 @@ __device__ __forceinline__ int q_of_col(int c) {
 
 // 16 bytes per lane from a buffer straight into LDS: lane L of the wave writes lds_base + 16 L.
 // (The address-space cast only exists in the device pass.)
+template <int AUX = 0>
 __device__ __forceinline__ void buffer_load_lds_b128(__amdgpu_buffer_rsrc_t rsrc, void *lds_base, unsigned voffset,
                                                      unsigned soffset) {
 #if defined(__HIP_DEVICE_COMPILE__)
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (void __attribute__((address_space(3))) *)(lds_base), 16, voffset,
-                                           soffset, 0, 0);
+                                           soffset, 0, AUX);
 #else
   (void)rsrc; (void)lds_base; (void)voffset; (void)soffset;
 #endif
 }
+
 
 // Two 8-byte LDS reads `stride` bytes apart, invisible to the compiler's wait-count bookkeeping.
 // They must be issued before any compiler-visible LDS read whose result is consumed later (LDS
@@ -114,9 +116,14 @@ __device__ __forceinline__ void wait_vmcnt() {
 // KS = 32-byte MFMA K steps per slab (packed weights only for KS = 4): a slab is BKT = 32 KS bytes of K.  With 128-byte
 // slabs every x row piece is a whole cache line (64-byte pieces are half lines, and the load path is bound by line
 // requests), a column group contributes two consecutive 1 KiB blocks, and there is one barrier per 4 K steps.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES, bool PK = false, int KS = 2>
+// WNT (packed weights): the weight loads carry the non-temporal bit -- planned when the launch streams tens of megabytes
+// of weights that at most two m-tiles read (GmmParams::w_nontemporal): a stream that is read once should not push x
+// out of the caches.  Whole kilobytes per instruction only: on row-major [E,N,K] weights with 64-byte slabs (half
+// lines) the bit costs 15 %.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES, bool PK = false, int KS = 2, bool WNT = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel(const GmmParams p) {
   static_assert(!PK || NK, "packed weights use the LDS-direct weight path");
+  static_assert(!WNT || PK, "non-temporal weight loads are for the packed layout");
   static_assert(KS == 2 || (KS == 4 && NK), "128-byte slabs are built for K-major weights");
   constexpr int BKT = 32 * KS;                      // bytes of K per slab
   constexpr int ROWS_PER_LOAD = 1024 / BKT;         // x rows one wave instruction (1 KiB) brings
@@ -285,7 +292,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
           // (the last one is zero padded)
           const int kblock = (k_first + kt) * KB_PER_SLAB + blk % KB_PER_SLAB;
           const unsigned kill_w = (kblock >= pk_blocks) ? OOB : 0u;
-          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, kblock * 1024);
+          buffer_load_lds_b128<WNT ? 2 : 0>(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, kblock * 1024);
         } else {
           const unsigned kill_b = (kbase + b_chunk[u] * 16 >= (unsigned)p.k) ? OOB : 0u;
           buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase);
@@ -620,13 +627,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
 }
 
 // ---- host launcher ---------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4, bool PK = false, int KS = 2>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4, bool PK = false, int KS = 2, bool WNT = false>
 static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
   constexpr int BKT = 32 * KS;
   const size_t loop_lds = (size_t)STAGES * BM * BKT + (size_t)(NK ? STAGES : KN_STAGES) * BN * BKT;
   const size_t epi_lds = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * 144;   // epilogue staging, 144-byte row pitch
   const size_t lds = (loop_lds > epi_lds ? loop_lds : epi_lds) + 3 * 1024;   // + epilogue operand table
-  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES, PK, KS>;
+  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES, PK, KS, WNT>;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -648,6 +655,8 @@ static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
 // K = 4096, N = 11008 packed: 26.0 against 28.8 us; 3 / 2 stages 26.7 / 34.1)
 template <int BM, int BN>
 static hipError_t launch_small(const GmmParams &p, bool nk, bool packed, hipStream_t stream) {
+  if (packed && p.w_nontemporal)
+    return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, true, 4, true>(p, stream) : launch_cfg<BM, BN, 2, 2, true, 4, true, 2, true>(p, stream);
   if (packed) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, true, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, true, 4, true>(p, stream);
   if (nk) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, false, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, true>(p, stream);
   return launch_cfg<BM, BN, 2, 2, false>(p, stream);
@@ -662,6 +671,7 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
         if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, true, stream);
         return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
       case TILE_128x256:   // four waves side by side, 128 x 64 each
+        if (p.w_nontemporal) return launch_cfg<128, 256, 1, 4, true, 3, true, 2, true>(p, stream);
         return p.wide_k_slabs ? launch_cfg<128, 256, 1, 4, true, 3, true, 4>(p, stream) : launch_cfg<128, 256, 1, 4, true, 3, true>(p, stream);
       case TILE_256x256: return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
       default: return hipErrorInvalidValue;

@@ -73,6 +73,7 @@ struct msco_gmm_op {
   int strip_groups = 16;
   int stream_tch = 1;        // packed W8A8: 16-row fragments per chunk (1: gmm_w8a8_stream_kernel, 2/4/8: the multi-row kernel)
   int wide_k_slabs = 0;      // small tile kernels on K-major weights: 128-byte K slabs
+  int w_nontemporal = 0;     // small tile kernels on packed weights: non-temporal weight loads
   size_t workspace_bytes = 0;
   unsigned *counters = nullptr;
   size_t counters_cap = 0;
@@ -142,6 +143,7 @@ void choose_plan(msco_gmm_op *op) {
   op->workspace_bytes = 0;
   op->tile_cfg = TILE_256x256;
   op->wide_k_slabs = 0;
+  op->w_nontemporal = 0;
 
   int family;
   // packed weights are K-contiguous per column like [E,N,K]: the same tile kernels read them
@@ -263,6 +265,16 @@ void choose_plan(msco_gmm_op *op) {
       // tiles, 46.8 us against 50.1 us)
       op->wide_k_slabs = k_major && t * want <= (num_cus > 0 ? num_cus : kTileTargetWorkgroups);
       if (tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;
+    }
+    if (op->tile_cfg == TILE_128x128 || op->tile_cfg == TILE_64x128 || op->tile_cfg == TILE_128x256) {
+      // Non-temporal weight loads: a weight stream of tens of megabytes that at most two m-tiles read should not push x
+      // out of the caches (E = 8 x 32 rows, 470 MB: 87.7 -> 79.4 us; M = 128, 45 MB: 20.8 -> 19.6 us); three m-tiles
+      // re-read it from the cache and lose badly without it there (M = 384: 35 -> 47 us), and a weight set the caches
+      // hold anyway gains nothing (M = 128, 16.8 MB: 13.8 -> 14.4 us).
+      int bm, bn;
+      tile_cfg_dims(op->tile_cfg, &bm, &bn);
+      const int64_t group_rows = e > 1 ? (m / e) + (m / e) / 2 : m;
+      op->w_nontemporal = is_packed(d) && e * k * n >= ((int64_t)32 << 20) && (group_rows + bm - 1) / bm <= 2;
     }
     if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
   }
@@ -507,6 +519,7 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   // the x rows staged through LDS, one row 11.85 -> 12.2 us, four rows per chunk (8 experts x 32 rows) 70.1 -> 70.4 us
   p.x_via_lds = (h->e > 0 ? (h->m + h->e - 1) / h->e : h->m) >= 8;
   p.wide_k_slabs = h->wide_k_slabs;
+  p.w_nontemporal = h->w_nontemporal;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t err = hipSuccess;
