@@ -413,7 +413,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_streamm_kernel(const G
 #pragma unroll
     for (int cg = 0; cg < SM_GROUPS; ++cg)
       wv[cg] = __builtin_amdgcn_raw_buffer_load_b128(rw, (live && cg < cg_count) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
-                                                     cg_base + cg * k_blocks * 1024, 0);
+                                                     cg_base + cg * k_blocks * 1024, kStreamAux);
 #pragma unroll
     for (int t = 0; t < TCH; ++t)
       xf[t] = __builtin_amdgcn_raw_buffer_load_b128(rx, k_ok ? xoff[t] + (unsigned)(kb * 64) : kBufferOob, 0, 0);

@@ -148,11 +148,12 @@ void choose_plan(msco_gmm_op *op) {
   int family;
   // packed weights are K-contiguous per column like [E,N,K]: the same tile kernels read them
   const bool k_major = d.transpose_b != 0 || is_packed(d);
-  // (row-major [E,N,K] weights have 16-row chunks only: a group that overflows its chunk streams its weights twice, so
-  // 1.5 x the average has to fit -- 128 rows over 8 experts: 111 us with 64 x 128 tiles against 140 us)
+  // (a group that overflows its 16-row chunk streams its weights twice, so on K-major weights 1.5 x the average has to
+  // fit; beyond that the 64 x 128 tile kernel with non-temporal weight loads is the better streamer -- 128 rows over 8
+  // experts, 470 MB of weights: 76 us against 82 us for the 32-row streaming kernel and 105 us for 16-row chunks;
+  // row-major [E,N,K]: 111 us against 140 us)
   const int64_t avg_rows = (m + (e > 0 ? e : 1) - 1) / (e > 0 ? e : 1);
-  const bool nk_row_major = d.transpose_b != 0 && !is_packed(d);
-  const bool many_small_groups = e > 1 && (nk_row_major ? avg_rows + avg_rows / 2 : avg_rows) <= kSkinnyRows &&
+  const bool many_small_groups = e > 1 && (k_major ? avg_rows + avg_rows / 2 : avg_rows) <= kSkinnyRows &&
                                  e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots;
   if (!aligned) {
     family = FAM_GENERIC;
@@ -230,7 +231,9 @@ void choose_plan(msco_gmm_op *op) {
     if (op->tile_cfg == TILE_128x128 || op->tile_cfg == TILE_64x128) {
       int bm, bn;
       tile_cfg_dims(op->tile_cfg, &bm, &bn);
-      const int64_t t = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+      // tiles the launch is expected to have: every group that holds rows has at least one m-tile
+      const int64_t groups_with_rows = std::min<int64_t>(e, m);
+      const int64_t t = std::max<int64_t>((m + bm - 1) / bm, groups_with_rows) * ((n + bn - 1) / bn);
       // t tiles x s slices run in ceil(t s / CUs) rounds (the operand ring takes most of a CU's LDS: one workgroup per
       // CU).  In units of one 64-byte K slab of a tile (0.2 us): a round costs its slabs plus 10 (prologue, epilogue),
       // a split adds 8 per slice for 64 x 128 tiles and 12 for 128 x 128 (its partial tile out and in, one round trip of
