@@ -53,6 +53,7 @@ struct GmmParams {
   int x_via_lds;            // packed-layout W8A8 decode kernel: stage the chunk's x rows through LDS (pays from about 8 rows per chunk)
   int wide_k_slabs;         // small tile kernels on K-major weights: 128-byte K slabs (planned when the workgroups run in one round)
   int w_nontemporal;        // small tile kernels on packed weights: non-temporal weight loads (a large weight stream that at most two m-tiles read)
+  int rows_lo, rows_hi;     // tile kernels: only groups with rows_lo < rows <= rows_hi are worked on (a launch pair splits the groups by size)
 };
 
 // ---- group_list --------------------------------------------------------------------------------

@@ -183,7 +183,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   for (int g0 = 0, carry = 0; g0 < p.e; g0 += 64) {
     int s0, e0;
     group_rows_chunk(p, g0, lane, carry, s0, e0);
-    const int upto = total + wave_scan_add(((e0 - s0 + T4_BM - 1) / T4_BM) * n_tiles, lane);
+    // (groups outside (rows_lo, rows_hi] have no tiles here: a second launch of the small tile kernel takes them)
+    const int rows_g = e0 - s0;
+    const int upto = total + wave_scan_add((rows_g > p.rows_lo && rows_g <= p.rows_hi) ? ((rows_g + T4_BM - 1) / T4_BM) * n_tiles : 0, lane);
     if (wave == 0 && g0 + lane < p.e) {
       meta_end[g0 + lane] = e0;
       meta_upto[g0 + lane] = upto;

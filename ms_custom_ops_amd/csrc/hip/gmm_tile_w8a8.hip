@@ -27,6 +27,8 @@
 //   x rows and [N,K] weights: row-major, 64 B per row, 16-byte chunk c of row r stored at chunk
 //     position c ^ ((r >> 2) & 3);
 //   [K,N] weights: 8 planes (one per 8 K rows) of BN slots x 8 bytes.
+#include <algorithm>
+
 #include "gmm_common.h"
 #include "gmm_kernels.h"
 
@@ -169,7 +171,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   for (int g0 = 0, carry = 0; g0 < p.e; g0 += 64) {
     int s0, e0;
     group_rows_chunk(p, g0, lane, carry, s0, e0);
-    const int t = wave_scan_add(((e0 - s0 + BM - 1) / BM) * n_tiles, lane);
+    const int rows_g = e0 - s0;   // (groups outside (rows_lo, rows_hi] have no tiles in this launch)
+    const int t = wave_scan_add((rows_g > p.rows_lo && rows_g <= p.rows_hi) ? ((rows_g + BM - 1) / BM) * n_tiles : 0, lane);
     total += wave_bcast(t, 63);
   }
   // K split across workgroups (small problems): the slices of one tile sit next to each other in the
@@ -187,7 +190,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   for (int g0 = 0, carry = 0, tiles_before = 0; g0 < p.e; g0 += 64) {
     int s0, e0;
     group_rows_chunk(p, g0, lane, carry, s0, e0);
-    const int tiles = ((e0 - s0 + BM - 1) / BM) * n_tiles;
+    const int rows_g = e0 - s0;
+    const int tiles = (rows_g > p.rows_lo && rows_g <= p.rows_hi) ? ((rows_g + BM - 1) / BM) * n_tiles : 0;
     const int upto = tiles_before + wave_scan_add(tiles, lane);      // tiles of groups 0 .. g0 + lane
     const int first = __popcll(__ballot(upto <= lid));              // `upto` is non-decreasing: first lane beyond lid
     if (first < 64) {
@@ -642,7 +646,9 @@ static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
     attr_set = true;
   }
   const long long n_tiles = (p.n + BN - 1) / BN;
-  const long long m_tiles_ub = (p.m + BM - 1) / BM + p.e;   // every non-empty group adds at most one partial tile
+  // every non-empty group adds at most one partial tile; a launch for the small groups only: that many tiles per group
+  const long long m_tiles_ub = p.rows_hi < p.m ? std::min<long long>((p.m + BM - 1) / BM + p.e, (long long)p.e * ((p.rows_hi + BM - 1) / BM))
+                                               : (p.m + BM - 1) / BM + p.e;
   const long long total_ub = m_tiles_ub * n_tiles;
   const long long grid = ((total_ub + kNumXcd - 1) / kNumXcd) * kNumXcd * (p.split_k > 1 ? p.split_k : 1);
   if (grid <= 0) return hipSuccess;

@@ -44,7 +44,7 @@ int env_int(const char *name, int fallback) {
 // Debug switches, read from the environment once per process (the first plan); planning itself reads no environment.
 struct Tuning {
   int print_plan, tile_cfg, tile_target_wgs, tile_split_k, stream_max_slots, skinny_wide16, stream_min_wgs, stream_groups,
-      skinny_target_wgs, skinny_split_k, tile_wide_k, stream_tch;
+      skinny_target_wgs, skinny_split_k, tile_wide_k, stream_tch, two_level;
 };
 const Tuning &tuning() {
   static const Tuning t = {env_int("MSCO_PRINT_PLAN", 0),        env_int("MSCO_TILE_CFG", -1),
@@ -52,7 +52,8 @@ const Tuning &tuning() {
                            env_int("MSCO_STREAM_MAX_SLOTS", 0),  env_int("MSCO_SKINNY_WIDE16", -1),
                            env_int("MSCO_STREAM_MIN_WGS", 0),    env_int("MSCO_STREAM_GROUPS", 0),
                            env_int("MSCO_SKINNY_TARGET_WGS", 0), env_int("MSCO_SKINNY_SPLIT_K", 0),
-                           env_int("MSCO_TILE_WIDE_K", -1),      env_int("MSCO_STREAM_TCH", 0)};
+                           env_int("MSCO_TILE_WIDE_K", -1),      env_int("MSCO_STREAM_TCH", 0),
+                           env_int("MSCO_TWO_LEVEL", 1)};
   return t;
 }
 int or_default(int v, int fallback) { return v > 0 ? v : fallback; }
@@ -74,6 +75,7 @@ struct msco_gmm_op {
   int stream_tch = 1;        // packed W8A8: 16-row fragments per chunk (1: gmm_w8a8_stream_kernel, 2/4/8: the multi-row kernel)
   int wide_k_slabs = 0;      // small tile kernels on K-major weights: 128-byte K slabs
   int w_nontemporal = 0;     // small tile kernels on packed weights: non-temporal weight loads
+  int small_group_rows = 0;  // > 0: the persistent kernel takes the groups with more rows, a second launch of 64 x 128 tiles the others
   size_t workspace_bytes = 0;
   unsigned *counters = nullptr;
   size_t counters_cap = 0;
@@ -144,6 +146,7 @@ void choose_plan(msco_gmm_op *op) {
   op->tile_cfg = TILE_256x256;
   op->wide_k_slabs = 0;
   op->w_nontemporal = 0;
+  op->small_group_rows = 0;
 
   int family;
   // packed weights are K-contiguous per column like [E,N,K]: the same tile kernels read them
@@ -281,6 +284,15 @@ void choose_plan(msco_gmm_op *op) {
     }
     if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
   }
+  // Many experts with uneven loads (a skewed routing) on packed weights: every group of a few rows costs the persistent
+  // kernel a whole 256-row m-tile per n-tile.  The groups of at most 64 rows go to a second launch of 64 x 128 tiles
+  // instead, which streams their weights once with non-temporal loads.  On the skewed 64-expert workload (49152 rows,
+  // K = 2048, N = 2816; 29 groups of at most 64 rows) the persistent kernel's tiles go from 10.2 to 8.9 per workgroup and the
+  // pair of launches measures 336 against 348 us; on [E,N,K] weights (no non-temporal loads) 347 against 350, not worth a
+  // launch.  Which groups are small only the device knows; with few experts the second launch would mostly find none.
+  if (family == FAM_TILE && op->tile_cfg == TILE_256x256_W4 && is_packed(d) && e >= 16 &&
+      (d.kernel_override == OV_AUTO || d.kernel_override == OV_TILE_256_W4) && tuning().two_level != 0)
+    op->small_group_rows = 64;
   op->stream_tch = 1;
   if (family == FAM_SKINNY && is_packed(d) && is_w8a8(d)) {
     // rows a group is expected to hold (shapes only): 16-row chunks up to 16 rows, else chunks of 32 / 64 / 128 rows
@@ -381,12 +393,13 @@ void choose_plan(msco_gmm_op *op) {
   const char *fam = family == FAM_TILE ? "tile" : family == FAM_SKINNY ? "skinny" : "generic";
   std::snprintf(buf, sizeof(buf),
                 "msco_gmm plan: kernel=%s%s%s%s layout=%s m=%lld k=%lld n=%lld e=%lld split_k=%d strips=%d "
-                "workspace=%zu",
+                "workspace=%zu%s",
                 is_w8a8(d) ? "w8a8_" : "a16w8_", (family == FAM_SKINNY && is_packed(d)) ? (op->stream_tch > 1 ? "stream_rows" : "stream") : fam,
                 family == FAM_TILE ? (std::string("_") + tile_cfg_name(op->tile_cfg)).c_str() : "",
                 (family == FAM_SKINNY && op->skinny_wide16) ? "_16w" : "",
                 is_packed(d) ? "packed" : d.transpose_b ? "[E,N,K]" : "[E,K,N]", (long long)m, (long long)k, (long long)n, (long long)e,
-                op->split_k, op->n_strips, op->workspace_bytes);
+                op->split_k, op->n_strips, op->workspace_bytes,
+                op->small_group_rows > 0 ? (" small_groups=" + std::to_string(op->small_group_rows) + ":tile_64x128").c_str() : "");
   op->info = buf;
 }
 
@@ -523,13 +536,24 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
   p.x_via_lds = (h->e > 0 ? (h->m + h->e - 1) / h->e : h->m) >= 8;
   p.wide_k_slabs = h->wide_k_slabs;
   p.w_nontemporal = h->w_nontemporal;
+  p.rows_lo = 0;
+  p.rows_hi = 0x7FFFFFFF;
 
   hipStream_t s = static_cast<hipStream_t>(stream);
   hipError_t err = hipSuccess;
   const bool nk = d.transpose_b != 0;
   const int layout = layout_of(d);
   if (is_w8a8(d)) {
-    if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, layout == 2, s);
+    if (h->family == FAM_TILE && h->small_group_rows > 0) {
+      GmmParams big = p, small = p;
+      big.rows_lo = h->small_group_rows;
+      small.rows_hi = h->small_group_rows;
+      small.split_k = 1;
+      small.wide_k_slabs = 0;              // (128-byte slabs measured slower here: 340 against 336 us)
+      small.w_nontemporal = layout == 2;   // each small group's weights are read by one m-tile
+      err = launch_tile_w8a8(big, h->tile_cfg, nk, layout == 2, s);
+      if (err == hipSuccess) err = launch_tile_w8a8(small, TILE_64x128, nk, layout == 2, s);
+    } else if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, layout == 2, s);
     else if (h->family == FAM_SKINNY && layout == 2) err = h->stream_tch > 1 ? launch_streamm_w8a8(p, h->stream_tch, s) : launch_stream_w8a8(p, s);
     else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
     else err = launch_generic_w8a8(p, layout, s);
