@@ -163,9 +163,21 @@ __device__ __forceinline__ T4Tile t4_locate(const int *meta_end, const int *meta
 // is (0).  The epilogue is bound by instruction issue, so the common forms get code of their own: 3 relu (one
 // instruction per value), 2 v * sigmoid(c v) with a uniform c (silu, fast gelu: five instructions, two of them
 // transcendental), 1 the tanh form of gelu (three more for its cubic).
-template <int MODE, bool PK, int ACT>
+//
+// WL: weight layout, 0 [E,N,K], 1 packed, 2 [E,K,N] (N a multiple of 256).  [E,K,N] rows are N-contiguous and an MFMA
+// operand wants 16 K-contiguous bytes per lane; the LDS transpose read of gfx950 (ds_read_b64_tr_b8) does that turn on
+// the way out of LDS.  Of a block of 16 lanes, lane i names 8 bytes M[i][0..7]; lane j receives byte b = M[2 b + j / 8][j % 8].
+// With lanes 2 b and 2 b + 1 pointing at the two 8-byte halves of one 16-column chunk of K row b, lane j gets K rows
+// 0 .. 7 of the column at byte j of that chunk, and two such reads (8 K rows apart) make the 16 bytes of the operand in
+// natural K order.  So a slab goes to LDS as it lies in memory -- K rows of 256 columns, one staging quad = 4 K rows,
+// lane L row L / 16, chunk slot L % 16 -- with two twists: slot s of row r holds chunk s ^ ((r % 8) << 1), so that the
+// eight rows of one transpose read (and both 16-lane blocks of a half wave) fall into different banks, and the middle
+// two dwords of every chunk are swapped on the way in, so that byte j of a chunk is column t4_col_of_q(j): the
+// epilogue's ownership of 8-column runs stays as it is.
+template <int MODE, int WL, int ACT>
 __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const GmmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
+  constexpr bool PK = WL == 1, KN = WL == 2;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -223,6 +235,8 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     if constexpr (PK) {
       const long long cg_bytes = (long long)k_blocks * 1024;
       return t4_rsrc(p.w + ((long long)t.grp * col_groups + t.n0 / 16) * cg_bytes, (long long)(col_groups - t.n0 / 16) * cg_bytes);
+    } else if constexpr (KN) {
+      return t4_rsrc(p.w + (long long)t.grp * w_elems + t.n0, w_elems - t.n0);
     } else {
       return t4_rsrc(p.w + (long long)t.grp * w_elems + (long long)t.n0 * p.k, (long long)(p.n - t.n0) * p.k);
     }
@@ -236,7 +250,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   // These lane constants are worked out again at the top of every tile from a lane id the compiler cannot see
   // through: kept across the epilogue they would cost it registers, and a spill there stalls the operand stream.
   const unsigned rows32 = 32u * (unsigned)p.k;
-  const unsigned b_step = PK ? 2u * (unsigned)k_blocks * 1024u : rows32;   // staging quad u -> u + 1: two column groups / 32 rows
+  const unsigned b_step = PK ? 2u * (unsigned)k_blocks * 1024u : KN ? 16u * (unsigned)p.n : rows32;   // staging quad u -> u + 1: two column groups / 32 rows / 16 K rows
   int d_chunk;
   unsigned a_voff0, b_voff0;
   // ---- fragment addressing ---------------------------------------------------------------------------
@@ -254,12 +268,18 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     const int d_row0 = 8 * wave + (ln >> 3);
     d_chunk = (ln & 7) ^ ((d_row0 >> 1) & 7);
     a_voff0 = (unsigned)d_row0 * (unsigned)p.k + d_chunk * 16;
-    b_voff0 = PK ? (unsigned)(((wave >> 1) * k_blocks + (wave & 1)) * 1024 + ln * 16)
-                 : (unsigned)t4_col_of_q(d_row0) * (unsigned)p.k + d_chunk * 16;   // LDS row rho feeds MFMA row rho % 32
+    const int w_krow = 4 * wave + (ln >> 4);   // [E,K,N]: K row of staging quad 0 that this lane carries
+    b_voff0 = PK   ? (unsigned)(((wave >> 1) * k_blocks + (wave & 1)) * 1024 + ln * 16)
+              : KN ? (unsigned)w_krow * (unsigned)p.n + (unsigned)(((ln & 15) ^ ((w_krow & 7) << 1)) * 16)
+                   : (unsigned)t4_col_of_q(d_row0) * (unsigned)p.k + d_chunk * 16;   // LDS row rho feeds MFMA row rho % 32
     const int swz = (q32 >> 1) & 7;
     x_lane = (unsigned)((wave_m * T4_WT + q32) * T4_BK + ((h ^ swz) << 4));
-    w_lane = PK ? (unsigned)(T4_W_BASE + wave_n * 16384 + (q32 >> 4) * 2048 + h * 256 + (t4_col_of_q(q32) & 15) * 16)
-                : (unsigned)(T4_W_BASE + (wave_n * T4_WT + q32) * T4_BK + ((h ^ swz) << 4));
+    // [E,K,N]: address lane i = ln % 16 of its block of 16 points at K row i / 2 (of the 16 that half h of the wave
+    // multiplies), half i % 2 of the chunk of this block's 16 columns; fragment f is an XOR with f << 5 away
+    w_lane = PK   ? (unsigned)(T4_W_BASE + wave_n * 16384 + (q32 >> 4) * 2048 + h * 256 + (t4_col_of_q(q32) & 15) * 16)
+             : KN ? (unsigned)(T4_W_BASE + (h * 16 + ((ln & 15) >> 1)) * 256 +
+                               (((wave_n * 8 + ((ln >> 4) & 1)) ^ (((ln & 15) >> 1) << 1)) * 16) + (ln & 1) * 8)
+                  : (unsigned)(T4_W_BASE + (wave_n * T4_WT + q32) * T4_BK + ((h ^ swz) << 4));
     st_x = (unsigned)(wave * 1024 + ln * 16);
     st_w = st_x + T4_W_BASE;
     asm volatile("" : "+v"(st_w));
@@ -288,6 +308,12 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     const unsigned kill = dead ? T4_OOB : 0u;
     if constexpr (OP == 0) {
       stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rx_n : rx_c, (a_voff0 + U * rows32) | kill, kbase, 0);
+    } else if constexpr (KN) {
+      // K rows 16 U + 4 wave + lane / 16 of the slab; the slab's first row goes into the scalar offset, which the buffer
+      // unit does not range-check, so rows past K are killed here (their x bytes read as zeros)
+      const bool dead_w = (ahead && !nxt.valid) || kbase + (unsigned)(16 * U + 4 * wave) + (unsigned)(lane >> 4) >= (unsigned)p.k;
+      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rw_n : rw_c, (b_voff0 + U * b_step) | (dead_w ? T4_OOB : 0u),
+                                                            kbase * (unsigned)p.n, 0);
     } else if constexpr (PK) {
       // K block 2 slab + wave % 2 of column groups 2 U + wave / 2; blocks past K do not exist (the last one is zero padded)
       const unsigned kb = 2u * (unsigned)(ahead ? s - k_slabs : s) + (unsigned)(wave & 1);
@@ -297,19 +323,37 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
       stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rw_n : rw_c, (b_voff0 + U * b_step) | kill, kbase, 0);
     }
   };
+  // a staging quad on its way to LDS ([E,K,N] weights: the middle dwords of the 16-column chunk change places)
+  auto put_quad = [&](unsigned addr, v4i v, auto op_c) {
+    if constexpr (KN && decltype(op_c)::value == 1) {
+      int y = v.y, z = v.z;
+      asm volatile("v_swap_b32 %0, %1" : "+v"(y), "+v"(z));
+      v.y = y;
+      v.z = z;
+    }
+    *reinterpret_cast<v4i *>(smem + addr) = v;
+  };
   // write quad (op, u) of slab s to its LDS stage and refill it with slab s + 2
   auto cycle_one = [&](int s, auto par_c, auto op_c, auto u_c) {
     constexpr int P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
-    *reinterpret_cast<v4i *>(smem + ((OP == 0 ? st_x : st_w) + (s & 1) * T4_OP_STAGE + U * 4096)) = stg[P][OP][U];
+    put_quad((OP == 0 ? st_x : st_w) + (s & 1) * T4_OP_STAGE + U * 4096, stg[P][OP][U], op_c);
     load_one(s + 2, par_c, op_c, u_c);
   };
   // the same for a slab whose successor lies inside the current tile and inside K: WS = stage written, soff = scalar
-  // offset of slab s + 2 (bytes of K; 16 times that in the packed weights)
-  auto cycle_clean = [&](auto ws_c, unsigned soff, auto par_c, auto op_c, auto u_c) {
+  // offset of slab s + 2 (bytes of K for x, soff_w for the weights: 16 times that in the packed layout, N times in [E,K,N])
+  auto cycle_clean = [&](auto ws_c, unsigned soff, unsigned soff_w, auto par_c, auto op_c, auto u_c) {
     constexpr int WS = decltype(ws_c)::value, P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
-    *reinterpret_cast<v4i *>(smem + ((OP == 0 ? st_x : st_w) + WS * T4_OP_STAGE + U * 4096)) = stg[P][OP][U];
+    put_quad((OP == 0 ? st_x : st_w) + WS * T4_OP_STAGE + U * 4096, stg[P][OP][U], op_c);
     if constexpr (OP == 0) stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rx_c, a_voff0 + U * rows32, soff, 0);
-    else stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rw_c, b_voff0 + U * b_step, PK ? soff * 16 : soff, 0);
+    else stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rw_c, b_voff0 + U * b_step, soff_w, 0);
+  };
+  // [E,K,N] weight fragment: two transpose reads, K rows 0 .. 7 and 8 .. 15 of the lane's column
+  auto read_tr = [&](unsigned addr) -> v4i {
+    typedef int v2i_t __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) v2i_t *lds_v2i;
+    const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(smem + addr));
+    const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(smem + addr + 2048));
+    return v4i{lo.x, lo.y, hi.x, hi.y};
   };
   // (qx = q << 5 arrives in a scalar the compiler cannot see through: hoisting the XORs out of the K
   // loop would park eight more addresses in registers that the loop does not have)
@@ -318,6 +362,8 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     if constexpr (PK) {
       // qx = q << 5: K block q / 2 is 1024 bytes on, chunk pair q % 2 another 512
       wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_OP_STAGE + (w_lane + (qx >> 6) * 1024 + ((qx >> 5) & 1) * 512) + F * 4096);
+    } else if constexpr (KN) {
+      wf[S][F] = read_tr(stage * T4_OP_STAGE + ((w_lane ^ (unsigned)(F << 5)) + (qx << 8)));   // K quarter q: 32 rows of 256 bytes on
     } else {
       wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_OP_STAGE + (w_lane ^ qx) + F * 32 * T4_BK);
     }
@@ -330,6 +376,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   auto read_w_clean = [&](auto stage_c, auto q_c, auto set_c, auto f_c) {
     constexpr int ST = decltype(stage_c)::value, Q = decltype(q_c)::value, S = decltype(set_c)::value, F = decltype(f_c)::value;
     if constexpr (PK) wf[S][F] = *reinterpret_cast<const v4i *>(smem + (w_lane + ST * T4_OP_STAGE + (Q >> 1) * 1024 + (Q & 1) * 512 + F * 4096));
+    else if constexpr (KN) wf[S][F] = read_tr((w_lane ^ (unsigned)(F << 5)) + ST * T4_OP_STAGE + Q * 8192);
     else wf[S][F] = *reinterpret_cast<const v4i *>(smem + ((w_lane ^ (unsigned)(Q << 5)) + ST * T4_OP_STAGE + F * 4096));
   };
   auto read_x_clean = [&](auto stage_c, auto q_c, auto set_c, auto i_c) {
@@ -432,8 +479,8 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
             acc[f][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[S][f], xf[S][i], acc[f][i], 0, 0, 0);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // DS read
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          // MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, KN ? 2 : 1, 0);   // DS read (a transposed weight fragment is two)
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -483,14 +530,15 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         constexpr int G = decltype(g_c)::value;
         const std::integral_constant<int, 2 * G> ua;
         const std::integral_constant<int, 2 * G + 1> ub;
+        const unsigned soff_w = PK ? soff * 16 : KN ? soff * (unsigned)p.n : soff;
         read_w_clean(rstage_c, rq_c, nxt_c, c0); read_x_clean(rstage_c, rq_c, nxt_c, c0);
-        cycle_clean(ws_c, soff, par_c, c0, ua);
+        cycle_clean(ws_c, soff, soff_w, par_c, c0, ua);
         read_x_clean(rstage_c, rq_c, nxt_c, c1); read_x_clean(rstage_c, rq_c, nxt_c, c2);
-        cycle_clean(ws_c, soff, par_c, c0, ub);
+        cycle_clean(ws_c, soff, soff_w, par_c, c0, ub);
         read_x_clean(rstage_c, rq_c, nxt_c, c3); read_w_clean(rstage_c, rq_c, nxt_c, c1);
-        cycle_clean(ws_c, soff, par_c, c1, ua);
+        cycle_clean(ws_c, soff, soff_w, par_c, c1, ua);
         read_w_clean(rstage_c, rq_c, nxt_c, c2); read_w_clean(rstage_c, rq_c, nxt_c, c3);
-        cycle_clean(ws_c, soff, par_c, c1, ub);
+        cycle_clean(ws_c, soff, soff_w, par_c, c1, ub);
         mfma_quarter(cur_c);
       };
       // slab kt in stage ST; soff3 / soff4: K offsets of slabs kt + 3 and kt + 4
@@ -710,9 +758,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   }
 }
 
-template <int MODE, bool PK, int ACT>
+template <int MODE, int WL, int ACT>
 static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t stream) {
-  auto kern = gmm_w8a8_tile4_nk_kernel<MODE, PK, ACT>;
+  auto kern = gmm_w8a8_tile4_nk_kernel<MODE, WL, ACT>;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -724,9 +772,10 @@ static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t strea
   return hipGetLastError();
 }
 
-hipError_t launch_tile4_w8a8_nk(const GmmParams &p, bool packed, hipStream_t stream) {
-  // the operand stream runs up to four slabs ahead inside one tile; the group table lives in LDS
-  if (p.k < 4 * T4_BK || p.e > T4_MAX_E) return hipErrorInvalidValue;
+hipError_t launch_tile4_w8a8(const GmmParams &p, int layout, hipStream_t stream) {
+  // the operand stream runs up to four slabs ahead inside one tile; the group table lives in LDS; [E,K,N] weights
+  // (layout 2) are read in whole 256-column rows
+  if (p.k < 4 * T4_BK || p.e > T4_MAX_E || layout < 0 || layout > 2 || (layout == 2 && p.n % T4_BN != 0)) return hipErrorInvalidValue;
   const long long n_tiles = (p.n + T4_BN - 1) / T4_BN;
   const long long m_tiles_ub = (p.m + T4_BM - 1) / T4_BM + p.e;   // every non-empty group adds at most one partial tile
   const long long total_ub = m_tiles_ub * n_tiles;
@@ -735,17 +784,19 @@ hipError_t launch_tile4_w8a8_nk(const GmmParams &p, bool packed, hipStream_t str
   if (grid <= 0) return hipSuccess;
   const int act = p.act_type == ACT_NONE ? 0 : p.act_type == ACT_RELU ? 3 : (p.act_type == ACT_SILU || p.act_type == ACT_FAST_GELU) ? 2 : 1;
   const unsigned g = (unsigned)grid;
-#define MSCO_T4_BY_ACT(MODE, PK)                                   \
-  (act == 0   ? t4_launch<MODE, PK, 0>(p, g, stream)               \
-   : act == 1 ? t4_launch<MODE, PK, 1>(p, g, stream)               \
-   : act == 2 ? t4_launch<MODE, PK, 2>(p, g, stream)               \
-              : t4_launch<MODE, PK, 3>(p, g, stream))
+#define MSCO_T4_BY_ACT(MODE, WL)                                   \
+  (act == 0   ? t4_launch<MODE, WL, 0>(p, g, stream)               \
+   : act == 1 ? t4_launch<MODE, WL, 1>(p, g, stream)               \
+   : act == 2 ? t4_launch<MODE, WL, 2>(p, g, stream)               \
+              : t4_launch<MODE, WL, 3>(p, g, stream))
+#define MSCO_T4_BY_LAYOUT(MODE) (layout == 1 ? MSCO_T4_BY_ACT(MODE, 1) : layout == 2 ? MSCO_T4_BY_ACT(MODE, 2) : MSCO_T4_BY_ACT(MODE, 0))
   switch (p.out_dtype) {
-    case DT_BF16: return packed ? MSCO_T4_BY_ACT(0, true) : MSCO_T4_BY_ACT(0, false);
-    case DT_F16: return packed ? MSCO_T4_BY_ACT(1, true) : MSCO_T4_BY_ACT(1, false);
-    case DT_I32: return packed ? t4_launch<2, true, 0>(p, g, stream) : t4_launch<2, false, 0>(p, g, stream);
+    case DT_BF16: return MSCO_T4_BY_LAYOUT(0);
+    case DT_F16: return MSCO_T4_BY_LAYOUT(1);
+    case DT_I32: return layout == 1 ? t4_launch<2, 1, 0>(p, g, stream) : layout == 2 ? t4_launch<2, 2, 0>(p, g, stream) : t4_launch<2, 0, 0>(p, g, stream);
     default: return hipErrorInvalidValue;
   }
+#undef MSCO_T4_BY_LAYOUT
 #undef MSCO_T4_BY_ACT
 }
 

@@ -674,7 +674,7 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
   if (packed) {
     switch (tile_cfg) {
       case TILE_256x256_W4:
-        if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, true, stream);
+        if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8(p, 1, stream);
         return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
       case TILE_128x256:   // four waves side by side, 128 x 64 each
         if (p.w_nontemporal) return launch_cfg<128, 256, 1, 4, true, 3, true, 2, true>(p, stream);
@@ -688,8 +688,8 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
       return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     case TILE_128x256:   // two 4-wave workgroups per CU; [N,K] weights only
       return nk ? launch_cfg<128, 256, 1, 4, true, 3>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
-    case TILE_256x256_W4:   // needs [N,K] weights, at least four 128-byte K slabs per tile, a group table that fits in LDS
-      if (nk && p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8_nk(p, false, stream);
+    case TILE_256x256_W4:   // needs at least four 128-byte K slabs per tile, a group table that fits in LDS, whole 256-column rows of [K,N] weights
+      if (p.k >= 512 && p.e <= 1024 && (nk || p.n % 256 == 0)) return launch_tile4_w8a8(p, nk ? 0 : 2, stream);
       return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     default:
       return hipErrorInvalidValue;

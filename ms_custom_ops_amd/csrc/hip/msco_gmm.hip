@@ -183,12 +183,15 @@ void choose_plan(msco_gmm_op *op) {
     auto group_tiles = [&](int bm, int bn) { return e * ((rows_per_group + bm - 1) / bm) * ((n + bn - 1) / bn); };
     const int64_t cover = rows_per_group + rows_per_group / 2;
     const int64_t busy = (num_cus > 0 ? num_cus : kTileTargetWorkgroups) * 3 / 4;
-    if (e > 1 && k_major && cover > 128 && cover <= 384 && k >= 512 && e <= 1024 && group_tiles(256, 256) >= busy) {
+    // (the persistent four-wave kernel: at least four 128-byte K slabs per tile, a group table that fits in LDS, K-major
+    // weights or [E,K,N] weights whose rows are whole 256-column pieces -- it turns those on the way out of LDS)
+    const bool w4_ok = (k_major || n % 256 == 0) && k >= 512 && e <= 1024;
+    if (e > 1 && w4_ok && cover > 128 && cover <= 384 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
     } else if (e > 1 && k_major && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
       // (128 x 256 tiles re-read x half as often: 64 / 96 rows per group 93 / 99 us against 100 / 111 us)
       op->tile_cfg = group_tiles(128, 256) >= busy ? TILE_128x256 : TILE_128x128;
-    } else if (e == 1 && k_major && k >= 512 && tiles(256, 256) >= busy * 2 / 3 && tiles(128, 256) > busy * 4 / 3) {
+    } else if (e == 1 && w4_ok && tiles(256, 256) >= busy * 2 / 3 && tiles(128, 256) > busy * 4 / 3) {
       // one group, K-major weights, a few hundred to a thousand rows: the persistent kernel already on half of the CUs
       // when 128 x 256 tiles would no longer run in one round (N = 11008: M = 768 / 1024: 47 / 52 us against 63 / 68 us
       // with 128 x 128 tiles) ...
@@ -198,8 +201,7 @@ void choose_plan(msco_gmm_op *op) {
       // M = 384, 129 tiles: 41 us against 35 us with 128 x 128)
       op->tile_cfg = TILE_128x256;
     } else if (rows_per_group >= 192 && tiles(256, 256) >= 256) {
-      // K-major weights take the persistent four-wave kernel when a tile has at least four 128-byte K slabs
-      op->tile_cfg = (k_major && k >= 512 && e <= 1024) ? TILE_256x256_W4 : TILE_256x256;
+      op->tile_cfg = w4_ok ? TILE_256x256_W4 : TILE_256x256;
     } else if (rows_per_group >= 96 && tiles(128, 128) >= 256) {
       op->tile_cfg = TILE_128x128;
     } else if (tiles(128, 128) >= 512) {
@@ -221,6 +223,9 @@ void choose_plan(msco_gmm_op *op) {
     case OV_GENERIC: family = FAM_GENERIC; break;
     default: break;
   }
+  // (what the persistent kernel cannot take runs the eight-wave kernel of the same tile shape; the plan says so)
+  if (family == FAM_TILE && op->tile_cfg == TILE_256x256_W4 && !(k >= 512 && e <= 1024 && (k_major || n % 256 == 0)))
+    op->tile_cfg = TILE_256x256;
   // the MFMA kernels address x and one group's weights through 32-bit buffer offsets
   const bool fits32 = (is_packed(d) ? (int64_t)packed_weight_bytes(k, n) : k * n) < ((int64_t)1 << 31) &&
                       m * k < ((int64_t)1 << 31);
