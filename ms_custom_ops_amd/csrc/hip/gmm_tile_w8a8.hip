@@ -44,6 +44,11 @@ constexpr int KN_RING = 3;    // [K,N] weight slabs in flight in registers
 // fragment read (16 consecutive rows, one logical chunk) cover all 16 slots of a 256-byte LDS cycle
 template <int BKT>
 __device__ __forceinline__ int swz(int r) { return BKT == 64 ? (r >> 2) & 3 : (r >> 1) & 7; }
+// [K,N] slabs read with transpose reads, K rows of BN bytes: a read touches 8 consecutive rows x the chunks of two
+// neighbouring 16-lane blocks, and those 16 pieces of 16 bytes have to fall into 16 different bank groups of the
+// 256-byte LDS cycle (rows of 128 bytes alias every second row)
+template <int BN>
+__device__ __forceinline__ int swz_kt(int r) { return BN == 256 ? (r & 7) << 1 : ((r >> 1) & 3) << 1; }
 
 // MFMA output row q (0..31) of a 32 x 32 block <-> weight column inside the block.  Lane half hh holds
 // rows q = 8 g + 4 hh + t (g = 0..3, t = 0..3); mapping them to columns 16 (g/2) + 8 hh + 4 (g%2) + t
@@ -81,6 +86,18 @@ __device__ __forceinline__ void lds_read_b64_pair(const unsigned char *p, int st
   asm volatile("ds_read_b64 %0, %1" : "=v"(hi) : "v"(a + (unsigned)stride));
 #else
   (void)p; (void)stride; lo = hi = uint2{0, 0};
+#endif
+}
+// The same with LDS transpose reads (ds_read_b64_tr_b8), STRIDE bytes apart.  Hand-written for the same reason: the
+// compiler takes the builtin for a read that any LDS-direct load in flight may alias and waits for all of them.
+template <int STRIDE>
+__device__ __forceinline__ void lds_read_tr8_pair(const unsigned char *p, uint2 &lo, uint2 &hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const unsigned a = (unsigned)(unsigned long)(const __attribute__((address_space(3))) unsigned char *)p;
+  asm volatile("ds_read_b64_tr_b8 %0, %1" : "=v"(lo) : "v"(a));
+  asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(hi) : "v"(a), "n"(STRIDE));
+#else
+  (void)p; lo = hi = uint2{0, 0};
 #endif
 }
 __device__ __forceinline__ void lds_write_b128(unsigned char *p, msco::v4i v) {
@@ -122,11 +139,19 @@ __device__ __forceinline__ void wait_vmcnt() {
 // of weights that at most two m-tiles read (GmmParams::w_nontemporal): a stream that is read once should not push x
 // out of the caches.  Whole kilobytes per instruction only: on row-major [E,N,K] weights with 64-byte slabs (half
 // lines) the bit costs 15 %.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES, bool PK = false, int KS = 2, bool WNT = false>
+// KT (with NK): the weights are [E,K,N] after all (N a multiple of 16) and take the LDS-direct path as they lie in
+// memory: a slab is BKT K rows of BN column bytes, one wave instruction brings 1024 / BN rows, lane L row L / (BN / 16),
+// slot L % (BN / 16), and slot s of row r holds the 16-column chunk s ^ swz_kt<BN>(r).  A weight fragment is two LDS
+// transpose reads (ds_read_b64_tr_b8: of a block of 16 lanes, lane i names 8 bytes M[i][0..7] and lane j receives
+// byte b = M[2 b + j / 8][j % 8]; with lanes 2 b and 2 b + 1 on the two halves of one chunk of K row b, lane j gets K
+// rows 0 .. 7 of the chunk's column j).  MFMA row q of a 32-column block is then column q itself, so a lane owns four
+// runs of 4 output columns instead of two of 8 and the epilogue parks 8-byte pieces.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES, bool PK = false, int KS = 2, bool WNT = false, bool KT = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel(const GmmParams p) {
   static_assert(!PK || NK, "packed weights use the LDS-direct weight path");
   static_assert(!WNT || PK, "non-temporal weight loads are for the packed layout");
   static_assert(KS == 2 || (KS == 4 && NK), "128-byte slabs are built for K-major weights");
+  static_assert(!KT || (NK && !PK && (BN == 128 || BN == 256)), "transpose reads: the LDS-direct path on [K,N] rows of 128 or 256 columns");
   constexpr int BKT = 32 * KS;                      // bytes of K per slab
   constexpr int ROWS_PER_LOAD = 1024 / BKT;         // x rows one wave instruction (1 KiB) brings
   constexpr int KB_PER_SLAB = BKT / 64;             // packed 1 KiB blocks of a column group per slab
@@ -242,8 +267,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   const int pk_blocks = (p.k + 63) / 64, pk_groups = (p.n + 15) / 16;   // packed layout: K blocks per column group, column groups
   const __amdgpu_buffer_rsrc_t rw =
     PK   ? make_rsrc(p.w + ((long long)grp * pk_groups + n0 / 16) * pk_blocks * 1024, (long long)(pk_groups - n0 / 16) * pk_blocks * 1024)
-    : NK ? make_rsrc(wg + (long long)n0 * p.k, (long long)(p.n - n0) * p.k)
-         : make_rsrc(wg + n0, w_elems - n0);
+    : (NK && !KT) ? make_rsrc(wg + (long long)n0 * p.k, (long long)(p.n - n0) * p.k)
+                  : make_rsrc(wg + n0, w_elems - n0);
 
   // ---- operands loaded straight into LDS (x rows, [N,K] weights) -----------------------------
   // One wave instruction fills 1 KiB of LDS = 16 rows x 64 B, lane L writing bytes [16 L, 16 L + 16).
@@ -267,7 +292,17 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   // column 32 * block + col_of_q(q) of the tile.
   unsigned b_voff[NK ? B_LD : 1];
   int b_chunk[NK ? B_LD : 1];                        // row-major weights: logical chunk of this lane in piece u
-  if constexpr (NK) {
+  constexpr int KT_SLOTS = BN / 16, KT_ROWS = 1024 / BN;   // [K,N] slabs: 16-column chunks per K row, K rows per piece
+  if constexpr (KT) {
+#pragma unroll
+    for (int u = 0; u < B_LD; ++u) {
+      const int krow = (wave * B_LD + u) * KT_ROWS + lane / KT_SLOTS;   // K row of the slab that this lane brings in piece u
+      const int chunk = (lane % KT_SLOTS) ^ swz_kt<BN>(krow);
+      b_chunk[u] = krow;                               // (the K tail is a matter of rows here)
+      // columns past N read as zero; the K row of the slab goes into the scalar offset, which nobody range-checks
+      b_voff[u] = (n0 + chunk * 16 < p.n) ? (unsigned)krow * (unsigned)p.n + chunk * 16 : OOB;
+    }
+  } else if constexpr (NK) {
 #pragma unroll
     for (int u = 0; u < B_LD; ++u) {
       const int blk = wave * B_LD + u;
@@ -297,6 +332,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
           const int kblock = (k_first + kt) * KB_PER_SLAB + blk % KB_PER_SLAB;
           const unsigned kill_w = (kblock >= pk_blocks) ? OOB : 0u;
           buffer_load_lds_b128<WNT ? 2 : 0>(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, kblock * 1024);
+        } else if constexpr (KT) {
+          const unsigned kill_b = (kbase + (unsigned)b_chunk[u] >= (unsigned)p.k) ? OOB : 0u;   // K rows past K
+          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase * (unsigned)p.n);
         } else {
           const unsigned kill_b = (kbase + b_chunk[u] * 16 >= (unsigned)p.k) ? OOB : 0u;
           buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase);
@@ -354,6 +392,16 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
       // chunk 2 kk + hh of the slab: block (2 kk + hh) / 4 of the column group's blocks in this slab, chunk % 4 inside it
       return *reinterpret_cast<const v4i *>(b + ((col >> 4) * KB_PER_SLAB + ((2 * kk + hh) >> 2)) * 1024 +
                                             ((2 * kk + hh) & 3) * 256 + (col & 15) * 16);
+    } else if constexpr (KT) {
+      // K rows 32 kk + 16 hh + 8 t + i / 2 (t = 0, 1: the two reads; i = lane % 16), half i % 2 of the chunk that holds the
+      // 16 columns of this lane's block of 16
+      const int i = lane & 15;
+      const int krow = 32 * kk + 16 * hh + (i >> 1);
+      const int chunk = (wave_n * WTN + 32 * f) / 16 + ((lane >> 4) & 1);
+      const unsigned char *b = lds_b + (kt % NSTAGE) * B_STAGE + krow * BN + ((chunk ^ swz_kt<BN>(krow)) << 4) + (i & 1) * 8;
+      uint2 lo, hi;
+      lds_read_tr8_pair<8 * BN>(b, lo, hi);   // (the caller orders these reads before its own and waits for them)
+      return v4i{(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
     } else if constexpr (NK) {
       const unsigned char *b = lds_b + (kt % NSTAGE) * B_STAGE;
       return *reinterpret_cast<const v4i *>(b + rho * BKT + (((2 * kk + hh) ^ swz<BKT>(rho)) << 4));
@@ -416,10 +464,10 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
       for (int i = 0; i < FM; ++i) xf[kk][i] = read_x(kt, i, kk);
-    if constexpr (!NK) {
+    if constexpr (!NK || KT) {
       // hand-issued weight reads: older than every x read, so one wait covers them
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk)
+      for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
         for (int f = 0; f < FN; ++f) lds_reads_done(wf[kk][f]);
     }
@@ -541,7 +589,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   lds_barrier();
 
   // ---- fused dequant epilogue --------------------------------------------------------------------
-  // acc[f][i][r] is output row 32 i + l32 and column 32 f + 16 (r / 8) + 8 hh + (r % 8) of the wave tile:
+  // acc[f][i][r] is output row 32 i + l32 and column 32 f + 16 (r / 8) + 8 hh + (r % 8) of the wave tile
+  // (transpose-read weights, KT: column 32 f + 8 (r / 4) + 4 hh + (r % 4), the MFMA's own row order):
   // lanes run along rows.  Each wave dequantises its values, parks them in a private LDS region
   // (rows of 128 payload bytes at a 144-byte pitch, conflict free both ways) and reads them back with
   // lanes running along columns, so every global store instruction writes 8 full 128-byte row segments.
@@ -563,24 +612,25 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
       if (raw && f != pass) continue;
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
-        const int cw = 32 * f + 16 * s2 + 8 * hh;            // column inside the wave tile
-        const int nb = n0 + wave_n * WTN + cw;
+        // accumulators 8 s2 .. 8 s2 + 7: one run of 8 columns, or (KT) two runs of 4, eight columns apart
+        const int cw = KT ? 32 * f + 16 * s2 + 4 * hh : 32 * f + 16 * s2 + 8 * hh;   // column inside the wave tile
+        constexpr int RUN2 = KT ? 8 : 4;                       // first column of accumulators 4 .. 7, relative to cw
         float sc[8];
         int bi[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          sc[j] = ep_scale[wave_n * WTN + cw + j];
-          bi[j] = ep_bias[wave_n * WTN + cw + j];
+          sc[j] = ep_scale[wave_n * WTN + cw + (j < 4 ? j : RUN2 + j - 4)];
+          bi[j] = ep_bias[wave_n * WTN + cw + (j < 4 ? j : RUN2 + j - 4)];
         }
 #pragma unroll
         for (int i = 0; i < FM; ++i) {
           unsigned char *dst = stage + (32 * i + l32) * EP_PITCH;
           if (raw) {
-            int *d = reinterpret_cast<int *>(dst + (16 * s2 + 8 * hh) * 4);
+            int *d = reinterpret_cast<int *>(dst + (cw - 32 * f) * 4);
             *reinterpret_cast<int4 *>(d) = make_int4(acc[f][i][8 * s2] + bi[0], acc[f][i][8 * s2 + 1] + bi[1],
                                                      acc[f][i][8 * s2 + 2] + bi[2], acc[f][i][8 * s2 + 3] + bi[3]);
-            *reinterpret_cast<int4 *>(d + 4) = make_int4(acc[f][i][8 * s2 + 4] + bi[4], acc[f][i][8 * s2 + 5] + bi[5],
-                                                         acc[f][i][8 * s2 + 6] + bi[6], acc[f][i][8 * s2 + 7] + bi[7]);
+            *reinterpret_cast<int4 *>(d + RUN2) = make_int4(acc[f][i][8 * s2 + 4] + bi[4], acc[f][i][8 * s2 + 5] + bi[5],
+                                                            acc[f][i][8 * s2 + 6] + bi[6], acc[f][i][8 * s2 + 7] + bi[7]);
           } else {
             float v[8];
 #pragma unroll
@@ -599,7 +649,12 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
               q.z = f32_to_f16_rne(v[4]) | ((unsigned)f32_to_f16_rne(v[5]) << 16);
               q.w = f32_to_f16_rne(v[6]) | ((unsigned)f32_to_f16_rne(v[7]) << 16);
             }
-            *reinterpret_cast<uint4 *>(dst + cw * 2) = q;
+            if constexpr (KT) {
+              *reinterpret_cast<uint2 *>(dst + cw * 2) = make_uint2(q.x, q.y);
+              *reinterpret_cast<uint2 *>(dst + (cw + RUN2) * 2) = make_uint2(q.z, q.w);
+            } else {
+              *reinterpret_cast<uint4 *>(dst + cw * 2) = q;
+            }
           }
         }
       }
@@ -631,13 +686,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
 }
 
 // ---- host launcher ---------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4, bool PK = false, int KS = 2, bool WNT = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4, bool PK = false, int KS = 2, bool WNT = false, bool KT = false>
 static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
   constexpr int BKT = 32 * KS;
   const size_t loop_lds = (size_t)STAGES * BM * BKT + (size_t)(NK ? STAGES : KN_STAGES) * BN * BKT;
   const size_t epi_lds = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * 144;   // epilogue staging, 144-byte row pitch
   const size_t lds = (loop_lds > epi_lds ? loop_lds : epi_lds) + 3 * 1024;   // + epilogue operand table
-  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES, PK, KS, WNT>;
+  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES, PK, KS, WNT, KT>;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -665,6 +720,10 @@ static hipError_t launch_small(const GmmParams &p, bool nk, bool packed, hipStre
     return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, true, 4, true>(p, stream) : launch_cfg<BM, BN, 2, 2, true, 4, true, 2, true>(p, stream);
   if (packed) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, true, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, true, 4, true>(p, stream);
   if (nk) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, false, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, true>(p, stream);
+  // [E,K,N] as stored: the LDS-direct path with transpose reads when the rows are whole 16-column chunks
+  if (p.n % 16 == 0)
+    return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, false, 4, false, true>(p, stream)
+                          : launch_cfg<BM, BN, 2, 2, true, 4, false, 2, false, true>(p, stream);
   return launch_cfg<BM, BN, 2, 2, false>(p, stream);
 }
 
@@ -685,11 +744,14 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
   }
   switch (tile_cfg) {
     case TILE_256x256:
+      if (!nk && p.n % 16 == 0) return launch_cfg<256, 256, 2, 4, true, 4, false, 2, false, true>(p, stream);
       return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
-    case TILE_128x256:   // two 4-wave workgroups per CU; [N,K] weights only
+    case TILE_128x256:   // two 4-wave workgroups per CU; K-major weights, or [K,N] rows of whole 16-column chunks
+      if (!nk && p.n % 16 == 0) return launch_cfg<128, 256, 1, 4, true, 3, false, 2, false, true>(p, stream);
       return nk ? launch_cfg<128, 256, 1, 4, true, 3>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     case TILE_256x256_W4:   // needs at least four 128-byte K slabs per tile, a group table that fits in LDS, whole 256-column rows of [K,N] weights
       if (p.k >= 512 && p.e <= 1024 && (nk || p.n % 256 == 0)) return launch_tile4_w8a8(p, nk ? 0 : 2, stream);
+      if (!nk && p.n % 16 == 0) return launch_cfg<256, 256, 2, 4, true, 4, false, 2, false, true>(p, stream);
       return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
     default:
       return hipErrorInvalidValue;
