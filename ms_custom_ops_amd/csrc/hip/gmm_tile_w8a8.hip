@@ -13,10 +13,10 @@
 //     stay in that XCD's L2.
 //   * Memory.  Operands are read through buffer descriptors (scalar base, one per-lane offset,
 //     out-of-range rows read as zero, so no clamping or branching in the loop) in 64-byte K slabs,
-//     three slabs ahead of the one being multiplied.  x rows and [N,K] weights go straight from
-//     memory into a 4-stage LDS ring (buffer_load ... lds), so slabs in flight cost no registers.
-//   * Weights stored [K,N] are held in a 3-deep register ring, transposed into K-contiguous MFMA
-//     fragments with v_perm_b32 and written to a 2-stage LDS buffer.
+//     three slabs ahead of the one being multiplied.  x rows and weights go straight from memory
+//     into a 4-stage LDS ring (buffer_load ... lds), so slabs in flight cost no registers.
+//   * Weights stored [K,N] lie in LDS as they lie in memory (K rows of BN column bytes) and are turned
+//     into K-contiguous MFMA fragments on the way out, by LDS transpose reads.
 //   * One LDS-only barrier per slab (it does not wait for the global loads in flight).
 //   * Operand roles.  The weights are the MFMA's first operand and x the second, so a lane owns one
 //     output row m and, after permuting which weight column feeds which MFMA row, two runs of 8
@@ -26,7 +26,7 @@
 // LDS layouts (a fragment read is 16 B per lane over 32 consecutive rows, conflict free per 16 lanes):
 //   x rows and [N,K] weights: row-major, 64 B per row, 16-byte chunk c of row r stored at chunk
 //     position c ^ ((r >> 2) & 3);
-//   [K,N] weights: 8 planes (one per 8 K rows) of BN slots x 8 bytes.
+//   [K,N] weights: K rows of BN bytes, 16-column chunk c of row r at chunk position c ^ swz_kt<BN>(r).
 #include <algorithm>
 
 #include "gmm_common.h"
@@ -37,8 +37,6 @@
 namespace msco {
 
 constexpr int BK = 64;        // bytes of K per slab = one MFMA K step
-constexpr int KN_STAGES = 2;  // LDS stages of the transposed [K,N] weight slab
-constexpr int KN_RING = 3;    // [K,N] weight slabs in flight in registers
 
 // rows of BKT bytes in LDS: 16-byte chunk c of row r sits at position c ^ swz<BKT>(r), so that the 16 lanes of a
 // fragment read (16 consecutive rows, one logical chunk) cover all 16 slots of a 256-byte LDS cycle
@@ -76,20 +74,10 @@ __device__ __forceinline__ void buffer_load_lds_b128(__amdgpu_buffer_rsrc_t rsrc
 }
 
 
-// Two 8-byte LDS reads `stride` bytes apart, invisible to the compiler's wait-count bookkeeping.
-// They must be issued before any compiler-visible LDS read whose result is consumed later (LDS
-// operations complete in order), and lds_reads_done() must precede the first use of the results.
-__device__ __forceinline__ void lds_read_b64_pair(const unsigned char *p, int stride, uint2 &lo, uint2 &hi) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  const unsigned a = (unsigned)(unsigned long)(const __attribute__((address_space(3))) unsigned char *)p;
-  asm volatile("ds_read_b64 %0, %1" : "=v"(lo) : "v"(a));
-  asm volatile("ds_read_b64 %0, %1" : "=v"(hi) : "v"(a + (unsigned)stride));
-#else
-  (void)p; (void)stride; lo = hi = uint2{0, 0};
-#endif
-}
-// The same with LDS transpose reads (ds_read_b64_tr_b8), STRIDE bytes apart.  Hand-written for the same reason: the
-// compiler takes the builtin for a read that any LDS-direct load in flight may alias and waits for all of them.
+// Two LDS transpose reads (ds_read_b64_tr_b8) STRIDE bytes apart, invisible to the compiler's wait-count bookkeeping:
+// the compiler takes the builtin for a read that any LDS-direct load in flight may alias and waits for all of them.
+// They must be issued before any compiler-visible LDS read whose result is consumed later (LDS operations complete in
+// order), and lds_reads_done() must precede the first use of the results.
 template <int STRIDE>
 __device__ __forceinline__ void lds_read_tr8_pair(const unsigned char *p, uint2 &lo, uint2 &hi) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -98,14 +86,6 @@ __device__ __forceinline__ void lds_read_tr8_pair(const unsigned char *p, uint2 
   asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(hi) : "v"(a), "n"(STRIDE));
 #else
   (void)p; lo = hi = uint2{0, 0};
-#endif
-}
-__device__ __forceinline__ void lds_write_b128(unsigned char *p, msco::v4i v) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  const unsigned a = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char *)p;
-  asm volatile("ds_write_b128 %0, %1" ::"v"(a), "v"(v) : "memory");
-#else
-  (void)p; (void)v;
 #endif
 }
 template <typename T>
@@ -128,7 +108,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 }
 
 // STAGES = depth of the LDS ring of the operands that are loaded straight into LDS (STAGES - 1 slabs in flight)
-// PK (with NK): weights in the packed layout (1 KiB blocks of 16 columns x 64 K bytes, byte 16 l + i of block (a, b) =
+// PK: weights in the packed layout (1 KiB blocks of 16 columns x 64 K bytes, byte 16 l + i of block (a, b) =
 // w[k = 64 b + 16 (l / 16) + i][n = 16 a + l % 16]).  A 64-byte K slab of the tile is then one block per column group:
 // the LDS-direct load of a block copies it as it lies, and a weight fragment is read at block (column / 16), chunk
 // 2 kk + hh, row (column % 16) -- conflict free without a swizzle.
@@ -139,25 +119,23 @@ __device__ __forceinline__ void wait_vmcnt() {
 // of weights that at most two m-tiles read (GmmParams::w_nontemporal): a stream that is read once should not push x
 // out of the caches.  Whole kilobytes per instruction only: on row-major [E,N,K] weights with 64-byte slabs (half
 // lines) the bit costs 15 %.
-// KT (with NK): the weights are [E,K,N] after all (N a multiple of 16) and take the LDS-direct path as they lie in
+// KT: the weights are [E,K,N] (N a multiple of 16) and take the LDS-direct path as they lie in
 // memory: a slab is BKT K rows of BN column bytes, one wave instruction brings 1024 / BN rows, lane L row L / (BN / 16),
 // slot L % (BN / 16), and slot s of row r holds the 16-column chunk s ^ swz_kt<BN>(r).  A weight fragment is two LDS
 // transpose reads (ds_read_b64_tr_b8: of a block of 16 lanes, lane i names 8 bytes M[i][0..7] and lane j receives
 // byte b = M[2 b + j / 8][j % 8]; with lanes 2 b and 2 b + 1 on the two halves of one chunk of K row b, lane j gets K
 // rows 0 .. 7 of the chunk's column j).  MFMA row q of a 32-column block is then column q itself, so a lane owns four
 // runs of 4 output columns instead of two of 8 and the epilogue parks 8-byte pieces.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES, bool PK = false, int KS = 2, bool WNT = false, bool KT = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool PK = false, int KS = 2, bool WNT = false, bool KT = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel(const GmmParams p) {
-  static_assert(!PK || NK, "packed weights use the LDS-direct weight path");
   static_assert(!WNT || PK, "non-temporal weight loads are for the packed layout");
-  static_assert(KS == 2 || (KS == 4 && NK), "128-byte slabs are built for K-major weights");
-  static_assert(!KT || (NK && !PK && (BN == 128 || BN == 256)), "transpose reads: the LDS-direct path on [K,N] rows of 128 or 256 columns");
+  static_assert(KS == 2 || KS == 4, "64- or 128-byte K slabs");
+  static_assert(!KT || (!PK && (BN == 128 || BN == 256)), "transpose reads: [K,N] rows of 128 or 256 columns");
   constexpr int BKT = 32 * KS;                      // bytes of K per slab
   constexpr int ROWS_PER_LOAD = 1024 / BKT;         // x rows one wave instruction (1 KiB) brings
   constexpr int KB_PER_SLAB = BKT / 64;             // packed 1 KiB blocks of a column group per slab
   constexpr int NSTAGE = STAGES;
   constexpr int AHEAD = STAGES - 1;                 // slabs requested ahead of the one being multiplied
-  static_assert(NK || STAGES == 4, "the [K,N] register ring is three slabs deep");
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int NT = NW * 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -167,20 +145,18 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   constexpr int A_STAGE = BM * BKT, B_STAGE = BN * BKT;
   constexpr int PANEL = 8;                          // m-tiles that share a streamed weight panel
   constexpr unsigned OOB = 0x80000000u;             // buffer offset that always reads zero
-  constexpr int VM_PER_SLAB = A_LD + (NK ? B_LD : 8);   // vector-memory loads a wave issues per slab
-  // [K,N] weight slab: 8 K-chunks of 8 rows x BN/4 column groups -> one 8(k) x 4(n)-byte block per thread
-  static_assert(NK || NT == 2 * BN, "one [K,N] block per thread");
+  constexpr int VM_PER_SLAB = A_LD + B_LD;          // vector-memory loads a wave issues per slab
   static_assert(FM >= 1 && FN >= 1 && A_LD >= 1 && B_LD >= 1, "tile shape");
   static_assert(BM % (ROWS_PER_LOAD * NW) == 0 && BN % (16 * NW) == 0, "row blocks per wave");
 
   // LDS: operand ring, reused by the epilogue staging; behind both, the tile's epilogue operands
-  constexpr int LOOP_LDS = NSTAGE * A_STAGE + (NK ? NSTAGE : KN_STAGES) * B_STAGE;
+  constexpr int LOOP_LDS = NSTAGE * (A_STAGE + B_STAGE);
   constexpr int EPI_LDS = NW * WTM * 144;
   constexpr int PARAM_OFF = LOOP_LDS > EPI_LDS ? LOOP_LDS : EPI_LDS;
   static_assert(BM <= 256 && BN <= 256, "epilogue operand table holds 256 entries");
   extern __shared__ __align__(16) unsigned char smem[];
   unsigned char *lds_a = smem;                      // [NSTAGE][BM * BKT], rows of BKT bytes, chunk c at c ^ swz<BKT>(row)
-  unsigned char *lds_b = smem + NSTAGE * A_STAGE;   // [N,K]: [NSTAGE][BN * BK] like x; [K,N]: [KN_STAGES][4][BN][16]
+  unsigned char *lds_b = smem + NSTAGE * A_STAGE;   // [NSTAGE][BN * BKT]: rows like x, packed blocks, or K rows of BN bytes ([K,N])
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -267,8 +243,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   const int pk_blocks = (p.k + 63) / 64, pk_groups = (p.n + 15) / 16;   // packed layout: K blocks per column group, column groups
   const __amdgpu_buffer_rsrc_t rw =
     PK   ? make_rsrc(p.w + ((long long)grp * pk_groups + n0 / 16) * pk_blocks * 1024, (long long)(pk_groups - n0 / 16) * pk_blocks * 1024)
-    : (NK && !KT) ? make_rsrc(wg + (long long)n0 * p.k, (long long)(p.n - n0) * p.k)
-                  : make_rsrc(wg + n0, w_elems - n0);
+    : KT ? make_rsrc(wg + n0, w_elems - n0)
+         : make_rsrc(wg + (long long)n0 * p.k, (long long)(p.n - n0) * p.k);
 
   // ---- operands loaded straight into LDS (x rows, [N,K] weights) -----------------------------
   // One wave instruction fills 1 KiB of LDS = 16 rows x 64 B, lane L writing bytes [16 L, 16 L + 16).
@@ -290,8 +266,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   }
   // [N,K] weights: LDS row rho = 32 * block + q feeds MFMA row q of that block and holds weight
   // column 32 * block + col_of_q(q) of the tile.
-  unsigned b_voff[NK ? B_LD : 1];
-  int b_chunk[NK ? B_LD : 1];                        // row-major weights: logical chunk of this lane in piece u
+  unsigned b_voff[B_LD];
+  int b_chunk[B_LD];                                 // [N,K] weights: logical chunk of this lane in piece u; [K,N]: its K row
   constexpr int KT_SLOTS = BN / 16, KT_ROWS = 1024 / BN;   // [K,N] slabs: 16-column chunks per K row, K rows per piece
   if constexpr (KT) {
 #pragma unroll
@@ -302,7 +278,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
       // columns past N read as zero; the K row of the slab goes into the scalar offset, which nobody range-checks
       b_voff[u] = (n0 + chunk * 16 < p.n) ? (unsigned)krow * (unsigned)p.n + chunk * 16 : OOB;
     }
-  } else if constexpr (NK) {
+  } else {
 #pragma unroll
     for (int u = 0; u < B_LD; ++u) {
       const int blk = wave * B_LD + u;
@@ -322,58 +298,22 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
       const unsigned kill_a = (kbase + a_chunk[u] * 16 >= (unsigned)p.k) ? OOB : 0u;
       buffer_load_lds_b128(rx, lds_a + stage * A_STAGE + blk * 1024, a_voff[u] | kill_a, kbase);
     }
-    if constexpr (NK) {
 #pragma unroll
-      for (int u = 0; u < B_LD; ++u) {
-        const int blk = wave * B_LD + u;
-        if constexpr (PK) {
-          // K block (k_first + kt) KB_PER_SLAB + blk % KB_PER_SLAB of the column group; blocks past K do not exist
-          // (the last one is zero padded)
-          const int kblock = (k_first + kt) * KB_PER_SLAB + blk % KB_PER_SLAB;
-          const unsigned kill_w = (kblock >= pk_blocks) ? OOB : 0u;
-          buffer_load_lds_b128<WNT ? 2 : 0>(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, kblock * 1024);
-        } else if constexpr (KT) {
-          const unsigned kill_b = (kbase + (unsigned)b_chunk[u] >= (unsigned)p.k) ? OOB : 0u;   // K rows past K
-          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase * (unsigned)p.n);
-        } else {
-          const unsigned kill_b = (kbase + b_chunk[u] * 16 >= (unsigned)p.k) ? OOB : 0u;
-          buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase);
-        }
+    for (int u = 0; u < B_LD; ++u) {
+      const int blk = wave * B_LD + u;
+      if constexpr (PK) {
+        // K block (k_first + kt) KB_PER_SLAB + blk % KB_PER_SLAB of the column group; blocks past K do not exist
+        // (the last one is zero padded)
+        const int kblock = (k_first + kt) * KB_PER_SLAB + blk % KB_PER_SLAB;
+        const unsigned kill_w = (kblock >= pk_blocks) ? OOB : 0u;
+        buffer_load_lds_b128<WNT ? 2 : 0>(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, kblock * 1024);
+      } else if constexpr (KT) {
+        const unsigned kill_b = (kbase + (unsigned)b_chunk[u] >= (unsigned)p.k) ? OOB : 0u;   // K rows past K
+        buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase * (unsigned)p.n);
+      } else {
+        const unsigned kill_b = (kbase + b_chunk[u] * 16 >= (unsigned)p.k) ? OOB : 0u;
+        buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase);
       }
-    }
-  };
-
-  // ---- [K,N] weights: registers -> v_perm transpose -> LDS -----------------------------------
-  // Thread (plane k8 = tid / (BN/4), i = tid % (BN/4)) loads 8 K rows x 4 columns (one dword per row),
-  // transposes them to 4 columns x 8 K bytes and writes 32 contiguous bytes into plane k8 of the LDS
-  // stage: plane k8 is an array of BN slots x 8 bytes, slot s = MFMA row feed position.  Its 4 columns
-  // are chosen so that they land in slots 4 i .. 4 i + 3: within a 32-column block, lane i % 8 takes the
-  // dword at column {0, 8, 4, 12, 16, 24, 20, 28}[i % 8] (all 8 dwords of the 32 bytes are covered, so
-  // the global loads stay fully coalesced).
-  const int kn_i = tid % (BN / 4), kn_k8 = tid / (BN / 4);
-  const int kn_col = 32 * (kn_i >> 3) + col_of_q(4 * (kn_i & 7));
-  // columns past N and K rows past K are turned into out-of-range offsets (they read as zero)
-  const unsigned bkn_voff = (n0 + kn_col < p.n) ? (unsigned)(8 * kn_k8) * (unsigned)p.n + kn_col : OOB;
-  unsigned rkn[NK ? 1 : KN_RING][8];
-  auto load_kn = [&](int kt, int slot) {
-    if constexpr (!NK) {
-      const int kabs = (k_first + kt) * BK;
-      const unsigned voff = (kabs + 8 * kn_k8 >= p.k) ? OOB : bkn_voff;
-#pragma unroll
-      for (int r = 0; r < 8; ++r)
-        rkn[slot][r] = __builtin_amdgcn_raw_buffer_load_b32(rw, voff, (kabs + r) * p.n, 0);
-    }
-  };
-  auto store_kn = [&](int kt, int slot) {
-    if constexpr (!NK) {
-      unsigned char *b = lds_b + (kt % KN_STAGES) * B_STAGE + kn_k8 * (BN * 8) + kn_i * 32;
-      unsigned lo[4], hi[4];
-      transpose4x4(rkn[slot][0], rkn[slot][1], rkn[slot][2], rkn[slot][3], lo[0], lo[1], lo[2], lo[3]);
-      transpose4x4(rkn[slot][4], rkn[slot][5], rkn[slot][6], rkn[slot][7], hi[0], hi[1], hi[2], hi[3]);
-      // hand-written stores for the same reason as the reads of this region (see read_w); the
-      // LDS-only barrier that follows waits for them
-      lds_write_b128(b, v4i{(int)lo[0], (int)hi[0], (int)lo[1], (int)hi[1]});
-      lds_write_b128(b + 16, v4i{(int)lo[2], (int)hi[2], (int)lo[3], (int)hi[3]});
     }
   };
 
@@ -402,19 +342,9 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
       uint2 lo, hi;
       lds_read_tr8_pair<8 * BN>(b, lo, hi);   // (the caller orders these reads before its own and waits for them)
       return v4i{(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
-    } else if constexpr (NK) {
+    } else {
       const unsigned char *b = lds_b + (kt % NSTAGE) * B_STAGE;
       return *reinterpret_cast<const v4i *>(b + rho * BKT + (((2 * kk + hh) ^ swz<BKT>(rho)) << 4));
-    } else {
-      // 16 K bytes of chunk c = 2 kk + hh: planes 2 c and 2 c + 1, 8 bytes each.  Read with
-      // hand-written ds_read_b64: the compiler makes every LDS read it knows about wait for all
-      // LDS-direct loads in flight unless it can tell them apart, and it cannot for this region
-      // (which those loads never write) -- that wait would serialise the whole operand pipeline.
-      // The caller orders these reads before its own and waits for them (read_w_done).
-      const unsigned char *b = lds_b + (kt % KN_STAGES) * B_STAGE + (2 * (2 * kk + hh)) * (BN * 8) + rho * 8;
-      uint2 lo, hi;
-      lds_read_b64_pair(b, BN * 8, lo, hi);
-      return v4i{(int)lo.x, (int)lo.y, (int)hi.x, (int)hi.y};
     }
   };
 
@@ -427,19 +357,16 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
       for (int r = 0; r < 16; ++r) acc[f][i][r] = 0;
 
   // ---- main loop ---------------------------------------------------------------------------------
-  // Slabs t+1 .. t+3 are in flight (LDS ring for the directly loaded operands, register ring for
-  // [K,N] weights) while slab t is multiplied.
+  // Slabs t+1 .. t+3 are in flight in the LDS ring while slab t is multiplied.
   //
-  // [N,K] weights with 8 waves: every SIMD hosts two waves, one from each half of the workgroup, and
+  // With 8 waves every SIMD hosts two waves, one from each half of the workgroup, and
   // the halves run half a step apart.  While one half issues its 16 MFMAs for slab t, the other half
   // does the memory side of its own step (requests slab t+3, reads its 12 operand fragments from
   // LDS).  Two workgroup barriers per step keep the halves in opposite phases, so the matrix pipe and
   // the LDS / memory pipes are busy at the same time instead of taking turns.  The half that runs
   // behind enters the loop through one extra barrier and the half that runs ahead leaves it through
-  // one, so all waves execute the same number.  [K,N] weights keep all waves in one phase with one
-  // barrier per slab: their register-staged weight loads stall now and then, and in the two-phase
-  // scheme such a stall stops both halves (measured slower).
-  constexpr bool PINGPONG = (NW == 8) && NK;
+  // one, so all waves execute the same number.  Four waves keep one phase with one barrier per slab.
+  constexpr bool PINGPONG = NW == 8;
   const bool behind = PINGPONG && wave >= NW / 2;
   auto phase_barrier = [&]() {
     __builtin_amdgcn_sched_barrier(0);
@@ -451,10 +378,8 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
   // the loop then issues the same number of loads, which keeps the vmcnt waits exact -- with
   // conditional requests the compiler has to assume the shortest path and waits for the loads it has
   // just issued.
-  auto step = [&](int kt, auto ring_slot) {
-    constexpr int SLOT = decltype(ring_slot)::value;          // == kt % KN_RING, compile-time for register indexing
+  auto step = [&](int kt) {
     issue_direct(kt + AHEAD);
-    load_kn(kt + 3, SLOT);                                    // (kt + 3) % 3 == kt % 3: that slot was emptied last step
     v4i xf[KS][FM], wf[KS][FN];
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk)
@@ -464,7 +389,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
     for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
       for (int i = 0; i < FM; ++i) xf[kk][i] = read_x(kt, i, kk);
-    if constexpr (!NK || KT) {
+    if constexpr (KT) {
       // hand-issued weight reads: older than every x read, so one wait covers them
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk)
@@ -489,34 +414,20 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
       __builtin_amdgcn_s_setprio(0);
       phase_barrier();
     } else {
-      store_kn(kt + 1, (SLOT + 1) % KN_RING);                 // its LDS stage held slab t-1, read before the last barrier
       wait_vmcnt<(AHEAD - 1) * VM_PER_SLAB>();                // only the loads of younger slabs may be outstanding
       lds_barrier();
     }
   };
 
   // prologue: slabs 0, 1, 2 requested; slab 0 published
-  issue_direct(0); load_kn(0, 0);
-  issue_direct(1); load_kn(1, 1);
-  if constexpr (AHEAD > 2) { issue_direct(2); load_kn(2, 2); }
-  store_kn(0, 0);
+  issue_direct(0);
+  issue_direct(1);
+  if constexpr (AHEAD > 2) issue_direct(2);
   wait_vmcnt<(AHEAD - 1) * VM_PER_SLAB>();
   lds_barrier();
   if (behind) phase_barrier();
 
-  if constexpr (NK) {
-    for (int kt = 0; kt < k_slabs; ++kt) step(kt, std::integral_constant<int, 0>{});
-  } else {
-    // unrolled by the register ring so that ring slots are compile-time register names
-    int kt = 0;
-    for (; kt + KN_RING <= k_slabs; kt += KN_RING) {
-      step(kt, std::integral_constant<int, 0>{});
-      step(kt + 1, std::integral_constant<int, 1>{});
-      step(kt + 2, std::integral_constant<int, 2>{});
-    }
-    if (kt < k_slabs) step(kt, std::integral_constant<int, 0>{});
-    if (kt + 1 < k_slabs) step(kt + 1, std::integral_constant<int, 1>{});
-  }
+  for (int kt = 0; kt < k_slabs; ++kt) step(kt);
   if (PINGPONG && !behind) phase_barrier();
 
   // ---- K split: partial tiles meet in the workspace, the last slice to arrive adds them up ----------
@@ -686,13 +597,13 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
 }
 
 // ---- host launcher ---------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool NK, int STAGES = 4, bool PK = false, int KS = 2, bool WNT = false, bool KT = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES = 4, bool PK = false, int KS = 2, bool WNT = false, bool KT = false>
 static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
   constexpr int BKT = 32 * KS;
-  const size_t loop_lds = (size_t)STAGES * BM * BKT + (size_t)(NK ? STAGES : KN_STAGES) * BN * BKT;
+  const size_t loop_lds = (size_t)STAGES * (BM + BN) * BKT;
   const size_t epi_lds = (size_t)WAVES_M * WAVES_N * (BM / WAVES_M) * 144;   // epilogue staging, 144-byte row pitch
   const size_t lds = (loop_lds > epi_lds ? loop_lds : epi_lds) + 3 * 1024;   // + epilogue operand table
-  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, NK, STAGES, PK, KS, WNT, KT>;
+  auto kern = gmm_w8a8_tile_kernel<BM, BN, WAVES_M, WAVES_N, STAGES, PK, KS, WNT, KT>;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -711,48 +622,43 @@ static hipError_t launch_cfg(const GmmParams &p, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// The small tile shapes on K-major weights (row-major [E,N,K] or packed) run 128-byte K slabs through a 4-stage ring
-// when the plan says so (GmmParams::wide_k_slabs: the workgroups fit one round; measured against 64-byte slabs on M = 256,
-// K = 4096, N = 11008 packed: 26.0 against 28.8 us; 3 / 2 stages 26.7 / 34.1)
+// The small tile shapes run 128-byte K slabs through a 4-stage ring when the plan says so (GmmParams::wide_k_slabs: the
+// workgroups fit one round; measured against 64-byte slabs on M = 256, K = 4096, N = 11008 packed: 26.0 against 28.8 us;
+// 3 / 2 stages 26.7 / 34.1).  layout: 0 [E,N,K], 1 packed, 2 [E,K,N] (transpose reads).
 template <int BM, int BN>
-static hipError_t launch_small(const GmmParams &p, bool nk, bool packed, hipStream_t stream) {
-  if (packed && p.w_nontemporal)
-    return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, true, 4, true>(p, stream) : launch_cfg<BM, BN, 2, 2, true, 4, true, 2, true>(p, stream);
-  if (packed) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, true, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, true, 4, true>(p, stream);
-  if (nk) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, false, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, true>(p, stream);
-  // [E,K,N] as stored: the LDS-direct path with transpose reads when the rows are whole 16-column chunks
-  if (p.n % 16 == 0)
-    return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, true, 4, false, 4, false, true>(p, stream)
-                          : launch_cfg<BM, BN, 2, 2, true, 4, false, 2, false, true>(p, stream);
-  return launch_cfg<BM, BN, 2, 2, false>(p, stream);
+static hipError_t launch_small(const GmmParams &p, int layout, hipStream_t stream) {
+  if (layout == 1 && p.w_nontemporal)
+    return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, true, 4, true>(p, stream) : launch_cfg<BM, BN, 2, 2, 4, true, 2, true>(p, stream);
+  if (layout == 1) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, true, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, 4, true>(p, stream);
+  if (layout == 0) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, false, 4>(p, stream) : launch_cfg<BM, BN, 2, 2>(p, stream);
+  return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, false, 4, false, true>(p, stream)
+                        : launch_cfg<BM, BN, 2, 2, 4, false, 2, false, true>(p, stream);
 }
 
+// nk: weights stored [E,N,K]; packed: the blocked layout; neither: [E,K,N] (N a multiple of 16, which the plan's
+// alignment rule guarantees for every MFMA kernel)
 hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool packed, hipStream_t stream) {
-  if (tile_cfg == TILE_128x128) return launch_small<128, 128>(p, nk, packed, stream);
-  if (tile_cfg == TILE_64x128) return launch_small<64, 128>(p, nk, packed, stream);
-  if (packed) {
-    switch (tile_cfg) {
-      case TILE_256x256_W4:
-        if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8(p, 1, stream);
-        return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
-      case TILE_128x256:   // four waves side by side, 128 x 64 each
-        if (p.w_nontemporal) return launch_cfg<128, 256, 1, 4, true, 3, true, 2, true>(p, stream);
-        return p.wide_k_slabs ? launch_cfg<128, 256, 1, 4, true, 3, true, 4>(p, stream) : launch_cfg<128, 256, 1, 4, true, 3, true>(p, stream);
-      case TILE_256x256: return launch_cfg<256, 256, 2, 4, true, 4, true>(p, stream);
-      default: return hipErrorInvalidValue;
-    }
+  const int layout = packed ? 1 : nk ? 0 : 2;
+  if (layout == 2 && p.n % 16 != 0) return hipErrorInvalidValue;
+  // the persistent kernel needs at least four 128-byte K slabs per tile, a group table that fits in LDS and, of [E,K,N]
+  // weights, whole 256-column rows; what it cannot take runs the eight-wave kernel of the same tile shape
+  if (tile_cfg == TILE_256x256_W4) {
+    if (p.k >= 512 && p.e <= 1024 && (layout != 2 || p.n % 256 == 0)) return launch_tile4_w8a8(p, layout, stream);
+    tile_cfg = TILE_256x256;
   }
   switch (tile_cfg) {
-    case TILE_256x256:
-      if (!nk && p.n % 16 == 0) return launch_cfg<256, 256, 2, 4, true, 4, false, 2, false, true>(p, stream);
-      return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
-    case TILE_128x256:   // two 4-wave workgroups per CU; K-major weights, or [K,N] rows of whole 16-column chunks
-      if (!nk && p.n % 16 == 0) return launch_cfg<128, 256, 1, 4, true, 3, false, 2, false, true>(p, stream);
-      return nk ? launch_cfg<128, 256, 1, 4, true, 3>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
-    case TILE_256x256_W4:   // needs at least four 128-byte K slabs per tile, a group table that fits in LDS, whole 256-column rows of [K,N] weights
-      if (p.k >= 512 && p.e <= 1024 && (nk || p.n % 256 == 0)) return launch_tile4_w8a8(p, nk ? 0 : 2, stream);
-      if (!nk && p.n % 16 == 0) return launch_cfg<256, 256, 2, 4, true, 4, false, 2, false, true>(p, stream);
-      return nk ? launch_cfg<256, 256, 2, 4, true>(p, stream) : launch_cfg<256, 256, 2, 4, false>(p, stream);
+    case TILE_128x128: return launch_small<128, 128>(p, layout, stream);
+    case TILE_64x128: return launch_small<64, 128>(p, layout, stream);
+    case TILE_256x256:   // eight waves, two per SIMD
+      return layout == 1 ? launch_cfg<256, 256, 2, 4, 4, true>(p, stream)
+           : layout == 0 ? launch_cfg<256, 256, 2, 4>(p, stream)
+                         : launch_cfg<256, 256, 2, 4, 4, false, 2, false, true>(p, stream);
+    case TILE_128x256:   // four waves side by side, 128 x 64 each; two workgroups per CU
+      if (layout == 1) {
+        if (p.w_nontemporal) return launch_cfg<128, 256, 1, 4, 3, true, 2, true>(p, stream);
+        return p.wide_k_slabs ? launch_cfg<128, 256, 1, 4, 3, true, 4>(p, stream) : launch_cfg<128, 256, 1, 4, 3, true>(p, stream);
+      }
+      return layout == 0 ? launch_cfg<128, 256, 1, 4, 3>(p, stream) : launch_cfg<128, 256, 1, 4, 3, false, 2, false, true>(p, stream);
     default:
       return hipErrorInvalidValue;
   }

@@ -55,6 +55,9 @@ def test_full_size_workload_bit_exact_and_checksums(device, name):
 
     acc, info = _launch(tx, tw, tg, None, None, None, wl.m, wl.k, wl.n, wl.e, cabi.DT_I32)
     assert _sha(acc.cpu().numpy()) == dig["acc"], info                       # int32 accumulators, bit-exact
+    # ([E,K,N] as stored: the prefill configurations run the persistent tile kernel through LDS transpose reads, a few
+    # hundred rows the small tiles on the same path)
+    assert "layout=[E,K,N]" in info and (("tile_256x256x128_w4" if wl.m >= 2048 else "skinny" if wl.m <= 16 else "tile_") in info), info
     bits, info = _launch(tx, tw, tg, ts, tp, tb, wl.m, wl.k, wl.n, wl.e, cabi.DT_BF16)
     assert _sha(bits.cpu().numpy().view(np.uint16)) == dig["bf16"], info     # bf16 output, bit-exact
 
