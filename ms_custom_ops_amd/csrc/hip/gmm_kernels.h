@@ -16,7 +16,7 @@ enum TileCfg : int {
 // MFMA tile kernel for W8A8 (prefill shapes).  nk: weights stored [E,N,K]; packed: the packed layout (nk is ignored).
 hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool packed, hipStream_t stream);
 const char *tile_cfg_name(int tile_cfg);
-hipError_t launch_tile4_w8a8(const GmmParams &p, int layout, hipStream_t stream);   // layout 0 [E,N,K], 1 packed, 2 [E,K,N] with N % 256 == 0
+hipError_t launch_tile4_w8a8(const GmmParams &p, int layout, hipStream_t stream);   // layout 0 [E,N,K], 1 packed, 2 [E,K,N] (N % 16 == 0)
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn);
 // K split across workgroups (p.split_k > 1; four-wave tile shapes only): partial tiles and arrival counters
 size_t tile_count_bound(int tile_cfg, int64_t m, int64_t n, int64_t e);

@@ -164,7 +164,7 @@ __device__ __forceinline__ T4Tile t4_locate(const int *meta_end, const int *meta
 // instruction per value), 2 v * sigmoid(c v) with a uniform c (silu, fast gelu: five instructions, two of them
 // transcendental), 1 the tanh form of gelu (three more for its cubic).
 //
-// WL: weight layout, 0 [E,N,K], 1 packed, 2 [E,K,N] (N a multiple of 256).  [E,K,N] rows are N-contiguous and an MFMA
+// WL: weight layout, 0 [E,N,K], 1 packed, 2 [E,K,N] (N a multiple of 16).  [E,K,N] rows are N-contiguous and an MFMA
 // operand wants 16 K-contiguous bytes per lane; the LDS transpose read of gfx950 (ds_read_b64_tr_b8) does that turn on
 // the way out of LDS.  Of a block of 16 lanes, lane i names 8 bytes M[i][0..7]; lane j receives byte b = M[2 b + j / 8][j % 8].
 // With lanes 2 b and 2 b + 1 pointing at the two 8-byte halves of one 16-column chunk of K row b, lane j gets K rows
@@ -236,10 +236,25 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
       const long long cg_bytes = (long long)k_blocks * 1024;
       return t4_rsrc(p.w + ((long long)t.grp * col_groups + t.n0 / 16) * cg_bytes, (long long)(col_groups - t.n0 / 16) * cg_bytes);
     } else if constexpr (KN) {
-      return t4_rsrc(p.w + (long long)t.grp * w_elems + t.n0, w_elems - t.n0);
+      return t4_rsrc(p.w + (long long)t.grp * w_elems + t.n0, w_elems - t.n0);   // (loads use w_rsrc_at: a window per slab)
     } else {
       return t4_rsrc(p.w + (long long)t.grp * w_elems + (long long)t.n0 * p.k, (long long)(p.n - t.n0) * p.k);
     }
+  };
+
+  // [E,K,N]: the window of a tile's weights from K row `krow0` on.  A slab's first row cannot go into the scalar offset
+  // of the load (the buffer unit range-checks the per-lane offset only, against the whole window): it goes into the
+  // base, and the window ends with the expert's matrix, so K rows past K and anything past the tensor read as zeros by
+  // the range check alone.  A chunk past N inside the matrix reads the next K row's bytes: columns that are never stored.
+  // (base and size of the tile's window are kept as scalars: K N < 2^31, so the size fits 32 bits)
+  struct T4Window {
+    const int8_t *base;
+    int bytes;
+  };
+  auto w_window = [&](const T4Tile &t) { return T4Window{p.w + (long long)t.grp * w_elems + t.n0, (int)w_elems - t.n0}; };
+  auto w_rsrc_at = [&](const T4Window &w, unsigned krow0) {
+    const unsigned off = krow0 * (unsigned)p.n;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(w.base + off), 0, max(w.bytes - (int)off, 0), 0x00020000);
   };
 
   // ---- global -> staging registers -------------------------------------------------------------------
@@ -298,6 +313,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
 
   T4Tile nxt = cur;        // tile that follows `cur` in this workgroup's walk (loads run ahead into it)
   __amdgpu_buffer_rsrc_t rx_c = x_rsrc(cur), rw_c = w_rsrc(cur), rx_n = rx_c, rw_n = rw_c;
+  T4Window ww_c = w_window(cur), ww_n = ww_c;   // ([E,K,N] only)
 
   // slab s of the current tile, or slab s - k_slabs of the next one
   auto load_one = [&](int s, auto par_c, auto op_c, auto u_c) {
@@ -309,11 +325,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     if constexpr (OP == 0) {
       stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rx_n : rx_c, (a_voff0 + U * rows32) | kill, kbase, 0);
     } else if constexpr (KN) {
-      // K rows 16 U + 4 wave + lane / 16 of the slab; the slab's first row goes into the scalar offset, which the buffer
-      // unit does not range-check, so rows past K are killed here (their x bytes read as zeros)
-      const bool dead_w = (ahead && !nxt.valid) || kbase + (unsigned)(16 * U + 4 * wave) + (unsigned)(lane >> 4) >= (unsigned)p.k;
-      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rw_n : rw_c, (b_voff0 + U * b_step) | (dead_w ? T4_OOB : 0u),
-                                                            kbase * (unsigned)p.n, 0);
+      // K rows 16 U + 4 wave + lane / 16 of the slab, in the window that starts with the slab (rows past K fall outside it)
+      const unsigned kill_w = (ahead && !nxt.valid) ? T4_OOB : 0u;
+      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc_at(ahead ? ww_n : ww_c, kbase), (b_voff0 + U * b_step) | kill_w, 0, 0);
     } else if constexpr (PK) {
       // K block 2 slab + wave % 2 of column groups 2 U + wave / 2; blocks past K do not exist (the last one is zero padded)
       const unsigned kb = 2u * (unsigned)(ahead ? s - k_slabs : s) + (unsigned)(wave & 1);
@@ -340,12 +354,13 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     load_one(s + 2, par_c, op_c, u_c);
   };
   // the same for a slab whose successor lies inside the current tile and inside K: WS = stage written, soff = scalar
-  // offset of slab s + 2 (bytes of K for x, soff_w for the weights: 16 times that in the packed layout, N times in [E,K,N])
-  auto cycle_clean = [&](auto ws_c, unsigned soff, unsigned soff_w, auto par_c, auto op_c, auto u_c) {
+  // offset of slab s + 2 (bytes of K for x, soff_w for the weights: 16 times that in the packed layout; [E,K,N]: the slab's
+  // own window rw_s and no offset)
+  auto cycle_clean = [&](auto ws_c, unsigned soff, __amdgpu_buffer_rsrc_t rw_s, unsigned soff_w, auto par_c, auto op_c, auto u_c) {
     constexpr int WS = decltype(ws_c)::value, P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
     put_quad((OP == 0 ? st_x : st_w) + WS * T4_OP_STAGE + U * 4096, stg[P][OP][U], op_c);
     if constexpr (OP == 0) stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rx_c, a_voff0 + U * rows32, soff, 0);
-    else stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rw_c, b_voff0 + U * b_step, soff_w, 0);
+    else stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rw_s, b_voff0 + U * b_step, soff_w, 0);
   };
   // [E,K,N] weight fragment: two transpose reads, K rows 0 .. 7 and 8 .. 15 of the lane's column
   auto read_tr = [&](unsigned addr) -> v4i {
@@ -412,7 +427,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   for (int ti = 0;; ++ti) {
     // the tile after this one: the operand stream crosses into it during the last slabs
     nxt = tile_at(ti + 1);
-    if (nxt.valid) { rx_n = x_rsrc(nxt); rw_n = w_rsrc(nxt); }
+    if (nxt.valid) { rx_n = x_rsrc(nxt); rw_n = w_rsrc(nxt); ww_n = w_window(nxt); }
     if (ti > 0) lane_constants();
 
     // Epilogue operands of this tile (scale and bias of its 256 columns, per-token scale of its 256
@@ -526,19 +541,19 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
       };
       // The same with stage, quarter and parity known at compile time, for slabs whose look-ahead stays inside the
       // current tile and inside K (loads need neither the next tile's descriptors nor a tail mask).
-      auto quarter_clean = [&](auto cur_c, auto nxt_c, auto rstage_c, auto rq_c, auto ws_c, unsigned soff, auto par_c, auto g_c) {
+      auto quarter_clean = [&](auto cur_c, auto nxt_c, auto rstage_c, auto rq_c, auto ws_c, unsigned soff, __amdgpu_buffer_rsrc_t rw_s, auto par_c, auto g_c) {
         constexpr int G = decltype(g_c)::value;
         const std::integral_constant<int, 2 * G> ua;
         const std::integral_constant<int, 2 * G + 1> ub;
-        const unsigned soff_w = PK ? soff * 16 : KN ? soff * (unsigned)p.n : soff;
+        const unsigned soff_w = PK ? soff * 16 : KN ? 0u : soff;
         read_w_clean(rstage_c, rq_c, nxt_c, c0); read_x_clean(rstage_c, rq_c, nxt_c, c0);
-        cycle_clean(ws_c, soff, soff_w, par_c, c0, ua);
+        cycle_clean(ws_c, soff, rw_s, soff_w, par_c, c0, ua);
         read_x_clean(rstage_c, rq_c, nxt_c, c1); read_x_clean(rstage_c, rq_c, nxt_c, c2);
-        cycle_clean(ws_c, soff, soff_w, par_c, c0, ub);
+        cycle_clean(ws_c, soff, rw_s, soff_w, par_c, c0, ub);
         read_x_clean(rstage_c, rq_c, nxt_c, c3); read_w_clean(rstage_c, rq_c, nxt_c, c1);
-        cycle_clean(ws_c, soff, soff_w, par_c, c1, ua);
+        cycle_clean(ws_c, soff, rw_s, soff_w, par_c, c1, ua);
         read_w_clean(rstage_c, rq_c, nxt_c, c2); read_w_clean(rstage_c, rq_c, nxt_c, c3);
-        cycle_clean(ws_c, soff, soff_w, par_c, c1, ub);
+        cycle_clean(ws_c, soff, rw_s, soff_w, par_c, c1, ub);
         mfma_quarter(cur_c);
       };
       // slab kt in stage ST; soff3 / soff4: K offsets of slabs kt + 3 and kt + 4
@@ -546,12 +561,14 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         constexpr int ST = decltype(stage_c)::value, PAR = decltype(par_c)::value;
         const std::integral_constant<int, ST ^ 1> other_stage;
         const std::integral_constant<int, PAR ^ 1> other;
-        quarter_clean(c0, c1, stage_c, c1, other_stage, soff3, par_c, c1);
-        quarter_clean(c1, c0, stage_c, c2, other_stage, soff3, par_c, c2);
-        quarter_clean(c0, c1, stage_c, c3, other_stage, soff3, par_c, c3);
+        // ([E,K,N]: one window per slab, made once per slab)
+        const __amdgpu_buffer_rsrc_t rw3 = KN ? w_rsrc_at(ww_c, soff3) : rw_c, rw4 = KN ? w_rsrc_at(ww_c, soff4) : rw_c;
+        quarter_clean(c0, c1, stage_c, c1, other_stage, soff3, rw3, par_c, c1);
+        quarter_clean(c1, c0, stage_c, c2, other_stage, soff3, rw3, par_c, c2);
+        quarter_clean(c0, c1, stage_c, c3, other_stage, soff3, rw3, par_c, c3);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         t4_barrier();
-        quarter_clean(c1, c0, other_stage, c0, stage_c, soff4, other, c0);
+        quarter_clean(c1, c0, other_stage, c0, stage_c, soff4, rw4, other, c0);
       };
       // iterations whose furthest request (group 0 of slab kt + 5) ends inside K
       const int k_clean = max(0, ((p.k / T4_BK - 4) / 2) * 2);
@@ -755,6 +772,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     cur = nxt;
     rx_c = rx_n;
     rw_c = rw_n;
+    ww_c = ww_n;
   }
 }
 
@@ -774,8 +792,8 @@ static hipError_t t4_launch(const GmmParams &p, unsigned grid, hipStream_t strea
 
 hipError_t launch_tile4_w8a8(const GmmParams &p, int layout, hipStream_t stream) {
   // the operand stream runs up to four slabs ahead inside one tile; the group table lives in LDS; [E,K,N] weights
-  // (layout 2) are read in whole 256-column rows
-  if (p.k < 4 * T4_BK || p.e > T4_MAX_E || layout < 0 || layout > 2 || (layout == 2 && p.n % T4_BN != 0)) return hipErrorInvalidValue;
+  // (layout 2) are read in 16-column chunks
+  if (p.k < 4 * T4_BK || p.e > T4_MAX_E || layout < 0 || layout > 2 || (layout == 2 && p.n % 16 != 0)) return hipErrorInvalidValue;
   const long long n_tiles = (p.n + T4_BN - 1) / T4_BN;
   const long long m_tiles_ub = (p.m + T4_BM - 1) / T4_BM + p.e;   // every non-empty group adds at most one partial tile
   const long long total_ub = m_tiles_ub * n_tiles;

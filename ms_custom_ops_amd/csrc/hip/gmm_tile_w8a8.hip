@@ -640,10 +640,10 @@ static hipError_t launch_small(const GmmParams &p, int layout, hipStream_t strea
 hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool packed, hipStream_t stream) {
   const int layout = packed ? 1 : nk ? 0 : 2;
   if (layout == 2 && p.n % 16 != 0) return hipErrorInvalidValue;
-  // the persistent kernel needs at least four 128-byte K slabs per tile, a group table that fits in LDS and, of [E,K,N]
-  // weights, whole 256-column rows; what it cannot take runs the eight-wave kernel of the same tile shape
+  // the persistent kernel needs at least four 128-byte K slabs per tile and a group table that fits in LDS; what it
+  // cannot take runs the eight-wave kernel of the same tile shape
   if (tile_cfg == TILE_256x256_W4) {
-    if (p.k >= 512 && p.e <= 1024 && (layout != 2 || p.n % 256 == 0)) return launch_tile4_w8a8(p, layout, stream);
+    if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8(p, layout, stream);
     tile_cfg = TILE_256x256;
   }
   switch (tile_cfg) {

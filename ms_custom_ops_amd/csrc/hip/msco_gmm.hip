@@ -150,10 +150,10 @@ void choose_plan(msco_gmm_op *op) {
 
   int family;
   // packed weights are K-contiguous per column like [E,N,K]: the same tile kernels read them
-  const bool k_major_stored = d.transpose_b != 0 || is_packed(d);
-  // [E,K,N] weights whose rows are whole 16-column chunks run the same LDS-direct tile kernels (transpose reads turn
-  // them on the way out of LDS) and follow the same tile rules; the decode kernels of that layout are its own
-  const bool k_major = k_major_stored || (is_w8a8(d) && n % 16 == 0);
+  // [E,K,N] weights run the same LDS-direct tile kernels as the K-major layouts (transpose reads turn them on the way
+  // out of LDS; rows of whole 16-column chunks, which the alignment rule guarantees) and follow the same tile rules;
+  // only the decode kernels of that layout are its own
+  const bool k_major = d.transpose_b != 0 || is_packed(d) || is_w8a8(d);
   // (a group that overflows its 16-row chunk streams its weights twice, so on K-major weights 1.5 x the average has to
   // fit; beyond that the 64 x 128 tile kernel with non-temporal weight loads is the better streamer -- 128 rows over 8
   // experts, 470 MB of weights: 76 us against 82 us for the 32-row streaming kernel and 105 us for 16-row chunks;
@@ -186,9 +186,8 @@ void choose_plan(msco_gmm_op *op) {
     auto group_tiles = [&](int bm, int bn) { return e * ((rows_per_group + bm - 1) / bm) * ((n + bn - 1) / bn); };
     const int64_t cover = rows_per_group + rows_per_group / 2;
     const int64_t busy = (num_cus > 0 ? num_cus : kTileTargetWorkgroups) * 3 / 4;
-    // (the persistent four-wave kernel: at least four 128-byte K slabs per tile, a group table that fits in LDS, K-major
-    // weights or [E,K,N] weights whose rows are whole 256-column pieces -- it turns those on the way out of LDS)
-    const bool w4_ok = (k_major_stored || n % 256 == 0) && k >= 512 && e <= 1024;
+    // (the persistent four-wave kernel: at least four 128-byte K slabs per tile, a group table that fits in LDS)
+    const bool w4_ok = k_major && k >= 512 && e <= 1024;
     if (e > 1 && w4_ok && cover > 128 && cover <= 384 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
     } else if (e > 1 && k_major && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
@@ -227,7 +226,7 @@ void choose_plan(msco_gmm_op *op) {
     default: break;
   }
   // (what the persistent kernel cannot take runs the eight-wave kernel of the same tile shape; the plan says so)
-  if (family == FAM_TILE && op->tile_cfg == TILE_256x256_W4 && !(k >= 512 && e <= 1024 && (k_major_stored || n % 256 == 0)))
+  if (family == FAM_TILE && op->tile_cfg == TILE_256x256_W4 && !(k >= 512 && e <= 1024))
     op->tile_cfg = TILE_256x256;
   // the MFMA kernels address x and one group's weights through 32-bit buffer offsets
   const bool fits32 = (is_packed(d) ? (int64_t)packed_weight_bytes(k, n) : k * n) < ((int64_t)1 << 31) &&
