@@ -32,6 +32,7 @@ CASES = [
     ("tile256", cabi.OV_TILE_256, False, False, RAGGED),
     ("tile256_w4", cabi.OV_TILE_256_W4, True, False, (700, 640, 512, 3, [300, 300, 700])),
     ("tile256_w4_packed", cabi.OV_TILE_256_W4, False, True, (700, 640, 512, 3, [300, 300, 700])),
+    ("tile256_w4_kn", cabi.OV_TILE_256_W4, False, False, (700, 640 + 48, 512 - 16, 3, [300, 300, 700])),   # [E,K,N] through transpose reads, K and N tails
 ]
 
 
