@@ -158,6 +158,10 @@ void choose_plan(msco_gmm_op *op) {
   // fit; beyond that the 64 x 128 tile kernel with non-temporal weight loads is the better streamer -- 128 rows over 8
   // experts, 470 MB of weights: 76 us against 82 us for the 32-row streaming kernel and 105 us for 16-row chunks;
   // row-major [E,N,K]: 111 us against 140 us)
+  // row-major [E,N,K] weights at decode sizes: a column's K bytes are contiguous and the columns are K bytes apart, which
+  // suits the 64 x 128 tile's LDS-direct loads better than the decode kernel's 64-byte row pieces (K = 4096, N = 11008,
+  // 1 / 16 rows: 15.8 / 15.9 us against 16.8 / 17.7 us; 32 rows over 8 experts, N = 14336: 103 against 115 us)
+  const bool nk_rows = is_w8a8(d) && d.transpose_b != 0 && !is_packed(d);
   const int64_t avg_rows = (m + (e > 0 ? e : 1) - 1) / (e > 0 ? e : 1);
   const bool many_small_groups = e > 1 && (k_major ? avg_rows + avg_rows / 2 : avg_rows) <= kSkinnyRows &&
                                  e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots;
@@ -165,7 +169,7 @@ void choose_plan(msco_gmm_op *op) {
     family = FAM_GENERIC;
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
-  } else if ((m <= kSkinnyMaxRows && !(e == 1 && m > (k_major ? 1 : 2) * kSkinnyRows)) || many_small_groups) {
+  } else if (((m <= kSkinnyMaxRows && !(e == 1 && m > (k_major ? 1 : 2) * kSkinnyRows)) || many_small_groups) && !nk_rows) {
     // decode: few rows in total, or groups of about one 16-row chunk each (the weights stream once per chunk).  The
     // grid enumerates every (group, chunk) a malformed-to-the-limit group_list could fill; beyond a thousand slots
     // the empty workgroups cost more than the tile kernel's partial tiles.  A single group of more than one 16-row
