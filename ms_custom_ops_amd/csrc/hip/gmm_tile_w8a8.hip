@@ -128,7 +128,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 // runs of 4 output columns instead of two of 8 and the epilogue parks 8-byte pieces.
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, bool PK = false, int KS = 2, bool WNT = false, bool KT = false>
 __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel(const GmmParams p) {
-  static_assert(!WNT || PK, "non-temporal weight loads are for the packed layout");
+  static_assert(!WNT || PK || KT, "non-temporal weight loads: whole kilobytes of whole lines per instruction (packed blocks, [K,N] rows)");
   static_assert(KS == 2 || KS == 4, "64- or 128-byte K slabs");
   static_assert(!KT || (!PK && (BN == 128 || BN == 256)), "transpose reads: [K,N] rows of 128 or 256 columns");
   constexpr int BKT = 32 * KS;                      // bytes of K per slab
@@ -309,7 +309,7 @@ __global__ void __launch_bounds__(WAVES_M *WAVES_N * 64, 2) gmm_w8a8_tile_kernel
         buffer_load_lds_b128<WNT ? 2 : 0>(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_w, kblock * 1024);
       } else if constexpr (KT) {
         const unsigned kill_b = (kbase + (unsigned)b_chunk[u] >= (unsigned)p.k) ? OOB : 0u;   // K rows past K
-        buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase * (unsigned)p.n);
+        buffer_load_lds_b128<WNT ? 2 : 0>(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase * (unsigned)p.n);
       } else {
         const unsigned kill_b = (kbase + b_chunk[u] * 16 >= (unsigned)p.k) ? OOB : 0u;
         buffer_load_lds_b128(rw, lds_b + stage * B_STAGE + blk * 1024, b_voff[u] | kill_b, kbase);
@@ -631,6 +631,9 @@ static hipError_t launch_small(const GmmParams &p, int layout, hipStream_t strea
     return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, true, 4, true>(p, stream) : launch_cfg<BM, BN, 2, 2, 4, true, 2, true>(p, stream);
   if (layout == 1) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, true, 4>(p, stream) : launch_cfg<BM, BN, 2, 2, 4, true>(p, stream);
   if (layout == 0) return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, false, 4>(p, stream) : launch_cfg<BM, BN, 2, 2>(p, stream);
+  if (p.w_nontemporal)
+    return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, false, 4, true, true>(p, stream)
+                          : launch_cfg<BM, BN, 2, 2, 4, false, 2, true, true>(p, stream);
   return p.wide_k_slabs ? launch_cfg<BM, BN, 2, 2, 4, false, 4, false, true>(p, stream)
                         : launch_cfg<BM, BN, 2, 2, 4, false, 2, false, true>(p, stream);
 }
@@ -658,6 +661,7 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
         if (p.w_nontemporal) return launch_cfg<128, 256, 1, 4, 3, true, 2, true>(p, stream);
         return p.wide_k_slabs ? launch_cfg<128, 256, 1, 4, 3, true, 4>(p, stream) : launch_cfg<128, 256, 1, 4, 3, true>(p, stream);
       }
+      if (layout == 2 && p.w_nontemporal) return launch_cfg<128, 256, 1, 4, 3, false, 2, true, true>(p, stream);
       return layout == 0 ? launch_cfg<128, 256, 1, 4, 3>(p, stream) : launch_cfg<128, 256, 1, 4, 3, false, 2, false, true>(p, stream);
     default:
       return hipErrorInvalidValue;

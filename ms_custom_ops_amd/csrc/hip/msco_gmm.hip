@@ -291,7 +291,10 @@ void choose_plan(msco_gmm_op *op) {
       int bm, bn;
       tile_cfg_dims(op->tile_cfg, &bm, &bn);
       const int64_t group_rows = e > 1 ? (m / e) + (m / e) / 2 : m;
-      op->w_nontemporal = is_packed(d) && e * k * n >= ((int64_t)32 << 20) && (group_rows + bm - 1) / bm <= 2;
+      // ([E,K,N] rows: a wave instruction brings whole lines too; 470 MB over 8 experts, 64 / 128 rows in all: 94 -> 84 us
+      // and 97 -> 87 us; on 45 MB it loses a little -- 32 rows 16.9 -> 17.3 us -- so the bar is higher there)
+      const int64_t nt_bytes = is_packed(d) ? ((int64_t)32 << 20) : ((int64_t)64 << 20);
+      op->w_nontemporal = (is_packed(d) || d.transpose_b == 0) && e * k * n >= nt_bytes && (group_rows + bm - 1) / bm <= 2;
     }
     if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
   }
