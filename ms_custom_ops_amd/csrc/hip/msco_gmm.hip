@@ -298,13 +298,14 @@ void choose_plan(msco_gmm_op *op) {
     }
     if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
   }
-  // Many experts with uneven loads (a skewed routing) on packed weights: every group of a few rows costs the persistent
-  // kernel a whole 256-row m-tile per n-tile.  The groups of at most 64 rows go to a second launch of 64 x 128 tiles
-  // instead, which streams their weights once with non-temporal loads.  On the skewed 64-expert workload (49152 rows,
-  // K = 2048, N = 2816; 29 groups of at most 64 rows) the persistent kernel's tiles go from 10.2 to 8.9 per workgroup and the
-  // pair of launches measures 336 against 348 us; on [E,N,K] weights (no non-temporal loads) 347 against 350, not worth a
-  // launch.  Which groups are small only the device knows; with few experts the second launch would mostly find none.
-  if (family == FAM_TILE && op->tile_cfg == TILE_256x256_W4 && is_packed(d) && e >= 16 &&
+  // Many experts with uneven loads (a skewed routing): every group of a few rows costs the persistent kernel a whole
+  // 256-row m-tile per n-tile.  The groups of at most 64 rows go to a second launch of 64 x 128 tiles instead, which
+  // streams their weights once with non-temporal loads.  On the skewed 64-expert workload (49152 rows, K = 2048, N = 2816;
+  // 29 groups of at most 64 rows) the persistent kernel's tiles go from 10.2 to 8.9 per workgroup and the pair of launches
+  // measures 336 against 348 us on packed weights and 340 against 352 us on [E,K,N]; on [E,N,K] weights (64-byte row
+  // pieces, no non-temporal loads) 347 against 350, not worth a launch.  Which groups are small only the device knows;
+  // with few experts the second launch would mostly find none.
+  if (family == FAM_TILE && op->tile_cfg == TILE_256x256_W4 && (is_packed(d) || d.transpose_b == 0) && e >= 16 &&
       (d.kernel_override == OV_AUTO || d.kernel_override == OV_TILE_256_W4) && tuning().two_level != 0)
     op->small_group_rows = 64;
   op->stream_tch = 1;
@@ -564,7 +565,7 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
       small.rows_hi = h->small_group_rows;
       small.split_k = 1;
       small.wide_k_slabs = 0;              // (128-byte slabs measured slower here: 340 against 336 us)
-      small.w_nontemporal = layout == 2;   // each small group's weights are read by one m-tile
+      small.w_nontemporal = layout == 2 || !nk;   // each small group's weights are read by one m-tile (packed, [E,K,N])
       err = launch_tile_w8a8(big, h->tile_cfg, nk, layout == 2, s);
       if (err == hipSuccess) err = launch_tile_w8a8(small, TILE_64x128, nk, layout == 2, s);
     } else if (h->family == FAM_TILE) err = launch_tile_w8a8(p, h->tile_cfg, nk, layout == 2, s);

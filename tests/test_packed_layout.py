@@ -261,7 +261,7 @@ def test_persistent_tile_kernel_random_shapes_both_layouts(device, seed):
 @pytest.mark.parametrize("e,seed", [(16, 0), (24, 1), (40, 2)])
 def test_many_uneven_groups_split_between_the_persistent_kernel_and_small_tiles(device, e, seed):
     # sixteen experts and more: the groups of at most 64 rows go to a second launch of 64 x 128 tiles, the others to the
-    # persistent kernel (packed weights only; [E,N,K] stays one launch); group sizes on both sides of the boundary
+    # persistent kernel (packed and [E,K,N] weights; [E,N,K] stays one launch); group sizes on both sides of the boundary
     from gpu_utils import run_w8a8
     rng = np.random.default_rng(7000 + seed)
     sizes = [0, 1, 63, 64, 65, 300, 64, 257] + [int(v) for v in rng.choice([0, 3, 17, 40, 64, 65, 100, 129, 420], e - 8)]
@@ -273,7 +273,10 @@ def test_many_uneven_groups_split_between_the_persistent_kernel_and_small_tiles(
     assert "tile_256x256x128_w4" in info and "small_groups=64:tile_64x128" in info and "layout=packed" in info, info
     ref = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt)
     bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", transpose_b=True, override=cabi.OV_TILE_256_W4, launches=2)   # stores [E,N,K]
-    assert "tile_256x256x128_w4" in info and "small_groups" not in info, info   # one launch on row-major weights
+    assert "tile_256x256x128_w4" in info and "small_groups" not in info, info   # one launch on [E,N,K] weights
+    assert np.array_equal(bits[:gl[-1]], ref[:gl[-1]]), info
+    bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", transpose_b=False, override=cabi.OV_TILE_256_W4, launches=2)   # [E,K,N] as stored
+    assert "tile_256x256x128_w4" in info and "small_groups=64:tile_64x128" in info and "layout=[E,K,N]" in info, info
     assert np.array_equal(bits[:gl[-1]], ref[:gl[-1]]), info
     assert (bits[gl[-1]:] == 0x7FC0).all()   # rows past the last boundary keep the fill value
 
