@@ -830,4 +830,202 @@ hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream) {
   return bf ? stream_launch_a16w8<true, 4>(p, grid, stream) : stream_launch_a16w8<false, 4>(p, grid, stream);
 }
 
+// ---- weight-only, more than 16 rows per group (packed weights) ------------------------------------------------
+// The multi-row shape of the W8A8 kernel above for 16-bit activations: a workgroup owns one chunk of 16 TCH rows of one
+// group (TCH = 2, 4) and a strip of four column groups over all of K; wave w takes K blocks w, w + 4, ...  Per K block a
+// wave converts its four weight blocks to 16-bit operands once and uses them for all TCH row fragments (8 TCH MFMAs, plus
+// 2 TCH against ones for the row sums that fold the offset into the epilogue), so a group's weights are streamed once per
+// 16 TCH rows instead of once per 16.  There is no K split (the grid of 64-column strips fills the chip): the four
+// waves' float32 tiles are added in wave order through LDS, which keeps the result reproducible run to run.
+namespace {
+template <int TCH>
+struct SamShape {
+  static constexpr int kRows = 16 * TCH;
+  static constexpr int kFrags = SM_GROUPS * TCH + TCH;        // 16 x 16 float32 fragments of the tile, then the row sums of the TCH row fragments
+  static constexpr size_t kLds = (size_t)kFrags * 64 * 16;   // float32 tile; later the 16-bit output tile (smaller)
+  static_assert((size_t)kRows * (SM_COLS + 8) * 2 <= kLds, "output tile fits the reduction tile");
+};
+}  // namespace
+
+template <bool BF16, int TCH>
+__global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_streamm_kernel(const GmmParams p) {
+  using S = SamShape<TCH>;
+  extern __shared__ __align__(16) unsigned char st_smem[];
+  v4f *tile = reinterpret_cast<v4f *>(st_smem);   // fragment f (cg * TCH + t; row sums: SM_GROUPS * TCH + t), lane at tile[f * 64 + lane]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c16 = lane & 15, h = lane >> 4;
+  const int strip = blockIdx.x;
+  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
+
+  int g_start, g_end;
+  group_range(p, grp, lane, g_start, g_end);
+  const int m0 = g_start + mc * S::kRows;
+  const int chunk_rows = min(S::kRows, g_end - m0);
+  if (chunk_rows <= 0) return;
+
+  const int n0 = strip * SM_COLS;
+  const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
+  const int cg_count = min(SM_GROUPS, col_groups - strip * SM_GROUPS);
+  const long long group_bytes = (long long)col_groups * k_blocks * 1024;
+  const __amdgpu_buffer_rsrc_t rw = buffer_over(p.w + (long long)grp * group_bytes, group_bytes);
+  // (a window over the chunk's rows: 16-bit x can be twice as many bytes as a 32-bit window holds)
+  const __amdgpu_buffer_rsrc_t rx = buffer_over(reinterpret_cast<const unsigned short *>(p.x) + (long long)m0 * p.k,
+                                                2ll * chunk_rows * p.k);
+  const int cg_base = strip * SM_GROUPS * k_blocks * 1024;
+
+  // row of fragment t in this lane (clamped into the chunk: rows past it are computed and never stored), byte offset
+  // of the lane's 16 K positions inside a block
+  unsigned xoff[TCH];
+#pragma unroll
+  for (int t = 0; t < TCH; ++t) xoff[t] = 2u * (unsigned)min(16 * t + c16, chunk_rows - 1) * (unsigned)p.k + 32u * (unsigned)h;
+
+  v4f acc[SM_GROUPS][TCH], rs[TCH];
+#pragma unroll
+  for (int t = 0; t < TCH; ++t) {
+    rs[t] = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int cg = 0; cg < SM_GROUPS; ++cg) acc[cg][t] = v4f{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // x fragments as in the 16-row kernel: for block b, lane (c, q), step s the 8 values x[c][64 b + 16 q + 8 s ..]
+  auto fetch = [&](int kb, v4i (&xf)[TCH][2], v4i (&wv)[SM_GROUPS]) {
+    const bool live = kb < k_blocks;
+    const bool k_ok = live && kb * 64 + 16 * h < p.k;   // K % 16 == 0: 16 K positions all inside or all outside
+#pragma unroll
+    for (int cg = 0; cg < SM_GROUPS; ++cg)
+      wv[cg] = __builtin_amdgcn_raw_buffer_load_b128(rw, (live && cg < cg_count) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
+                                                     cg_base + cg * k_blocks * 1024, kStreamAux);
+#pragma unroll
+    for (int t = 0; t < TCH; ++t) {
+      xf[t][0] = __builtin_amdgcn_raw_buffer_load_b128(rx, k_ok ? xoff[t] + (unsigned)(kb * 128) : kBufferOob, 0, 0);
+      xf[t][1] = __builtin_amdgcn_raw_buffer_load_b128(rx, k_ok ? xoff[t] + (unsigned)(kb * 128) + 16u : kBufferOob, 0, 0);
+    }
+  };
+  const unsigned ones = BF16 ? 0x3F803F80u : 0x3C003C00u;
+  const v4i ones_frag = v4i{(int)ones, (int)ones, (int)ones, (int)ones};
+  // (a block that was not loaded reads as w + 128 = 128 everywhere: its x fragments are zeros, so it adds nothing)
+  auto multiply = [&](const v4i (&xf)[TCH][2], const v4i (&wv)[SM_GROUPS]) {
+#pragma unroll
+    for (int cg = 0; cg < SM_GROUPS; ++cg) {
+      const unsigned d0 = (unsigned)wv[cg][0] ^ 0x80808080u, d1 = (unsigned)wv[cg][1] ^ 0x80808080u;   // w + 128 as unsigned bytes
+      const unsigned d2 = (unsigned)wv[cg][2] ^ 0x80808080u, d3 = (unsigned)wv[cg][3] ^ 0x80808080u;
+      const v4i w0 = sa_frag<BF16>(d0, d1), w1 = sa_frag<BF16>(d2, d3);
+#pragma unroll
+      for (int t = 0; t < TCH; ++t) {
+        acc[cg][t] = sa_mfma<BF16>(xf[t][0], w0, acc[cg][t]);
+        acc[cg][t] = sa_mfma<BF16>(xf[t][1], w1, acc[cg][t]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < TCH; ++t) {
+      rs[t] = sa_mfma<BF16>(xf[t][0], ones_frag, rs[t]);
+      rs[t] = sa_mfma<BF16>(xf[t][1], ones_frag, rs[t]);
+    }
+  };
+
+  // thread tid will own fragments f = j * 4 + wave (j = 0 .. TCH - 1) at its lane position: rows 16 t + 4 h + r, column
+  // 16 cg + c.  Their antiquant scale and offset are requested behind the first operand loads (16-bit elements: the word
+  // that holds them, branch-free; decoded in the epilogue).
+  v4i xa[TCH][2], wa[SM_GROUPS], xb[TCH][2], wb[SM_GROUPS];
+  int kb = wave;
+  fetch(kb, xa, wa);
+  unsigned sc_word[TCH], of_word[TCH];
+  {
+    const __amdgpu_buffer_rsrc_t rs_sc = buffer_over(p.aq_scale, p.aq_scale ? 2ll * p.e * p.n : 0);
+    const __amdgpu_buffer_rsrc_t rs_of = buffer_over(p.aq_offset, p.aq_offset ? 2ll * p.e * p.n : 0);
+#pragma unroll
+    for (int j = 0; j < TCH; ++j) {
+      const int cg = (j * ST_WAVES + wave) / TCH;
+      const int n = n0 + 16 * cg + c16;
+      const bool live = cg < cg_count && n < p.n;
+      const unsigned byte = 2u * (unsigned)((long long)grp * p.n + n);
+      sc_word[j] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_sc, live ? (byte & ~3u) : kBufferOob, 0, 0);
+      of_word[j] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_of, live ? (byte & ~3u) : kBufferOob, 0, 0);
+    }
+  }
+  // two K blocks in flight per wave: the loads of the next block are issued before this one is multiplied
+  for (; kb < k_blocks; kb += 2 * ST_WAVES) {
+    fetch(kb + ST_WAVES, xb, wb);   // past K: masked, zeros
+    multiply(xa, wa);
+    fetch(kb + 2 * ST_WAVES, xa, wa);
+    multiply(xb, wb);
+  }
+
+  // the four waves' tiles and row sums, added in wave order (every lane only touches its own slots)
+#pragma unroll
+  for (int w = 0; w < ST_WAVES; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int cg = 0; cg < SM_GROUPS; ++cg)
+#pragma unroll
+        for (int t = 0; t < TCH; ++t) {
+          v4f *slot = tile + (cg * TCH + t) * 64 + lane;
+          *slot = w == 0 ? acc[cg][t] : *slot + acc[cg][t];
+        }
+#pragma unroll
+      for (int t = 0; t < TCH; ++t) {
+        v4f *slot = tile + (SM_GROUPS * TCH + t) * 64 + lane;
+        *slot = w == 0 ? rs[t] : *slot + rs[t];
+      }
+    }
+    __syncthreads();
+  }
+
+  v4f v[TCH], xs[TCH];
+#pragma unroll
+  for (int j = 0; j < TCH; ++j) {
+    const int f = j * ST_WAVES + wave;
+    v[j] = tile[f * 64 + lane];
+    xs[j] = tile[(SM_GROUPS * TCH + f % TCH) * 64 + lane];
+  }
+
+  // ---- epilogue: out = s * (sum_k x (w + 128) + (o - 128) sum_k x) ---------------------------------------------
+  unsigned short(*tile_out)[SM_COLS + 8] = reinterpret_cast<unsigned short(*)[SM_COLS + 8]>(st_smem);
+  __syncthreads();   // every thread holds its part of the float32 tile: the LDS tile can be reused
+#pragma unroll
+  for (int j = 0; j < TCH; ++j) {
+    const int f = j * ST_WAVES + wave, cg = f / TCH, t = f % TCH;
+    const int cl = 16 * cg + c16, n = n0 + cl;
+    if (cg < cg_count && n < p.n) {
+      const bool upper = ((long long)grp * p.n + n) & 1;   // which half of its word the element is
+      const float sc = p.aq_scale ? sa_half_like<BF16>((unsigned short)(upper ? sc_word[j] >> 16 : sc_word[j])) : 1.0f;
+      const float of = p.aq_offset ? sa_half_like<BF16>((unsigned short)(upper ? of_word[j] >> 16 : of_word[j])) : 0.0f;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = 16 * t + 4 * h + r;
+        if (row < chunk_rows) tile_out[row][cl] = half_out(p, fmaf(of - 128.0f, xs[j][r], v[j][r]) * sc);
+      }
+    }
+  }
+  __syncthreads();
+  // whole-row stores: 16 TCH rows x 8 pieces of 8 columns
+  for (int item = tid; item < S::kRows * 8; item += ST_THREADS) {
+    const int row = item >> 3, c8 = (item & 7) * 8;
+    const int n = n0 + c8;
+    if (row < chunk_rows && c8 < 16 * cg_count && n < p.n) {
+      const uint4 q = *reinterpret_cast<const uint4 *>(&tile_out[row][c8]);
+      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned short *>(p.out) + (long long)(m0 + row) * p.n + n) = q;
+    }
+  }
+}
+
+template <bool BF16, int TCH>
+static hipError_t streamm_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
+  hipLaunchKernelGGL((gmm_a16w8_streamm_kernel<BF16, TCH>), grid, dim3(ST_THREADS), SamShape<TCH>::kLds, stream, p);
+  return hipGetLastError();
+}
+
+// tch = 16-row fragments per chunk (2 or 4); p.max_chunks counts chunks of 16 tch rows, p.n_strips strips of 64 columns
+hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, hipStream_t stream) {
+  if (p.m == 0) return hipSuccess;
+  if (p.split_k != 1) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), 1u);
+  const bool bf = p.x_dtype == DT_BF16;
+  if (tch == 4) return bf ? streamm_launch_a16w8<true, 4>(p, grid, stream) : streamm_launch_a16w8<false, 4>(p, grid, stream);
+  if (tch == 2) return bf ? streamm_launch_a16w8<true, 2>(p, grid, stream) : streamm_launch_a16w8<false, 2>(p, grid, stream);
+  return hipErrorInvalidValue;
+}
+
 }  // namespace msco

@@ -72,7 +72,7 @@ struct msco_gmm_op {
   int skinny_cols = kSkinnyCols;
   int n_strips = 0;
   int strip_groups = 16;
-  int stream_tch = 1;        // packed W8A8: 16-row fragments per chunk (1: gmm_w8a8_stream_kernel, 2/4/8: the multi-row kernel)
+  int stream_tch = 1;        // packed weights: 16-row fragments per chunk (1: the 16-row streaming kernels, 2/4/8: the multi-row ones; weight-only up to 4)
   int wide_k_slabs = 0;      // small tile kernels on K-major weights: 128-byte K slabs
   int w_nontemporal = 0;     // small tile kernels on packed weights: non-temporal weight loads
   int small_group_rows = 0;  // > 0: the persistent kernel takes the groups with more rows, a second launch of 64 x 128 tiles the others
@@ -320,6 +320,16 @@ void choose_plan(msco_gmm_op *op) {
     while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch = op->stream_tch == 1 ? 2 : op->stream_tch * 2;
     if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8) op->stream_tch = tuning().stream_tch;
+  } else if (family == FAM_SKINNY && is_packed(d) && is_a16w8(d)) {
+    // weight-only on packed weights: chunks of 32 or 64 rows by the same estimate (its multi-row kernel holds at most four
+    // row fragments in registers); larger groups stream their weights once per 64 rows (8 experts, K = 4096, N = 14336,
+    // 128 / 512 / 2048 rows: 111 / 334 / 1307 us with 16-row chunks)
+    const int64_t avg = (m + e - 1) / e;
+    const int64_t rows = e == 1 ? m : avg + avg / 2;
+    op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : 4;
+    while (op->stream_tch < 4 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
+      op->stream_tch *= 2;
+    if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4) op->stream_tch = tuning().stream_tch;
   }
   if (family == FAM_SKINNY) {
     // grid.y enumerates (group, chunk of 16 * stream_tch rows)
@@ -387,6 +397,7 @@ void choose_plan(msco_gmm_op *op) {
       const int slice_blocks = is_w8a8(d) ? 128 : 64;
       want = std::max(want, (int)(((k + 63) / 64 + slice_blocks - 1) / slice_blocks));
     }
+    if (is_packed(d) && op->stream_tch > 1 && !is_w8a8(d)) want = 1;   // the multi-row weight-only kernel walks all of K
     op->split_k = want;
     if (!is_packed(d)) op->skinny_cols = wide16 ? 128 : kSkinnyCols;
     if (is_packed(d)) {
@@ -573,7 +584,8 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
     else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
     else err = launch_generic_w8a8(p, layout, s);
   } else {
-    if (h->family == FAM_SKINNY) err = layout == 2 ? launch_stream_a16w8(p, s) : launch_skinny_a16w8(p, s);
+    if (h->family == FAM_SKINNY && layout == 2) err = h->stream_tch > 1 ? launch_streamm_a16w8(p, h->stream_tch, s) : launch_stream_a16w8(p, s);
+    else if (h->family == FAM_SKINNY) err = launch_skinny_a16w8(p, s);
     else err = launch_generic_a16w8(p, layout, s);
   }
   return err == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;

@@ -12,7 +12,7 @@ c1          single group,  M=128  K=4096 N=4096, zero int32 bias
 c2_m{M}     dense linear,  K=4096 N=11008, M in {1, 16, 256, 2048}, int32 bias in [-1000, 1000]
 c3          MoE E=8 top-2 over 4096 tokens (8192 rows), K=4096 N=14336
 c4          MoE E=64 top-6 over 8192 tokens (49152 rows), Zipf(1.2) expert popularity, K=2048 N=2816
-c5          weight-only decode, E=8 top-2 over 16 tokens (32 rows), bf16 x, K=4096 N=14336
+c5          weight-only decode, E=8 top-2 over 16 tokens (32 rows), bf16 x, K=4096 N=14336 (c5_t<T>: T tokens)
 c3_decode   the c3 layer at decode time: E=8 top-2 over 16 tokens (32 rows), int8 x, K=4096 N=14336 (not one of the
             published configurations: c3's weights with c5's routing, the W8A8 counterpart of c5)
 """
@@ -130,8 +130,8 @@ def make(name: str, *, scale_down: int = 1) -> Workload:
         counts = np.diff(np.concatenate([[0], gl]))
         meta = {"empty_groups": int((counts == 0).sum()), "max_over_mean": float(counts.max() / counts.mean())}
         return Workload(name, "w8a8", m, k, n, e, x, w, s, pt, None, None, gl, meta)
-    if name == "c5":
-        t, e, top_k = 16, 8, 2
+    if name == "c5" or name.startswith("c5_t"):   # c5_t<T>: the weight-only layer of c5 with T tokens (c5 = c5_t16)
+        t, e, top_k = (16 if name == "c5" else int(name[4:])), 8, 2
         k, n = 4096 // sd, 14336 // sd
         m = t * top_k
         x = f32_to_bf16_bits(np.random.randn(m, k).astype(np.float32))
