@@ -831,27 +831,33 @@ hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream) {
 }
 
 // ---- weight-only, more than 16 rows per group (packed weights) ------------------------------------------------
-// The multi-row shape of the W8A8 kernel above for 16-bit activations: a workgroup owns one chunk of 16 TCH rows of one
-// group (TCH = 2, 4) and a strip of four column groups over all of K; wave w takes K blocks w, w + 4, ...  Per K block a
-// wave converts its four weight blocks to 16-bit operands once and uses them for all TCH row fragments (8 TCH MFMAs, plus
-// 2 TCH against ones for the row sums that fold the offset into the epilogue), so a group's weights are streamed once per
-// 16 TCH rows instead of once per 16.  There is no K split (the grid of 64-column strips fills the chip): the four
-// waves' float32 tiles are added in wave order through LDS, which keeps the result reproducible run to run.
+// A workgroup owns one chunk of 16 TCH rows of one group (TCH = 2, 4, 8) and a strip of 4 G column groups (G = 2, 4: 128
+// or 256 columns; TCH = 8 with G = 2 only, for registers) over all of K; wave w owns column groups w G .. w G + G - 1 of the strip and walks every K block, so its
+// accumulators are complete sums: no K split, no reduction between waves, the same float32 summation order run to run.
+// Per K block the workgroup brings the chunk's x slab (16 TCH rows x 64 K, 16-bit) into LDS once -- every wave needs
+// all of it, and 16-bit x is twice the bytes of the weights it meets -- while each wave requests its G weight blocks,
+// converts them to 16-bit operands once and uses them for all TCH row fragments (2 G TCH MFMAs, plus 2 TCH against ones
+// for the row sums that fold the offset into the epilogue).  A group's weights are streamed once per 16 TCH rows
+// instead of once per 16.  LDS rows of 128 payload bytes at a 144-byte pitch: the 16 lanes of a fragment read (16
+// consecutive rows, one 16-byte chunk) fall into 16 different bank groups.
 namespace {
-template <int TCH>
+template <int TCH, int G>
 struct SamShape {
   static constexpr int kRows = 16 * TCH;
-  static constexpr int kFrags = SM_GROUPS * TCH + TCH;        // 16 x 16 float32 fragments of the tile, then the row sums of the TCH row fragments
-  static constexpr size_t kLds = (size_t)kFrags * 64 * 16;   // float32 tile; later the 16-bit output tile (smaller)
-  static_assert((size_t)kRows * (SM_COLS + 8) * 2 <= kLds, "output tile fits the reduction tile");
+  static constexpr int kCols = 64 * G;                         // 4 waves x G column groups x 16
+  static constexpr int kPitch = 144;                           // bytes of an x row in LDS (64 K x 2 bytes + 16)
+  static constexpr int kStage = kRows * kPitch;                // one K block of the chunk's x
+  static constexpr int kPieces = kRows * 8 / ST_THREADS;       // 16-byte pieces of a slab per thread
+  static constexpr size_t kOut = (size_t)kRows * (kCols + 8) * 2;   // 16-bit output tile of the epilogue
+  static constexpr size_t kLds = 2 * kStage > kOut ? 2 * kStage : kOut;
+  static_assert(kPieces >= 1, "slab pieces per thread");
 };
 }  // namespace
 
-template <bool BF16, int TCH>
-__global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_streamm_kernel(const GmmParams p) {
-  using S = SamShape<TCH>;
+template <bool BF16, int TCH, int G>
+__global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const GmmParams p) {
+  using S = SamShape<TCH, G>;
   extern __shared__ __align__(16) unsigned char st_smem[];
-  v4f *tile = reinterpret_cast<v4f *>(st_smem);   // fragment f (cg * TCH + t; row sums: SM_GROUPS * TCH + t), lane at tile[f * 64 + lane]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -865,50 +871,64 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_streamm_kernel(const 
   const int chunk_rows = min(S::kRows, g_end - m0);
   if (chunk_rows <= 0) return;
 
-  const int n0 = strip * SM_COLS;
+  const int n0 = strip * S::kCols;
   const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
-  const int cg_count = min(SM_GROUPS, col_groups - strip * SM_GROUPS);
+  const int cg0 = strip * 4 * G + wave * G;                          // this wave's first column group
+  const int cg_count = max(0, min(G, col_groups - cg0));
   const long long group_bytes = (long long)col_groups * k_blocks * 1024;
   const __amdgpu_buffer_rsrc_t rw = buffer_over(p.w + (long long)grp * group_bytes, group_bytes);
   // (a window over the chunk's rows: 16-bit x can be twice as many bytes as a 32-bit window holds)
   const __amdgpu_buffer_rsrc_t rx = buffer_over(reinterpret_cast<const unsigned short *>(p.x) + (long long)m0 * p.k,
                                                 2ll * chunk_rows * p.k);
-  const int cg_base = strip * SM_GROUPS * k_blocks * 1024;
 
-  // row of fragment t in this lane (clamped into the chunk: rows past it are computed and never stored), byte offset
-  // of the lane's 16 K positions inside a block
-  unsigned xoff[TCH];
+  // the slab pieces this thread carries: piece i = tid + 256 u is row i / 8 (clamped into the chunk: rows past it are
+  // computed and never stored), 16-byte chunk i % 8 of the block's 128 bytes
+  unsigned x_src[S::kPieces], x_dst[S::kPieces];
 #pragma unroll
-  for (int t = 0; t < TCH; ++t) xoff[t] = 2u * (unsigned)min(16 * t + c16, chunk_rows - 1) * (unsigned)p.k + 32u * (unsigned)h;
+  for (int u = 0; u < S::kPieces; ++u) {
+    const int i = tid + ST_THREADS * u, row = i >> 3, chunk = i & 7;
+    x_src[u] = 2u * (unsigned)min(row, chunk_rows - 1) * (unsigned)p.k + 16u * (unsigned)chunk;
+    x_dst[u] = (unsigned)(row * S::kPitch + chunk * 16);
+  }
+  auto load_x = [&](int kb, v4i (&xr)[S::kPieces]) {
+#pragma unroll
+    for (int u = 0; u < S::kPieces; ++u) {
+      const int chunk = (tid + ST_THREADS * u) & 7;
+      const bool ok = kb < k_blocks && kb * 64 + 8 * chunk < p.k;   // K % 16 == 0: a chunk's 8 K positions are all inside or all outside
+      xr[u] = __builtin_amdgcn_raw_buffer_load_b128(rx, ok ? x_src[u] + (unsigned)(kb * 128) : kBufferOob, 0, 0);
+    }
+  };
+  auto store_x = [&](int stage, const v4i (&xr)[S::kPieces]) {
+#pragma unroll
+    for (int u = 0; u < S::kPieces; ++u) *reinterpret_cast<v4i *>(st_smem + stage * S::kStage + x_dst[u]) = xr[u];
+  };
+  auto load_w = [&](int kb, v4i (&wv)[G]) {
+#pragma unroll
+    for (int cg = 0; cg < G; ++cg)
+      wv[cg] = __builtin_amdgcn_raw_buffer_load_b128(rw, (kb < k_blocks && cg < cg_count) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
+                                                     (cg0 + cg) * k_blocks * 1024, kStreamAux);
+  };
 
-  v4f acc[SM_GROUPS][TCH], rs[TCH];
+  v4f acc[G][TCH], rs[TCH];
 #pragma unroll
   for (int t = 0; t < TCH; ++t) {
     rs[t] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int cg = 0; cg < SM_GROUPS; ++cg) acc[cg][t] = v4f{0.f, 0.f, 0.f, 0.f};
+    for (int cg = 0; cg < G; ++cg) acc[cg][t] = v4f{0.f, 0.f, 0.f, 0.f};
   }
-
-  // x fragments as in the 16-row kernel: for block b, lane (c, q), step s the 8 values x[c][64 b + 16 q + 8 s ..]
-  auto fetch = [&](int kb, v4i (&xf)[TCH][2], v4i (&wv)[SM_GROUPS]) {
-    const bool live = kb < k_blocks;
-    const bool k_ok = live && kb * 64 + 16 * h < p.k;   // K % 16 == 0: 16 K positions all inside or all outside
-#pragma unroll
-    for (int cg = 0; cg < SM_GROUPS; ++cg)
-      wv[cg] = __builtin_amdgcn_raw_buffer_load_b128(rw, (live && cg < cg_count) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
-                                                     cg_base + cg * k_blocks * 1024, kStreamAux);
-#pragma unroll
-    for (int t = 0; t < TCH; ++t) {
-      xf[t][0] = __builtin_amdgcn_raw_buffer_load_b128(rx, k_ok ? xoff[t] + (unsigned)(kb * 128) : kBufferOob, 0, 0);
-      xf[t][1] = __builtin_amdgcn_raw_buffer_load_b128(rx, k_ok ? xoff[t] + (unsigned)(kb * 128) + 16u : kBufferOob, 0, 0);
-    }
-  };
   const unsigned ones = BF16 ? 0x3F803F80u : 0x3C003C00u;
   const v4i ones_frag = v4i{(int)ones, (int)ones, (int)ones, (int)ones};
-  // (a block that was not loaded reads as w + 128 = 128 everywhere: its x fragments are zeros, so it adds nothing)
-  auto multiply = [&](const v4i (&xf)[TCH][2], const v4i (&wv)[SM_GROUPS]) {
+  // x fragments as in the 16-row kernel: lane (c, q), step s holds the 8 values x[16 t + c][64 b + 16 q + 8 s ..], i.e.
+  // chunk 2 q + s of row 16 t + c.  (A block that was not loaded reads as w + 128 = 128: its x is zeros, it adds nothing.)
+  auto multiply = [&](int stage, const v4i (&wv)[G]) {
+    v4i xf[TCH][2];
 #pragma unroll
-    for (int cg = 0; cg < SM_GROUPS; ++cg) {
+    for (int t = 0; t < TCH; ++t)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+        xf[t][s2] = *reinterpret_cast<const v4i *>(st_smem + stage * S::kStage + (16 * t + c16) * S::kPitch + (2 * h + s2) * 16);
+#pragma unroll
+    for (int cg = 0; cg < G; ++cg) {
       const unsigned d0 = (unsigned)wv[cg][0] ^ 0x80808080u, d1 = (unsigned)wv[cg][1] ^ 0x80808080u;   // w + 128 as unsigned bytes
       const unsigned d2 = (unsigned)wv[cg][2] ^ 0x80808080u, d3 = (unsigned)wv[cg][3] ^ 0x80808080u;
       const v4i w0 = sa_frag<BF16>(d0, d1), w1 = sa_frag<BF16>(d2, d3);
@@ -925,107 +945,100 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_streamm_kernel(const 
     }
   };
 
-  // thread tid will own fragments f = j * 4 + wave (j = 0 .. TCH - 1) at its lane position: rows 16 t + 4 h + r, column
-  // 16 cg + c.  Their antiquant scale and offset are requested behind the first operand loads (16-bit elements: the word
-  // that holds them, branch-free; decoded in the epilogue).
-  v4i xa[TCH][2], wa[SM_GROUPS], xb[TCH][2], wb[SM_GROUPS];
-  int kb = wave;
-  fetch(kb, xa, wa);
-  unsigned sc_word[TCH], of_word[TCH];
+  // slab 0 to LDS, slab 1 and the weights of blocks 0 and 1 on their way
+  v4i xr[S::kPieces], wa[G], wb[G];
+  load_x(0, xr);
+  load_w(0, wa);
+  // antiquant scale and offset of this lane's G output columns, requested behind the first operand loads (16-bit
+  // elements: the word that holds them, branch-free; decoded in the epilogue)
+  unsigned sc_word[G], of_word[G];
   {
     const __amdgpu_buffer_rsrc_t rs_sc = buffer_over(p.aq_scale, p.aq_scale ? 2ll * p.e * p.n : 0);
     const __amdgpu_buffer_rsrc_t rs_of = buffer_over(p.aq_offset, p.aq_offset ? 2ll * p.e * p.n : 0);
 #pragma unroll
-    for (int j = 0; j < TCH; ++j) {
-      const int cg = (j * ST_WAVES + wave) / TCH;
-      const int n = n0 + 16 * cg + c16;
+    for (int cg = 0; cg < G; ++cg) {
+      const int n = 16 * (cg0 + cg) + c16;
       const bool live = cg < cg_count && n < p.n;
       const unsigned byte = 2u * (unsigned)((long long)grp * p.n + n);
-      sc_word[j] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_sc, live ? (byte & ~3u) : kBufferOob, 0, 0);
-      of_word[j] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_of, live ? (byte & ~3u) : kBufferOob, 0, 0);
+      sc_word[cg] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_sc, live ? (byte & ~3u) : kBufferOob, 0, 0);
+      of_word[cg] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_of, live ? (byte & ~3u) : kBufferOob, 0, 0);
     }
   }
-  // two K blocks in flight per wave: the loads of the next block are issued before this one is multiplied
-  for (; kb < k_blocks; kb += 2 * ST_WAVES) {
-    fetch(kb + ST_WAVES, xb, wb);   // past K: masked, zeros
-    multiply(xa, wa);
-    fetch(kb + 2 * ST_WAVES, xa, wa);
-    multiply(xb, wb);
+  // (LDS-only barrier: __syncthreads would also wait for the operand loads that are in flight on purpose)
+  auto slab_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+  store_x(0, xr);
+  load_x(1, xr);
+  slab_barrier();
+  // One barrier per K block: the slab of block kb + 1 is written to the other stage (which every wave finished reading
+  // before the last barrier) while block kb is multiplied, and the requests run two blocks ahead.
+  for (int kb = 0; kb < k_blocks; kb += 2) {
+    load_w(kb + 1, wb);
+    multiply(0, wa);
+    store_x(1, xr);
+    load_x(kb + 2, xr);
+    slab_barrier();
+    load_w(kb + 2, wa);
+    multiply(1, wb);   // (past K: zeros times 128)
+    store_x(0, xr);
+    load_x(kb + 3, xr);
+    slab_barrier();
   }
 
-  // the four waves' tiles and row sums, added in wave order (every lane only touches its own slots)
+  // ---- epilogue: out = s * (sum_k x (w + 128) + (o - 128) sum_k x); lane (c, h) holds rows 16 t + 4 h + r of column
+  // 16 cg + c of its wave's column groups.  The output tile is staged in LDS (the slabs are done with) for whole-row stores.
+  unsigned short(*tile_out)[S::kCols + 8] = reinterpret_cast<unsigned short(*)[S::kCols + 8]>(st_smem);
 #pragma unroll
-  for (int w = 0; w < ST_WAVES; ++w) {
-    if (wave == w) {
-#pragma unroll
-      for (int cg = 0; cg < SM_GROUPS; ++cg)
-#pragma unroll
-        for (int t = 0; t < TCH; ++t) {
-          v4f *slot = tile + (cg * TCH + t) * 64 + lane;
-          *slot = w == 0 ? acc[cg][t] : *slot + acc[cg][t];
-        }
-#pragma unroll
-      for (int t = 0; t < TCH; ++t) {
-        v4f *slot = tile + (SM_GROUPS * TCH + t) * 64 + lane;
-        *slot = w == 0 ? rs[t] : *slot + rs[t];
-      }
-    }
-    __syncthreads();
-  }
-
-  v4f v[TCH], xs[TCH];
-#pragma unroll
-  for (int j = 0; j < TCH; ++j) {
-    const int f = j * ST_WAVES + wave;
-    v[j] = tile[f * 64 + lane];
-    xs[j] = tile[(SM_GROUPS * TCH + f % TCH) * 64 + lane];
-  }
-
-  // ---- epilogue: out = s * (sum_k x (w + 128) + (o - 128) sum_k x) ---------------------------------------------
-  unsigned short(*tile_out)[SM_COLS + 8] = reinterpret_cast<unsigned short(*)[SM_COLS + 8]>(st_smem);
-  __syncthreads();   // every thread holds its part of the float32 tile: the LDS tile can be reused
-#pragma unroll
-  for (int j = 0; j < TCH; ++j) {
-    const int f = j * ST_WAVES + wave, cg = f / TCH, t = f % TCH;
-    const int cl = 16 * cg + c16, n = n0 + cl;
+  for (int cg = 0; cg < G; ++cg) {
+    const int n = 16 * (cg0 + cg) + c16, cl = 16 * (wave * G + cg) + c16;
     if (cg < cg_count && n < p.n) {
       const bool upper = ((long long)grp * p.n + n) & 1;   // which half of its word the element is
-      const float sc = p.aq_scale ? sa_half_like<BF16>((unsigned short)(upper ? sc_word[j] >> 16 : sc_word[j])) : 1.0f;
-      const float of = p.aq_offset ? sa_half_like<BF16>((unsigned short)(upper ? of_word[j] >> 16 : of_word[j])) : 0.0f;
+      const float sc = p.aq_scale ? sa_half_like<BF16>((unsigned short)(upper ? sc_word[cg] >> 16 : sc_word[cg])) : 1.0f;
+      const float of = p.aq_offset ? sa_half_like<BF16>((unsigned short)(upper ? of_word[cg] >> 16 : of_word[cg])) : 0.0f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int row = 16 * t + 4 * h + r;
-        if (row < chunk_rows) tile_out[row][cl] = half_out(p, fmaf(of - 128.0f, xs[j][r], v[j][r]) * sc);
-      }
+      for (int t = 0; t < TCH; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = 16 * t + 4 * h + r;
+          if (row < chunk_rows) tile_out[row][cl] = half_out(p, fmaf(of - 128.0f, rs[t][r], acc[cg][t][r]) * sc);
+        }
     }
   }
   __syncthreads();
-  // whole-row stores: 16 TCH rows x 8 pieces of 8 columns
-  for (int item = tid; item < S::kRows * 8; item += ST_THREADS) {
-    const int row = item >> 3, c8 = (item & 7) * 8;
+  // whole-row stores: 16 TCH rows x pieces of 8 columns
+  constexpr int ROW_PIECES = S::kCols / 8;
+  for (int item = tid; item < S::kRows * ROW_PIECES; item += ST_THREADS) {
+    const int row = item / ROW_PIECES, c8 = (item % ROW_PIECES) * 8;
     const int n = n0 + c8;
-    if (row < chunk_rows && c8 < 16 * cg_count && n < p.n) {
+    if (row < chunk_rows && n < p.n) {   // N % 16 == 0: 8 columns all inside or all outside
       const uint4 q = *reinterpret_cast<const uint4 *>(&tile_out[row][c8]);
       *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned short *>(p.out) + (long long)(m0 + row) * p.n + n) = q;
     }
   }
 }
 
-template <bool BF16, int TCH>
-static hipError_t streamm_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
-  hipLaunchKernelGGL((gmm_a16w8_streamm_kernel<BF16, TCH>), grid, dim3(ST_THREADS), SamShape<TCH>::kLds, stream, p);
+template <bool BF16, int TCH, int G>
+static hipError_t rows_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
+  using S = SamShape<TCH, G>;
+  hipLaunchKernelGGL((gmm_a16w8_rows_kernel<BF16, TCH, G>), grid, dim3(ST_THREADS), S::kLds, stream, p);
   return hipGetLastError();
 }
 
-// tch = 16-row fragments per chunk (2 or 4); p.max_chunks counts chunks of 16 tch rows, p.n_strips strips of 64 columns
+// tch = 16-row fragments per chunk (2, 4 or 8); p.max_chunks counts chunks of 16 tch rows; p.strip_groups = column groups
+// per strip (8 or 16: two or four per wave; 8 for tch = 8), p.n_strips strips
 hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
-  if (p.split_k != 1) return hipErrorInvalidValue;
+  if (p.split_k != 1 || (p.strip_groups != 8 && p.strip_groups != 16) || (tch != 2 && tch != 4 && tch != 8) ||
+      (tch == 8 && p.strip_groups != 8))
+    return hipErrorInvalidValue;
   const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), 1u);
   const bool bf = p.x_dtype == DT_BF16;
-  if (tch == 4) return bf ? streamm_launch_a16w8<true, 4>(p, grid, stream) : streamm_launch_a16w8<false, 4>(p, grid, stream);
-  if (tch == 2) return bf ? streamm_launch_a16w8<true, 2>(p, grid, stream) : streamm_launch_a16w8<false, 2>(p, grid, stream);
-  return hipErrorInvalidValue;
+  const bool wide = p.strip_groups == 16;
+#define MSCO_ROWS_BY(TCH)                                                                                                   \
+  (bf ? (wide ? rows_launch_a16w8<true, TCH, 4>(p, grid, stream) : rows_launch_a16w8<true, TCH, 2>(p, grid, stream))      \
+      : (wide ? rows_launch_a16w8<false, TCH, 4>(p, grid, stream) : rows_launch_a16w8<false, TCH, 2>(p, grid, stream)))
+  if (tch == 8) return bf ? rows_launch_a16w8<true, 8, 2>(p, grid, stream) : rows_launch_a16w8<false, 8, 2>(p, grid, stream);
+  return tch == 4 ? MSCO_ROWS_BY(4) : MSCO_ROWS_BY(2);
+#undef MSCO_ROWS_BY
 }
 
 }  // namespace msco

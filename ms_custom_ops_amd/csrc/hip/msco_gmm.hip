@@ -321,15 +321,14 @@ void choose_plan(msco_gmm_op *op) {
       op->stream_tch = op->stream_tch == 1 ? 2 : op->stream_tch * 2;
     if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8) op->stream_tch = tuning().stream_tch;
   } else if (family == FAM_SKINNY && is_packed(d) && is_a16w8(d)) {
-    // weight-only on packed weights: chunks of 32 or 64 rows by the same estimate (its multi-row kernel holds at most four
-    // row fragments in registers); larger groups stream their weights once per 64 rows (8 experts, K = 4096, N = 14336,
-    // 128 / 512 / 2048 rows: 111 / 334 / 1307 us with 16-row chunks)
+    // weight-only on packed weights: chunks of 32, 64 or 128 rows by the same estimate; larger groups stream their weights
+    // once per 128 rows (8 experts, K = 4096, N = 14336, 128 / 512 / 2048 rows: 111 / 334 / 1307 us with 16-row chunks)
     const int64_t avg = (m + e - 1) / e;
     const int64_t rows = e == 1 ? m : avg + avg / 2;
-    op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : 4;
-    while (op->stream_tch < 4 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
+    op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
+    while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch *= 2;
-    if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4) op->stream_tch = tuning().stream_tch;
+    if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8) op->stream_tch = tuning().stream_tch;
   }
   if (family == FAM_SKINNY) {
     // grid.y enumerates (group, chunk of 16 * stream_tch rows)
@@ -348,7 +347,15 @@ void choose_plan(msco_gmm_op *op) {
     if (forced_variant >= 0 && is_w8a8(d)) wide16 = forced_variant != 0;
     op->skinny_wide16 = wide16;
     int want, cap;
-    if (is_packed(d) && op->stream_tch > 1) {
+    if (is_packed(d) && op->stream_tch > 1 && !is_w8a8(d)) {
+      // multi-row weight-only kernel: strips of 16 column groups (four per wave) when they still give every CU two
+      // workgroups, else of 8; every workgroup walks all of K
+      const int64_t col_groups = (n + 15) / 16;
+      op->strip_groups = (op->stream_tch < 8 && ((col_groups + 15) / 16) * active >= 2 * (int64_t)num_cus) ? 16 : 8;   // (128-row chunks: two column groups per wave, for registers)
+      op->n_strips = (int)((col_groups + op->strip_groups - 1) / op->strip_groups);
+      op->skinny_cols = op->strip_groups * 16;
+      want = cap = 1;
+    } else if (is_packed(d) && op->stream_tch > 1) {
       // multi-row kernel: strips of four column groups, K split until about two workgroups per CU stream operands
       const int64_t col_groups = (n + 15) / 16, k_blocks = (k + 63) / 64;
       op->strip_groups = 4;
