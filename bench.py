@@ -507,10 +507,12 @@ def main():
                              ("c5", "packed"), ("c3_decode", "kn"), ("c3_decode", "packed"),
                              # the headline MoE layer at serving batch sizes (T tokens, top-2 of 8): bound by the 470 MB of weights
                              ("c3_t64", "packed"), ("c3_t128", "packed"), ("c3_t256", "packed"), ("c3_t512", "packed"),
-                             ("c3_t1024", "packed")]:
+                             ("c3_t1024", "packed"),
+                             # the weight-only layer beyond decode: chunks of 32 .. 128 rows share a pass over the weights
+                             ("c5_t64", "packed"), ("c5_t256", "packed")]:
             w2 = workloads.make(name)
             w_bytes = w2.w.nbytes
-            hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5", "c3_decode") or name.startswith("c3_t")
+            hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5", "c3_decode") or name.startswith(("c3_t", "c5_t"))
             copies = max(1, int(np.ceil(ROTATE_BYTES / w_bytes))) if hbm_bound_guess else 1
             p2 = DeviceProblem(w2, layout, copies)
             _, sec, _ = p2.time(max(20, min(200, args.steps)), args.warmup)
