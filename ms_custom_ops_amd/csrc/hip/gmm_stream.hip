@@ -882,7 +882,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
                                                 2ll * chunk_rows * p.k);
 
   // the slab pieces this thread carries: piece i = tid + 256 u is row i / 8 (clamped into the chunk: rows past it are
-  // computed and never stored), 16-byte chunk i % 8 of the block's 128 bytes
+  // computed at most and never stored), 16-byte chunk i % 8 of the block's 128 bytes
   unsigned x_src[S::kPieces], x_dst[S::kPieces];
 #pragma unroll
   for (int u = 0; u < S::kPieces; ++u) {
@@ -920,10 +920,12 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
   const v4i ones_frag = v4i{(int)ones, (int)ones, (int)ones, (int)ones};
   // x fragments as in the 16-row kernel: lane (c, q), step s holds the 8 values x[16 t + c][64 b + 16 q + 8 s ..], i.e.
   // chunk 2 q + s of row 16 t + c.  (A block that was not loaded reads as w + 128 = 128: its x is zeros, it adds nothing.)
-  auto multiply = [&](int stage, const v4i (&wv)[G]) {
-    v4i xf[TCH][2];
+  // LIVE = row fragments that hold rows of the chunk (a compile-time count: the others are neither read nor multiplied)
+  auto multiply = [&](auto live_c, int stage, const v4i (&wv)[G]) {
+    constexpr int LIVE = decltype(live_c)::value;
+    v4i xf[LIVE][2];
 #pragma unroll
-    for (int t = 0; t < TCH; ++t)
+    for (int t = 0; t < LIVE; ++t)
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
         xf[t][s2] = *reinterpret_cast<const v4i *>(st_smem + stage * S::kStage + (16 * t + c16) * S::kPitch + (2 * h + s2) * 16);
@@ -933,13 +935,13 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
       const unsigned d2 = (unsigned)wv[cg][2] ^ 0x80808080u, d3 = (unsigned)wv[cg][3] ^ 0x80808080u;
       const v4i w0 = sa_frag<BF16>(d0, d1), w1 = sa_frag<BF16>(d2, d3);
 #pragma unroll
-      for (int t = 0; t < TCH; ++t) {
+      for (int t = 0; t < LIVE; ++t) {
         acc[cg][t] = sa_mfma<BF16>(xf[t][0], w0, acc[cg][t]);
         acc[cg][t] = sa_mfma<BF16>(xf[t][1], w1, acc[cg][t]);
       }
     }
 #pragma unroll
-    for (int t = 0; t < TCH; ++t) {
+    for (int t = 0; t < LIVE; ++t) {
       rs[t] = sa_mfma<BF16>(xf[t][0], ones_frag, rs[t]);
       rs[t] = sa_mfma<BF16>(xf[t][1], ones_frag, rs[t]);
     }
@@ -971,17 +973,42 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
   slab_barrier();
   // One barrier per K block: the slab of block kb + 1 is written to the other stage (which every wave finished reading
   // before the last barrier) while block kb is multiplied, and the requests run two blocks ahead.
-  for (int kb = 0; kb < k_blocks; kb += 2) {
-    load_w(kb + 1, wb);
-    multiply(0, wa);
-    store_x(1, xr);
-    load_x(kb + 2, xr);
-    slab_barrier();
-    load_w(kb + 2, wa);
-    multiply(1, wb);   // (past K: zeros times 128)
-    store_x(0, xr);
-    load_x(kb + 3, xr);
-    slab_barrier();
+  auto k_loop = [&](auto live_c) {
+    for (int kb = 0; kb < k_blocks; kb += 2) {
+      load_w(kb + 1, wb);
+      multiply(live_c, 0, wa);
+      store_x(1, xr);
+      load_x(kb + 2, xr);
+      slab_barrier();
+      load_w(kb + 2, wa);
+      multiply(live_c, 1, wb);   // (past K: zeros times 128)
+      store_x(0, xr);
+      load_x(kb + 3, xr);
+      slab_barrier();
+    }
+  };
+  // one copy of the loop per number of row fragments that hold rows (the last chunk of a group is rarely full, and on
+  // 128-row chunks the matrix pipe is what bounds this kernel)
+  // (32-row chunks keep one loop: two copies measured slower there, 87 against 80 us at 64 tokens)
+  const int live = (chunk_rows + 15) / 16;   // 1 .. TCH, the same for the whole workgroup
+  if constexpr (TCH <= 2) {
+    const std::integral_constant<int, TCH> all;
+    for (int kb = 0; kb < k_blocks; kb += 2) {
+      load_w(kb + 1, wb);
+      multiply(all, 0, wa);
+      store_x(1, xr);
+      load_x(kb + 2, xr);
+      slab_barrier();
+      load_w(kb + 2, wa);
+      multiply(all, 1, wb);
+      store_x(0, xr);
+      load_x(kb + 3, xr);
+      slab_barrier();
+    }
+  } else {
+    static_for<TCH>([&](auto i_c) {
+      if (live == decltype(i_c)::value + 1) k_loop(std::integral_constant<int, decltype(i_c)::value + 1>{});
+    });
   }
 
   // ---- epilogue: out = s * (sum_k x (w + 128) + (o - 128) sum_k x); lane (c, h) holds rows 16 t + 4 h + r of column
