@@ -973,43 +973,32 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
   slab_barrier();
   // One barrier per K block: the slab of block kb + 1 is written to the other stage (which every wave finished reading
   // before the last barrier) while block kb is multiplied, and the requests run two blocks ahead.
-  auto k_loop = [&](auto live_c) {
-    for (int kb = 0; kb < k_blocks; kb += 2) {
-      load_w(kb + 1, wb);
-      multiply(live_c, 0, wa);
-      store_x(1, xr);
-      load_x(kb + 2, xr);
-      slab_barrier();
-      load_w(kb + 2, wa);
-      multiply(live_c, 1, wb);   // (past K: zeros times 128)
-      store_x(0, xr);
-      load_x(kb + 3, xr);
-      slab_barrier();
-    }
-  };
-  // one copy of the loop per number of row fragments that hold rows (the last chunk of a group is rarely full, and on
-  // 128-row chunks the matrix pipe is what bounds this kernel)
-  // (32-row chunks keep one loop: two copies measured slower there, 87 against 80 us at 64 tokens)
-  const int live = (chunk_rows + 15) / 16;   // 1 .. TCH, the same for the whole workgroup
-  if constexpr (TCH <= 2) {
-    const std::integral_constant<int, TCH> all;
-    for (int kb = 0; kb < k_blocks; kb += 2) {
-      load_w(kb + 1, wb);
-      multiply(all, 0, wa);
-      store_x(1, xr);
-      load_x(kb + 2, xr);
-      slab_barrier();
-      load_w(kb + 2, wa);
-      multiply(all, 1, wb);
-      store_x(0, xr);
-      load_x(kb + 3, xr);
-      slab_barrier();
-    }
-  } else {
-    static_for<TCH>([&](auto i_c) {
-      if (live == decltype(i_c)::value + 1) k_loop(std::integral_constant<int, decltype(i_c)::value + 1>{});
-    });
+  // One copy of the loop per number of row fragments that hold rows (the last chunk of a group is rarely full, and on
+  // 64- and 128-row chunks the matrix pipe is what bounds this kernel); 32-row chunks keep one loop (two copies measured
+  // slower there, 87 against 80 us at 64 tokens).  Written out rather than wrapped in a lambda: called through one, the
+  // same loop came out of the scheduler 8 % slower.
+  const int live = (TCH <= 2) ? TCH : (chunk_rows + 15) / 16;   // 1 .. TCH, the same for the whole workgroup
+#define MSCO_ROWS_LOOP(LIVE)                                               \
+  if constexpr (LIVE <= TCH) {                                             \
+    if (live == LIVE) {                                                    \
+      const std::integral_constant<int, (LIVE <= TCH ? LIVE : 1)> live_c;  \
+      for (int kb = 0; kb < k_blocks; kb += 2) {                           \
+        load_w(kb + 1, wb);                                                \
+        multiply(live_c, 0, wa);                                           \
+        store_x(1, xr);                                                    \
+        load_x(kb + 2, xr);                                                \
+        slab_barrier();                                                    \
+        load_w(kb + 2, wa);                                                \
+        multiply(live_c, 1, wb); /* (past K: zeros times 128) */           \
+        store_x(0, xr);                                                    \
+        load_x(kb + 3, xr);                                                \
+        slab_barrier();                                                    \
+      }                                                                    \
+    }                                                                      \
   }
+  MSCO_ROWS_LOOP(1) MSCO_ROWS_LOOP(2) MSCO_ROWS_LOOP(3) MSCO_ROWS_LOOP(4)
+  MSCO_ROWS_LOOP(5) MSCO_ROWS_LOOP(6) MSCO_ROWS_LOOP(7) MSCO_ROWS_LOOP(8)
+#undef MSCO_ROWS_LOOP
 
   // ---- epilogue: out = s * (sum_k x (w + 128) + (o - 128) sum_k x); lane (c, h) holds rows 16 t + 4 h + r of column
   // 16 cg + c of its wave's column groups.  The output tile is staged in LDS (the slabs are done with) for whole-row stores.
