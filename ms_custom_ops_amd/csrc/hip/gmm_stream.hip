@@ -840,23 +840,35 @@ hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream) {
 // for the row sums that fold the offset into the epilogue).  A group's weights are streamed once per 16 TCH rows
 // instead of once per 16.  LDS rows of 128 payload bytes at a 144-byte pitch: the 16 lanes of a fragment read (16
 // consecutive rows, one 16-byte chunk) fall into 16 different bank groups.
+//
+// KN: the weights are row-major [E,K,N] instead of packed.  Then the workgroup also brings the strip's weight slab (64 K
+// rows x 64 G column bytes, whole lines) into LDS as it lies in memory, and a wave gets the operand of a 16 x 16 x 32
+// MFMA with one LDS transpose read (ds_read_b64_tr_b8: of a block of 16 lanes, lane i names 8 bytes M[i][0..7] and lane j
+// receives byte b = M[2 b + j / 8][j % 8]; with lanes 2 b and 2 b + 1 on the two halves of the 16 column bytes of K row
+// b, lane j of block q holds K rows 8 q .. 8 q + 7 of column j): lane group q then multiplies K positions 32 s + 8 q ..
+// of step s, and reads x chunk 4 s + q instead of 2 q + s.  Weight rows sit at a pitch of 64 G + 16 bytes (the 8 rows
+// of a block's read, and the two blocks of a half wave, in different bank groups).
 namespace {
-template <int TCH, int G>
+template <int TCH, int G, bool KN = false>
 struct SamShape {
   static constexpr int kRows = 16 * TCH;
   static constexpr int kCols = 64 * G;                         // 4 waves x G column groups x 16
   static constexpr int kPitch = 144;                           // bytes of an x row in LDS (64 K x 2 bytes + 16)
   static constexpr int kStage = kRows * kPitch;                // one K block of the chunk's x
   static constexpr int kPieces = kRows * 8 / ST_THREADS;       // 16-byte pieces of a slab per thread
+  static constexpr int kWPitch = kCols + 16;                   // [E,K,N]: bytes of a weight K row in LDS
+  static constexpr int kWStage = KN ? 64 * kWPitch : 0;        // [E,K,N]: one K block of the strip's weights
+  static constexpr int kWPieces = 64 * kCols / 16 / ST_THREADS;   // its 16-byte pieces per thread (= G)
+  static constexpr int kSlabs = 2 * (kStage + kWStage);        // two stages of operands
   static constexpr size_t kOut = (size_t)kRows * (kCols + 8) * 2;   // 16-bit output tile of the epilogue
-  static constexpr size_t kLds = 2 * kStage > kOut ? 2 * kStage : kOut;
-  static_assert(kPieces >= 1, "slab pieces per thread");
+  static constexpr size_t kLds = kSlabs > kOut ? kSlabs : kOut;
+  static_assert(kPieces >= 1 && kWPieces == G, "slab pieces per thread");
 };
 }  // namespace
 
-template <bool BF16, int TCH, int G>
+template <bool BF16, int TCH, int G, bool KN = false>
 __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const GmmParams p) {
-  using S = SamShape<TCH, G>;
+  using S = SamShape<TCH, G, KN>;
   extern __shared__ __align__(16) unsigned char st_smem[];
 
   const int tid = threadIdx.x;
@@ -875,11 +887,16 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
   const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
   const int cg0 = strip * 4 * G + wave * G;                          // this wave's first column group
   const int cg_count = max(0, min(G, col_groups - cg0));
-  const long long group_bytes = (long long)col_groups * k_blocks * 1024;
-  const __amdgpu_buffer_rsrc_t rw = buffer_over(p.w + (long long)grp * group_bytes, group_bytes);
+  const long long group_bytes = KN ? (long long)p.k * p.n : (long long)col_groups * k_blocks * 1024;
+  // ([E,K,N]: the window starts at the strip's first column and ends with the expert's matrix; every offset goes into
+  // the range-checked per-lane part, so K rows past K read as zeros, and a chunk past N reads bytes of the next K row
+  // into columns that are never stored)
+  const __amdgpu_buffer_rsrc_t rw = KN ? buffer_over(p.w + (long long)grp * group_bytes + n0, group_bytes - n0)
+                                       : buffer_over(p.w + (long long)grp * group_bytes, group_bytes);
   // (a window over the chunk's rows: 16-bit x can be twice as many bytes as a 32-bit window holds)
   const __amdgpu_buffer_rsrc_t rx = buffer_over(reinterpret_cast<const unsigned short *>(p.x) + (long long)m0 * p.k,
                                                 2ll * chunk_rows * p.k);
+  unsigned char *w_smem = st_smem + 2 * S::kStage;   // [E,K,N]: the two weight stages behind the two x stages
 
   // the slab pieces this thread carries: piece i = tid + 256 u is row i / 8 (clamped into the chunk: rows past it are
   // computed at most and never stored), 16-byte chunk i % 8 of the block's 128 bytes
@@ -902,11 +919,30 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
 #pragma unroll
     for (int u = 0; u < S::kPieces; ++u) *reinterpret_cast<v4i *>(st_smem + stage * S::kStage + x_dst[u]) = xr[u];
   };
+  // packed: this wave's G blocks of K block kb, straight into the registers they are multiplied from.  [E,K,N]: this
+  // thread's G pieces of the strip's slab (piece i = tid + 256 u: K row i / (4 G), 16-byte chunk i % (4 G)), on their way to LDS
   auto load_w = [&](int kb, v4i (&wv)[G]) {
 #pragma unroll
-    for (int cg = 0; cg < G; ++cg)
-      wv[cg] = __builtin_amdgcn_raw_buffer_load_b128(rw, (kb < k_blocks && cg < cg_count) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
-                                                     (cg0 + cg) * k_blocks * 1024, kStreamAux);
+    for (int cg = 0; cg < G; ++cg) {
+      if constexpr (KN) {
+        const int i = tid + ST_THREADS * cg, row = i / (4 * G), chunk = i % (4 * G);
+        const bool ok = kb < k_blocks && n0 + 16 * chunk < p.n;
+        wv[cg] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? (unsigned)(kb * 64 + row) * (unsigned)p.n + 16u * (unsigned)chunk : kBufferOob,
+                                                       0, kStreamAux);
+      } else {
+        wv[cg] = __builtin_amdgcn_raw_buffer_load_b128(rw, (kb < k_blocks && cg < cg_count) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
+                                                       (cg0 + cg) * k_blocks * 1024, kStreamAux);
+      }
+    }
+  };
+  auto store_w = [&](int stage, const v4i (&wv)[G]) {
+    if constexpr (KN) {
+#pragma unroll
+      for (int u = 0; u < G; ++u) {
+        const int i = tid + ST_THREADS * u, row = i / (4 * G), chunk = i % (4 * G);
+        *reinterpret_cast<v4i *>(w_smem + stage * S::kWStage + row * S::kWPitch + chunk * 16) = wv[u];
+      }
+    }
   };
 
   v4f acc[G][TCH], rs[TCH];
@@ -928,11 +964,22 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
     for (int t = 0; t < LIVE; ++t)
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2)
-        xf[t][s2] = *reinterpret_cast<const v4i *>(st_smem + stage * S::kStage + (16 * t + c16) * S::kPitch + (2 * h + s2) * 16);
+        xf[t][s2] = *reinterpret_cast<const v4i *>(st_smem + stage * S::kStage + (16 * t + c16) * S::kPitch + (KN ? 4 * s2 + h : 2 * h + s2) * 16);
 #pragma unroll
     for (int cg = 0; cg < G; ++cg) {
-      const unsigned d0 = (unsigned)wv[cg][0] ^ 0x80808080u, d1 = (unsigned)wv[cg][1] ^ 0x80808080u;   // w + 128 as unsigned bytes
-      const unsigned d2 = (unsigned)wv[cg][2] ^ 0x80808080u, d3 = (unsigned)wv[cg][3] ^ 0x80808080u;
+      unsigned d0, d1, d2, d3;   // w + 128 as unsigned bytes: the lane's 8 K positions of step 0, then of step 1
+      if constexpr (KN) {
+        typedef int v2i_t __attribute__((ext_vector_type(2)));
+        typedef __attribute__((address_space(3))) v2i_t *lds_v2i;
+        const unsigned char *src = w_smem + stage * S::kWStage + (8 * h + (c16 >> 1)) * S::kWPitch + 16 * (wave * G + cg) + (c16 & 1) * 8;
+        const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(src));
+        const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(src + 32 * S::kWPitch));
+        d0 = (unsigned)lo.x ^ 0x80808080u; d1 = (unsigned)lo.y ^ 0x80808080u;
+        d2 = (unsigned)hi.x ^ 0x80808080u; d3 = (unsigned)hi.y ^ 0x80808080u;
+      } else {
+        d0 = (unsigned)wv[cg][0] ^ 0x80808080u; d1 = (unsigned)wv[cg][1] ^ 0x80808080u;
+        d2 = (unsigned)wv[cg][2] ^ 0x80808080u; d3 = (unsigned)wv[cg][3] ^ 0x80808080u;
+      }
       const v4i w0 = sa_frag<BF16>(d0, d1), w1 = sa_frag<BF16>(d2, d3);
 #pragma unroll
       for (int t = 0; t < LIVE; ++t) {
@@ -970,6 +1017,10 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
   auto slab_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
   store_x(0, xr);
   load_x(1, xr);
+  if constexpr (KN) {   // (the weights take the same road as x: registers -> LDS, one block ahead of the multiply)
+    store_w(0, wa);
+    load_w(1, wa);
+  }
   slab_barrier();
   // One barrier per K block: the slab of block kb + 1 is written to the other stage (which every wave finished reading
   // before the last barrier) while block kb is multiplied, and the requests run two blocks ahead.
@@ -983,15 +1034,17 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
     if (live == LIVE) {                                                    \
       const std::integral_constant<int, (LIVE <= TCH ? LIVE : 1)> live_c;  \
       for (int kb = 0; kb < k_blocks; kb += 2) {                           \
-        load_w(kb + 1, wb);                                                \
+        if constexpr (!KN) load_w(kb + 1, wb);                             \
         multiply(live_c, 0, wa);                                           \
         store_x(1, xr);                                                    \
         load_x(kb + 2, xr);                                                \
+        if constexpr (KN) { store_w(1, wa); load_w(kb + 2, wa); }          \
         slab_barrier();                                                    \
-        load_w(kb + 2, wa);                                                \
-        multiply(live_c, 1, wb); /* (past K: zeros times 128) */           \
+        if constexpr (!KN) load_w(kb + 2, wa);                             \
+        multiply(live_c, 1, KN ? wa : wb); /* (past K: zeros times 128) */ \
         store_x(0, xr);                                                    \
         load_x(kb + 3, xr);                                                \
+        if constexpr (KN) { store_w(0, wa); load_w(kb + 3, wa); }          \
         slab_barrier();                                                    \
       }                                                                    \
     }                                                                      \
@@ -1032,17 +1085,27 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
   }
 }
 
-template <bool BF16, int TCH, int G>
+template <bool BF16, int TCH, int G, bool KN = false>
 static hipError_t rows_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
-  using S = SamShape<TCH, G>;
-  hipLaunchKernelGGL((gmm_a16w8_rows_kernel<BF16, TCH, G>), grid, dim3(ST_THREADS), S::kLds, stream, p);
+  using S = SamShape<TCH, G, KN>;
+  auto kern = gmm_a16w8_rows_kernel<BF16, TCH, G, KN>;
+  if constexpr (S::kLds > 64 * 1024) {
+    static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
+    if (!attr_set) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::kLds);
+      if (e != hipSuccess) return e;
+      attr_set = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(ST_THREADS), S::kLds, stream, p);
   return hipGetLastError();
 }
 
 // tch = 16-row fragments per chunk (2, 4 or 8); p.max_chunks counts chunks of 16 tch rows; p.strip_groups = column groups
 // per strip (8 or 16: two or four per wave; 8 for tch = 8), p.n_strips strips
-hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, hipStream_t stream) {
+hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, bool packed, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
+  if (!packed && p.n % 16 != 0) return hipErrorInvalidValue;   // [E,K,N] rows of whole 16-column chunks
   if (p.split_k != 1 || (p.strip_groups != 8 && p.strip_groups != 16) || (tch != 2 && tch != 4 && tch != 8) ||
       (tch == 8 && p.strip_groups != 8))
     return hipErrorInvalidValue;
@@ -1052,6 +1115,12 @@ hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, hipStream_t stream)
 #define MSCO_ROWS_BY(TCH)                                                                                                   \
   (bf ? (wide ? rows_launch_a16w8<true, TCH, 4>(p, grid, stream) : rows_launch_a16w8<true, TCH, 2>(p, grid, stream))      \
       : (wide ? rows_launch_a16w8<false, TCH, 4>(p, grid, stream) : rows_launch_a16w8<false, TCH, 2>(p, grid, stream)))
+  if (!packed) {   // (registers: 64-row chunks with two column groups per wave only, no 128-row chunks)
+    if (tch == 4 && !wide) return bf ? rows_launch_a16w8<true, 4, 2, true>(p, grid, stream) : rows_launch_a16w8<false, 4, 2, true>(p, grid, stream);
+    if (tch == 2 && wide) return bf ? rows_launch_a16w8<true, 2, 4, true>(p, grid, stream) : rows_launch_a16w8<false, 2, 4, true>(p, grid, stream);
+    if (tch == 2) return bf ? rows_launch_a16w8<true, 2, 2, true>(p, grid, stream) : rows_launch_a16w8<false, 2, 2, true>(p, grid, stream);
+    return hipErrorInvalidValue;
+  }
   if (tch == 8) return bf ? rows_launch_a16w8<true, 8, 2>(p, grid, stream) : rows_launch_a16w8<false, 8, 2>(p, grid, stream);
   return tch == 4 ? MSCO_ROWS_BY(4) : MSCO_ROWS_BY(2);
 #undef MSCO_ROWS_BY

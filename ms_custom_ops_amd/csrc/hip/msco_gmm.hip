@@ -320,15 +320,18 @@ void choose_plan(msco_gmm_op *op) {
     while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch = op->stream_tch == 1 ? 2 : op->stream_tch * 2;
     if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8) op->stream_tch = tuning().stream_tch;
-  } else if (family == FAM_SKINNY && is_packed(d) && is_a16w8(d)) {
-    // weight-only on packed weights: chunks of 32, 64 or 128 rows by the same estimate; larger groups stream their weights
-    // once per 128 rows (8 experts, K = 4096, N = 14336, 128 / 512 / 2048 rows: 111 / 334 / 1307 us with 16-row chunks)
+  } else if (family == FAM_SKINNY && is_a16w8(d) && (is_packed(d) || (d.transpose_b == 0 && n % 16 == 0))) {
+    // weight-only on packed or [E,K,N] weights: chunks of 32, 64 or 128 rows by the same estimate (64 at most on [E,K,N],
+    // whose weight slab shares the registers); larger groups stream their weights once per chunk (8 experts, K = 4096,
+    // N = 14336, 128 / 512 / 2048 rows: 111 / 334 / 1307 us with 16-row chunks)
+    const int tch_max = is_packed(d) ? 8 : 4;
     const int64_t avg = (m + e - 1) / e;
     const int64_t rows = e == 1 ? m : avg + avg / 2;
-    op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
-    while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
+    op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : (rows <= 64 || tch_max == 4) ? 4 : 8;
+    while (op->stream_tch < tch_max && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch *= 2;
-    if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8) op->stream_tch = tuning().stream_tch;
+    if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || (tuning().stream_tch == 8 && tch_max == 8))
+      op->stream_tch = tuning().stream_tch;
   }
   if (family == FAM_SKINNY) {
     // grid.y enumerates (group, chunk of 16 * stream_tch rows)
@@ -347,11 +350,13 @@ void choose_plan(msco_gmm_op *op) {
     if (forced_variant >= 0 && is_w8a8(d)) wide16 = forced_variant != 0;
     op->skinny_wide16 = wide16;
     int want, cap;
-    if (is_packed(d) && op->stream_tch > 1 && !is_w8a8(d)) {
+    if (op->stream_tch > 1 && !is_w8a8(d)) {
       // multi-row weight-only kernel: strips of 16 column groups (four per wave) when they still give every CU two
-      // workgroups, else of 8; every workgroup walks all of K
+      // workgroups, else of 8; every workgroup walks all of K.  (For registers: 128-row chunks, and 64-row chunks on
+      // [E,K,N] weights, with two column groups per wave.)
       const int64_t col_groups = (n + 15) / 16;
-      op->strip_groups = (op->stream_tch < 8 && ((col_groups + 15) / 16) * active >= 2 * (int64_t)num_cus) ? 16 : 8;   // (128-row chunks: two column groups per wave, for registers)
+      const bool narrow = op->stream_tch == 8 || (!is_packed(d) && op->stream_tch == 4);
+      op->strip_groups = (!narrow && ((col_groups + 15) / 16) * active >= 2 * (int64_t)num_cus) ? 16 : 8;
       op->n_strips = (int)((col_groups + op->strip_groups - 1) / op->strip_groups);
       op->skinny_cols = op->strip_groups * 16;
       want = cap = 1;
@@ -404,9 +409,9 @@ void choose_plan(msco_gmm_op *op) {
       const int slice_blocks = is_w8a8(d) ? 128 : 64;
       want = std::max(want, (int)(((k + 63) / 64 + slice_blocks - 1) / slice_blocks));
     }
-    if (is_packed(d) && op->stream_tch > 1 && !is_w8a8(d)) want = 1;   // the multi-row weight-only kernel walks all of K
+    if (op->stream_tch > 1 && !is_w8a8(d)) want = 1;   // the multi-row weight-only kernel walks all of K
     op->split_k = want;
-    if (!is_packed(d)) op->skinny_cols = wide16 ? 128 : kSkinnyCols;
+    if (!is_packed(d) && !(op->stream_tch > 1 && !is_w8a8(d))) op->skinny_cols = wide16 ? 128 : kSkinnyCols;
     if (is_packed(d)) {
       // the packed-layout kernels keep a full 16 x 256 partial tile per (strip, K slice) whatever the strip's width
       const size_t tile_bytes = !is_w8a8(d)           ? stream_a16w8_tile_bytes()
@@ -415,6 +420,8 @@ void choose_plan(msco_gmm_op *op) {
       const size_t tiles = op->stream_tch > 1 ? (size_t)e * op->max_chunks * op->n_strips
                                               : skinny_counter_count(m, n, e, op->skinny_cols);
       op->workspace_bytes = op->split_k > 1 ? tiles * (size_t)op->split_k * tile_bytes : 0;
+    } else if (op->stream_tch > 1 && !is_w8a8(d)) {
+      op->workspace_bytes = 0;   // (the multi-row weight-only kernel has no K split)
     } else {
       op->workspace_bytes = is_w8a8(d) ? skinny_workspace_bytes(m, n, e, op->split_k, op->skinny_cols)
                                        : a16w8_workspace_bytes(m, n, e, op->split_k);
@@ -427,7 +434,8 @@ void choose_plan(msco_gmm_op *op) {
   std::snprintf(buf, sizeof(buf),
                 "msco_gmm plan: kernel=%s%s%s%s layout=%s m=%lld k=%lld n=%lld e=%lld split_k=%d strips=%d "
                 "workspace=%zu%s",
-                is_w8a8(d) ? "w8a8_" : "a16w8_", (family == FAM_SKINNY && is_packed(d)) ? (op->stream_tch > 1 ? "stream_rows" : "stream") : fam,
+                is_w8a8(d) ? "w8a8_" : "a16w8_", (family == FAM_SKINNY && is_packed(d)) ? (op->stream_tch > 1 ? "stream_rows" : "stream")
+                : (family == FAM_SKINNY && op->stream_tch > 1)    ? "skinny_rows" : fam,
                 family == FAM_TILE ? (std::string("_") + tile_cfg_name(op->tile_cfg)).c_str() : "",
                 (family == FAM_SKINNY && op->skinny_wide16) ? "_16w" : "",
                 is_packed(d) ? "packed" : d.transpose_b ? "[E,N,K]" : "[E,K,N]", (long long)m, (long long)k, (long long)n, (long long)e,
@@ -591,7 +599,8 @@ int msco_gmm_launch(msco_gmm_handle h, const void *const *inputs, void *out, voi
     else if (h->family == FAM_SKINNY) err = launch_skinny_w8a8(p, nk, h->skinny_wide16 != 0, s);
     else err = launch_generic_w8a8(p, layout, s);
   } else {
-    if (h->family == FAM_SKINNY && layout == 2) err = h->stream_tch > 1 ? launch_streamm_a16w8(p, h->stream_tch, s) : launch_stream_a16w8(p, s);
+    if (h->family == FAM_SKINNY && h->stream_tch > 1) err = launch_streamm_a16w8(p, h->stream_tch, layout == 2, s);
+    else if (h->family == FAM_SKINNY && layout == 2) err = launch_stream_a16w8(p, s);
     else if (h->family == FAM_SKINNY) err = launch_skinny_a16w8(p, s);
     else err = launch_generic_a16w8(p, layout, s);
   }

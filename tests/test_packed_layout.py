@@ -238,9 +238,32 @@ def test_weight_only_multi_row_streaming_kernel_within_tolerance(device, dtype, 
     ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
     assert (np.abs(got[:last] - exact[:last]) <= ulp * np.abs(exact[:last]) + 1e-5 * mag[:last]).all(), info
     assert (bits[last:] == 0x7FC0).all()   # rows past the last boundary keep the fill value
-    # and the same inputs through the row-major 16-row kernel agree to the same bound (two float32 summation orders)
+    # and the same inputs through the row-major kernel agree to the same bound (two float32 summation orders)
     bits_rm, _ = run_a16w8(x, w, s, o, gl, dtype=dtype)
     assert (np.abs(to_f(bits_rm).astype(np.float64)[:last] - got[:last]) <= 2 * ulp * np.abs(exact[:last]) + 2e-5 * mag[:last]).all()
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("m,k,n,e,gl", [
+    (150, 1024 + 64, 272, 3, [70, 70, 150]),                # chunks of 64 rows: 64 + 6 rows, an empty group, 64 + 16; N tail
+    (64, 2048, 128, 1, [64]),                               # one full chunk of four row fragments
+    (33, 512 + 16, 64, 2, [20, 33]),                        # chunks of 32 rows, K not a multiple of 64
+    (300, 4096, 512, 4, [10, 100, 100, 300]),               # groups of 10, 90, 0 and 200 rows in chunks of 64
+    (160, 256, 14336, 8, [20, 40, 60, 80, 100, 120, 140, 160]),   # chunks of 32 rows, wide N: strips of 256 columns
+])
+def test_weight_only_multi_row_kernel_on_row_major_weights(device, dtype, m, k, n, e, gl):
+    """The same on [E,K,N] weights as stored: the strip's weight slab goes through LDS and transpose reads turn it into
+    MFMA operands.  Tolerance as above; the 16-row kernel of this layout (forced) agrees to the same bound."""
+    from gpu_utils import run_a16w8
+    x, w, s, o, exact, mag, to_f, last = _weight_only_case(24, m, k, n, e, gl, dtype)
+    bits, info = run_a16w8(x, w, s, o, gl, dtype=dtype)
+    assert "a16w8_skinny_rows" in info and "layout=[E,K,N]" in info and "split_k=1 " in info, info
+    got = to_f(bits).astype(np.float64)
+    ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
+    assert (np.abs(got[:last] - exact[:last]) <= ulp * np.abs(exact[:last]) + 1e-5 * mag[:last]).all(), info
+    assert (bits[last:] == 0x7FC0).all()   # rows past the last boundary keep the fill value
+    bits_p, _ = run_a16w8(x, w, s, o, gl, dtype=dtype, packed=True)   # the packed layout's kernel: another summation order
+    assert (np.abs(to_f(bits_p).astype(np.float64)[:last] - got[:last]) <= 2 * ulp * np.abs(exact[:last]) + 2e-5 * mag[:last]).all()
 
 
 def test_weight_only_generic_kernel_on_packed_weights(device):
