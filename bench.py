@@ -509,7 +509,7 @@ def main():
                              ("c3_t64", "packed"), ("c3_t128", "packed"), ("c3_t256", "packed"), ("c3_t512", "packed"),
                              ("c3_t1024", "packed"),
                              # the weight-only layer beyond decode: chunks of 32 .. 128 rows share a pass over the weights
-                             ("c5_t64", "packed"), ("c5_t256", "packed")]:
+                             ("c5_t64", "packed"), ("c5_t256", "packed"), ("c5_t256", "kn")]:
             w2 = workloads.make(name)
             w_bytes = w2.w.nbytes
             hbm_bound_guess = name in ("c1", "c2_m256", "c2_m16", "c2_m1", "c5", "c3_decode") or name.startswith(("c3_t", "c5_t"))
