@@ -266,6 +266,31 @@ def test_weight_only_multi_row_kernel_on_row_major_weights(device, dtype, m, k, 
     assert (np.abs(to_f(bits_p).astype(np.float64)[:last] - got[:last]) <= 2 * ulp * np.abs(exact[:last]) + 2e-5 * mag[:last]).all()
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_weight_only_rows_kernels_random_shapes(device, seed):
+    # a seeded sweep over the shapes of the multi-row weight-only kernels: K with odd and even block counts and 16..48-byte
+    # tails, N from one column group to several strips with tails, ragged group lists with empty groups and sizes on both
+    # sides of the 32 / 64 / 128-row chunks; packed weights and [E,K,N], both 16-bit types, against the float64 golden
+    from gpu_utils import run_a16w8
+    rng = np.random.default_rng(9000 + seed)
+    k = int(rng.integers(1, 20)) * 64 + int(rng.choice([0, 0, 16, 32, 48]))
+    n = int(rng.integers(1, 40)) * 16
+    e = int(rng.choice([1, 2, 3, 5, 8]))
+    m = int(rng.integers(17 * e, 140 * e))
+    cuts = np.sort(rng.integers(0, m + 1, e - 1)) if e > 1 else np.array([], dtype=np.int64)
+    gl = [int(v) for v in cuts] + [m - int(rng.choice([0, 0, 5]))]
+    gl = [int(v) for v in np.maximum.accumulate(gl)]
+    dtype = "bf16" if seed % 2 == 0 else "f16"
+    x, w, s, o, exact, mag, to_f, last = _weight_only_case(100 + seed, m, k, n, e, gl, dtype)
+    ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
+    for packed in (True, False):
+        bits, info = run_a16w8(x, w, s, o, gl, dtype=dtype, packed=packed)
+        assert ("a16w8_stream_rows" if packed else "a16w8_skinny_rows") in info, info
+        got = to_f(bits).astype(np.float64)
+        assert (np.abs(got[:last] - exact[:last]) <= ulp * np.abs(exact[:last]) + 1e-5 * mag[:last]).all(), info
+        assert (bits[last:] == 0x7FC0).all(), info
+
+
 def test_weight_only_generic_kernel_on_packed_weights(device):
     from gpu_utils import run_a16w8
     x, w, s, o, exact, mag, to_f, last = _weight_only_case(22, 12, 200, 48, 2, [5, 12], "bf16")
