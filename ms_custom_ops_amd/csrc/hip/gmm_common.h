@@ -270,19 +270,6 @@ __device__ __forceinline__ void transpose4x4(unsigned r0, unsigned r1, unsigned 
   c3 = perm(hi23, hi01, 0x07060302u);
 }
 
-// Transpose a 16 (rows, k) x 8 (cols, n) byte block held as 16 uint2 row pieces into 8 column
-// fragments of 16 k-bytes each (v4i = k 0..3, 4..7, 8..11, 12..15).
-__device__ __forceinline__ void transpose16x8(const uint2 (&r)[16], v4i (&frag)[8]) {
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    unsigned c0, c1, c2, c3;
-    transpose4x4(r[4 * q].x, r[4 * q + 1].x, r[4 * q + 2].x, r[4 * q + 3].x, c0, c1, c2, c3);
-    frag[0][q] = (int)c0; frag[1][q] = (int)c1; frag[2][q] = (int)c2; frag[3][q] = (int)c3;
-    transpose4x4(r[4 * q].y, r[4 * q + 1].y, r[4 * q + 2].y, r[4 * q + 3].y, c0, c1, c2, c3);
-    frag[4][q] = (int)c0; frag[5][q] = (int)c1; frag[6][q] = (int)c2; frag[7][q] = (int)c3;
-  }
-}
-
 // f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>), in order
 template <typename F, int... I>
 __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {

@@ -36,8 +36,6 @@
 
 namespace msco {
 
-constexpr int BK = 64;        // bytes of K per slab = one MFMA K step
-
 // rows of BKT bytes in LDS: 16-byte chunk c of row r sits at position c ^ swz<BKT>(r), so that the 16 lanes of a
 // fragment read (16 consecutive rows, one logical chunk) cover all 16 slots of a 256-byte LDS cycle
 template <int BKT>
@@ -54,10 +52,6 @@ __device__ __forceinline__ int swz_kt(int r) { return BN == 256 ? (r & 7) << 1 :
 __device__ __forceinline__ int col_of_q(int q) {
   const int g = q >> 3, hh = (q >> 2) & 1, t = q & 3;
   return 16 * (g >> 1) + 8 * hh + 4 * (g & 1) + t;
-}
-__device__ __forceinline__ int q_of_col(int c) {
-  const int a = c >> 4, hh = (c >> 3) & 1, b = (c >> 2) & 1, t = c & 3;
-  return 8 * (2 * a + b) + 4 * hh + t;
 }
 
 // 16 bytes per lane from a buffer straight into LDS: lane L of the wave writes lds_base + 16 L.

@@ -126,12 +126,6 @@ int check_desc(const msco_gmm_desc &d) {
   return MSCO_ERR_UNSUPPORTED;
 }
 
-int pow2_at_least(int v) {
-  int p = 1;
-  while (p < v) p <<= 1;
-  return p;
-}
-
 void choose_plan(msco_gmm_op *op) {
   const msco_gmm_desc &d = op->desc;
   const int num_cus = op->num_cus;
