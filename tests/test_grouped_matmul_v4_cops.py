@@ -81,6 +81,36 @@ def test_v4_float32_scale_output_dtype_rules(device, mode):
 
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_v4_a16w8_beyond_decode_sizes(device, mode, dtype):
+    """The a16w8 form of the reference's test (test_grouped_matmul_v4_cops.py:139-192) at serving batch sizes: 300 rows
+    over 4 experts (groups of 10, 90, 0 and 180 rows, the last boundary below M) through the operator in both modes --
+    the [E,K,N] weights take the multi-row kernel (one pass over a group's weights per 64 rows)."""
+    rng = np.random.default_rng(5)
+    m, k, n, e = 300, 512, 256, 4
+    ends = np.array([10, 100, 100, 280], dtype=np.int64)
+    x = _t(rng.uniform(-4, 4, (m, k)).astype(np.float32), dtype)
+    w = rng.integers(-127, 128, (e, k, n)).astype(np.int8)
+    s = _t(rng.uniform(0.005, 0.02, (e, n)).astype(np.float32), dtype)
+    o = _t(rng.integers(-8, 9, (e, n)).astype(np.float32), dtype)
+    with ms_custom_ops.exec_mode(mode):
+        res = ms_custom_ops.grouped_matmul_v4_cops([x], [_t(w)], None, None, None, [s], [o], None, _t(ends), None, None,
+                                                   None, 3, 0, 0)
+    assert res[0].dtype == dtype and res[0].shape == (m, n)
+    xf, sf, of = x.float().cpu().numpy(), s.float().cpu().numpy(), o.float().cpu().numpy()
+    last = int(ends[-1])
+    exact = O.a16w8_grouped_f64(xf, w, sf, of, ends)[:last]
+    mag = np.zeros_like(exact)
+    starts = np.concatenate([[0], ends[:-1]])
+    for g in range(e):
+        a, b = int(starts[g]), int(ends[g])
+        mag[a:b] = np.abs(xf[a:b].astype(np.float64)) @ (np.abs(w[g].astype(np.float64) + of[g]) * np.abs(sf[g]))
+    got = res[0][:last].float().cpu().numpy().astype(np.float64)
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    assert (np.abs(got - exact) <= ulp * np.abs(exact) + 1e-5 * mag).all()
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_v4_a16w8_last_boundary_below_m(device, mode, dtype):
     """a16w8 with scale 0.01 and offset 1, group_list [1,3,10,14,18,22,24,30] over 32 rows: only the first
     30 rows are defined (test_grouped_matmul_v4_cops.py:139-192)."""
