@@ -841,7 +841,8 @@ hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream) {
 // instead of once per 16.  LDS rows of 128 payload bytes at a 144-byte pitch: the 16 lanes of a fragment read (16
 // consecutive rows, one 16-byte chunk) fall into 16 different bank groups.
 //
-// KN: the weights are row-major [E,K,N] instead of packed.  Then the workgroup also brings the strip's weight slab (64 K
+// KN (32-row chunks only; larger chunks of this layout have the kernel below): the weights are row-major [E,K,N] instead
+// of packed.  Then the workgroup also brings the strip's weight slab (64 K
 // rows x 64 G column bytes, whole lines) into LDS as it lies in memory, and a wave gets the operand of a 16 x 16 x 32
 // MFMA with one LDS transpose read (ds_read_b64_tr_b8: of a block of 16 lanes, lane i names 8 bytes M[i][0..7] and lane j
 // receives byte b = M[2 b + j / 8][j % 8]; with lanes 2 b and 2 b + 1 on the two halves of the 16 column bytes of K row
@@ -1101,13 +1102,281 @@ static hipError_t rows_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStr
   return hipGetLastError();
 }
 
+// ---- weight-only, row-major [E,K,N] weights, 64- and 128-row chunks: 32 x 32 x 16 MFMAs ---------------------------
+// The 16 x 16 x 32 forms above run at half the rate of the 32 x 32 forms, and a 128-row chunk of them does not fit the
+// register file.  Here a workgroup owns a chunk of 32 TR rows (TR = 2, 4) and a strip of 128 GP columns; wave w owns the GP
+// blocks of 32 columns w GP .. w GP + GP - 1 and all rows, again over all of K.  Both slabs go through LDS as they lie in
+// memory.  Of a 16-K step, lane l of an x fragment holds row l % 32, K positions 8 (l / 32) .. + 7 (one 16-byte read),
+// and of a weight fragment column l % 32 at the same K positions: one transpose read, with the four blocks of 16 lanes
+// on (K half, column half) = (l / 32, l / 16 % 2).  Weight rows sit at a pitch of 128 GP + 32 bytes: the 8 rows and the
+// two column halves a pass reads fall into 16 different bank groups.
+// The row sums of x come from the vector unit instead of an MFMA against ones (which would cost a quarter of the matrix
+// time here): a thread adds up the 8 values of every slab piece it carries to LDS (always the same row), and 8 neighbouring
+// threads combine their sums at the end.
+namespace {
+typedef float v16f __attribute__((ext_vector_type(16)));
+template <int TR, int GP>
+struct Rows32Shape {
+  static constexpr int kRows = 32 * TR;
+  static constexpr int kCols = 128 * GP;                       // 4 waves x GP blocks of 32 columns
+  static constexpr int kPitch = 144;                           // bytes of an x row in LDS (64 K x 2 bytes + 16)
+  static constexpr int kStage = kRows * kPitch;                // one K block of the chunk's x
+  static constexpr int kPieces = kRows * 8 / ST_THREADS;       // 16-byte pieces of an x slab per thread
+  static constexpr int kWPitch = kCols + 32;                   // bytes of a weight K row in LDS
+  static constexpr int kWStage = 64 * kWPitch;                 // one K block of the strip's weights
+  static constexpr int kWPieces = 64 * kCols / 16 / ST_THREADS;   // its 16-byte pieces per thread (= 2 GP)
+  static constexpr int kSlabs = 2 * (kStage + kWStage);        // two stages of operands
+  static constexpr int kOut = kRows * (kCols + 8) * 2;         // 16-bit output tile of the epilogue
+  static constexpr int kTile = kSlabs > kOut ? kSlabs : kOut;
+  static constexpr size_t kLds = (size_t)kTile + kRows * 4;    // + the chunk's row sums of x
+  static_assert(kPieces >= 1 && kWPieces == 2 * GP, "slab pieces per thread");
+};
+template <bool BF16>
+__device__ __forceinline__ v16f rows32_mfma(const v4i &a, const v4i &b, const v16f &c) {
+  if constexpr (BF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+  }
+}
+// the sum of the 8 16-bit values of a slab piece, in float32, element 0 first
+template <bool BF16>
+__device__ __forceinline__ float rows32_sum8(const v4i &v) {
+  float s = 0.f;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const unsigned w = (unsigned)v[d];
+    s += sa_half_like<BF16>((unsigned short)w);
+    s += sa_half_like<BF16>((unsigned short)(w >> 16));
+  }
+  return s;
+}
+}  // namespace
+
+template <bool BF16, int TR, int GP>
+__global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const GmmParams p) {
+  using S = Rows32Shape<TR, GP>;
+  extern __shared__ __align__(16) unsigned char st_smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int c32 = lane & 31, kh = lane >> 5;
+  const int strip = blockIdx.x;
+  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
+
+  int g_start, g_end;
+  group_range(p, grp, lane, g_start, g_end);
+  const int m0 = g_start + mc * S::kRows;
+  const int chunk_rows = min(S::kRows, g_end - m0);
+  if (chunk_rows <= 0) return;
+
+  const int n0 = strip * S::kCols;
+  const int k_blocks = (p.k + 63) / 64;
+  const long long group_bytes = (long long)p.k * p.n;
+  // (windows as in the kernel above: the weights from the strip's first column to the end of the expert's matrix, K rows
+  // past K read as zeros; x over the chunk's rows)
+  const __amdgpu_buffer_rsrc_t rw = buffer_over(p.w + (long long)grp * group_bytes + n0, group_bytes - n0);
+  const __amdgpu_buffer_rsrc_t rx = buffer_over(reinterpret_cast<const unsigned short *>(p.x) + (long long)m0 * p.k,
+                                                2ll * chunk_rows * p.k);
+  unsigned char *w_smem = st_smem + 2 * S::kStage;
+
+  // x slab piece u of this thread: row tid / 8 + 32 u, 16-byte chunk tid % 8 of the block's 128 bytes (rows past the chunk
+  // lie outside the window and read as zeros)
+  const int x_chunk = tid & 7;
+  const unsigned x_src = 2u * (unsigned)(tid >> 3) * (unsigned)p.k + 16u * (unsigned)x_chunk;
+  const unsigned x_dst = (unsigned)((tid >> 3) * S::kPitch + x_chunk * 16);
+  float x_sum[S::kPieces];
+#pragma unroll
+  for (int u = 0; u < S::kPieces; ++u) x_sum[u] = 0.f;
+  auto load_x = [&](int kb, v4i (&xr)[S::kPieces]) {
+    const bool ok = kb < k_blocks && kb * 64 + 8 * x_chunk < p.k;   // K % 16 == 0: a chunk's 8 K positions are all inside or all outside
+#pragma unroll
+    for (int u = 0; u < S::kPieces; ++u)
+      xr[u] = __builtin_amdgcn_raw_buffer_load_b128(rx, ok ? x_src + (unsigned)(64 * u) * (unsigned)p.k + (unsigned)(kb * 128) : kBufferOob, 0, 0);
+  };
+  auto store_x = [&](int stage, const v4i (&xr)[S::kPieces]) {   // (every piece passes here once: its share of the row sum)
+#pragma unroll
+    for (int u = 0; u < S::kPieces; ++u) {
+      *reinterpret_cast<v4i *>(st_smem + stage * S::kStage + x_dst + 32 * u * S::kPitch) = xr[u];
+      x_sum[u] += rows32_sum8<BF16>(xr[u]);
+    }
+  };
+  // weight slab piece i = tid + 256 u: K row i / (8 GP), 16-byte chunk i % (8 GP) of the strip's columns
+  auto load_w = [&](int kb, v4i (&wv)[S::kWPieces]) {
+#pragma unroll
+    for (int u = 0; u < S::kWPieces; ++u) {
+      const int i = tid + ST_THREADS * u, row = i / (8 * GP), chunk = i % (8 * GP);
+      const bool ok = kb < k_blocks && n0 + 16 * chunk < p.n;
+      wv[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? (unsigned)(kb * 64 + row) * (unsigned)p.n + 16u * (unsigned)chunk : kBufferOob,
+                                                    0, kStreamAux);
+    }
+  };
+  auto store_w = [&](int stage, const v4i (&wv)[S::kWPieces]) {
+#pragma unroll
+    for (int u = 0; u < S::kWPieces; ++u) {
+      const int i = tid + ST_THREADS * u, row = i / (8 * GP), chunk = i % (8 * GP);
+      *reinterpret_cast<v4i *>(w_smem + stage * S::kWStage + row * S::kWPitch + chunk * 16) = wv[u];
+    }
+  };
+
+  v16f acc[GP][TR];
+#pragma unroll
+  for (int gp = 0; gp < GP; ++gp)
+#pragma unroll
+    for (int t = 0; t < TR; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[gp][t][v] = 0.f;
+
+  // this lane's corner of the two slabs: x row l % 32 at chunk l / 32; of the weights the 8 bytes it names for a transpose
+  // read (K row 8 (l / 32) + (l % 16) / 2, column half l / 16 % 2, byte half l % 2 of the wave's first block)
+  const unsigned x_lane = (unsigned)(c32 * S::kPitch + kh * 16);
+  const unsigned w_lane = (unsigned)((8 * kh + ((lane & 15) >> 1)) * S::kWPitch + 32 * wave * GP + 16 * ((lane >> 4) & 1) + 8 * (lane & 1));
+  // LIVE = 32-row fragments that hold rows of the chunk (a compile-time count: the others are neither read nor multiplied)
+  auto multiply = [&](auto live_c, int stage) {
+    constexpr int LIVE = decltype(live_c)::value;
+    typedef int v2i_t __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) v2i_t *lds_v2i;
+    const unsigned char *xs = st_smem + stage * S::kStage + x_lane;
+    const unsigned char *ws = w_smem + stage * S::kWStage + w_lane;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      v4i xf[LIVE];
+#pragma unroll
+      for (int t = 0; t < LIVE; ++t) xf[t] = *reinterpret_cast<const v4i *>(xs + 32 * t * S::kPitch + 32 * s);
+#pragma unroll
+      for (int gp = 0; gp < GP; ++gp) {
+        const v2i_t w8 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(ws + 16 * s * S::kWPitch + 32 * gp));
+        const v4i wf = sa_frag<BF16>((unsigned)w8.x ^ 0x80808080u, (unsigned)w8.y ^ 0x80808080u);   // w + 128, exact in 16 bits
+#pragma unroll
+        for (int t = 0; t < LIVE; ++t) acc[gp][t] = rows32_mfma<BF16>(xf[t], wf, acc[gp][t]);
+      }
+    }
+  };
+
+  v4i xr[S::kPieces], wr[S::kWPieces];
+  load_x(0, xr);
+  load_w(0, wr);
+  // antiquant scale and offset of this lane's GP output columns (16-bit elements: the word that holds them)
+  unsigned sc_word[GP], of_word[GP];
+  {
+    const __amdgpu_buffer_rsrc_t rs_sc = buffer_over(p.aq_scale, p.aq_scale ? 2ll * p.e * p.n : 0);
+    const __amdgpu_buffer_rsrc_t rs_of = buffer_over(p.aq_offset, p.aq_offset ? 2ll * p.e * p.n : 0);
+#pragma unroll
+    for (int gp = 0; gp < GP; ++gp) {
+      const int n = n0 + 32 * (wave * GP + gp) + c32;
+      const unsigned byte = 2u * (unsigned)((long long)grp * p.n + n);
+      sc_word[gp] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_sc, n < p.n ? (byte & ~3u) : kBufferOob, 0, 0);
+      of_word[gp] = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rs_of, n < p.n ? (byte & ~3u) : kBufferOob, 0, 0);
+    }
+  }
+  // (LDS-only barrier: __syncthreads would also wait for the operand loads that are in flight on purpose)
+  auto slab_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+  store_x(0, xr);
+  load_x(1, xr);
+  store_w(0, wr);
+  load_w(1, wr);
+  slab_barrier();
+  // One barrier per K block, the requests two blocks ahead, one copy of the loop per number of live row fragments.
+  const int live = (chunk_rows + 31) / 32;   // 1 .. TR, the same for the whole workgroup
+#define MSCO_ROWS32_LOOP(LIVE)                                             \
+  if constexpr (LIVE <= TR) {                                              \
+    if (live == LIVE) {                                                    \
+      const std::integral_constant<int, (LIVE <= TR ? LIVE : 1)> live_c;   \
+      for (int kb = 0; kb < k_blocks; kb += 2) {                           \
+        multiply(live_c, 0);                                               \
+        store_x(1, xr);                                                    \
+        load_x(kb + 2, xr);                                                \
+        store_w(1, wr);                                                    \
+        load_w(kb + 2, wr);                                                \
+        slab_barrier();                                                    \
+        multiply(live_c, 1); /* (past K: zeros times anything finite) */   \
+        store_x(0, xr);                                                    \
+        load_x(kb + 3, xr);                                                \
+        store_w(0, wr);                                                    \
+        load_w(kb + 3, wr);                                                \
+        slab_barrier();                                                    \
+      }                                                                    \
+    }                                                                      \
+  }
+  MSCO_ROWS32_LOOP(1) MSCO_ROWS32_LOOP(2) MSCO_ROWS32_LOOP(3) MSCO_ROWS32_LOOP(4)
+#undef MSCO_ROWS32_LOOP
+
+  // ---- row sums: the 8 chunks of a row sit with 8 neighbouring threads
+  float *row_sum = reinterpret_cast<float *>(st_smem + S::kTile);
+#pragma unroll
+  for (int u = 0; u < S::kPieces; ++u) {
+    float v = x_sum[u];
+    v += __shfl_xor(v, 1);
+    v += __shfl_xor(v, 2);
+    v += __shfl_xor(v, 4);
+    if ((tid & 7) == 0) row_sum[(tid + ST_THREADS * u) >> 3] = v;
+  }
+  __syncthreads();
+
+  // ---- epilogue: out = s * (sum_k x (w + 128) + (o - 128) sum_k x); lane l holds column l % 32 of its wave's blocks and
+  // rows 32 t + 8 j + 4 (l / 32) + r in accumulator element 4 j + r.  The output tile is staged in LDS (the slabs are
+  // done with) for whole-row stores.
+  unsigned short(*tile_out)[S::kCols + 8] = reinterpret_cast<unsigned short(*)[S::kCols + 8]>(st_smem);
+  float sc[GP], of[GP];
+#pragma unroll
+  for (int gp = 0; gp < GP; ++gp) {
+    const int n = n0 + 32 * (wave * GP + gp) + c32;
+    const bool upper = ((long long)grp * p.n + n) & 1;   // which half of its word the element is
+    sc[gp] = p.aq_scale ? sa_half_like<BF16>((unsigned short)(upper ? sc_word[gp] >> 16 : sc_word[gp])) : 1.0f;
+    of[gp] = (p.aq_offset ? sa_half_like<BF16>((unsigned short)(upper ? of_word[gp] >> 16 : of_word[gp])) : 0.0f) - 128.0f;
+  }
+#pragma unroll
+  for (int t = 0; t < TR; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row0 = 32 * t + 8 * j + 4 * kh;
+      if (row0 < chunk_rows) {
+        // (rows past the chunk and columns past N land in the tile as well: the row stores below leave them out)
+        const v4f xs4 = *reinterpret_cast<const v4f *>(&row_sum[row0]);
+#pragma unroll
+        for (int gp = 0; gp < GP; ++gp) {
+          const int cl = 32 * (wave * GP + gp) + c32;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) tile_out[row0 + r][cl] = half_out(p, fmaf(of[gp], xs4[r], acc[gp][t][4 * j + r]) * sc[gp]);
+        }
+      }
+    }
+  __syncthreads();
+  // whole-row stores: pieces of 8 columns
+  constexpr int ROW_PIECES = S::kCols / 8;
+  for (int item = tid; item < S::kRows * ROW_PIECES; item += ST_THREADS) {
+    const int row = item / ROW_PIECES, c8 = (item % ROW_PIECES) * 8;
+    const int n = n0 + c8;
+    if (row < chunk_rows && n < p.n) {   // N % 16 == 0: 8 columns all inside or all outside
+      const uint4 q = *reinterpret_cast<const uint4 *>(&tile_out[row][c8]);
+      *reinterpret_cast<uint4 *>(reinterpret_cast<unsigned short *>(p.out) + (long long)(m0 + row) * p.n + n) = q;
+    }
+  }
+}
+
+template <bool BF16, int TR, int GP>
+static hipError_t rows32_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
+  using S = Rows32Shape<TR, GP>;
+  auto kern = gmm_a16w8_rows32_kernel<BF16, TR, GP>;
+  if constexpr (S::kLds > 64 * 1024) {
+    static std::atomic<bool> attr_set{false};   // (idempotent, as above)
+    if (!attr_set) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::kLds);
+      if (e != hipSuccess) return e;
+      attr_set = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(ST_THREADS), S::kLds, stream, p);
+  return hipGetLastError();
+}
+
 // tch = 16-row fragments per chunk (2, 4 or 8); p.max_chunks counts chunks of 16 tch rows; p.strip_groups = column groups
-// per strip (8 or 16: two or four per wave; 8 for tch = 8), p.n_strips strips
+// per strip (8 or 16: strips of 128 or 256 columns; 8 for tch = 8 on packed weights), p.n_strips strips
 hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, bool packed, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
   if (!packed && p.n % 16 != 0) return hipErrorInvalidValue;   // [E,K,N] rows of whole 16-column chunks
   if (p.split_k != 1 || (p.strip_groups != 8 && p.strip_groups != 16) || (tch != 2 && tch != 4 && tch != 8) ||
-      (tch == 8 && p.strip_groups != 8))
+      (tch == 8 && packed && p.strip_groups != 8))
     return hipErrorInvalidValue;
   const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), 1u);
   const bool bf = p.x_dtype == DT_BF16;
@@ -1115,11 +1384,15 @@ hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, bool packed, hipStr
 #define MSCO_ROWS_BY(TCH)                                                                                                   \
   (bf ? (wide ? rows_launch_a16w8<true, TCH, 4>(p, grid, stream) : rows_launch_a16w8<true, TCH, 2>(p, grid, stream))      \
       : (wide ? rows_launch_a16w8<false, TCH, 4>(p, grid, stream) : rows_launch_a16w8<false, TCH, 2>(p, grid, stream)))
-  if (!packed) {   // (registers: 64-row chunks with two column groups per wave only, no 128-row chunks)
-    if (tch == 4 && !wide) return bf ? rows_launch_a16w8<true, 4, 2, true>(p, grid, stream) : rows_launch_a16w8<false, 4, 2, true>(p, grid, stream);
-    if (tch == 2 && wide) return bf ? rows_launch_a16w8<true, 2, 4, true>(p, grid, stream) : rows_launch_a16w8<false, 2, 4, true>(p, grid, stream);
-    if (tch == 2) return bf ? rows_launch_a16w8<true, 2, 2, true>(p, grid, stream) : rows_launch_a16w8<false, 2, 2, true>(p, grid, stream);
-    return hipErrorInvalidValue;
+  if (!packed) {   // 32-row chunks on 16 x 16 x 32 MFMAs, 64- and 128-row chunks on 32 x 32 x 16
+#define MSCO_ROWS32_BY(TR)                                                                                                  \
+  (bf ? (wide ? rows32_launch_a16w8<true, TR, 2>(p, grid, stream) : rows32_launch_a16w8<true, TR, 1>(p, grid, stream))    \
+      : (wide ? rows32_launch_a16w8<false, TR, 2>(p, grid, stream) : rows32_launch_a16w8<false, TR, 1>(p, grid, stream)))
+    if (tch == 8) return MSCO_ROWS32_BY(4);
+    if (tch == 4) return MSCO_ROWS32_BY(2);
+#undef MSCO_ROWS32_BY
+    return wide ? (bf ? rows_launch_a16w8<true, 2, 4, true>(p, grid, stream) : rows_launch_a16w8<false, 2, 4, true>(p, grid, stream))
+                : (bf ? rows_launch_a16w8<true, 2, 2, true>(p, grid, stream) : rows_launch_a16w8<false, 2, 2, true>(p, grid, stream));
   }
   if (tch == 8) return bf ? rows_launch_a16w8<true, 8, 2>(p, grid, stream) : rows_launch_a16w8<false, 8, 2>(p, grid, stream);
   return tch == 4 ? MSCO_ROWS_BY(4) : MSCO_ROWS_BY(2);

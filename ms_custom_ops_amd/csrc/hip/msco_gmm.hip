@@ -72,7 +72,7 @@ struct msco_gmm_op {
   int skinny_cols = kSkinnyCols;
   int n_strips = 0;
   int strip_groups = 16;
-  int stream_tch = 1;        // packed weights: 16-row fragments per chunk (1: the 16-row streaming kernels, 2/4/8: the multi-row ones; weight-only up to 4)
+  int stream_tch = 1;        // packed and, weight-only, [E,K,N] weights: 16-row fragments per chunk (1: the 16-row streaming kernels, 2/4/8: the multi-row ones)
   int wide_k_slabs = 0;      // small tile kernels on K-major weights: 128-byte K slabs
   int w_nontemporal = 0;     // small tile kernels on packed weights: non-temporal weight loads
   int small_group_rows = 0;  // > 0: the persistent kernel takes the groups with more rows, a second launch of 64 x 128 tiles the others
@@ -315,16 +315,15 @@ void choose_plan(msco_gmm_op *op) {
       op->stream_tch = op->stream_tch == 1 ? 2 : op->stream_tch * 2;
     if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8) op->stream_tch = tuning().stream_tch;
   } else if (family == FAM_SKINNY && is_a16w8(d) && (is_packed(d) || (d.transpose_b == 0 && n % 16 == 0))) {
-    // weight-only on packed or [E,K,N] weights: chunks of 32, 64 or 128 rows by the same estimate (64 at most on [E,K,N],
-    // whose weight slab shares the registers); larger groups stream their weights once per chunk (8 experts, K = 4096,
-    // N = 14336, 128 / 512 / 2048 rows: 111 / 334 / 1307 us with 16-row chunks)
-    const int tch_max = is_packed(d) ? 8 : 4;
+    // weight-only on packed or [E,K,N] weights: chunks of 32, 64 or 128 rows by the same estimate; larger groups stream
+    // their weights once per chunk (8 experts, K = 4096, N = 14336, 128 / 512 / 2048 rows: 111 / 334 / 1307 us with
+    // 16-row chunks)
     const int64_t avg = (m + e - 1) / e;
     const int64_t rows = e == 1 ? m : avg + avg / 2;
-    op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : (rows <= 64 || tch_max == 4) ? 4 : 8;
-    while (op->stream_tch < tch_max && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
+    op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
+    while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch *= 2;
-    if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || (tuning().stream_tch == 8 && tch_max == 8))
+    if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8)
       op->stream_tch = tuning().stream_tch;
   }
   if (family == FAM_SKINNY) {
@@ -345,11 +344,11 @@ void choose_plan(msco_gmm_op *op) {
     op->skinny_wide16 = wide16;
     int want, cap;
     if (op->stream_tch > 1 && !is_w8a8(d)) {
-      // multi-row weight-only kernel: strips of 16 column groups (four per wave) when they still give every CU two
-      // workgroups, else of 8; every workgroup walks all of K.  (For registers: 128-row chunks, and 64-row chunks on
-      // [E,K,N] weights, with two column groups per wave.)
+      // multi-row weight-only kernels: strips of 16 column groups (256 columns) when they still give every CU two
+      // workgroups, else of 8; every workgroup walks all of K.  (For registers: 128-row chunks on packed weights with
+      // strips of 8.)
       const int64_t col_groups = (n + 15) / 16;
-      const bool narrow = op->stream_tch == 8 || (!is_packed(d) && op->stream_tch == 4);
+      const bool narrow = is_packed(d) && op->stream_tch == 8;
       op->strip_groups = (!narrow && ((col_groups + 15) / 16) * active >= 2 * (int64_t)num_cus) ? 16 : 8;
       op->n_strips = (int)((col_groups + op->strip_groups - 1) / op->strip_groups);
       op->skinny_cols = op->strip_groups * 16;

@@ -248,12 +248,17 @@ def test_weight_only_multi_row_streaming_kernel_within_tolerance(device, dtype, 
     (150, 1024 + 64, 272, 3, [70, 70, 150]),                # chunks of 64 rows: 64 + 6 rows, an empty group, 64 + 16; N tail
     (64, 2048, 128, 1, [64]),                               # one full chunk of four row fragments
     (33, 512 + 16, 64, 2, [20, 33]),                        # chunks of 32 rows, K not a multiple of 64
-    (300, 4096, 512, 4, [10, 100, 100, 300]),               # groups of 10, 90, 0 and 200 rows in chunks of 64
+    (300, 4096, 512, 4, [10, 100, 100, 300]),               # chunks of 128 rows: groups of 10, 90, 0 and 200 (128 + 72) rows
     (160, 256, 14336, 8, [20, 40, 60, 80, 100, 120, 140, 160]),   # chunks of 32 rows, wide N: strips of 256 columns
+    (260, 1024 + 48, 400, 2, [129, 260]),                   # chunks of 128 rows: 128 + 1 and 128 + 3 rows, K and N tails
+    (700, 512, 4096, 2, [300, 700]),                        # chunks of 128 rows, strips of 128 columns
+    (320, 256, 14336, 8, [40, 80, 120, 160, 200, 240, 280, 320]),       # chunks of 64 rows, strips of 256 columns
+    (1200, 320, 8192, 8, [100, 250, 400, 550, 700, 850, 1000, 1200]),   # chunks of 128 rows, strips of 256 columns
 ])
 def test_weight_only_multi_row_kernel_on_row_major_weights(device, dtype, m, k, n, e, gl):
     """The same on [E,K,N] weights as stored: the strip's weight slab goes through LDS and transpose reads turn it into
-    MFMA operands.  Tolerance as above; the 16-row kernel of this layout (forced) agrees to the same bound."""
+    MFMA operands (16 x 16 x 32 on 32-row chunks, 32 x 32 x 16 on 64- and 128-row chunks).  Tolerance as above; the
+    packed layout's kernel agrees to the same bound."""
     from gpu_utils import run_a16w8
     x, w, s, o, exact, mag, to_f, last = _weight_only_case(24, m, k, n, e, gl, dtype)
     bits, info = run_a16w8(x, w, s, o, gl, dtype=dtype)
