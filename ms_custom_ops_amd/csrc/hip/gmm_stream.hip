@@ -831,9 +831,9 @@ hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream) {
 }
 
 // ---- weight-only, more than 16 rows per group (packed weights) ------------------------------------------------
-// A workgroup owns one chunk of 16 TCH rows of one group (TCH = 2, 4, 8) and a strip of 4 G column groups (G = 2, 4: 128
-// or 256 columns; TCH = 8 with G = 2 only, for registers) over all of K; wave w owns column groups w G .. w G + G - 1 of the strip and walks every K block, so its
-// accumulators are complete sums: no K split, no reduction between waves, the same float32 summation order run to run.
+// A workgroup owns one chunk of 16 TCH rows of one group (TCH = 2, 4; 128-row chunks have the kernel below) and a strip
+// of 4 G column groups (G = 2, 4: 128 or 256 columns) over all of K; wave w owns column groups w G .. w G + G - 1 of the
+// strip and walks every K block, so its accumulators are complete sums: no K split, no reduction between waves, the same float32 summation order run to run.
 // Per K block the workgroup brings the chunk's x slab (16 TCH rows x 64 K, 16-bit) into LDS once -- every wave needs
 // all of it, and 16-bit x is twice the bytes of the weights it meets -- while each wave requests its G weight blocks,
 // converts them to 16-bit operands once and uses them for all TCH row fragments (2 G TCH MFMAs, plus 2 TCH against ones
@@ -1051,7 +1051,6 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
     }                                                                      \
   }
   MSCO_ROWS_LOOP(1) MSCO_ROWS_LOOP(2) MSCO_ROWS_LOOP(3) MSCO_ROWS_LOOP(4)
-  MSCO_ROWS_LOOP(5) MSCO_ROWS_LOOP(6) MSCO_ROWS_LOOP(7) MSCO_ROWS_LOOP(8)
 #undef MSCO_ROWS_LOOP
 
   // ---- epilogue: out = s * (sum_k x (w + 128) + (o - 128) sum_k x); lane (c, h) holds rows 16 t + 4 h + r of column
@@ -1102,20 +1101,22 @@ static hipError_t rows_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStr
   return hipGetLastError();
 }
 
-// ---- weight-only, row-major [E,K,N] weights, 64- and 128-row chunks: 32 x 32 x 16 MFMAs ---------------------------
-// The 16 x 16 x 32 forms above run at half the rate of the 32 x 32 forms, and a 128-row chunk of them does not fit the
-// register file.  Here a workgroup owns a chunk of 32 TR rows (TR = 2, 4) and a strip of 128 GP columns; wave w owns the GP
-// blocks of 32 columns w GP .. w GP + GP - 1 and all rows, again over all of K.  Both slabs go through LDS as they lie in
-// memory.  Of a 16-K step, lane l of an x fragment holds row l % 32, K positions 8 (l / 32) .. + 7 (one 16-byte read),
+// ---- weight-only, 64- and 128-row chunks on [E,K,N] weights, 128-row chunks on packed weights: 32 x 32 x 16 MFMAs ----
+// The 16 x 16 x 32 forms above run at half the rate of the 32 x 32 forms, and a 128-row chunk of them fills the register
+// file at 128 columns.  Here a workgroup owns a chunk of 32 TR rows (TR = 2, 4) and a strip of 128 GP columns; wave w owns
+// the GP blocks of 32 columns w GP .. w GP + GP - 1 and all rows, again over all of K.  Both slabs go through LDS as they
+// lie in memory.  Of a 16-K step, lane l of an x fragment holds row l % 32, K positions 8 (l / 32) .. + 7 (one 16-byte read),
 // and of a weight fragment column l % 32 at the same K positions: one transpose read, with the four blocks of 16 lanes
 // on (K half, column half) = (l / 32, l / 16 % 2).  Weight rows sit at a pitch of 128 GP + 32 bytes: the 8 rows and the
-// two column halves a pass reads fall into 16 different bank groups.
+// two column halves a pass reads fall into 16 different bank groups.  PK: packed weights.  A block of 16 columns x 64 K
+// keeps its lane order in LDS, and the same fragment is a plain 8-byte read (no transpose: a packed lane already holds 16
+// consecutive K positions of one column).
 // The row sums of x come from the vector unit instead of an MFMA against ones (which would cost a quarter of the matrix
 // time here): a thread adds up the 8 values of every slab piece it carries to LDS (always the same row), and 8 neighbouring
 // threads combine their sums at the end.
 namespace {
 typedef float v16f __attribute__((ext_vector_type(16)));
-template <int TR, int GP>
+template <int TR, int GP, bool PK = false>
 struct Rows32Shape {
   static constexpr int kRows = 32 * TR;
   static constexpr int kCols = 128 * GP;                       // 4 waves x GP blocks of 32 columns
@@ -1123,7 +1124,8 @@ struct Rows32Shape {
   static constexpr int kStage = kRows * kPitch;                // one K block of the chunk's x
   static constexpr int kPieces = kRows * 8 / ST_THREADS;       // 16-byte pieces of an x slab per thread
   static constexpr int kWPitch = kCols + 32;                   // bytes of a weight K row in LDS
-  static constexpr int kWStage = 64 * kWPitch;                 // one K block of the strip's weights
+  static constexpr int kWBlock = 1024 + 8;                     // packed: bytes of a 16-column block in LDS
+  static constexpr int kWStage = PK ? (kCols / 16) * kWBlock : 64 * kWPitch;   // one K block of the strip's weights
   static constexpr int kWPieces = 64 * kCols / 16 / ST_THREADS;   // its 16-byte pieces per thread (= 2 GP)
   static constexpr int kSlabs = 2 * (kStage + kWStage);        // two stages of operands
   static constexpr int kOut = kRows * (kCols + 8) * 2;         // 16-bit output tile of the epilogue
@@ -1153,9 +1155,9 @@ __device__ __forceinline__ float rows32_sum8(const v4i &v) {
 }
 }  // namespace
 
-template <bool BF16, int TR, int GP>
+template <bool BF16, int TR, int GP, bool PK = false>
 __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const GmmParams p) {
-  using S = Rows32Shape<TR, GP>;
+  using S = Rows32Shape<TR, GP, PK>;
   extern __shared__ __align__(16) unsigned char st_smem[];
 
   const int tid = threadIdx.x;
@@ -1171,11 +1173,12 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
   if (chunk_rows <= 0) return;
 
   const int n0 = strip * S::kCols;
-  const int k_blocks = (p.k + 63) / 64;
-  const long long group_bytes = (long long)p.k * p.n;
+  const int k_blocks = (p.k + 63) / 64, col_groups = (p.n + 15) / 16;
+  const long long group_bytes = PK ? (long long)col_groups * k_blocks * 1024 : (long long)p.k * p.n;
   // (windows as in the kernel above: the weights from the strip's first column to the end of the expert's matrix, K rows
-  // past K read as zeros; x over the chunk's rows)
-  const __amdgpu_buffer_rsrc_t rw = buffer_over(p.w + (long long)grp * group_bytes + n0, group_bytes - n0);
+  // past K read as zeros -- packed: the expert's blocks; x over the chunk's rows)
+  const __amdgpu_buffer_rsrc_t rw = PK ? buffer_over(p.w + (long long)grp * group_bytes, group_bytes)
+                                       : buffer_over(p.w + (long long)grp * group_bytes + n0, group_bytes - n0);
   const __amdgpu_buffer_rsrc_t rx = buffer_over(reinterpret_cast<const unsigned short *>(p.x) + (long long)m0 * p.k,
                                                 2ll * chunk_rows * p.k);
   unsigned char *w_smem = st_smem + 2 * S::kStage;
@@ -1201,21 +1204,36 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
       x_sum[u] += rows32_sum8<BF16>(xr[u]);
     }
   };
-  // weight slab piece i = tid + 256 u: K row i / (8 GP), 16-byte chunk i % (8 GP) of the strip's columns
+  // weight slab piece i = tid + 256 u: K row i / (8 GP), 16-byte chunk i % (8 GP) of the strip's columns.  Packed: lane
+  // i % 64 of the strip's block i / 64 = wave + 4 u (a block is 16 columns x 64 K, lane (q, c) holding K positions 16 q ..
+  // 16 q + 15 of column c), kept in LDS at a pitch of 1024 + 8 bytes, hence written in two halves
   auto load_w = [&](int kb, v4i (&wv)[S::kWPieces]) {
 #pragma unroll
     for (int u = 0; u < S::kWPieces; ++u) {
-      const int i = tid + ST_THREADS * u, row = i / (8 * GP), chunk = i % (8 * GP);
-      const bool ok = kb < k_blocks && n0 + 16 * chunk < p.n;
-      wv[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? (unsigned)(kb * 64 + row) * (unsigned)p.n + 16u * (unsigned)chunk : kBufferOob,
-                                                    0, kStreamAux);
+      if constexpr (PK) {
+        const int cg = strip * (8 * GP) + wave + 4 * u;
+        wv[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, (kb < k_blocks && cg < col_groups) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
+                                                      min(cg, col_groups - 1) * k_blocks * 1024, kStreamAux);
+      } else {
+        const int i = tid + ST_THREADS * u, row = i / (8 * GP), chunk = i % (8 * GP);
+        const bool ok = kb < k_blocks && n0 + 16 * chunk < p.n;
+        wv[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? (unsigned)(kb * 64 + row) * (unsigned)p.n + 16u * (unsigned)chunk : kBufferOob,
+                                                      0, kStreamAux);
+      }
     }
   };
   auto store_w = [&](int stage, const v4i (&wv)[S::kWPieces]) {
 #pragma unroll
     for (int u = 0; u < S::kWPieces; ++u) {
-      const int i = tid + ST_THREADS * u, row = i / (8 * GP), chunk = i % (8 * GP);
-      *reinterpret_cast<v4i *>(w_smem + stage * S::kWStage + row * S::kWPitch + chunk * 16) = wv[u];
+      if constexpr (PK) {
+        typedef int v2i_t __attribute__((ext_vector_type(2)));
+        unsigned char *dst = w_smem + stage * S::kWStage + (wave + 4 * u) * S::kWBlock + lane * 16;
+        *reinterpret_cast<v2i_t *>(dst) = v2i_t{wv[u][0], wv[u][1]};
+        *reinterpret_cast<v2i_t *>(dst + 8) = v2i_t{wv[u][2], wv[u][3]};
+      } else {
+        const int i = tid + ST_THREADS * u, row = i / (8 * GP), chunk = i % (8 * GP);
+        *reinterpret_cast<v4i *>(w_smem + stage * S::kWStage + row * S::kWPitch + chunk * 16) = wv[u];
+      }
     }
   };
 
@@ -1230,7 +1248,10 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
   // this lane's corner of the two slabs: x row l % 32 at chunk l / 32; of the weights the 8 bytes it names for a transpose
   // read (K row 8 (l / 32) + (l % 16) / 2, column half l / 16 % 2, byte half l % 2 of the wave's first block)
   const unsigned x_lane = (unsigned)(c32 * S::kPitch + kh * 16);
-  const unsigned w_lane = (unsigned)((8 * kh + ((lane & 15) >> 1)) * S::kWPitch + 32 * wave * GP + 16 * ((lane >> 4) & 1) + 8 * (lane & 1));
+  // (packed: of block 2 (w GP + gp) + (l % 32) / 16, the lane of K group s and column l % 16, its half l / 32 -- a plain
+  // 8-byte read; the 8-byte skew between blocks puts the two blocks of a pass into different banks)
+  const unsigned w_lane = PK ? (unsigned)((2 * wave * GP + (c32 >> 4)) * S::kWBlock + (c32 & 15) * 16 + 8 * kh)
+                             : (unsigned)((8 * kh + ((lane & 15) >> 1)) * S::kWPitch + 32 * wave * GP + 16 * ((lane >> 4) & 1) + 8 * (lane & 1));
   // LIVE = 32-row fragments that hold rows of the chunk (a compile-time count: the others are neither read nor multiplied)
   auto multiply = [&](auto live_c, int stage) {
     constexpr int LIVE = decltype(live_c)::value;
@@ -1245,7 +1266,9 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
       for (int t = 0; t < LIVE; ++t) xf[t] = *reinterpret_cast<const v4i *>(xs + 32 * t * S::kPitch + 32 * s);
 #pragma unroll
       for (int gp = 0; gp < GP; ++gp) {
-        const v2i_t w8 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(ws + 16 * s * S::kWPitch + 32 * gp));
+        v2i_t w8;
+        if constexpr (PK) w8 = *reinterpret_cast<const v2i_t *>(ws + 256 * s + 2 * S::kWBlock * gp);
+        else w8 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(ws + 16 * s * S::kWPitch + 32 * gp));
         const v4i wf = sa_frag<BF16>((unsigned)w8.x ^ 0x80808080u, (unsigned)w8.y ^ 0x80808080u);   // w + 128, exact in 16 bits
 #pragma unroll
         for (int t = 0; t < LIVE; ++t) acc[gp][t] = rows32_mfma<BF16>(xf[t], wf, acc[gp][t]);
@@ -1354,10 +1377,10 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
   }
 }
 
-template <bool BF16, int TR, int GP>
+template <bool BF16, int TR, int GP, bool PK = false>
 static hipError_t rows32_launch_a16w8(const GmmParams &p, const dim3 &grid, hipStream_t stream) {
-  using S = Rows32Shape<TR, GP>;
-  auto kern = gmm_a16w8_rows32_kernel<BF16, TR, GP>;
+  using S = Rows32Shape<TR, GP, PK>;
+  auto kern = gmm_a16w8_rows32_kernel<BF16, TR, GP, PK>;
   if constexpr (S::kLds > 64 * 1024) {
     static std::atomic<bool> attr_set{false};   // (idempotent, as above)
     if (!attr_set) {
@@ -1371,12 +1394,11 @@ static hipError_t rows32_launch_a16w8(const GmmParams &p, const dim3 &grid, hipS
 }
 
 // tch = 16-row fragments per chunk (2, 4 or 8); p.max_chunks counts chunks of 16 tch rows; p.strip_groups = column groups
-// per strip (8 or 16: strips of 128 or 256 columns; 8 for tch = 8 on packed weights), p.n_strips strips
+// per strip (8 or 16: strips of 128 or 256 columns), p.n_strips strips
 hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, bool packed, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
   if (!packed && p.n % 16 != 0) return hipErrorInvalidValue;   // [E,K,N] rows of whole 16-column chunks
-  if (p.split_k != 1 || (p.strip_groups != 8 && p.strip_groups != 16) || (tch != 2 && tch != 4 && tch != 8) ||
-      (tch == 8 && packed && p.strip_groups != 8))
+  if (p.split_k != 1 || (p.strip_groups != 8 && p.strip_groups != 16) || (tch != 2 && tch != 4 && tch != 8))
     return hipErrorInvalidValue;
   const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), 1u);
   const bool bf = p.x_dtype == DT_BF16;
@@ -1394,7 +1416,9 @@ hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, bool packed, hipStr
     return wide ? (bf ? rows_launch_a16w8<true, 2, 4, true>(p, grid, stream) : rows_launch_a16w8<false, 2, 4, true>(p, grid, stream))
                 : (bf ? rows_launch_a16w8<true, 2, 2, true>(p, grid, stream) : rows_launch_a16w8<false, 2, 2, true>(p, grid, stream));
   }
-  if (tch == 8) return bf ? rows_launch_a16w8<true, 8, 2>(p, grid, stream) : rows_launch_a16w8<false, 8, 2>(p, grid, stream);
+  if (tch == 8)   // 128-row chunks: the 32 x 32 x 16 kernel, the packed blocks through LDS
+    return wide ? (bf ? rows32_launch_a16w8<true, 4, 2, true>(p, grid, stream) : rows32_launch_a16w8<false, 4, 2, true>(p, grid, stream))
+                : (bf ? rows32_launch_a16w8<true, 4, 1, true>(p, grid, stream) : rows32_launch_a16w8<false, 4, 1, true>(p, grid, stream));
   return tch == 4 ? MSCO_ROWS_BY(4) : MSCO_ROWS_BY(2);
 #undef MSCO_ROWS_BY
 }

@@ -345,11 +345,9 @@ void choose_plan(msco_gmm_op *op) {
     int want, cap;
     if (op->stream_tch > 1 && !is_w8a8(d)) {
       // multi-row weight-only kernels: strips of 16 column groups (256 columns) when they still give every CU two
-      // workgroups, else of 8; every workgroup walks all of K.  (For registers: 128-row chunks on packed weights with
-      // strips of 8.)
+      // workgroups, else of 8; every workgroup walks all of K.
       const int64_t col_groups = (n + 15) / 16;
-      const bool narrow = is_packed(d) && op->stream_tch == 8;
-      op->strip_groups = (!narrow && ((col_groups + 15) / 16) * active >= 2 * (int64_t)num_cus) ? 16 : 8;
+      op->strip_groups = ((col_groups + 15) / 16) * active >= 2 * (int64_t)num_cus ? 16 : 8;
       op->n_strips = (int)((col_groups + op->strip_groups - 1) / op->strip_groups);
       op->skinny_cols = op->strip_groups * 16;
       want = cap = 1;

@@ -226,9 +226,11 @@ def test_weight_only_streaming_kernel_within_tolerance(device, dtype, m, k, n, e
     (33, 512 + 16, 64, 2, [20, 33]),                        # chunks of 32 rows, K not a multiple of 64
     (300, 4096, 512, 4, [10, 100, 100, 300]),               # chunks of 128 rows: groups of 10, 90, 0 and 200 (128 + 72) rows
     (260, 1024 + 48, 400, 2, [129, 260]),                   # 128 + 1 and 128 + 3 rows, K and N tails
+    (1200, 320, 8192, 8, [100, 250, 400, 550, 700, 850, 1000, 1200]),   # chunks of 128 rows, strips of 256 columns
 ])
 def test_weight_only_multi_row_streaming_kernel_within_tolerance(device, dtype, m, k, n, e, gl):
-    """More than 16 rows per group on packed weights: chunks of 32, 64 or 128 rows share one pass over the group's weights.
+    """More than 16 rows per group on packed weights: chunks of 32, 64 or 128 rows share one pass over the group's weights
+    (128-row chunks on 32 x 32 x 16 MFMAs, the packed blocks through LDS).
     Same tolerance as the 16-row kernel, against the float64 value of the reference's a16w8 golden."""
     from gpu_utils import run_a16w8
     x, w, s, o, exact, mag, to_f, last = _weight_only_case(23, m, k, n, e, gl, dtype)
