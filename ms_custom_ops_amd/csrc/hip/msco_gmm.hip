@@ -323,6 +323,12 @@ void choose_plan(msco_gmm_op *op) {
     op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
     while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch *= 2;
+    // One group whose column strips do not fill the chip: the multi-row kernels have no K split, every workgroup walks
+    // all of K, and below 64 rows the 16-row kernels with their K split are faster although they stream the weights once
+    // per 16 rows (K = 4096, N = 11008, 32 / 64 rows: packed 24 / 41 us against 49 / 51; [E,K,N] 32 us against 39 at 32
+    // rows, where 64 rows do best in 32-row chunks, 40 us against 48 and 50).
+    if (e == 1 && m <= 64 && (n + 127) / 128 < num_cus)
+      op->stream_tch = (is_packed(d) || m <= 32) ? 1 : 2;
     if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8)
       op->stream_tch = tuning().stream_tch;
   }

@@ -222,7 +222,7 @@ def test_weight_only_streaming_kernel_within_tolerance(device, dtype, m, k, n, e
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
 @pytest.mark.parametrize("m,k,n,e,gl", [
     (150, 1024 + 64, 272, 3, [70, 70, 150]),                # chunks of 64 rows: 64 + 6 rows, an empty group, 64 + 16; N tail
-    (64, 2048, 128, 1, [64]),                               # one full chunk of four row fragments
+    (80, 2048, 128, 2, [64, 80]),                           # one full chunk of 64 rows and a quarter of one
     (33, 512 + 16, 64, 2, [20, 33]),                        # chunks of 32 rows, K not a multiple of 64
     (300, 4096, 512, 4, [10, 100, 100, 300]),               # chunks of 128 rows: groups of 10, 90, 0 and 200 (128 + 72) rows
     (260, 1024 + 48, 400, 2, [129, 260]),                   # 128 + 1 and 128 + 3 rows, K and N tails
@@ -248,7 +248,7 @@ def test_weight_only_multi_row_streaming_kernel_within_tolerance(device, dtype, 
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
 @pytest.mark.parametrize("m,k,n,e,gl", [
     (150, 1024 + 64, 272, 3, [70, 70, 150]),                # chunks of 64 rows: 64 + 6 rows, an empty group, 64 + 16; N tail
-    (64, 2048, 128, 1, [64]),                               # one full chunk of four row fragments
+    (80, 2048, 128, 2, [64, 80]),                           # one full chunk of 64 rows and a quarter of one
     (33, 512 + 16, 64, 2, [20, 33]),                        # chunks of 32 rows, K not a multiple of 64
     (300, 4096, 512, 4, [10, 100, 100, 300]),               # chunks of 128 rows: groups of 10, 90, 0 and 200 (128 + 72) rows
     (160, 256, 14336, 8, [20, 40, 60, 80, 100, 120, 140, 160]),   # chunks of 32 rows, wide N: strips of 256 columns
@@ -292,7 +292,8 @@ def test_weight_only_rows_kernels_random_shapes(device, seed):
     ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
     for packed in (True, False):
         bits, info = run_a16w8(x, w, s, o, gl, dtype=dtype, packed=packed)
-        assert ("a16w8_stream_rows" if packed else "a16w8_skinny_rows") in info, info
+        if not (e == 1 and m <= 64):   # (one small group goes back to the 16-row kernels and their K split)
+            assert ("a16w8_stream_rows" if packed else "a16w8_skinny_rows") in info, info
         got = to_f(bits).astype(np.float64)
         assert (np.abs(got[:last] - exact[:last]) <= ulp * np.abs(exact[:last]) + 1e-5 * mag[:last]).all(), info
         assert (bits[last:] == 0x7FC0).all(), info
