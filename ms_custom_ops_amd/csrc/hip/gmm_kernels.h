@@ -39,6 +39,7 @@ hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream);   // K s
 hipError_t launch_streamm_w8a8(const GmmParams &p, int tch, hipStream_t stream);
 hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, bool packed, hipStream_t stream);   // weight-only, 32 / 64 / 128 rows per chunk (tch = 2, 4, 8), packed or [E,K,N] weights, no K split
 size_t streamm_tile_bytes(int tch);   // workspace bytes of one (chunk, strip, K slice) partial tile
+size_t rows32_a16w8_slice_bytes(int strip_groups);   // workspace bytes of one (chunk, strip, K slice) partial tile of the 128-row weight-only kernel
 size_t stream_a16w8_tile_bytes();   // workspace bytes of one (strip, K slice) partial tile of the weight-only kernel
 int stream_blocks_per_wave(int64_t k, int split_k);
 size_t packed_weight_bytes(int64_t k, int64_t n);   // bytes of one group's weights in the packed layout

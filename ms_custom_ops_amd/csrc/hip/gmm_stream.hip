@@ -1130,7 +1130,8 @@ struct Rows32Shape {
   static constexpr int kSlabs = 2 * (kStage + kWStage);        // two stages of operands
   static constexpr int kOut = kRows * (kCols + 8) * 2;         // 16-bit output tile of the epilogue
   static constexpr int kTile = kSlabs > kOut ? kSlabs : kOut;
-  static constexpr size_t kLds = (size_t)kTile + kRows * 4;    // + the chunk's row sums of x
+  static constexpr size_t kLds = (size_t)kTile + kRows * 4 + 16;   // + the chunk's row sums of x + the K split's ticket
+  static constexpr size_t kSliceWords = (size_t)kRows * kCols / 2 + kRows / 2;   // 64-bit words of a K slice's partial tile
   static_assert(kPieces >= 1 && kWPieces == 2 * GP, "slab pieces per thread");
 };
 template <bool BF16>
@@ -1174,6 +1175,9 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
 
   const int n0 = strip * S::kCols;
   const int k_blocks = (p.k + 63) / 64, col_groups = (p.n + 15) / 16;
+  // K slice of this workgroup (grid.z slices of whole blocks; one past the end of K adds zeros)
+  const int ks = blockIdx.z, slice_blocks = (k_blocks + p.split_k - 1) / p.split_k;
+  const int kb0 = ks * slice_blocks, kb_end = min(k_blocks, kb0 + slice_blocks);
   const long long group_bytes = PK ? (long long)col_groups * k_blocks * 1024 : (long long)p.k * p.n;
   // (windows as in the kernel above: the weights from the strip's first column to the end of the expert's matrix, K rows
   // past K read as zeros -- packed: the expert's blocks; x over the chunk's rows)
@@ -1192,7 +1196,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
 #pragma unroll
   for (int u = 0; u < S::kPieces; ++u) x_sum[u] = 0.f;
   auto load_x = [&](int kb, v4i (&xr)[S::kPieces]) {
-    const bool ok = kb < k_blocks && kb * 64 + 8 * x_chunk < p.k;   // K % 16 == 0: a chunk's 8 K positions are all inside or all outside
+    const bool ok = kb < kb_end && kb * 64 + 8 * x_chunk < p.k;   // K % 16 == 0: a chunk's 8 K positions are all inside or all outside
 #pragma unroll
     for (int u = 0; u < S::kPieces; ++u)
       xr[u] = __builtin_amdgcn_raw_buffer_load_b128(rx, ok ? x_src + (unsigned)(64 * u) * (unsigned)p.k + (unsigned)(kb * 128) : kBufferOob, 0, 0);
@@ -1212,11 +1216,11 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
     for (int u = 0; u < S::kWPieces; ++u) {
       if constexpr (PK) {
         const int cg = strip * (8 * GP) + wave + 4 * u;
-        wv[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, (kb < k_blocks && cg < col_groups) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
+        wv[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, (kb < kb_end && cg < col_groups) ? (unsigned)(kb * 1024 + lane * 16) : kBufferOob,
                                                       min(cg, col_groups - 1) * k_blocks * 1024, kStreamAux);
       } else {
         const int i = tid + ST_THREADS * u, row = i / (8 * GP), chunk = i % (8 * GP);
-        const bool ok = kb < k_blocks && n0 + 16 * chunk < p.n;
+        const bool ok = kb < kb_end && n0 + 16 * chunk < p.n;
         wv[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, ok ? (unsigned)(kb * 64 + row) * (unsigned)p.n + 16u * (unsigned)chunk : kBufferOob,
                                                       0, kStreamAux);
       }
@@ -1277,8 +1281,8 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
   };
 
   v4i xr[S::kPieces], wr[S::kWPieces];
-  load_x(0, xr);
-  load_w(0, wr);
+  load_x(kb0, xr);
+  load_w(kb0, wr);
   // antiquant scale and offset of this lane's GP output columns (16-bit elements: the word that holds them)
   unsigned sc_word[GP], of_word[GP];
   {
@@ -1295,9 +1299,9 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
   // (LDS-only barrier: __syncthreads would also wait for the operand loads that are in flight on purpose)
   auto slab_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
   store_x(0, xr);
-  load_x(1, xr);
+  load_x(kb0 + 1, xr);
   store_w(0, wr);
-  load_w(1, wr);
+  load_w(kb0 + 1, wr);
   slab_barrier();
   // One barrier per K block, the requests two blocks ahead, one copy of the loop per number of live row fragments.
   const int live = (chunk_rows + 31) / 32;   // 1 .. TR, the same for the whole workgroup
@@ -1305,7 +1309,7 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
   if constexpr (LIVE <= TR) {                                              \
     if (live == LIVE) {                                                    \
       const std::integral_constant<int, (LIVE <= TR ? LIVE : 1)> live_c;   \
-      for (int kb = 0; kb < k_blocks; kb += 2) {                           \
+      for (int kb = kb0; kb < kb_end; kb += 2) {                           \
         multiply(live_c, 0);                                               \
         store_x(1, xr);                                                    \
         load_x(kb + 2, xr);                                                \
@@ -1335,6 +1339,75 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
     if ((tid & 7) == 0) row_sum[(tid + ST_THREADS * u) >> 3] = v;
   }
   __syncthreads();
+
+  if (p.split_k > 1) {
+    // float32 partials through the workspace, added in slice order by the last arriver: 64-bit word i of thread t at
+    // i * 256 + t (accumulator elements 2 i, 2 i + 1 in (gp, t, element) order), the row sums behind them
+    typedef long long i64;
+    constexpr int WORDS = GP * TR * 8;
+    unsigned *s_ticket = reinterpret_cast<unsigned *>(st_smem + S::kTile + S::kRows * 4);
+    const long long tile = ((long long)grp * p.max_chunks + mc) * p.n_strips + strip;
+    i64 *base = reinterpret_cast<i64 *>(p.partial) + tile * p.split_k * (long long)S::kSliceWords;
+    i64 *mine = base + (long long)ks * (long long)S::kSliceWords;
+    auto pack = [](float lo, float hi) { return (i64)(((unsigned long long)__float_as_uint(hi) << 32) | __float_as_uint(lo)); };
+#pragma unroll
+    for (int gp = 0; gp < GP; ++gp)
+#pragma unroll
+      for (int t = 0; t < TR; ++t)
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          __hip_atomic_store(mine + ((gp * TR + t) * 8 + i) * ST_THREADS + tid, pack(acc[gp][t][2 * i], acc[gp][t][2 * i + 1]),
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid < S::kRows / 2)
+      __hip_atomic_store(mine + WORDS * ST_THREADS + tid, pack(row_sum[2 * tid], row_sum[2 * tid + 1]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    publish_partials_and_sync();
+    if (tid == 0) *s_ticket = __hip_atomic_fetch_add(&p.counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (*s_ticket != (unsigned)(p.split_k - 1)) return;
+    if (tid == 0) __hip_atomic_store(&p.counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // (as many loads in flight as the registers hold -- every round is a round trip to memory: blocks of up to 32 words,
+    // two slices at a time where the accumulators leave room)
+    constexpr int WB = WORDS < 32 ? WORDS : 32, NS = WORDS >= 64 ? 1 : 2;
+#pragma unroll
+    for (int gp = 0; gp < GP; ++gp)
+#pragma unroll
+      for (int t = 0; t < TR; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[gp][t][v] = 0.f;
+#pragma unroll
+    for (int b0 = 0; b0 < WORDS; b0 += WB) {
+      for (int s0 = 0; s0 < p.split_k; s0 += NS) {
+        i64 w[NS][WB];
+#pragma unroll
+        for (int u = 0; u < NS; ++u) {
+          const i64 *src = base + (long long)min(s0 + u, p.split_k - 1) * (long long)S::kSliceWords + b0 * ST_THREADS + tid;
+#pragma unroll
+          for (int i = 0; i < WB; ++i) w[u][i] = __hip_atomic_load(src + i * ST_THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int u = 0; u < NS; ++u)
+          if (s0 + u < p.split_k) {
+#pragma unroll
+            for (int i = 0; i < WB; ++i) {
+              const int word = b0 + i;   // (gp TR + t) 8 + pair
+              acc[word / (8 * TR)][(word / 8) % TR][2 * (word % 8)] += __uint_as_float((unsigned)(unsigned long long)w[u][i]);
+              acc[word / (8 * TR)][(word / 8) % TR][2 * (word % 8) + 1] += __uint_as_float((unsigned)((unsigned long long)w[u][i] >> 32));
+            }
+          }
+      }
+    }
+    if (tid < S::kRows / 2) {   // (these threads read their two row sums above, before the barrier)
+      float lo = 0.f, hi = 0.f;
+      for (int sl = 0; sl < p.split_k; ++sl) {
+        const i64 w = __hip_atomic_load(base + (long long)sl * (long long)S::kSliceWords + WORDS * ST_THREADS + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        lo += __uint_as_float((unsigned)(unsigned long long)w);
+        hi += __uint_as_float((unsigned)((unsigned long long)w >> 32));
+      }
+      row_sum[2 * tid] = lo;
+      row_sum[2 * tid + 1] = hi;
+    }
+    __syncthreads();
+  }
 
   // ---- epilogue: out = s * (sum_k x (w + 128) + (o - 128) sum_k x); lane l holds column l % 32 of its wave's blocks and
   // rows 32 t + 8 j + 4 (l / 32) + r in accumulator element 4 j + r.  The output tile is staged in LDS (the slabs are
@@ -1393,14 +1466,18 @@ static hipError_t rows32_launch_a16w8(const GmmParams &p, const dim3 &grid, hipS
   return hipGetLastError();
 }
 
+// workspace bytes of one (chunk, strip, K slice) partial tile of the 128-row kernel: accumulators and row sums
+size_t rows32_a16w8_slice_bytes(int strip_groups) { return ((size_t)128 * 16 * strip_groups + 128) * 4; }
+
 // tch = 16-row fragments per chunk (2, 4 or 8); p.max_chunks counts chunks of 16 tch rows; p.strip_groups = column groups
 // per strip (8 or 16: strips of 128 or 256 columns), p.n_strips strips
 hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, bool packed, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
   if (!packed && p.n % 16 != 0) return hipErrorInvalidValue;   // [E,K,N] rows of whole 16-column chunks
-  if (p.split_k != 1 || (p.strip_groups != 8 && p.strip_groups != 16) || (tch != 2 && tch != 4 && tch != 8))
+  if ((p.strip_groups != 8 && p.strip_groups != 16) || (tch != 2 && tch != 4 && tch != 8) || p.split_k < 1 ||
+      (p.split_k > 1 && tch != 8))   // (a K split: 128-row chunks only)
     return hipErrorInvalidValue;
-  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), 1u);
+  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
   const bool bf = p.x_dtype == DT_BF16;
   const bool wide = p.strip_groups == 16;
 #define MSCO_ROWS_BY(TCH)                                                                                                   \

@@ -357,6 +357,15 @@ void choose_plan(msco_gmm_op *op) {
       op->n_strips = (int)((col_groups + op->strip_groups - 1) / op->strip_groups);
       op->skinny_cols = op->strip_groups * 16;
       want = cap = 1;
+      // One group whose strips leave most CUs idle: 128-row chunks with a K split (slices of at least 8 blocks) up to
+      // about two workgroups per CU.  K = 4096, N = 11008, 128 / 256 / 512 rows without it: 59 / 61 / 83 us.
+      const int64_t base = (int64_t)op->n_strips * active, k_blocks = (k + 63) / 64;
+      if (e == 1 && base < num_cus && tuning().stream_tch == 0) {
+        op->stream_tch = 8;
+        op->max_chunks = (int)((m + 127) / 128);
+        want = (int)std::min<int64_t>(kTargetWorkgroups / std::max<int64_t>((int64_t)op->n_strips * op->max_chunks, 1), kMaxSplitK);
+        cap = std::max<int>(1, (int)(k_blocks / 8));
+      }
     } else if (is_packed(d) && op->stream_tch > 1) {
       // multi-row kernel: strips of four column groups, K split until about two workgroups per CU stream operands
       const int64_t col_groups = (n + 15) / 16, k_blocks = (k + 63) / 64;
@@ -406,10 +415,12 @@ void choose_plan(msco_gmm_op *op) {
       const int slice_blocks = is_w8a8(d) ? 128 : 64;
       want = std::max(want, (int)(((k + 63) / 64 + slice_blocks - 1) / slice_blocks));
     }
-    if (op->stream_tch > 1 && !is_w8a8(d)) want = 1;   // the multi-row weight-only kernel walks all of K
+    if (op->stream_tch > 1 && !is_w8a8(d) && !(e == 1 && op->stream_tch == 8)) want = 1;   // the multi-row weight-only kernels walk all of K, but for one group in 128-row chunks
     op->split_k = want;
     if (!is_packed(d) && !(op->stream_tch > 1 && !is_w8a8(d))) op->skinny_cols = wide16 ? 128 : kSkinnyCols;
-    if (is_packed(d)) {
+    if (op->stream_tch > 1 && !is_w8a8(d)) {
+      op->workspace_bytes = op->split_k > 1 ? (size_t)e * op->max_chunks * op->n_strips * op->split_k * rows32_a16w8_slice_bytes(op->strip_groups) : 0;
+    } else if (is_packed(d)) {
       // the packed-layout kernels keep a full 16 x 256 partial tile per (strip, K slice) whatever the strip's width
       const size_t tile_bytes = !is_w8a8(d)           ? stream_a16w8_tile_bytes()
                                 : op->stream_tch > 1 ? streamm_tile_bytes(op->stream_tch)
@@ -417,8 +428,6 @@ void choose_plan(msco_gmm_op *op) {
       const size_t tiles = op->stream_tch > 1 ? (size_t)e * op->max_chunks * op->n_strips
                                               : skinny_counter_count(m, n, e, op->skinny_cols);
       op->workspace_bytes = op->split_k > 1 ? tiles * (size_t)op->split_k * tile_bytes : 0;
-    } else if (op->stream_tch > 1 && !is_w8a8(d)) {
-      op->workspace_bytes = 0;   // (the multi-row weight-only kernel has no K split)
     } else {
       op->workspace_bytes = is_w8a8(d) ? skinny_workspace_bytes(m, n, e, op->split_k, op->skinny_cols)
                                        : a16w8_workspace_bytes(m, n, e, op->split_k);

@@ -273,6 +273,32 @@ def test_weight_only_multi_row_kernel_on_row_major_weights(device, dtype, m, k, 
     assert (np.abs(to_f(bits_p).astype(np.float64)[:last] - got[:last]) <= 2 * ulp * np.abs(exact[:last]) + 2e-5 * mag[:last]).all()
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("packed", [True, False])
+@pytest.mark.parametrize("m,k,n,last", [
+    (128, 4096, 1024, 128),          # one full 128-row chunk, 8 strips: K in 8 slices
+    (200, 1024 + 64, 400, 190),      # two chunks (128 + 62 rows), K and N tails, 17 blocks in slices of 9 and 8
+    (70, 512 + 16, 2048, 70),        # 9 blocks: one slice
+    (300, 8192, 256, 300),           # three chunks (the last with two live row fragments), 128 blocks in 8 slices
+])
+def test_weight_only_one_group_k_split(device, dtype, packed, m, k, n, last):
+    """One group of more than 64 rows whose column strips leave most CUs idle: 128-row chunks with a K split, partial
+    accumulators and row sums through the workspace, added in slice order by the last arriver.  Same tolerance against
+    the float64 golden; a second launch on the same inputs gives the same bits (one summation order, counters back at zero)."""
+    from gpu_utils import run_a16w8
+    x, w, s, o, exact, mag, to_f, last_row = _weight_only_case(31, m, k, n, 1, [last], dtype)
+    bits, info = run_a16w8(x, w, s, o, [last], dtype=dtype, packed=packed)
+    assert ("a16w8_stream_rows" if packed else "a16w8_skinny_rows") in info, info
+    if k >= 1024:
+        assert "split_k=1 " not in info, info
+    got = to_f(bits).astype(np.float64)
+    ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
+    assert (np.abs(got[:last_row] - exact[:last_row]) <= ulp * np.abs(exact[:last_row]) + 1e-5 * mag[:last_row]).all(), info
+    assert (bits[last_row:] == 0x7FC0).all()
+    bits2, _ = run_a16w8(x, w, s, o, [last], dtype=dtype, packed=packed)
+    assert (bits2 == bits).all()
+
+
 @pytest.mark.parametrize("seed", range(10))
 def test_weight_only_rows_kernels_random_shapes(device, seed):
     # a seeded sweep over the shapes of the multi-row weight-only kernels: K with odd and even block counts and 16..48-byte
