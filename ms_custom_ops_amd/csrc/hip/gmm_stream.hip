@@ -1398,10 +1398,18 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
     }
     if (tid < S::kRows / 2) {   // (these threads read their two row sums above, before the barrier)
       float lo = 0.f, hi = 0.f;
-      for (int sl = 0; sl < p.split_k; ++sl) {
-        const i64 w = __hip_atomic_load(base + (long long)sl * (long long)S::kSliceWords + WORDS * ST_THREADS + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        lo += __uint_as_float((unsigned)(unsigned long long)w);
-        hi += __uint_as_float((unsigned)((unsigned long long)w >> 32));
+      for (int s0 = 0; s0 < p.split_k; s0 += 8) {   // (eight loads in flight: one round trip for any split the plan makes)
+        i64 w[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          w[u] = __hip_atomic_load(base + (long long)min(s0 + u, p.split_k - 1) * (long long)S::kSliceWords + WORDS * ST_THREADS + tid,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < p.split_k) {
+            lo += __uint_as_float((unsigned)(unsigned long long)w[u]);
+            hi += __uint_as_float((unsigned)((unsigned long long)w[u] >> 32));
+          }
       }
       row_sum[2 * tid] = lo;
       row_sum[2 * tid + 1] = hi;
