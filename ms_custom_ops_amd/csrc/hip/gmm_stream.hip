@@ -20,6 +20,9 @@
 // MFMA, nothing else.  Per column group a wave parks its partial tile in LDS; afterwards the four waves'
 // tiles are added in wave order.  K split across workgroups, arrival counter and epilogue are those of the
 // row-major decode kernels.
+//
+// Further down: the multi-row forms for groups of more than 16 rows (W8A8 on packed weights; weight-only on packed and
+// on row-major [E,K,N] weights, the latter two with the chunk's x -- and where it pays the weights -- staged in LDS).
 #include <type_traits>
 #include <utility>
 
