@@ -323,12 +323,11 @@ void choose_plan(msco_gmm_op *op) {
     op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
     while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch *= 2;
-    // One group whose column strips do not fill the chip: the multi-row kernels have no K split, every workgroup walks
-    // all of K, and below 64 rows the 16-row kernels with their K split are faster although they stream the weights once
-    // per 16 rows (K = 4096, N = 11008, 32 / 64 rows: packed 24 / 41 us against 49 / 51; [E,K,N] 32 us against 39 at 32
-    // rows, where 64 rows do best in 32-row chunks, 40 us against 48 and 50).
-    if (e == 1 && m <= 64 && (n + 127) / 128 < num_cus)
-      op->stream_tch = (is_packed(d) || m <= 32) ? 1 : 2;
+    // One group whose column strips do not fill the chip: the multi-row kernels walk all of K in every workgroup (only
+    // the 128-row form has a K split, below), and for few rows the 16-row kernels with their K split are faster
+    // although they stream the weights once per 16 rows (K = 4096, N = 11008, 32 / 64 rows: packed 24 / 41 us against
+    // 49 / 51; [E,K,N] 32 us against 39 at 32 rows -- its 33 to 64 rows go on to the 128-row form, 39 us against 48).
+    if (e == 1 && (n + 127) / 128 < num_cus && m <= (is_packed(d) ? 64 : 32)) op->stream_tch = 1;
     if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8)
       op->stream_tch = tuning().stream_tch;
   }
@@ -351,7 +350,7 @@ void choose_plan(msco_gmm_op *op) {
     int want, cap;
     if (op->stream_tch > 1 && !is_w8a8(d)) {
       // multi-row weight-only kernels: strips of 16 column groups (256 columns) when they still give every CU two
-      // workgroups, else of 8; every workgroup walks all of K.
+      // workgroups, else of 8; every workgroup walks all of K (one exception below).
       const int64_t col_groups = (n + 15) / 16;
       op->strip_groups = ((col_groups + 15) / 16) * active >= 2 * (int64_t)num_cus ? 16 : 8;
       op->n_strips = (int)((col_groups + op->strip_groups - 1) / op->strip_groups);
