@@ -145,7 +145,10 @@ MSCO_API int msco_gmm_create(const msco_gmm_desc *desc, msco_gmm_handle *out_han
 
 /* Fix the shapes (shape-dependent work of Resize: kernel choice, grid, workspace size).
  * m = rows of x, k = reduction length, n = output columns, e = number of groups.
- * Replaces UpdateShape + Tiling + GetWorkspaceSize.  May be called again with new shapes. */
+ * Replaces UpdateShape + Tiling + GetWorkspaceSize.  May be called again with new shapes, but only while no launch
+ * of this handle is in flight on any stream: planning re-zeroes (with a synchronous hipMemset) the arrival counters
+ * that a split-K launch of the handle reduces through, and may free and re-allocate them.  Callers that re-plan per
+ * shape keep one handle per (shape, stream), as the operator layer's plan cache does. */
 MSCO_API int msco_gmm_plan(msco_gmm_handle h, int64_t m, int64_t k, int64_t n, int64_t e, size_t *workspace_bytes);
 
 /* Enqueue the computation.  inputs[MSCO_IN_COUNT] are device pointers (NULL = absent);

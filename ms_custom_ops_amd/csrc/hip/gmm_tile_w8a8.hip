@@ -665,7 +665,7 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
 const char *tile_cfg_name(int tile_cfg) {
   switch (tile_cfg) {
     case TILE_256x256: return "256x256x64";
-    case TILE_128x128: return "128x128";   // 128-byte K slabs on K-major weights, 64-byte on [E,K,N]
+    case TILE_128x128: return "128x128";   // (64- or 128-byte K slabs: the plan's wide_k_slabs, whatever the layout)
     case TILE_64x128: return "64x128";
     case TILE_128x256: return "128x256x64";
     case TILE_256x256_W4: return "256x256x128_w4";

@@ -143,40 +143,39 @@ void choose_plan(msco_gmm_op *op) {
   op->small_group_rows = 0;
 
   int family;
-  // packed weights are K-contiguous per column like [E,N,K]: the same tile kernels read them
-  // [E,K,N] weights run the same LDS-direct tile kernels as the K-major layouts (transpose reads turn them on the way
-  // out of LDS; rows of whole 16-column chunks, which the alignment rule guarantees) and follow the same tile rules;
-  // only the decode kernels of that layout are its own
-  const bool k_major = d.transpose_b != 0 || is_packed(d) || is_w8a8(d);
-  // (a group that overflows its 16-row chunk streams its weights twice, so on K-major weights 1.5 x the average has to
-  // fit; beyond that the 64 x 128 tile kernel with non-temporal weight loads is the better streamer -- 128 rows over 8
-  // experts, 470 MB of weights: 76 us against 82 us for the 32-row streaming kernel and 105 us for 16-row chunks;
-  // row-major [E,N,K]: 111 us against 140 us)
+  // All three W8A8 weight layouts follow the same tile rules: packed weights are K-contiguous per column like [E,N,K],
+  // and [E,K,N] weights run the same LDS-direct tile kernels (transpose reads turn them on the way out of LDS; rows of
+  // whole 16-column chunks, which the alignment rule guarantees).  Only the decode kernels are per layout.
+  // (a group that overflows its 16-row chunk streams its weights twice, so 1.5 x the average has to fit; beyond that
+  // the 64 x 128 tile kernel with non-temporal weight loads is the better streamer -- 128 rows over 8 experts, 470 MB
+  // of weights: 76 us against 82 us for the 32-row streaming kernel and 105 us for 16-row chunks; row-major [E,N,K]:
+  // 111 us against 140 us)
   // row-major [E,N,K] weights at decode sizes: a column's K bytes are contiguous and the columns are K bytes apart, which
   // suits the 64 x 128 tile's LDS-direct loads better than the decode kernel's 64-byte row pieces (K = 4096, N = 11008,
   // 1 / 16 rows: 15.8 / 15.9 us against 16.8 / 17.7 us; 32 rows over 8 experts, N = 14336: 103 against 115 us)
   const bool nk_rows = is_w8a8(d) && d.transpose_b != 0 && !is_packed(d);
   const int64_t avg_rows = (m + (e > 0 ? e : 1) - 1) / (e > 0 ? e : 1);
-  const bool many_small_groups = e > 1 && (k_major ? avg_rows + avg_rows / 2 : avg_rows) <= kSkinnyRows &&
+  const bool many_small_groups = e > 1 && avg_rows + avg_rows / 2 <= kSkinnyRows &&
                                  e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots;
   if (!aligned) {
     family = FAM_GENERIC;
   } else if (is_a16w8(d)) {
     family = FAM_SKINNY;  // the weight-only path is a decode path; large M re-streams weights per 16 rows
-  } else if (((m <= kSkinnyMaxRows && !(e == 1 && m > (k_major ? 1 : 2) * kSkinnyRows)) || many_small_groups) && !nk_rows) {
+  } else if (((m <= kSkinnyMaxRows && !(e == 1 && m > kSkinnyRows)) || many_small_groups) && !nk_rows) {
     // decode: few rows in total, or groups of about one 16-row chunk each (the weights stream once per chunk).  The
     // grid enumerates every (group, chunk) a malformed-to-the-limit group_list could fill; beyond a thousand slots
     // the empty workgroups cost more than the tile kernel's partial tiles.  A single group of more than one 16-row
-    // chunk (two on [E,K,N] weights) takes the small tile kernel with a K split instead (measured on packed weights,
-    // K = 4096, N = 11008: 32 / 48 / 64 rows 17.1 / 17.5 / 18.0 us against 18.7 / 24.4 / 26.3 us of the multi-row
-    // streaming kernel, which stays for several groups of a few dozen rows each).
+    // chunk takes the small tile kernel with a K split instead (measured on packed weights, K = 4096, N = 11008:
+    // 32 / 48 / 64 rows 17.1 / 17.5 / 18.0 us against 18.7 / 24.4 / 26.3 us of the multi-row streaming kernel, which
+    // stays for several groups of a few dozen rows each; [E,K,N] weights, same shape, 17 / 32 / 64 rows: 16.5 / 16.9 /
+    // 18.3 us).
     family = FAM_SKINNY;
   } else {
     family = FAM_TILE;
     // tile shape from shapes only: average rows per group and how many tiles fill 256 CUs
     const int64_t rows_per_group = m / (e > 0 ? e : 1);
     auto tiles = [&](int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
-    // several groups on K-major weights, a few dozen to a few hundred rows each: the launch is bound by the weight
+    // several groups, a few dozen to a few hundred rows each: the launch is bound by the weight
     // stream (every group's matrix is read once per m-tile of the group), so the m-tile should hold a whole group --
     // real routings are uneven, hence 1.5 x the average -- as long as there are tiles for most CUs.  Measured (E = 8,
     // K = 4096, N = 14336, packed; 64 x 128 / 128 x 128 / 256 x 256 tiles): 64 rows per group 112 / 97 / 100 us, 128 rows per
@@ -185,18 +184,18 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t cover = rows_per_group + rows_per_group / 2;
     const int64_t busy = (num_cus > 0 ? num_cus : kTileTargetWorkgroups) * 3 / 4;
     // (the persistent four-wave kernel: at least four 128-byte K slabs per tile, a group table that fits in LDS)
-    const bool w4_ok = k_major && k >= 512 && e <= 1024;
+    const bool w4_ok = k >= 512 && e <= 1024;
     if (e > 1 && w4_ok && cover > 128 && cover <= 384 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
-    } else if (e > 1 && k_major && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
+    } else if (e > 1 && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
       // (128 x 256 tiles re-read x half as often: 64 / 96 rows per group 93 / 99 us against 100 / 111 us)
       op->tile_cfg = group_tiles(128, 256) >= busy ? TILE_128x256 : TILE_128x128;
     } else if (e == 1 && w4_ok && tiles(256, 256) >= busy * 2 / 3 && tiles(128, 256) > busy * 4 / 3) {
-      // one group, K-major weights, a few hundred to a thousand rows: the persistent kernel already on half of the CUs
+      // one group, a few hundred to a thousand rows: the persistent kernel already on half of the CUs
       // when 128 x 256 tiles would no longer run in one round (N = 11008: M = 768 / 1024: 47 / 52 us against 63 / 68 us
       // with 128 x 128 tiles) ...
       op->tile_cfg = TILE_256x256_W4;
-    } else if (e == 1 && k_major && tiles(128, 256) >= busy * 4 / 5 && tiles(128, 256) <= busy * 4 / 3) {
+    } else if (e == 1 && tiles(128, 256) >= busy * 4 / 5 && tiles(128, 256) <= busy * 4 / 3) {
       // ... and 128 x 256 tiles while they do and fill most of the chip (M = 448 .. 640: 40 - 42 us against 45 - 47 us;
       // M = 384, 129 tiles: 41 us against 35 us with 128 x 128)
       op->tile_cfg = TILE_128x256;
@@ -206,8 +205,8 @@ void choose_plan(msco_gmm_op *op) {
       op->tile_cfg = TILE_128x128;
     } else if (tiles(128, 128) >= 512) {
       op->tile_cfg = TILE_128x128;
-    } else if (k_major && rows_per_group >= 192 && tiles(128, 128) > kTileSplitMaxTiles) {
-      // K-major weights, a few hundred rows: 128 x 128 tiles on at least half of the CUs beat twice as many 64 x 128
+    } else if (rows_per_group >= 192 && tiles(128, 128) > kTileSplitMaxTiles) {
+      // a few hundred rows: 128 x 128 tiles on at least half of the CUs beat twice as many 64 x 128
       // tiles (measured: M = 256, N = 11008: 32 us against 44 us); with fewer tiles the K split of the small tile wins
       op->tile_cfg = TILE_128x128;
     } else {
@@ -257,12 +256,9 @@ void choose_plan(msco_gmm_op *op) {
         return rounds * (slabs + 10 + exchange);
       };
       int want = 1;
-      if (t <= kTileSplitMaxTiles && k_major) {
+      if (t <= kTileSplitMaxTiles) {
         for (int sl = 2; sl <= std::min(kMaxSplitK, cap); ++sl)
           if (split_cost(sl) < split_cost(want)) want = sl;
-      } else if (t <= kTileSplitMaxTiles) {
-        // [E,K,N] weights (64-byte slabs, two workgroups per CU, register-transposed weights): about one workgroup per CU
-        want = std::max(1, std::min(std::min((int)((cus + t / 2) / std::max<int64_t>(t, 1)), kMaxSplitK), cap));
       }
       const int forced_split = d.force_split_k > 0 ? d.force_split_k : tuning().tile_split_k;
       if (forced_split > 0) want = std::min(forced_split, cap);
@@ -274,8 +270,8 @@ void choose_plan(msco_gmm_op *op) {
       // 128-byte K slabs (a 4-stage ring of them takes most of a CU's LDS: one workgroup per CU) when the workgroups
       // run in one round; more tiles than CUs keep 64-byte slabs and two workgroups per CU (M = 512, N = 11008: 344
       // tiles, 46.8 us against 50.1 us)
-      op->wide_k_slabs = k_major && t * want <= (num_cus > 0 ? num_cus : kTileTargetWorkgroups);
-      if (tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;
+      op->wide_k_slabs = t * want <= (num_cus > 0 ? num_cus : kTileTargetWorkgroups);
+      if (tuning().tile_wide_k >= 0) op->wide_k_slabs = tuning().tile_wide_k != 0;
     }
     if (op->tile_cfg == TILE_128x128 || op->tile_cfg == TILE_64x128 || op->tile_cfg == TILE_128x256) {
       // Non-temporal weight loads: a weight stream of tens of megabytes that at most two m-tiles read should not push x
@@ -290,7 +286,7 @@ void choose_plan(msco_gmm_op *op) {
       const int64_t nt_bytes = is_packed(d) ? ((int64_t)32 << 20) : ((int64_t)64 << 20);
       op->w_nontemporal = (is_packed(d) || d.transpose_b == 0) && e * k * n >= nt_bytes && (group_rows + bm - 1) / bm <= 2;
     }
-    if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0 && k_major) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
+    if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
   }
   // Many experts with uneven loads (a skewed routing): every group of a few rows costs the persistent kernel a whole
   // 256-row m-tile per n-tile.  The groups of at most 64 rows go to a second launch of 64 x 128 tiles instead, which

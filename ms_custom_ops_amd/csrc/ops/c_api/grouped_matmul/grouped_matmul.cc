@@ -132,7 +132,7 @@ TypeId InferGroupedMatmulOutputType(TypeId x_dtype, TypeId weight_dtype, TypeId 
 
 // What this backend does not implement is refused up front with a precise message.
 static void CheckBackendSupport(TypeId x_dtype, bool has_scale, bool has_antiquant, TypeId bias_dtype, bool bias_none,
-                                bool transpose_a, int64_t x_format) {
+                                int64_t x_format) {
   if (x_dtype != kNumberTypeInt8) {
     MS_LOG_EXCEPTION << "For GroupedMatmul, the HIP backend implements the quantized int8 path only, but got x dtype:"
                      << x_dtype;
@@ -146,9 +146,6 @@ static void CheckBackendSupport(TypeId x_dtype, bool has_scale, bool has_antiqua
   }
   if (!bias_none && bias_dtype != kNumberTypeInt32) {
     MS_LOG_EXCEPTION << "For GroupedMatmul, the quantized path takes an int32 'bias', but got:" << bias_dtype;
-  }
-  if (transpose_a) {
-    MS_LOG_EXCEPTION << "For GroupedMatmul, transpose_a=True is not implemented by the HIP backend.";
   }
   if (x_format != static_cast<int64_t>(DataFormat::ND)) {
     MS_LOG_EXCEPTION << "For GroupedMatmul, x_format must be 0 (ND) on the HIP backend, but got:" << x_format;
@@ -241,9 +238,18 @@ class CustomGroupedMatmul : public HipGmmKernelMod {
  protected:
   // backend order {x, weight, bias, scale, group_list, per_token_scale, antiquant_scale}, the order
   // the reference hands to its kernel object (grouped_matmul.cc:201-207)
+  // transpose_a (ops/c_api/grouped_matmul/grouped_matmul.cc:73-74,216-218 of the reference): x arrives [K, M].  The
+  // kernels read K-contiguous rows, so Launch turns it into [M, K] in a workspace slice of its own; here x is
+  // presented with the shape it will have then.
   TensorList GetBackendInputs(const KernelTensorList &inputs) override {
     auto t = [&](GroupedMatmulInputIndex i) { return inputs[I(i)].tensor; };
-    return {t(GroupedMatmulInputIndex::kGmmXIndex),          t(GroupedMatmulInputIndex::kGmmWeightIndex),
+    ms::Tensor x = t(GroupedMatmulInputIndex::kGmmXIndex);
+    transpose_x_ = inputs[I(GroupedMatmulInputIndex::kGmmTransposeAIndex)].GetValueWithCheck<bool>();
+    if (transpose_x_) {
+      CheckContiguous(kernel_name_, {x}, true);
+      x = x.Slice(0, ShapeVector{x.shape()[kIndex1], x.shape()[kIndex0]});
+    }
+    return {x,          t(GroupedMatmulInputIndex::kGmmWeightIndex),
             t(GroupedMatmulInputIndex::kGmmBiasIndex),       t(GroupedMatmulInputIndex::kGmmScaleIndex),
             t(GroupedMatmulInputIndex::kGmmGroupListIndex),  t(GroupedMatmulInputIndex::kGmmPerTokenScaleIndex),
             t(GroupedMatmulInputIndex::kGmmAntiquantScaleIndex), ms::Tensor()};
@@ -251,12 +257,11 @@ class CustomGroupedMatmul : public HipGmmKernelMod {
 
   msco_gmm_desc CreateKernel(const KernelTensorList &inputs, const TensorList &in,
                              const std::vector<ms::Tensor> &outputs) override {
-    const bool ta = inputs[I(GroupedMatmulInputIndex::kGmmTransposeAIndex)].GetValueWithCheck<bool>();
     const bool tb = inputs[I(GroupedMatmulInputIndex::kGmmTransposeBIndex)].GetValueWithCheck<bool>();
     const int64_t x_format = inputs[I(GroupedMatmulInputIndex::kGmmXFormatIndex)].GetValueWithCheck<int64_t>();
     CheckBackendSupport(in[MSCO_IN_X].data_type(), in[MSCO_IN_SCALE].is_defined(),
                         in[MSCO_IN_ANTIQUANT_SCALE].is_defined(), in[MSCO_IN_BIAS].data_type(),
-                        !in[MSCO_IN_BIAS].is_defined(), ta, x_format);
+                        !in[MSCO_IN_BIAS].is_defined(), x_format);
     const GmmProblem pb = MakeGroupedMatmulProblem(in, tb);
     CheckOptionalShapes(in, pb.m, pb.n, pb.e);
     return MakeGroupedMatmulDesc(in, outputs.at(0).data_type(), tb);
@@ -289,7 +294,7 @@ class GroupedMatmulRunner : public HipGmmPyboostRunner {
   msco_gmm_desc CreateKernel(const TensorList &in, const TensorList &outputs) override {
     CheckBackendSupport(in[MSCO_IN_X].data_type(), in[MSCO_IN_SCALE].is_defined(),
                         in[MSCO_IN_ANTIQUANT_SCALE].is_defined(), in[MSCO_IN_BIAS].data_type(), !with_bias_,
-                        transpose_a_, static_cast<int64_t>(x_format_));
+                        static_cast<int64_t>(x_format_));
     const GmmProblem pb = MakeGroupedMatmulProblem(in, transpose_b_);
     CheckOptionalShapes(in, pb.m, pb.n, pb.e);
     return MakeGroupedMatmulDesc(in, outputs.at(0).data_type(), transpose_b_);
@@ -317,7 +322,20 @@ std::vector<ms::Tensor> hip_grouped_matmul(const ms::Tensor &x, const ms::Tensor
   runner->SetParam(transpose_a, transpose_b, bias.has_value());
   runner->SetXFormat(static_cast<DataFormat>(x_format));
 
-  std::vector<ms::Tensor> inputs = {x,
+  auto out_shape = InferGroupedMatmulOutputShape(x.shape(), weight.shape(), group_list.shape(), transpose_a,
+                                                 transpose_b, x.data_type());
+  // transpose_a: x arrives [K, M]; the kernels read K-contiguous rows, so it is turned into [M, K] once
+  ms::Tensor x_rows = x;
+  if (transpose_a && x.data_type() == kNumberTypeInt8) {
+    CheckContiguous(op_name, {x}, true);
+    const int64_t k = x.shape()[kIndex0], m = x.shape()[kIndex1];
+    x_rows = AllocateTensor(kNumberTypeInt8, ShapeVector{m, k});
+    if (m > 0 && k > 0) {
+      const int rc = msco_transpose_2d(x.GetDataPtr(), x_rows.GetDataPtr(), 1, k, m, 1, CurrentStream());
+      if (rc != MSCO_OK) MS_LOG_EXCEPTION << "For " << op_name << ", transposing x failed: " << msco_status_string(rc);
+    }
+  }
+  std::vector<ms::Tensor> inputs = {x_rows,
                                     weight,
                                     GetTensorOrEmpty(bias),
                                     GetTensorOrEmpty(scale),
@@ -325,8 +343,6 @@ std::vector<ms::Tensor> hip_grouped_matmul(const ms::Tensor &x, const ms::Tensor
                                     GetTensorOrEmpty(per_token_scale),
                                     GetTensorOrEmpty(antiquant_scale),
                                     ms::Tensor()};
-  auto out_shape = InferGroupedMatmulOutputShape(x.shape(), weight.shape(), group_list.shape(), transpose_a,
-                                                 transpose_b, x.data_type());
   auto out_type = InferGroupedMatmulOutputType(
     x.data_type(), weight.data_type(), group_list.data_type(), inputs[MSCO_IN_BIAS].data_type(), !bias.has_value(),
     inputs[MSCO_IN_SCALE].data_type(), !scale.has_value(), inputs[MSCO_IN_PER_TOKEN_SCALE].data_type(),

@@ -1,5 +1,6 @@
 #include "ops/framework/hip_backend/hip_gmm_runner.h"
 
+#include <algorithm>
 #include <cstring>
 #include <sstream>
 
@@ -132,7 +133,10 @@ std::vector<size_t> HipGmmKernelMod::Resize(const KernelTensorList &inputs, cons
   problem_ = GetProblem(inputs, backend_inputs, outputs);
   plan_stream_ = CurrentStream();
   plan_ = GmmPlanCache::GetInstance().GetOrCreate(kernel_name_, desc_, problem_, plan_stream_);
-  return plan_->workspace_bytes ? std::vector<size_t>{plan_->workspace_bytes} : std::vector<size_t>{};
+  std::vector<size_t> sizes;
+  if (plan_->workspace_bytes) sizes.push_back(plan_->workspace_bytes);
+  if (transpose_x_) sizes.push_back(static_cast<size_t>(std::max<int64_t>(problem_.m * problem_.k, 1)));
+  return sizes;
 }
 
 bool HipGmmKernelMod::Launch(const KernelTensorList &inputs, const std::vector<ms::Tensor> &workspace,
@@ -148,8 +152,21 @@ bool HipGmmKernelMod::Launch(const KernelTensorList &inputs, const std::vector<m
   for (size_t i = 0; i < backend_inputs.size() && i < MSCO_IN_COUNT; ++i) {
     addrs[i] = backend_inputs[i].is_defined() ? backend_inputs[i].GetDataPtr() : nullptr;
   }
-  void *ws = workspace.empty() ? nullptr : workspace[0].GetDataPtr();
-  const size_t ws_bytes = workspace.empty() ? 0 : workspace[0].nbytes();
+  const bool has_ws = plan_->workspace_bytes > 0;
+  if (workspace.size() != (has_ws ? 1u : 0u) + (transpose_x_ ? 1u : 0u)) {
+    MS_LOG_EXCEPTION << "For " << kernel_name_ << ", Launch got " << workspace.size() << " workspace tensors, Resize asked for "
+                     << (has_ws ? 1 : 0) + (transpose_x_ ? 1 : 0);
+  }
+  void *ws = has_ws ? workspace[0].GetDataPtr() : nullptr;
+  const size_t ws_bytes = has_ws ? workspace[0].nbytes() : 0;
+  if (transpose_x_) {
+    void *rows = workspace.back().GetDataPtr();
+    if (problem_.m > 0 && problem_.k > 0) {
+      const int rc = msco_transpose_2d(addrs[MSCO_IN_X], rows, 1, problem_.k, problem_.m, 1, stream);
+      if (rc != MSCO_OK) MS_LOG_EXCEPTION << "For " << kernel_name_ << ", transposing x failed: " << msco_status_string(rc);
+    }
+    addrs[MSCO_IN_X] = rows;
+  }
   const GmmPlanPtr plan = plan_;   // the launch drops the GIL: another thread's Resize may replace plan_ meanwhile
   LaunchPlan(kernel_name_, plan, addrs, outputs.at(0).GetDataPtr(), ws, ws_bytes, stream);
   return true;

@@ -105,6 +105,9 @@ class HipGmmKernelMod : public KernelMod {
   virtual GmmProblem GetProblem(const KernelTensorList &inputs, const TensorList &backend_inputs,
                                 const std::vector<ms::Tensor> &outputs) = 0;
   std::string kernel_name_;
+  // set by GetBackendInputs when x arrives [K, M] and was presented as [M, K]: Resize asks for one more workspace
+  // slice of M K bytes (the last one) and Launch transposes x into it first
+  bool transpose_x_{false};
   GmmPlanPtr plan_;
   void *plan_stream_{nullptr};   // the stream plan_ belongs to (kernel objects are per stream)
   msco_gmm_desc desc_{};         // what Resize planned for: Launch fetches the plan of its own stream with these

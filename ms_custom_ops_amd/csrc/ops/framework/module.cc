@@ -4,6 +4,7 @@
 #include "ops/framework/module.h"
 
 #include <map>
+#include <memory>
 #include <mutex>
 #include <sstream>
 
@@ -98,17 +99,35 @@ std::string InputSignature(const KernelTensorList &inputs) {
 }
 
 // One kernel module per operator, as a graph holds one per node: Init ran once, Resize runs again only when the
-// input signature changes (docs/ops_develop_guide.md:193-197).
+// input signature changes (docs/ops_develop_guide.md:193-197).  A module keeps what Resize planned in its members
+// and Launch reads them, so a node's Resize, workspace allocation and Launch form one critical section under the
+// node's own mutex: a second thread (or a re-entrant call) with another signature waits for the pending Launch
+// instead of re-planning the module under it.
 struct GraphNode {
+  std::mutex mu;   // taken with the GIL released (see LockNode), held across Resize .. Launch
   std::shared_ptr<KernelMod> kernel;
   std::string signature;
   std::vector<size_t> workspace_sizes;
   size_t inits{0}, resizes{0}, launches{0};
 };
-std::mutex g_nodes_mu;
-std::map<std::string, GraphNode> &GraphNodes() {
-  static auto *nodes = new std::map<std::string, GraphNode>();   // leaked: kernel modules may hold device state
+std::mutex g_nodes_mu;   // guards the map only
+std::map<std::string, std::unique_ptr<GraphNode>> &GraphNodes() {
+  static auto *nodes = new std::map<std::string, std::unique_ptr<GraphNode>>();   // leaked: kernel modules may hold device state
   return *nodes;
+}
+GraphNode &NodeOf(const std::string &name) {
+  std::lock_guard<std::mutex> lock(g_nodes_mu);
+  auto &slot = GraphNodes()[name];
+  if (slot == nullptr) slot = std::make_unique<GraphNode>();
+  return *slot;
+}
+// Lock order is node mutex first, interpreter lock second.  The launch below drops the interpreter lock while it
+// holds the node mutex, so a thread must never wait for the node mutex while it holds the interpreter lock.
+std::unique_lock<std::mutex> LockNode(GraphNode &node) {
+  std::unique_lock<std::mutex> lock(node.mu, std::defer_lock);
+  py::gil_scoped_release no_gil;
+  lock.lock();
+  return lock;
 }
 
 // Graph-mode execution of one registered op: the reference's compile-time infer plus the kernel
@@ -124,34 +143,28 @@ std::vector<ms::Tensor> GraphRun(const std::string &name, const py::list &args) 
   if (shapes.size() != types.size()) MS_LOG_EXCEPTION << "For " << name << ", infer returned mismatching outputs.";
   std::vector<ms::Tensor> outputs;
   for (size_t i = 0; i < shapes.size(); ++i) outputs.push_back(AllocateTensor(types[i], shapes[i]));
-  std::shared_ptr<KernelMod> kernel;
-  std::vector<size_t> ws_sizes;
-  {
-    std::lock_guard<std::mutex> lock(g_nodes_mu);
-    GraphNode &node = GraphNodes()[name];
-    if (node.kernel == nullptr) {
-      node.kernel = reg->kernel_mod();
-      if (!node.kernel->Init(inputs, outputs)) {
-        node.kernel = nullptr;
-        MS_LOG_EXCEPTION << "For " << name << ", KernelMod::Init failed.";
-      }
-      ++node.inits;
-      node.signature.clear();
+  GraphNode &node = NodeOf(name);
+  std::unique_lock<std::mutex> lock = LockNode(node);
+  if (node.kernel == nullptr) {
+    node.kernel = reg->kernel_mod();
+    if (!node.kernel->Init(inputs, outputs)) {
+      node.kernel = nullptr;
+      MS_LOG_EXCEPTION << "For " << name << ", KernelMod::Init failed.";
     }
-    const std::string signature = InputSignature(inputs);
-    if (node.resizes == 0 || signature != node.signature) {
-      node.signature.clear();                       // stays empty if Resize throws: the next call plans again
-      node.workspace_sizes = node.kernel->Resize(inputs, outputs);
-      node.signature = signature;
-      ++node.resizes;
-    }
-    ++node.launches;
-    kernel = node.kernel;
-    ws_sizes = node.workspace_sizes;
+    ++node.inits;
+    node.signature.clear();
   }
+  const std::string signature = InputSignature(inputs);
+  if (node.resizes == 0 || signature != node.signature) {
+    node.signature.clear();                       // stays empty if Resize throws: the next call plans again
+    node.workspace_sizes = node.kernel->Resize(inputs, outputs);
+    node.signature = signature;
+    ++node.resizes;
+  }
+  ++node.launches;
   std::vector<ms::Tensor> workspace;
-  for (size_t sz : ws_sizes) workspace.push_back(AllocateTensor(kNumberTypeInt8, ShapeVector{static_cast<int64_t>(sz)}));
-  if (!kernel->Launch(inputs, workspace, outputs, CurrentStream())) {
+  for (size_t sz : node.workspace_sizes) workspace.push_back(AllocateTensor(kNumberTypeInt8, ShapeVector{static_cast<int64_t>(sz)}));
+  if (!node.kernel->Launch(inputs, workspace, outputs, CurrentStream())) {
     MS_LOG_EXCEPTION << "For " << name << ", KernelMod::Launch failed.";
   }
   return outputs;
@@ -198,11 +211,16 @@ PYBIND11_MODULE(MS_EXTENSION_NAME, m) {
     return py::make_tuple(c.hits(), c.misses(), c.size());
   });
   m.def("_graph_node_stats", [](const std::string &name) -> py::tuple {
-    std::lock_guard<std::mutex> lock(ms_custom_ops::g_nodes_mu);
-    auto &nodes = ms_custom_ops::GraphNodes();
-    auto it = nodes.find(name);
-    if (it == nodes.end()) return py::make_tuple(0, 0, 0);
-    return py::make_tuple(it->second.inits, it->second.resizes, it->second.launches);
+    ms_custom_ops::GraphNode *node = nullptr;
+    {
+      std::lock_guard<std::mutex> lock(ms_custom_ops::g_nodes_mu);
+      auto &nodes = ms_custom_ops::GraphNodes();
+      auto it = nodes.find(name);
+      if (it == nodes.end()) return py::make_tuple(0, 0, 0);
+      node = it->second.get();
+    }
+    std::unique_lock<std::mutex> lock = ms_custom_ops::LockNode(*node);
+    return py::make_tuple(node->inits, node->resizes, node->launches);
   }, "(Init, Resize, Launch) calls of an operator's graph-mode kernel module so far");
   m.def("_plan_cache_clear", []() { ms_custom_ops::GmmPlanCache::GetInstance().Clear(); });
   m.def("_backend_abi_version", []() { return msco_gmm_abi_version(); });

@@ -26,14 +26,25 @@ CASES = [
     ("skinny_nk", cabi.OV_SKINNY, True, False, RAGGED),
     ("skinny_16w", cabi.OV_AUTO, False, False, (16, 512, 384, 1, [16])),
     ("stream", cabi.OV_AUTO, False, True, (24, 512, 384, 4, [5, 5, 17, 24])),
-    ("stream_rows", cabi.OV_AUTO, False, True, (48, 512, 384, 1, [48])),
+    ("stream_rows", cabi.OV_AUTO, False, True, (48, 512, 384, 2, [20, 48])),
     ("tile64", cabi.OV_TILE_64, True, False, RAGGED),
     ("tile128", cabi.OV_TILE_128, False, False, RAGGED),
     ("tile256", cabi.OV_TILE_256, False, False, RAGGED),
     ("tile256_w4", cabi.OV_TILE_256_W4, True, False, (700, 640, 512, 3, [300, 300, 700])),
     ("tile256_w4_packed", cabi.OV_TILE_256_W4, False, True, (700, 640, 512, 3, [300, 300, 700])),
     ("tile256_w4_kn", cabi.OV_TILE_256_W4, False, False, (700, 640 + 48, 512 - 16, 3, [300, 300, 700])),   # [E,K,N] through transpose reads, K and N tails
+    # 128 x 256 tiles (several groups of about a hundred rows, enough columns to fill the chip with them)
+    ("tile128x256", cabi.OV_AUTO, True, False, (800, 256, 6144, 8, [90, 200, 310, 400, 400, 530, 700, 800])),
+    ("tile128x256_packed", cabi.OV_AUTO, False, True, (800, 256, 6144, 8, [90, 200, 310, 400, 400, 530, 700, 800])),
+    # sixteen uneven groups: the persistent kernel takes the large ones, a second launch of 64 x 128 tiles the small ones
+    ("two_launches_packed", cabi.OV_TILE_256_W4, False, True,
+     (1200, 512, 512, 16, [300, 303, 303, 373, 437, 502, 503, 783, 783, 800, 830, 900, 964, 1100, 1101, 1200])),
+    ("two_launches_kn", cabi.OV_TILE_256_W4, False, False,
+     (1200, 512, 512, 16, [300, 303, 303, 373, 437, 502, 503, 783, 783, 800, 830, 900, 964, 1100, 1101, 1200])),
 ]
+# what the plan of a case has to name, so that the case keeps reaching the code it is there for
+PLAN_MUST_NAME = {"tile128x256": "128x256", "tile128x256_packed": "128x256", "two_launches_packed": "small_groups=64",
+                  "two_launches_kn": "small_groups=64", "stream_rows": "stream_rows"}
 
 
 def _reference(x, w, gl, bias, scale, pt, act):
@@ -69,6 +80,7 @@ def test_fused_activation_every_kernel_family(name, override, transpose_b, packe
         bits, info = run_w8a8(x, w, gl, bias, scale, pt, out=out, transpose_b=transpose_b, override=override, packed=packed,
                               act_type=act, launches=2)
         got = O.bf16_bits_to_f32(bits) if out == "bf16" else bits.view(np.float16).astype(np.float32)
+        assert PLAN_MUST_NAME.get(name, "") in info, info
         if act == O.ACT_RELU:
             want = O.f32_to_bf16_bits(ref64.astype(np.float32)) if out == "bf16" else O.f32_to_f16(ref64.astype(np.float32)).view(np.uint16)
             assert np.array_equal(bits[:last], want[:last]), info
@@ -76,13 +88,26 @@ def test_fused_activation_every_kernel_family(name, override, transpose_b, packe
             _assert_close(got[:last], ref64[:last], out, info)
 
 
+# weight-only shapes (m, k, e, group_list, what the plan must name): the 16-row decode kernels, the multi-row kernels
+# with chunks of 32, 64 and 128 rows, and one group of 200 rows whose 128-row chunks split K across workgroups (the
+# epilogue then runs in the last arriver)
+A16_SHAPES = [
+    (32, 512, 4, [7, 7, 20, 32], ""),
+    (40, 512, 2, [20, 40], "_rows"),
+    (48, 512, 2, [40, 48], "_rows"),
+    (130, 512, 2, [100, 130], "_rows"),
+    (200, 1024, 1, [200], "_rows"),
+]
+
+
 @pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("packed", [False, True])
-def test_fused_activation_weight_only(act, packed):
+@pytest.mark.parametrize("shape", A16_SHAPES, ids=[f"m{s[0]}e{s[2]}" for s in A16_SHAPES])
+def test_fused_activation_weight_only(act, packed, shape):
     from gpu_utils import run_a16w8
     rng = np.random.default_rng(3)
-    m, k, n, e = 32, 512, 384, 4
-    gl = [7, 7, 20, 32]
+    m, k, e, gl, must_name = shape
+    n = 384
     xf = rng.standard_normal((m, k)).astype(np.float32)
     x_bits = O.f32_to_bf16_bits(xf)
     w = rng.integers(-127, 128, (e, k, n), dtype=np.int8)
@@ -92,6 +117,7 @@ def test_fused_activation_weight_only(act, packed):
     exact = O.a16w8_grouped_f64(xv, w, sv, ov, gl)
     plain, info = run_a16w8(x_bits, w, s_bits, o_bits, gl, packed=packed)
     bits, info = run_a16w8(x_bits, w, s_bits, o_bits, gl, packed=packed, act_type=act)
+    assert must_name in info and (m != 200 or "split_k=1 " not in info), info
     got = O.bf16_bits_to_f32(bits).astype(np.float64)
     # the matmul itself is floating point (tolerance 2^-7 |exact| + 1e-5 sum|terms|, as for the plain weight-only path);
     # the activations are 1.13-Lipschitz, so the same allowance carries through them, plus the output rounding

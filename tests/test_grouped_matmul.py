@@ -86,6 +86,32 @@ def test_gmm_real_moe_shape(device, trans_b):
     custom_grouped_matmul(1024, 5120, 1344, 8, trans_b=trans_b, with_pertoken_scale=True, out_dtype=torch.bfloat16)
 
 
+@pytest.mark.parametrize("exec_mode", MODES)
+@pytest.mark.parametrize("shape", [[40, 64, 128, 8], [1000, 512, 256, 8]])
+def test_gmm_transpose_a(device, exec_mode, shape):
+    """transpose_a=True: x arrives [K, M] (the reference passes the flag down to its kernel,
+    ops/c_api/grouped_matmul/grouped_matmul.cc:73-74,216-218); same result as the [M, K] call, bit for bit, twice in a
+    row (the graph-mode module keeps its extra workspace slice across calls) and with a second shape."""
+    m, k, n, e = shape
+    rng = np.random.default_rng(m)
+    x = rng.integers(-127, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, (e, k, n), dtype=np.int8)
+    s = (rng.random((e, n)) / 1000).astype(np.float32)
+    ps = rng.random(m).astype(np.float32)
+    b = rng.integers(-10, 10, (e, n)).astype(np.int32)
+    gl = O.random_group_list(m, e, rng).astype(np.int32)
+    ref = O.grouped_matmul_w8a8(x, w, gl, b, s, ps)
+    xt = _t(x.T)   # [K, M], contiguous
+    with ms_custom_ops.exec_mode(exec_mode):
+        for _ in range(2):
+            out = ms_custom_ops.grouped_matmul(xt, _t(w), _t(gl), _t(b), _t(s), _t(ps), None, True, False,
+                                               output_dtype=torch.bfloat16)
+            assert out.shape == (m, n)
+            assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), ref)
+        with pytest.raises(RuntimeError, match="must have the same dimension of 'k'"):
+            ms_custom_ops.grouped_matmul(_t(x), _t(w), _t(gl), _t(b), _t(s), _t(ps), None, True, False)
+
+
 def test_gmm_errors(device):
     x = torch.zeros(32, 64, dtype=torch.int8, device="cuda")
     w = torch.zeros(8, 64, 128, dtype=torch.int8, device="cuda")
