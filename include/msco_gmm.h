@@ -195,6 +195,14 @@ MSCO_API int msco_gmm_a8w4(const int8_t *x, const void *weight, const int32_t *g
                            const float *weight_scale, void *out, int64_t m, int64_t k, int64_t n, int64_t e,
                            int64_t group_size, void *stream);
 
+/* 4-bit weights of grouped_matmul_v4_cops widened to int8 on the device.  The reference hands its qint4x2 weight
+ * [E, K, N / 2] to aclnnGroupedMatmulV4 as an int4 tensor of shape [E, K, N] (UnifyWeightShape,
+ * ops/c_api/grouped_matmul_v4_cops/grouped_matmul_v4_cops.cc:56-66,274-295); this backend multiplies int8, so the op
+ * layer widens the nibbles first: byte i of src holds element 2 i in its low nibble and element 2 i + 1 in its high
+ * nibble (tests/st/test_grouped_matmul_v4_cops.py:458-460), each a signed 4-bit value; dst receives 2 * src_bytes
+ * int8 values.  Both pointers 16-byte aligned.  Enqueued on the given stream, nothing is allocated. */
+MSCO_API int msco_unpack_int4(const void *src, void *dst, int64_t src_bytes, void *stream);
+
 /* Weight prepack, once at load time -- the counterpart of the reference's trans_data ND -> FRACTAL_NZ step
  * (ops/c_api/trans_data/trans_data.cc:203-223, shape contract ops/c_api/trans_data/trans_data.md:45-99).
  * src is [e,k,n] int8 (or [e,n,k] when src_transposed); dst receives e * msco_packed_weight_bytes(k, n) bytes in the

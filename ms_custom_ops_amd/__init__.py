@@ -50,7 +50,8 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
 
 __all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "grouped_matmul_w4", "quant_batch_matmul", "moe_init_routing_v2", "moe_init_routing_quant",
            "moe_token_unpermute", "set_context", "get_context", "exec_mode",
-           "GRAPH_MODE", "PYNATIVE_MODE", "dtype_to_type_id", "type_id_to_dtype", "plan_cache_stats", "trans_data"]
+           "GRAPH_MODE", "PYNATIVE_MODE", "dtype_to_type_id", "type_id_to_dtype", "plan_cache_stats", "trans_data",
+           "qint4x2", "QInt4x2", "as_qint4x2"]
 
 GRAPH_MODE = 0
 PYNATIVE_MODE = 1
@@ -103,10 +104,33 @@ def exec_mode(mode: int):
         set_context(prev)
 
 
+qint4x2 = 50   # TypeId of MindSpore's packed 4-bit type (two signed 4-bit values per stored element)
+
+
+class QInt4x2:
+    """Marks an int8 / uint8 tensor as qint4x2 data (torch has no 4-bit dtype): every byte holds two signed 4-bit values,
+    the even-indexed one in the low nibble, and the stored shape is the logical shape with the last axis halved -- what
+    ``Tensor(w_int4_np, dtype=ms.qint4x2)`` is in the reference (tests/st/test_grouped_matmul_v4_cops.py:458-460,479)."""
+
+    def __init__(self, tensor: torch.Tensor):
+        if not isinstance(tensor, torch.Tensor) or tensor.dtype not in (torch.int8, torch.uint8):
+            raise TypeError("qint4x2 data is carried by an int8 or uint8 tensor")
+        self.tensor = tensor
+
+
+def as_qint4x2(tensor: torch.Tensor) -> QInt4x2:
+    return QInt4x2(tensor)
+
+
 # ---- framework hooks: PyTorch owns device memory and streams -------------------------------------
 def _wrap(t: Optional[torch.Tensor]):
     if t is None:
         return None
+    if isinstance(t, QInt4x2):
+        w = t.tensor
+        if not w.is_cuda:
+            raise ValueError("ms_custom_ops_amd operators take GPU tensors; got a tensor on " + str(w.device))
+        return _C.Tensor(w.data_ptr(), qint4x2, list(w.shape), list(w.stride()), w)
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"expected a torch.Tensor, got {type(t).__name__}")
     if not t.is_cuda:

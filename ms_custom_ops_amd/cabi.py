@@ -34,7 +34,7 @@ WL_ROW_MAJOR, WL_PACKED = 0, 1
 
 EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco_gmm_plan_info", "msco_gmm_destroy",
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
-                    "msco_packed_weight_bytes", "msco_pack_weight", "msco_gmm_a8w4",
+                    "msco_packed_weight_bytes", "msco_pack_weight", "msco_gmm_a8w4", "msco_unpack_int4",
                     "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_init_routing_v2_quant",
                     "msco_moe_token_unpermute", "msco_probe_mfma", "msco_probe_read", "msco_gmm_launch_static")
 STATIC_WORKSPACE_BYTES = 32 << 20
@@ -94,6 +94,8 @@ def load():
         lib.msco_moe_init_routing_v2.restype = ctypes.c_int
         lib.msco_moe_init_routing_v2.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_size_t] + [ctypes.c_int64] * 4 + \
                                                 [ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_unpack_int4.restype = ctypes.c_int
+        lib.msco_unpack_int4.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         lib.msco_gmm_a8w4.restype = ctypes.c_int
         lib.msco_gmm_a8w4.argtypes = [ctypes.c_void_p] * 6 + [ctypes.c_int64] * 5 + [ctypes.c_void_p]
         lib.msco_moe_init_routing_v2_quant.restype = ctypes.c_int
@@ -144,6 +146,12 @@ def gmm_a8w4(x: int, weight: int, group_list: int, x_scale: int, weight_scale: i
     vp = lambda v: ctypes.c_void_p(v if v else None)
     _check("msco_gmm_a8w4", load().msco_gmm_a8w4(vp(x), vp(weight), vp(group_list), vp(x_scale), vp(weight_scale), vp(out),
                                                  m, k, n, e, group_size, vp(stream)))
+
+
+def unpack_int4(src: int, dst: int, src_bytes: int, stream: Optional[int] = None):
+    """Raw-pointer call of msco_unpack_int4 (see include/msco_gmm.h): src_bytes bytes of nibble pairs -> 2 * src_bytes int8."""
+    vp = lambda v: ctypes.c_void_p(v if v else None)
+    _check("msco_unpack_int4", load().msco_unpack_int4(vp(src), vp(dst), src_bytes, vp(stream)))
 
 
 def probe_mfma(operands: int, sink: int, iters: int, stream: Optional[int] = None):

@@ -192,8 +192,55 @@ __global__ void __launch_bounds__(256) gmm_a8w4_kernel(const int8_t *x, const un
   }
 }
 
+// 4-bit values widened to int8: 16 source bytes (32 nibbles) -> 32 bytes per thread, low nibble first, sign extended
+__global__ void __launch_bounds__(256) unpack_int4_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, long long pieces,
+                                                          const unsigned char *src_tail, signed char *dst_tail, int tail_bytes) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  auto widen = [](unsigned w, unsigned &lo, unsigned &hi) {
+    // bytes b0 b1 b2 b3 of w -> lo = {b0.lo, b0.hi, b1.lo, b1.hi}, hi = {b2.lo, b2.hi, b3.lo, b3.hi}, each nibble sign extended
+    const unsigned even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+    const unsigned l = __builtin_amdgcn_perm(odd, even, 0x05010400u);   // e0 o0 e1 o1
+    const unsigned h = __builtin_amdgcn_perm(odd, even, 0x07030602u);   // e2 o2 e3 o3
+    // sign extension of a 4-bit value held in a byte: (v ^ 8) - 8, per byte without carries between bytes
+    lo = ((l ^ 0x08080808u) | 0x80808080u) - 0x08080808u;
+    lo ^= 0x80808080u;
+    hi = ((h ^ 0x08080808u) | 0x80808080u) - 0x08080808u;
+    hi ^= 0x80808080u;
+  };
+  if (i < pieces) {
+    const uint4 v = src[i];
+    uint4 a, b;
+    widen(v.x, a.x, a.y); widen(v.y, a.z, a.w); widen(v.z, b.x, b.y); widen(v.w, b.z, b.w);
+    dst[2 * i] = a;
+    dst[2 * i + 1] = b;
+  }
+  if (i < tail_bytes) {   // the last bytes of a source whose size is not a multiple of 16
+    const unsigned char t = src_tail[i];
+    const int lo = t & 15, hi = t >> 4;
+    dst_tail[2 * i] = (signed char)(lo >= 8 ? lo - 16 : lo);
+    dst_tail[2 * i + 1] = (signed char)(hi >= 8 ? hi - 16 : hi);
+  }
+}
+
 }  // namespace
 }  // namespace msco
+
+extern "C" int msco_unpack_int4(const void *src, void *dst, int64_t src_bytes, void *stream) {
+  using namespace msco;
+  if (src_bytes < 0) return MSCO_ERR_SHAPE;
+  if (src_bytes == 0) return MSCO_OK;
+  if (src == nullptr || dst == nullptr) return MSCO_ERR_INVALID_ARG;
+  if ((reinterpret_cast<uintptr_t>(src) & 15) != 0 || (reinterpret_cast<uintptr_t>(dst) & 15) != 0) return MSCO_ERR_INVALID_ARG;
+  const long long pieces = src_bytes / 16;
+  const int tail = (int)(src_bytes % 16);
+  const long long threads = pieces > tail ? pieces : tail;
+  if ((threads + 255) / 256 > 0x7FFFFFFFll) return MSCO_ERR_SHAPE;
+  const unsigned char *s8 = static_cast<const unsigned char *>(src);
+  hipLaunchKernelGGL(unpack_int4_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), pieces, s8 + pieces * 16,
+                     static_cast<signed char *>(dst) + pieces * 32, tail);
+  return hipGetLastError() == hipSuccess ? MSCO_OK : MSCO_ERR_DEVICE;
+}
 
 extern "C" int msco_gmm_a8w4(const int8_t *x, const void *weight, const int32_t *group_list, const float *x_scale,
                              const float *weight_scale, void *out, int64_t m, int64_t k, int64_t n, int64_t e,

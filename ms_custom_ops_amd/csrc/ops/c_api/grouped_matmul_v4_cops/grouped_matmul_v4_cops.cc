@@ -9,9 +9,11 @@
 // The reference forwards the twelve lists to aclnnGroupedMatmulV4 (:359-363); here
 //   * group_type 0 (one x [M,K], one weight [E,K,N], one output [M,N]) is one grouped launch of the
 //     HIP backend: W8A8 with per-channel scale / per-token scale / int32 bias, or weight-only
-//     (bf16/f16 x, int8 weight, antiquant scale and offset [E,N]);
+//     (bf16/f16 x, int8 weight, antiquant scale and offset [E,N]); with a qint4x2 weight [E,K,N/2] (A8W4,
+//     tests/st/test_grouped_matmul_v4_cops.py:429-485) the nibble pairs are widened to int8 on the device first
+//     (msco_unpack_int4) and the W8A8 launch multiplies them: exact, at the price of one more pass over the weights;
 //   * group_type -1 (independent x[i] @ weight[i]) is one dense launch per pair.
-// Not implemented on this backend and refused with a message: float x float matmuls, int4 weights,
+// Not implemented on this backend and refused with a message: float x float matmuls,
 // uint64 scales with int8 output, `offset`, the activation inputs, group_type 1.  act_type selects an activation
 // fused into the epilogue (0 none, 1 relu, 2 gelu_tanh, 4 fast_gelu, 5 silu: the values of CANN's GMMActType, which the
 // reference passes through without naming them).
@@ -63,7 +65,13 @@ void CheckV4Support(const V4Args &a) {
   }
   const TypeId xt = a.x[0].data_type(), wt = a.weight[0].data_type();
   if (wt == kNumberTypeInt4) {
-    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", int4 weights are not implemented by the HIP backend.";
+    // A8W4 (tests/st/test_grouped_matmul_v4_cops.py:429-485): int8 x, qint4x2 weight [E, K, N / 2], one output
+    if (xt != kNumberTypeInt8 || a.group_type != kGroupTypeSingleOutput || a.weight_format != kNdFormat) {
+      MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", int4 weights are implemented for Int8 'x', group_type 0 "
+                       << "and weight_format 'ND' only, but got x dtype " << xt << ", group_type " << a.group_type
+                       << ", weight_format '" << a.weight_format << "'.";
+    }
+    return;
   }
   if (wt != kNumberTypeInt8) {
     MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName
@@ -81,6 +89,10 @@ struct OneLaunch {
   GmmProblem problem{};
   const void *addrs[MSCO_IN_COUNT] = {nullptr};
   void *out{nullptr};
+  // 4-bit weights: the nibble pairs (int4_bytes bytes at int4_src) are widened to int8 in a staging buffer of twice that
+  // size first, and addrs[MSCO_IN_WEIGHT] is set to the staging buffer
+  const void *int4_src{nullptr};
+  size_t int4_bytes{0};
 };
 const char *const kBackendOpName = "GroupedMatmulV4";
 
@@ -90,6 +102,7 @@ OneLaunch BuildOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &b
                    const ms::Tensor &group_list, int64_t group_list_type, const ms::Tensor &out, int64_t m, int64_t k,
                    int64_t n, int64_t e, bool packed, int64_t act_type) {
   const TypeId xt = x.data_type();
+  const bool int4 = w.data_type() == kNumberTypeInt4;
   OneLaunch one;
   one.problem = GmmProblem{m, k, n, e};
   one.out = out.GetDataPtr();
@@ -110,6 +123,11 @@ OneLaunch BuildOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &b
   d.act_type = static_cast<int32_t>(act_type);
   addrs[MSCO_IN_X] = x.GetDataPtr();
   addrs[MSCO_IN_WEIGHT] = w.GetDataPtr();
+  if (int4) {
+    one.int4_src = w.GetDataPtr();
+    one.int4_bytes = w.nbytes();
+    addrs[MSCO_IN_WEIGHT] = nullptr;   // the staging buffer, set by the caller
+  }
   addrs[MSCO_IN_GROUP_LIST] = group_list.is_defined() ? group_list.GetDataPtr() : nullptr;
   auto expect_en = [&](const ms::Tensor &t, const char *name) {
     if (t.is_defined() && t.numel() != e * n) {
@@ -124,7 +142,18 @@ OneLaunch BuildOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &b
     const bool raw = out.data_type() == kNumberTypeInt32;
     expect_en(bias, "bias");
     expect_en(scale, "scale");
-    if (bias.is_defined() && bias.data_type() != kNumberTypeInt32) {
+    if (int4) {
+      // The reference kernel multiplies the nibbles unsigned and needs bias = 8 * sum_k w[k, n] * scale[n] (Float32,
+      // tests/st/test_grouped_matmul_v4_cops.py:463) to compensate; here they are multiplied signed, so the term is
+      // checked for its type and not read (the expected value of the test, :467-476, contains no bias either).
+      if (bias.is_defined() && bias.data_type() != kNumberTypeFloat32) {
+        MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << " with A8W4, 'bias' must be Float32, but got "
+                           << bias.data_type();
+      }
+      if (!scale.is_defined() || out.data_type() == kNumberTypeInt32) {
+        MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << " with A8W4, 'scale' must be given.";
+      }
+    } else if (bias.is_defined() && bias.data_type() != kNumberTypeInt32) {
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", the quantized path takes an Int32 'bias', but got "
                          << bias.data_type();
     }
@@ -132,10 +161,10 @@ OneLaunch BuildOne(const ms::Tensor &x, const ms::Tensor &w, const ms::Tensor &b
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", 'per_token_scale' must be Float32 with M = " << m
                          << " elements, but got " << per_token.data_type() << " " << per_token.shape();
     }
-    d.bias_dtype = bias.is_defined() ? MSCO_DT_I32 : MSCO_DT_NONE;
+    d.bias_dtype = (bias.is_defined() && !int4) ? MSCO_DT_I32 : MSCO_DT_NONE;
     d.scale_dtype = (!raw && scale.is_defined()) ? ToBackendDtype(scale.data_type()) : MSCO_DT_NONE;
     d.per_token_dtype = (!raw && per_token.is_defined()) ? MSCO_DT_F32 : MSCO_DT_NONE;
-    addrs[MSCO_IN_BIAS] = bias.is_defined() ? bias.GetDataPtr() : nullptr;
+    addrs[MSCO_IN_BIAS] = d.bias_dtype != MSCO_DT_NONE ? bias.GetDataPtr() : nullptr;
     addrs[MSCO_IN_SCALE] = d.scale_dtype != MSCO_DT_NONE ? scale.GetDataPtr() : nullptr;
     addrs[MSCO_IN_PER_TOKEN_SCALE] = d.per_token_dtype != MSCO_DT_NONE ? per_token.GetDataPtr() : nullptr;
   } else {
@@ -181,7 +210,10 @@ std::vector<OneLaunch> BuildLaunches(const V4Args &a, const TensorVec &outputs) 
                          << (packed ? "[E, N/16, ceil(K/64), 1024] (prepacked by trans_data)" : "[E, K, N]") << ", but got "
                          << x.shape() << " and " << w.shape();
     }
-    const int64_t m = x.shape()[0], k = x.shape()[1], e = w.shape()[0], n = packed ? w.shape()[1] * 16 : w.shape()[2];
+    // (qint4x2: two 4-bit values per stored element along N -- UnifyWeightShape of the reference,
+    // ops/c_api/grouped_matmul_v4_cops/grouped_matmul_v4_cops.cc:56-66,274-295)
+    const int64_t n_mul = w.data_type() == kNumberTypeInt4 ? 2 : 1;
+    const int64_t m = x.shape()[0], k = x.shape()[1], e = w.shape()[0], n = packed ? w.shape()[1] * 16 : w.shape()[2] * n_mul;
     const int64_t wk = packed ? (w.shape()[2] == (k + 63) / 64 ? k : w.shape()[2] * 64) : w.shape()[1];
     if (wk != k) {
       MS_EXCEPTION_VALUE << "For " << kGroupedMatmulV4CopsName << ", the K dimension of 'x' and 'weight' must be equal, "
@@ -226,11 +258,25 @@ std::vector<OneLaunch> BuildLaunches(const V4Args &a, const TensorVec &outputs) 
   return launches;
 }
 
+// 4-bit weights -> int8 in `staging` (2 * int4_bytes bytes), which becomes the launch's weight
+void WidenInt4(OneLaunch &one, void *staging, void *stream) {
+  const int rc = msco_unpack_int4(one.int4_src, staging, static_cast<int64_t>(one.int4_bytes), stream);
+  if (rc != MSCO_OK) {
+    MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", widening the 4-bit weights failed: " << msco_status_string(rc);
+  }
+  one.addrs[MSCO_IN_WEIGHT] = staging;
+}
+
 // Pynative: plan (cached), take the workspace from the framework's allocator, launch.
 void RunGroupedMatmulV4(const V4Args &a, const TensorVec &outputs) {
   void *stream = CurrentStream();
-  for (const OneLaunch &one : BuildLaunches(a, outputs)) {
+  for (OneLaunch &one : BuildLaunches(a, outputs)) {
     auto plan = GmmPlanCache::GetInstance().GetOrCreate(kBackendOpName, one.desc, one.problem, stream);
+    ms::Tensor widened;
+    if (one.int4_bytes > 0) {
+      widened = AllocateTensor(kNumberTypeInt8, ShapeVector{static_cast<int64_t>(2 * one.int4_bytes)});
+      WidenInt4(one, widened.GetDataPtr(), stream);
+    }
     ms::Tensor workspace;
     if (plan->workspace_bytes > 0) {
       workspace = AllocateTensor(kNumberTypeInt8, ShapeVector{static_cast<int64_t>(plan->workspace_bytes)});
@@ -280,22 +326,33 @@ class GroupedMatmulV4CopsHip : public KernelMod {
     void *stream = CurrentStream();
     for (const OneLaunch &one : BuildLaunches(ArgsFromGraphInputs(inputs), outputs)) {
       sizes.push_back(GmmPlanCache::GetInstance().GetOrCreate(kBackendOpName, one.desc, one.problem, stream)->workspace_bytes);
+      if (one.int4_bytes > 0) sizes.push_back(2 * one.int4_bytes);   // 4-bit weights widened to int8: one more slice
     }
     return sizes;
   }
 
   bool Launch(const KernelTensorList &inputs, const std::vector<ms::Tensor> &workspace, const std::vector<ms::Tensor> &outputs,
               void *stream) override {
-    const std::vector<OneLaunch> launches = BuildLaunches(ArgsFromGraphInputs(inputs), outputs);
-    for (size_t i = 0; i < launches.size(); ++i) {
+    std::vector<OneLaunch> launches = BuildLaunches(ArgsFromGraphInputs(inputs), outputs);
+    size_t slot = 0;   // workspace slices in Resize's order: per launch the plan's, then the widened weights if any
+    for (size_t li = 0; li < launches.size(); ++li) {
       // the plan of the stream this launch goes to (a cache hit unless the stream changed since Resize)
-      auto plan = GmmPlanCache::GetInstance().GetOrCreate(kBackendOpName, launches[i].desc, launches[i].problem, stream);
+      auto plan = GmmPlanCache::GetInstance().GetOrCreate(kBackendOpName, launches[li].desc, launches[li].problem, stream);
+      const size_t i = slot++;
+      if (launches[li].int4_bytes > 0) {
+        const size_t w_slot = slot++;
+        if (w_slot >= workspace.size() || workspace[w_slot].nbytes() < 2 * launches[li].int4_bytes) {
+          MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", Launch got no workspace for the widened 4-bit weights of launch "
+                           << li << ": Resize must run when shapes change.";
+        }
+        WidenInt4(launches[li], workspace[w_slot].GetDataPtr(), stream);
+      }
       const bool have = i < workspace.size() && workspace[i].is_defined();
       if (plan->workspace_bytes > 0 && (!have || workspace[i].nbytes() < plan->workspace_bytes)) {
         MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", Launch got no workspace of " << plan->workspace_bytes
-                         << " bytes for launch " << i << ": Resize must run when shapes change.";
+                         << " bytes for launch " << li << ": Resize must run when shapes change.";
       }
-      LaunchPlan(kBackendOpName, plan, launches[i].addrs, launches[i].out, have ? workspace[i].GetDataPtr() : nullptr,
+      LaunchPlan(kBackendOpName, plan, launches[li].addrs, launches[li].out, have ? workspace[i].GetDataPtr() : nullptr,
                  have ? workspace[i].nbytes() : 0, stream);
     }
     return true;

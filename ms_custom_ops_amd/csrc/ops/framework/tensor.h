@@ -62,6 +62,7 @@ inline std::string TypeIdToString(TypeId t) {
 inline size_t TypeIdSize(TypeId t) {
   switch (t) {
     case kNumberTypeBool: case kNumberTypeInt8: case kNumberTypeUInt8: return 1;
+    case kNumberTypeInt4: return 1;   // qint4x2 storage: one byte per element of the stored shape (two 4-bit values)
     case kNumberTypeInt16: case kNumberTypeUInt16: case kNumberTypeFloat16: case kNumberTypeBFloat16: return 2;
     case kNumberTypeInt32: case kNumberTypeUInt32: case kNumberTypeFloat32: return 4;
     case kNumberTypeInt64: case kNumberTypeUInt64: case kNumberTypeFloat64: return 8;

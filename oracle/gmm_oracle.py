@@ -313,6 +313,30 @@ def golden_v4_perchannel_bias(x, w, scale, bias, counts):
     return np.concatenate(parts, axis=0)
 
 
+def encode_scale_uint64(scale_f32) -> np.ndarray:
+    """float32 scales -> the uint64 wire format of the V4 A8W4 test (float32 bits zero-extended,
+    tests/st/test_grouped_matmul_v4_cops.py:462)."""
+    return np.frombuffer(np.ascontiguousarray(scale_f32, dtype=np.float32).tobytes(), dtype=np.uint32).astype(np.uint64).reshape(np.shape(scale_f32))
+
+
+def golden_v4_a8w4(x, w, scale_u64, per_token, counts):
+    """The reference's expected value for grouped_matmul_v4_cops with 4-bit weights, literally
+    (tests/st/test_grouped_matmul_v4_cops.py:467-476): x int8 [m, k]; w the int8 VALUES [e, k, n] in [-8, 7] (the op itself
+    receives them as pack_int4(w), two per byte along n, :458-460); scale_u64 [e, 1, n] float32 bits in uint64; per_token
+    float32 [m, 1]; counts int64 [e].  float32 [sum(counts), n]; the test's float32 bias (:463) does not enter."""
+    index = np.cumsum(counts)
+    x_split = np.split(x, index, axis=0)
+    pt_split = np.split(per_token, index, axis=0)
+    scale_fp32 = np.asarray(scale_u64).astype(np.uint32)
+    scale_fp32.dtype = np.float32
+    out = []
+    for i in range(w.shape[0]):
+        mm = np.matmul(x_split[i].astype(np.int32), w[i].astype(np.int32)).astype(np.float32)
+        mm = mm * scale_fp32[i] * pt_split[i]
+        out.append(mm)
+    return np.concatenate(out, axis=0)
+
+
 def golden_v4_a16w8(x, w, antiquant_scale, antiquant_offset, ends):
     """test_grouped_matmul_v4_cops.py:166-174: matmul(x_g, (w_g + o_g) * s_g) in the dtype numpy picks
     (x's float dtype); only rows below the last boundary exist."""

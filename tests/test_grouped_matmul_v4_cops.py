@@ -244,3 +244,92 @@ def test_graph_kernel_module_inits_once_resizes_on_new_shapes_and_reads_fresh_te
     run(64, 4)          # new shape: planned again, same kernel module
     assert stats() == (inits0, resizes0 + 1, launches0 + 3)
     assert inits0 == 1
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("output_dtype", [torch.float16, torch.bfloat16, None])
+def test_v4_a8w4_reference_case(device, mode, output_dtype):
+    """The reference's A8W4 case (tests/st/test_grouped_matmul_v4_cops.py:429-485): int8 x, qint4x2 weight [e, k, n / 2]
+    (two nibbles per byte along n), uint64-encoded per-channel scale [e, 1, n], per-token scale [m, 1], float32 bias
+    (the reference kernel's compensation term, not part of the expected value), counts list; same seed, shapes and
+    tolerance; output float16 / bfloat16 (bfloat16 when output_dtype is not given).  This build's bar on top: the
+    output is one rounding of the oracle's exact float32 value, bit for bit."""
+    np.random.seed(1)
+    e, m, k, n = 8, 32, 256, 128
+    x_np = np.random.randint(-5, 5, size=(m, k)).astype(np.int8)
+    w_np = np.random.randint(-5, 5, size=(e, k, n)).astype(np.int8)
+    w_int4_np = O.pack_int4(w_np)
+    assert w_int4_np.shape == (e, k, n // 2)
+    scale_np = np.random.normal(0, 0.01, size=(e, 1, n)).astype(np.float32)
+    scale_u64 = O.encode_scale_uint64(scale_np)
+    bias_np = 8 * (w_np.astype(np.float32) * scale_np).sum(axis=1)
+    pertoken_np = np.random.normal(0, 0.01, (m, 1)).astype(np.float32)
+    counts = np.array([1, 2, 7, 4, 4, 4, 2, 8], dtype=np.int64)
+    expect = O.golden_v4_a8w4(x_np, w_np, scale_u64, pertoken_np, counts)
+    # (torch moves uint64 only as raw bytes on some builds: the bits travel as int64 and are viewed back)
+    scale_t = torch.from_numpy(scale_u64.view(np.int64)).cuda().view(torch.uint64)
+    with ms_custom_ops.exec_mode(mode):
+        for _ in range(2):   # the second call reuses the graph-mode module and its extra workspace slice
+            out = ms_custom_ops.grouped_matmul_v4_cops(
+                [_t(x_np)], [ms_custom_ops.as_qint4x2(_t(w_int4_np))], bias=[_t(bias_np)], scale=[scale_t],
+                per_token_scale=[_t(pertoken_np)], group_list=_t(counts), split_item=3, group_type=0, group_list_type=1,
+                output_dtype=output_dtype)[0]
+            assert out.shape == (m, n) and out.dtype == (output_dtype or torch.bfloat16)
+            cnt = expect.shape[0]
+            np.testing.assert_allclose(expect, out[:cnt].float().cpu().numpy(), rtol=5e-3, atol=5e-3)   # the reference's bar
+            if out.dtype == torch.float16:
+                assert np.array_equal(out.cpu().numpy().view(np.uint16), O.f32_to_f16(expect).view(np.uint16))
+            else:
+                assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), O.f32_to_bf16_bits(expect))
+
+
+def test_v4_a8w4_full_nibble_range_ragged_groups_and_rules(device):
+    """Every 4-bit value (-8 .. 7), int8 x over its whole range, empty groups, a K that is not a multiple of 64 and a
+    byte count that is not a multiple of 16 per row; then the argument rules."""
+    rng = np.random.default_rng(11)
+    e, m, k, n = 8, 50, 96, 48
+    x = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-8, 8, (e, k, n), dtype=np.int8)
+    assert w.min() == -8 and w.max() == 7
+    scale = rng.uniform(1e-3, 1e-2, (e, 1, n)).astype(np.float32)
+    pt = rng.uniform(1e-3, 1e-2, (m, 1)).astype(np.float32)
+    counts = np.array([0, 9, 0, 17, 1, 0, 20, 3], dtype=np.int64)
+    expect = O.golden_v4_a8w4(x, w, O.encode_scale_uint64(scale), pt, counts)
+    scale_t = torch.from_numpy(O.encode_scale_uint64(scale).view(np.int64)).cuda().view(torch.uint64)
+    f = ms_custom_ops.grouped_matmul_v4_cops
+    wq = ms_custom_ops.as_qint4x2(_t(O.pack_int4(w)))
+    for mode in MODES:
+        with ms_custom_ops.exec_mode(mode):
+            out = f([_t(x)], [wq], scale=[scale_t], per_token_scale=[_t(pt)], group_list=_t(counts), split_item=3,
+                    group_type=0, group_list_type=1, output_dtype=torch.float16)[0]
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), O.f32_to_f16(expect).view(np.uint16))
+    # cumulative list (group_list_type 0) gives the same rows
+    out = f([_t(x)], [wq], scale=[scale_t], per_token_scale=[_t(pt)], group_list=_t(np.cumsum(counts)), split_item=3,
+            group_type=0, group_list_type=0)[0]
+    assert out.dtype == torch.bfloat16
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), O.f32_to_bf16_bits(expect))
+    with pytest.raises(ValueError, match="the output type must be in"):
+        f([_t(x)], [wq], scale=[scale_t], group_list=_t(counts), split_item=3, group_type=0, group_list_type=1,
+          output_dtype=torch.float32)
+    with pytest.raises(ValueError, match="'scale' must be given"):
+        f([_t(x)], [wq], group_list=_t(counts), split_item=3, group_type=0, group_list_type=1)
+    with pytest.raises(ValueError, match="'bias' must be Float32"):
+        f([_t(x)], [wq], bias=[_t(np.zeros((e, n), np.int32))], scale=[scale_t], group_list=_t(counts), split_item=3,
+          group_type=0, group_list_type=1)
+    with pytest.raises(RuntimeError, match="int4 weights are implemented for"):
+        f([_t(x)], [ms_custom_ops.as_qint4x2(_t(O.pack_int4(w[0])))], scale=[scale_t[0]], group_type=-1)
+    with pytest.raises(TypeError, match="carried by an int8 or uint8"):
+        ms_custom_ops.as_qint4x2(_t(x).int())
+
+
+def test_unpack_int4_through_the_c_abi(device):
+    """msco_unpack_int4 against the oracle's unpack, sizes that end inside a 16-byte piece included."""
+    from ms_custom_ops_amd import cabi
+    rng = np.random.default_rng(2)
+    for nbytes in (1, 15, 16, 17, 4096 + 5, 1 << 20):
+        src = rng.integers(0, 256, nbytes, dtype=np.uint8)
+        t = torch.from_numpy(src).cuda()
+        dst = torch.full((2 * nbytes + 16,), 99, dtype=torch.int8, device="cuda")
+        cabi.unpack_int4(t.data_ptr(), dst.data_ptr(), nbytes, torch.cuda.current_stream().cuda_stream)
+        got = dst.cpu().numpy()
+        assert np.array_equal(got[:2 * nbytes], O.unpack_int4(src)) and (got[2 * nbytes:] == 99).all()

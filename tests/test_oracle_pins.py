@@ -421,3 +421,42 @@ def test_count_compare_counts_like_the_reference_comparator():
     # relative to the expected value, sign and scale free
     assert O.count_compare(np.array([-100.3]), np.array([-100.0]), 0.004)
     assert not O.count_compare(np.array([-100.5] * 1000), np.array([-100.0] * 1000), 0.004)
+
+
+def test_v4_a8w4_golden_against_exact_integers_a_scalar_loop_and_the_wire_formats():
+    """golden_v4_a8w4 / encode_scale_uint64 (tests/st/test_grouped_matmul_v4_cops.py:453-476) pinned by what the formula
+    fixes: the integer sums in exact Python integers, each of the two products rounded to float32 once; constant scales
+    give the plain integer matmul; the exact-path oracle of the W8A8 op on the same values agrees bit for bit; nibble
+    pairs along n by hand."""
+    rng = np.random.default_rng(5)
+    e, m, k, n = 4, 11, 48, 16
+    counts = np.array([3, 0, 6, 2], dtype=np.int64)
+    x = rng.integers(-128, 128, (m, k), dtype=np.int8)
+    w = rng.integers(-8, 8, (e, k, n), dtype=np.int8)
+    scale = rng.normal(0, 0.01, (e, 1, n)).astype(np.float32)
+    pt = rng.normal(0, 0.01, (m, 1)).astype(np.float32)
+    su = O.encode_scale_uint64(scale)
+    assert su.dtype == np.uint64 and su.shape == (e, 1, n) and (su >> np.uint64(32) == 0).all()
+    assert np.array_equal((su & np.uint64(0xFFFFFFFF)).astype(np.uint32).view(np.float32), scale)
+    got = O.golden_v4_a8w4(x, w, su, pt, counts)
+    assert got.dtype == np.float32 and got.shape == (m, n)
+    ends = np.cumsum(counts)
+    for row in range(m):
+        g = int(np.searchsorted(ends, row, side="right"))
+        for col in range(n):
+            acc = sum(int(x[row, kk]) * int(w[g, kk, col]) for kk in range(k))
+            want = np.float32(np.float32(np.float32(acc) * scale[g, 0, col]) * pt[row, 0])
+            assert got[row, col] == want, (row, col)
+    # the exact-path oracle of the int8 op on the same 4-bit values: same bits
+    ref = O.grouped_matmul_w8a8(x, w, ends, None, scale.reshape(e, n), pt.reshape(m), out_dtype="f32")
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    # scale 1 and per-token 1: the integer matmul itself
+    ones = O.golden_v4_a8w4(x, w, O.encode_scale_uint64(np.ones((e, 1, n), np.float32)), np.ones((m, 1), np.float32), counts)
+    for g, (a, b) in enumerate(zip(np.concatenate([[0], ends[:-1]]), ends)):
+        assert np.array_equal(ones[a:b], (x[a:b].astype(np.int64) @ w[g].astype(np.int64)).astype(np.float32))
+    # the packing of the test (:458-460): flattened, element 2 i in the low nibble, 2 i + 1 in the high one = pairs along n
+    wn = np.array([[[1, -1, 7, -8]]], dtype=np.int8)
+    flat = wn.reshape(-1) & 0x000F
+    literal = (flat[0::2] | (flat[1::2] << 4)).reshape(1, 1, 2)
+    assert np.array_equal(literal.astype(np.uint8), np.array([[[0xF1, 0x87]]], dtype=np.uint8))
+    assert np.array_equal(O.pack_int4(wn), literal.astype(np.uint8)) and np.array_equal(O.unpack_int4(O.pack_int4(w)), w)
