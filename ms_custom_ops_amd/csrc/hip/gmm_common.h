@@ -141,6 +141,33 @@ __device__ __forceinline__ void group_range(const GmmParams &p, int grp, int lan
   g_end = wave_bcast(end, grp - g0);
 }
 
+// Dispatch slot -> (group, chunk of rows_per_chunk rows) for the decode kernels: the grid's y extent enumerates only the
+// chunks that hold rows, group after group, so that many experts with few rows cost no empty workgroups.  Returns false
+// for a slot past the last chunk.  The number of chunks is at most min(E, M) + M / rows_per_chunk for any group_list
+// (every group with rows has at most one partial chunk), which is what the launchers size grid.y by.  Every lane of the
+// wave must call it; grp, mc and the row range come back wave-uniform.
+__device__ __forceinline__ bool chunk_of_slot(const GmmParams &p, int slot, int rows_per_chunk, int lane, int &grp, int &mc,
+                                              int &g_start, int &g_end) {
+  int carry = 0, seen = 0;
+  for (int g0 = 0; g0 < p.e; g0 += 64) {
+    int s0, e0;
+    group_rows_chunk(p, g0, lane, carry, s0, e0);
+    const int chunks = (e0 - s0 + rows_per_chunk - 1) / rows_per_chunk;   // 0 for empty groups and for lanes past E
+    const int upto = seen + wave_scan_add(chunks, lane);                  // chunks up to and including this lane's group
+    const unsigned long long beyond = __ballot(upto > slot);               // `upto` is non-decreasing
+    if (beyond != 0) {
+      const int first = __builtin_amdgcn_readfirstlane((int)__builtin_ctzll(beyond));
+      grp = g0 + first;
+      mc = slot - (wave_bcast(upto, first) - wave_bcast(chunks, first));
+      g_start = wave_bcast(s0, first);
+      g_end = wave_bcast(e0, first);
+      return true;
+    }
+    seen = wave_bcast(upto, 63);
+  }
+  return false;
+}
+
 // ---- number formats ----------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned short b) { return __uint_as_float((unsigned)b << 16); }
 

@@ -22,6 +22,16 @@ void tile_cfg_dims(int tile_cfg, int *bm, int *bn);
 size_t tile_count_bound(int tile_cfg, int64_t m, int64_t n, int64_t e);
 size_t tile_workspace_bytes(int tile_cfg, int64_t m, int64_t n, int64_t e, int split_k);
 
+// grid.y of the decode kernels: an upper bound, for any group_list, of the number of chunks of rows_per_chunk rows that
+// hold rows (see chunk_of_slot in gmm_common.h)
+inline unsigned chunk_slots(const GmmParams &p, int rows_per_chunk) {
+  const long long per_group = ((long long)p.m + rows_per_chunk - 1) / rows_per_chunk;
+  const long long all = (long long)p.e * (per_group > 1 ? per_group : 1);
+  const long long held = (p.m < p.e ? p.m : p.e) + p.m / rows_per_chunk;
+  const long long slots = all < held ? all : held;
+  return (unsigned)(slots > 1 ? slots : 1);
+}
+
 // Skinny (decode) kernels: one workgroup streams a 128-column weight strip of one group over a K
 // range; waves split K and reduce through LDS, workgroups split K and reduce through the workspace.
 // wide16: the 16-wave / 128-column-strip variant for small weight sets, else 4 waves / 256-column strips

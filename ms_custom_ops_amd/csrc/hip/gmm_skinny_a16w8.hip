@@ -78,13 +78,11 @@ __global__ void __launch_bounds__(AW_THREADS, 4) gmm_a16w8_skinny_kernel(const G
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15, h = lane >> 4;
   const int strip = blockIdx.x, ks = blockIdx.z;
-  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;   // first chunks of all groups are dispatched first
-
-  int g_start, g_end;
-  group_range(p, grp, lane, g_start, g_end);
+  // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
+  int grp, mc, g_start, g_end;
+  if (!chunk_of_slot(p, (int)blockIdx.y, kSkinnyRows, lane, grp, mc, g_start, g_end)) return;
   const int m0 = g_start + mc * kSkinnyRows;
   const int chunk_rows = min(kSkinnyRows, g_end - m0);
-  if (chunk_rows <= 0) return;
 
   const int n0 = strip * AW_COLS;
   const int8_t *wg = p.w + (long long)grp * p.k * p.n;
@@ -250,7 +248,7 @@ size_t a16w8_workspace_bytes(int64_t m, int64_t n, int64_t e, int split_k) {
 
 hipError_t launch_skinny_a16w8(const GmmParams &p, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
-  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  const dim3 grid((unsigned)p.n_strips, chunk_slots(p, kSkinnyRows), (unsigned)p.split_k);
   if (p.x_dtype == DT_BF16) {
     hipLaunchKernelGGL(gmm_a16w8_skinny_kernel<true>, grid, dim3(AW_THREADS), 0, stream, p);
   } else {

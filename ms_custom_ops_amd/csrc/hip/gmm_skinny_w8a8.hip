@@ -42,13 +42,11 @@ __global__ void __launch_bounds__(SK_THREADS, NK ? 3 : 4) gmm_w8a8_skinny_kernel
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: scalar loop control
   const int c16 = lane & 15, h = lane >> 4;
   const int strip = blockIdx.x, ks = blockIdx.z;
-  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;   // first chunks of all groups are dispatched first
-
-  int g_start, g_end;
-  group_range(p, grp, lane, g_start, g_end);
+  // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
+  int grp, mc, g_start, g_end;
+  if (!chunk_of_slot(p, (int)blockIdx.y, kSkinnyRows, lane, grp, mc, g_start, g_end)) return;
   const int m0 = g_start + mc * kSkinnyRows;
   const int chunk_rows = min(kSkinnyRows, g_end - m0);
-  if (chunk_rows <= 0) return;
 
   const int n0 = strip * SK_COLS;
   const int8_t *xg = reinterpret_cast<const int8_t *>(p.x);
@@ -245,13 +243,11 @@ __global__ void __launch_bounds__(W16_THREADS) gmm_w8a8_skinny16_kernel(const Gm
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: scalar loop control
   const int c16 = lane & 15, h = lane >> 4;
   const int strip = blockIdx.x, ks = blockIdx.z;
-  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;   // first chunks of all groups are dispatched first
-
-  int g_start, g_end;
-  group_range(p, grp, lane, g_start, g_end);
+  // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
+  int grp, mc, g_start, g_end;
+  if (!chunk_of_slot(p, (int)blockIdx.y, kSkinnyRows, lane, grp, mc, g_start, g_end)) return;
   const int m0 = g_start + mc * kSkinnyRows;
   const int chunk_rows = min(kSkinnyRows, g_end - m0);
-  if (chunk_rows <= 0) return;
 
   const int n0 = strip * W16_COLS;
   const int8_t *wg = p.w + (long long)grp * p.k * p.n;
@@ -454,11 +450,11 @@ hipError_t launch_skinny_w8a8(const GmmParams &p, bool nk, bool wide16, hipStrea
       if (e != hipSuccess) return e;
       attr_done[nk] = true;
     }
-    const dim3 grid((unsigned)((p.n + W16_COLS - 1) / W16_COLS), (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+    const dim3 grid((unsigned)((p.n + W16_COLS - 1) / W16_COLS), chunk_slots(p, kSkinnyRows), (unsigned)p.split_k);
     hipLaunchKernelGGL(kern, grid, dim3(W16_THREADS), W16_LDS, stream, p);
     return hipGetLastError();
   }
-  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  const dim3 grid((unsigned)p.n_strips, chunk_slots(p, kSkinnyRows), (unsigned)p.split_k);
   if (nk) {
     hipLaunchKernelGGL(gmm_w8a8_skinny_kernel<true>, grid, dim3(SK_THREADS), 0, stream, p);
   } else {

@@ -106,13 +106,11 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_stream_kernel(const Gm
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15, h = lane >> 4;
   const int strip = blockIdx.x, ks = blockIdx.z;
-  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;   // first chunks of all groups are dispatched first
-
-  int g_start, g_end;
-  group_range(p, grp, lane, g_start, g_end);
+  // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
+  int grp, mc, g_start, g_end;
+  if (!chunk_of_slot(p, (int)blockIdx.y, kSkinnyRows, lane, grp, mc, g_start, g_end)) return;
   const int m0 = g_start + mc * kSkinnyRows;
   const int chunk_rows = min(kSkinnyRows, g_end - m0);
-  if (chunk_rows <= 0) return;
 
   const int n0 = strip * p.strip_groups * 16;
   const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
@@ -335,7 +333,7 @@ hipError_t launch_stream_w8a8(const GmmParams &p, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
   const int nb = stream_blocks_per_wave(p.k, p.split_k);
   if (nb > 32 || p.strip_groups < 1 || p.strip_groups > ST_GROUPS) return hipErrorInvalidValue;   // the plan splits K until a slice has at most 128 blocks
-  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  const dim3 grid((unsigned)p.n_strips, chunk_slots(p, kSkinnyRows), (unsigned)p.split_k);
   if (nb > 16) return stream_launch_w8a8<32, false>(p, grid, stream);   // (a 128-block slice of 16 rows would need 128 KiB of LDS)
   if (p.x_via_lds) {
     if (nb > 8) return stream_launch_w8a8<16, true>(p, grid, stream);
@@ -378,13 +376,11 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_w8a8_streamm_kernel(const G
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15, h = lane >> 4;
   const int strip = blockIdx.x, ks = blockIdx.z;
-  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
-
-  int g_start, g_end;
-  group_range(p, grp, lane, g_start, g_end);
+  // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
+  int grp, mc, g_start, g_end;
+  if (!chunk_of_slot(p, (int)blockIdx.y, S::kRows, lane, grp, mc, g_start, g_end)) return;
   const int m0 = g_start + mc * S::kRows;
   const int chunk_rows = min(S::kRows, g_end - m0);
-  if (chunk_rows <= 0) return;
 
   for (int i = tid; i < S::kTileInts / 4; i += ST_THREADS) reinterpret_cast<v4i *>(tile)[i] = v4i{0, 0, 0, 0};
 
@@ -543,7 +539,7 @@ static hipError_t streamm_launch(const GmmParams &p, const dim3 &grid, hipStream
 // tch = 16-row fragments per chunk (2, 4 or 8); p.max_chunks counts chunks of 16 tch rows, p.n_strips strips of 64 columns
 hipError_t launch_streamm_w8a8(const GmmParams &p, int tch, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
-  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  const dim3 grid((unsigned)p.n_strips, chunk_slots(p, 16 * tch), (unsigned)p.split_k);
   if (tch == 8) return streamm_launch<8>(p, grid, stream);
   if (tch == 4) return streamm_launch<4>(p, grid, stream);
   if (tch == 2) return streamm_launch<2>(p, grid, stream);
@@ -609,13 +605,11 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_stream_kernel(const G
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15, h = lane >> 4;
   const int strip = blockIdx.x, ks = blockIdx.z;
-  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
-
-  int g_start, g_end;
-  group_range(p, grp, lane, g_start, g_end);
+  // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
+  int grp, mc, g_start, g_end;
+  if (!chunk_of_slot(p, (int)blockIdx.y, kSkinnyRows, lane, grp, mc, g_start, g_end)) return;
   const int m0 = g_start + mc * kSkinnyRows;
   const int chunk_rows = min(kSkinnyRows, g_end - m0);
-  if (chunk_rows <= 0) return;
 
   const int n0 = strip * p.strip_groups * 16;
   const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
@@ -826,7 +820,7 @@ hipError_t launch_stream_a16w8(const GmmParams &p, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
   const int nb = stream_blocks_per_wave(p.k, p.split_k);
   if (nb > 16 || p.strip_groups < 1 || p.strip_groups > ST_GROUPS) return hipErrorInvalidValue;   // slices of at most 64 blocks
-  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  const dim3 grid((unsigned)p.n_strips, chunk_slots(p, kSkinnyRows), (unsigned)p.split_k);
   const bool bf = p.x_dtype == DT_BF16;
   if (nb > 8) return bf ? stream_launch_a16w8<true, 16>(p, grid, stream) : stream_launch_a16w8<false, 16>(p, grid, stream);
   if (nb > 4) return bf ? stream_launch_a16w8<true, 8>(p, grid, stream) : stream_launch_a16w8<false, 8>(p, grid, stream);
@@ -879,13 +873,11 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows_kernel(const Gmm
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15, h = lane >> 4;
   const int strip = blockIdx.x;
-  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
-
-  int g_start, g_end;
-  group_range(p, grp, lane, g_start, g_end);
+  // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
+  int grp, mc, g_start, g_end;
+  if (!chunk_of_slot(p, (int)blockIdx.y, S::kRows, lane, grp, mc, g_start, g_end)) return;
   const int m0 = g_start + mc * S::kRows;
   const int chunk_rows = min(S::kRows, g_end - m0);
-  if (chunk_rows <= 0) return;
 
   const int n0 = strip * S::kCols;
   const int col_groups = (p.n + 15) / 16, k_blocks = (p.k + 63) / 64;
@@ -1168,13 +1160,11 @@ __global__ void __launch_bounds__(ST_THREADS, 2) gmm_a16w8_rows32_kernel(const G
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c32 = lane & 31, kh = lane >> 5;
   const int strip = blockIdx.x;
-  const int grp = (int)blockIdx.y % p.e, mc = (int)blockIdx.y / p.e;
-
-  int g_start, g_end;
-  group_range(p, grp, lane, g_start, g_end);
+  // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
+  int grp, mc, g_start, g_end;
+  if (!chunk_of_slot(p, (int)blockIdx.y, S::kRows, lane, grp, mc, g_start, g_end)) return;
   const int m0 = g_start + mc * S::kRows;
   const int chunk_rows = min(S::kRows, g_end - m0);
-  if (chunk_rows <= 0) return;
 
   const int n0 = strip * S::kCols;
   const int k_blocks = (p.k + 63) / 64, col_groups = (p.n + 15) / 16;
@@ -1488,7 +1478,7 @@ hipError_t launch_streamm_a16w8(const GmmParams &p, int tch, bool packed, hipStr
   if ((p.strip_groups != 8 && p.strip_groups != 16) || (tch != 2 && tch != 4 && tch != 8) || p.split_k < 1 ||
       (p.split_k > 1 && tch != 8))   // (a K split: 128-row chunks only)
     return hipErrorInvalidValue;
-  const dim3 grid((unsigned)p.n_strips, (unsigned)(p.e * p.max_chunks), (unsigned)p.split_k);
+  const dim3 grid((unsigned)p.n_strips, chunk_slots(p, 16 * tch), (unsigned)p.split_k);
   const bool bf = p.x_dtype == DT_BF16;
   const bool wide = p.strip_groups == 16;
 #define MSCO_ROWS_BY(TCH)                                                                                                   \

@@ -153,10 +153,14 @@ void choose_plan(msco_gmm_op *op) {
   // row-major [E,N,K] weights at decode sizes: a column's K bytes are contiguous and the columns are K bytes apart, which
   // suits the 64 x 128 tile's LDS-direct loads better than the decode kernel's 64-byte row pieces (K = 4096, N = 11008,
   // 1 / 16 rows: 15.8 / 15.9 us against 16.8 / 17.7 us; 32 rows over 8 experts, N = 14336: 103 against 115 us)
-  const bool nk_rows = is_w8a8(d) && d.transpose_b != 0 && !is_packed(d);
+  // (with hundreds of experts and a few rows the decode kernel wins again: 40 rows over 256 experts, K = 512, N = 7168:
+  // 42 us against 95 us)
+  const bool nk_rows = is_w8a8(d) && d.transpose_b != 0 && !is_packed(d) && e <= 32;
   const int64_t avg_rows = (m + (e > 0 ? e : 1) - 1) / (e > 0 ? e : 1);
+  // (the decode kernels' grid enumerates the chunks that hold rows -- at most min(E, M) + M / 16 of them -- so experts
+  // without rows cost nothing)
   const bool many_small_groups = e > 1 && avg_rows + avg_rows / 2 <= kSkinnyRows &&
-                                 e * ((m + kSkinnyRows - 1) / kSkinnyRows) <= kSkinnyMaxChunkSlots;
+                                 std::min<int64_t>(m, e) + m / kSkinnyRows <= kSkinnyMaxChunkSlots;
   if (!aligned) {
     family = FAM_GENERIC;
   } else if (is_a16w8(d)) {
@@ -306,8 +310,8 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t avg = (m + e - 1) / e;
     const int64_t rows = e == 1 ? m : avg + avg / 2;
     op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
-    // fewer, larger chunks when the (group, chunk) grid would be mostly empty slots
-    while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
+    // fewer, larger chunks when there would be more chunks than the grid should enumerate
+    while (op->stream_tch < 8 && std::min<int64_t>(m, e) + m / (16 * op->stream_tch) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch = op->stream_tch == 1 ? 2 : op->stream_tch * 2;
     if (tuning().stream_tch == 1 || tuning().stream_tch == 2 || tuning().stream_tch == 4 || tuning().stream_tch == 8) op->stream_tch = tuning().stream_tch;
   } else if (family == FAM_SKINNY && is_a16w8(d) && (is_packed(d) || (d.transpose_b == 0 && n % 16 == 0))) {
@@ -317,7 +321,7 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t avg = (m + e - 1) / e;
     const int64_t rows = e == 1 ? m : avg + avg / 2;
     op->stream_tch = rows <= 16 ? 1 : rows <= 32 ? 2 : rows <= 64 ? 4 : 8;
-    while (op->stream_tch < 8 && e * ((m + 16 * op->stream_tch - 1) / (16 * op->stream_tch)) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
+    while (op->stream_tch < 8 && std::min<int64_t>(m, e) + m / (16 * op->stream_tch) > or_default(tuning().stream_max_slots, (int)kSkinnyMaxChunkSlots))
       op->stream_tch *= 2;
     // One group whose column strips do not fill the chip: the multi-row kernels walk all of K in every workgroup (only
     // the 128-row form has a K split, below), and for few rows the 16-row kernels with their K split are faster

@@ -15,6 +15,12 @@ c4          MoE E=64 top-6 over 8192 tokens (49152 rows), Zipf(1.2) expert popul
 c5          weight-only decode, E=8 top-2 over 16 tokens (32 rows), bf16 x, K=4096 N=14336 (c5_t<T>: T tokens)
 c3_decode   the c3 layer at decode time: E=8 top-2 over 16 tokens (32 rows), int8 x, K=4096 N=14336 (not one of the
             published configurations: c3's weights with c5's routing, the W8A8 counterpart of c5)
+ref_m{M}_k{K}_n{N}_e{E}
+            the shapes the reference's own tests time or call "real": M rows cut into E groups at sorted random
+            boundaries (empty groups allowed), per-channel and per-token scales -- E=8, M=1024, K=5120, N in {2688, 1344}
+            (tests/st/test_grouped_matmul.py:325-345) and E=256 with (M, K, N) in {(40, 512, 7168), (1024, 2048, 7168),
+            (1024, 7168, 4096)} (:190-204).  Weights beyond 1 GiB are not drawn on the host: ``w`` is None and
+            ``meta["w_shape"]`` says what to draw on the device (timing only).
 """
 from __future__ import annotations
 
@@ -142,6 +148,16 @@ def make(name: str, *, scale_down: int = 1) -> Workload:
         logits = np.random.randn(t, e)
         gl, _, _ = route_topk(logits, top_k, e)
         return Workload(name, "a16w8", m, k, n, e, x, w, s, None, None, off, gl, {"offset_int8": off_i8})
+    if name.startswith("ref_m"):
+        parts = dict((p[0], int(p[1:])) for p in name[4:].split("_"))
+        m, k, n, e = parts["m"], parts["k"] // sd, parts["n"] // sd, parts["e"]
+        x = _int8((m, k))
+        big = e * k * n > (1 << 30)
+        w = None if big else _int8((e, k, n))
+        s = _scale((e, n)); pt = _scale((m,))
+        cuts = np.sort(np.random.randint(0, m + 1, size=e - 1))   # duplicates allowed: empty groups (test_grouped_matmul.py:162-169)
+        gl = np.concatenate([cuts, [m]]).astype(np.int64)
+        return Workload(name, "w8a8", m, k, n, e, x, w, s, pt, None, None, gl, {"w_shape": (e, k, n)})
     raise KeyError(name)
 
 
@@ -155,5 +171,7 @@ def algorithmic_work(wl: Workload) -> Dict[str, float]:
     b = m * wl.k * sx + nonempty * wl.k * wl.n + m * wl.n * 2 + wl.group_list.nbytes
     for extra in (wl.scale, wl.per_token, wl.bias, wl.offset):
         if extra is not None:
-            b += extra.nbytes
+            # per-group rows ([E, N]) are read for the groups that hold rows only
+            per_group = extra.ndim == 2 and extra.shape[0] == wl.e and wl.e > 1
+            b += extra.nbytes * nonempty // wl.e if per_group else extra.nbytes
     return {"ops": 2.0 * m * wl.k * wl.n, "bytes": float(b), "rows": m, "nonempty_groups": nonempty}
