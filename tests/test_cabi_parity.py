@@ -257,3 +257,34 @@ def test_weight_only_scaled_c5_and_constant_scale_case(device, dtype):
     ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
     assert (np.abs(got - exact) <= ulp * np.abs(exact) + 1e-5 * mag).all(), info
     assert "skinny" in info
+
+
+@pytest.mark.parametrize("m", [40, 300])
+@pytest.mark.parametrize("layout", ["kn", "nk", "packed"])
+def test_hundreds_of_experts_few_rows_decode_kernels_enumerate_only_chunks_with_rows(device, m, layout):
+    """256 experts, 40 and 300 rows (the reference's DeepSeek-shaped cases, tests/st/test_grouped_matmul.py:190-204, at a
+    small K and N): most experts hold no row, some hold more than one 16-row chunk.  The decode kernels' grid counts
+    chunks that hold rows, not experts; every layout stays bit-exact, for cumulative and for count lists."""
+    from gpu_utils import run_w8a8
+    e, k, n = 256, 128, 272
+    rng, x, w, bias, scale, pt = _inputs(40 + m, m, k, n, e)
+    counts = np.zeros(e, dtype=np.int64)
+    hit = rng.choice(e, size=m // 5, replace=False)
+    if m > 40:
+        counts[hit[0]] = 37                          # one expert with several 16-row chunks
+    for _ in range(m - 5 - int(counts.sum())):       # (five rows stay behind the last boundary)
+        counts[hit[rng.integers(1, len(hit))]] += 1
+    ends = np.cumsum(counts)
+    last = int(ends[-1])
+    assert last == m - 5 and (counts == 0).sum() > e // 2 and (m == 40 or counts.max() > 32)
+    ref = O.grouped_matmul_w8a8(x, w, ends, bias, scale, pt)
+    ref_acc = O.grouped_matmul_w8a8(x, w, ends, bias, out_dtype="i32")
+    for gl, gl_type in ((ends, 0), (counts, 1)):
+        bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", transpose_b=layout == "nk", packed=layout == "packed",
+                              group_list_type=gl_type, launches=2)
+        assert ("skinny" in info or "stream" in info), info
+        assert np.array_equal(bits[:last], ref[:last]), info
+        assert (bits[last:] == 0x7FC0).all(), info     # rows past the last boundary are not written
+        acc, info = run_w8a8(x, w, gl, bias, out="i32", transpose_b=layout == "nk", packed=layout == "packed",
+                             group_list_type=gl_type)
+        assert np.array_equal(acc[:last], ref_acc[:last]), info
