@@ -153,9 +153,10 @@ void choose_plan(msco_gmm_op *op) {
   // row-major [E,N,K] weights at decode sizes: a column's K bytes are contiguous and the columns are K bytes apart, which
   // suits the 64 x 128 tile's LDS-direct loads better than the decode kernel's 64-byte row pieces (K = 4096, N = 11008,
   // 1 / 16 rows: 15.8 / 15.9 us against 16.8 / 17.7 us; 32 rows over 8 experts, N = 14336: 103 against 115 us)
-  // (with hundreds of experts and a few rows the decode kernel wins again: 40 rows over 256 experts, K = 512, N = 7168:
-  // 42 us against 95 us)
-  const bool nk_rows = is_w8a8(d) && d.transpose_b != 0 && !is_packed(d) && e <= 32;
+  // (a few rows over hundreds of experts are the decode kernel's again -- 40 rows over 256 experts, K = 512, N = 7168: 41 us
+  // against 95 us -- but not a thousand rows over them: K = 2048, N = 7168: 635 against 595 us, K = 7168, N = 4096: 1467
+  // against 1244 us)
+  const bool nk_rows = is_w8a8(d) && d.transpose_b != 0 && !is_packed(d) && !(e > 32 && m <= kSkinnyMaxRows);
   const int64_t avg_rows = (m + (e > 0 ? e : 1) - 1) / (e > 0 ? e : 1);
   // (the decode kernels' grid enumerates the chunks that hold rows -- at most min(E, M) + M / 16 of them -- so experts
   // without rows cost nothing)
