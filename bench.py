@@ -54,7 +54,8 @@ def parse():
                          "nk=[E,N,K] (prepacked once by a transpose), kn=[E,K,N] as generated")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--zero-operands", action="store_true", help="with --probe <workload>: all-zero x and weights (same kernel, nothing toggles)")
+    ap.add_argument("--zero-operands", nargs="?", const="both", default=None, choices=["both", "x", "w"],
+                    help="with --probe <workload>: all-zero x and weights, or only one of them (same kernel, less or nothing toggles)")
     ap.add_argument("--probe", default=None, help="workload name, `copy` or `moe` (the routing / un-permutation pair): launches only, for counter collection")
     return ap.parse_args()
 
@@ -75,8 +76,10 @@ class DeviceProblem:
             w0 = torch.randint(-127, 128, tuple(wl.meta["w_shape"]), dtype=torch.int8, device=dev)
         else:
             w0 = t(wl.w)
-        if zero_operands:   # same shapes, routing and kernel, operands that toggle nothing: a timing yardstick only
+        # same shapes, routing and kernel, operands that toggle nothing: a timing yardstick only (True or "both", "x", "w")
+        if zero_operands in (True, "both", "x"):
             self.x.zero_()
+        if zero_operands in (True, "both", "w"):
             w0.zero_()
         self.prepack_ms = None
         if nk:

@@ -58,6 +58,34 @@ def build_backend(verbose: bool = False) -> str:
     return BACKEND_LIB
 
 
+ATTRIBUTION_BUILDS = {"noepi": 1, "nomfma": 2, "nomfma_noepi": 3, "nostore": 4}
+
+
+def build_attribution(verbose: bool = False):
+    """Measurement builds of the backend, never the shipped one: lib/attr/libmsco_gmm_<name>.so is libmsco_gmm.so with
+    one part of the persistent tile kernel taken out (MSCO_TILE4_ATTR in gmm_tile4_w8a8.hip), so that timing the rest
+    says what that part costs.  Select one with MSCO_GMM_LIB=<path>; their results are wrong on purpose."""
+    build_backend(verbose)
+    hipcc = _hipcc()
+    hip_dir = os.path.join(CSRC, "hip")
+    out_dir = os.path.join(LIB_DIR, "attr")
+    os.makedirs(out_dir, exist_ok=True)
+    others = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in HIP_SOURCES if s != "gmm_tile4_w8a8.hip"]
+
+    def build_one(item):
+        name, mask = item
+        obj = os.path.join(out_dir, "gmm_tile4_w8a8_%s.o" % name)
+        _run([hipcc] + HIP_FLAGS + ["-DMSCO_BUILDING_LIB", "-DMSCO_TILE4_ATTR=%d" % mask, "-I", INCLUDE, "-I", hip_dir, "-c",
+                                    os.path.join(hip_dir, "gmm_tile4_w8a8.hip"), "-o", obj])
+        lib = os.path.join(out_dir, "libmsco_gmm_%s.so" % name)
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + others + [obj])
+        os.remove(obj)
+        return lib
+
+    with cf.ThreadPoolExecutor(max_workers=4) as pool:
+        return list(pool.map(build_one, ATTRIBUTION_BUILDS.items()))
+
+
 def pybind_module_path() -> str:
     suffix = sysconfig.get_config_var("EXT_SUFFIX") or ".so"
     return os.path.join(PKG_DIR, "ms_custom_ops" + suffix)
@@ -97,5 +125,6 @@ def build_all(verbose: bool = False):
 
 
 if __name__ == "__main__":
-    for path in build_all(verbose="-v" in sys.argv):
+    paths = build_attribution("-v" in sys.argv) if "--attribution" in sys.argv else build_all(verbose="-v" in sys.argv)
+    for path in paths:
         print("built", path)

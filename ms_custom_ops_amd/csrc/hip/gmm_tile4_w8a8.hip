@@ -55,6 +55,14 @@ constexpr int T4_W_BASE = 2 * T4_OP_STAGE;       // x stages 0 and 1, then weigh
                                                  // together fit the 16-bit offset field of an LDS instruction
 constexpr int T4_RING = 2 * T4_W_BASE;           // 128 KiB
 constexpr int T4_LD = T4_BM / 8 / T4_NW;         // staging quads (8 rows x 128 B per wave) per operand and slab
+// Attribution builds, never the shipped library: MSCO_TILE4_ATTR is a bit mask that takes one part of the kernel out
+// so that timing the rest says what that part costs (results are then wrong on purpose).  1: the epilogue sits behind
+// a branch that no launch takes (its code and registers stay); 2: every MFMA becomes an empty statement that keeps
+// both operand fragments alive (loads, LDS traffic and barriers unchanged); 4: the epilogue computes everything and
+// its output stores become empty statements.
+#ifndef MSCO_TILE4_ATTR
+#define MSCO_TILE4_ATTR 0
+#endif
 constexpr int T4_EP_PITCH = 144;                 // epilogue staging: 128 payload bytes per row
 constexpr int T4_PARAM_OFF = T4_RING;            // epilogue operand tables (scale, bias, per-token; two tiles) behind the ring
 constexpr int T4_PARAM_BYTES = 3 * 1024;
@@ -491,7 +499,11 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         for (int f = 0; f < T4_F; ++f)
 #pragma unroll
           for (int i = 0; i < T4_F; ++i)
+#if MSCO_TILE4_ATTR & 2
+            asm volatile("" ::"v"(wf[S][f]), "v"(xf[S][i]));
+#else
             acc[f][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[S][f], xf[S][i], acc[f][i], 0, 0, 0);
+#endif
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          // MFMA
@@ -591,6 +603,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     // 128 payload bytes at a 144-byte pitch), read back with lanes along columns, store full 128-byte
     // row segments.  The operand ring is live (it already holds the next tile), so only the small
     // region behind it is used.  The table was published by the barriers of the slabs since kt == 2.
+#if MSCO_TILE4_ATTR & 1
+    if (p.m == -12345)
+#endif
     {
       // (lane-derived values are laundered through an empty asm: otherwise every LDS address below is
       // loop invariant, gets computed before the tile loop and has to survive the K loop in a register
@@ -649,7 +664,15 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         const unsigned v0 = (n_first < p.n ? v_row : T4_OOB) + PIECE * 128;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
+#if MSCO_TILE4_ATTR & 4
+          {
+            const v4i val = __builtin_bit_cast(v4i, rb[t]);
+            const unsigned off = v0 + (unsigned)(32 * I + 8 * t) * pitch;
+            asm volatile("" ::"v"(val), "v"(off));
+          }
+#else
           __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, rb[t]), rs_out, v0 + (unsigned)(32 * I + 8 * t) * pitch, 0, 0);
+#endif
       };
       auto load_scales = [&](auto piece_c) {
         constexpr int PIECE = decltype(piece_c)::value;

@@ -282,7 +282,8 @@ def test_hundreds_of_experts_few_rows_decode_kernels_enumerate_only_chunks_with_
     for gl, gl_type in ((ends, 0), (counts, 1)):
         bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", transpose_b=layout == "nk", packed=layout == "packed",
                               group_list_type=gl_type, launches=2)
-        assert ("skinny" in info or "stream" in info), info
+        # ([E,N,K] weights beyond 64 rows stay with the small tile kernel, whose tiles are cut per group as well)
+        assert ("skinny" in info or "stream" in info or (layout == "nk" and m > 64 and "tile_64x128" in info)), info
         assert np.array_equal(bits[:last], ref[:last]), info
         assert (bits[last:] == 0x7FC0).all(), info     # rows past the last boundary are not written
         acc, info = run_w8a8(x, w, gl, bias, out="i32", transpose_b=layout == "nk", packed=layout == "packed",
