@@ -15,8 +15,9 @@ all three.
 Prints ONE JSON line.  Besides the contract keys it carries
   roofline      the dominant kernel's achieved algorithmic rate against the MI355X peak,
   cpu_baseline  the numpy restatement of the reference golden timed on this box's host cores,
-  sweep         the other configurations (dense decode / prefill sweep, skewed MoE, weight-only
-                decode) as TOPS and GB/s with their roofline fractions, per weight layout.
+  sweep         the other configurations (dense decode / prefill sweep, skewed MoE, weight-only decode, serving sizes,
+                the reference's own timing shapes) per weight layout, one row each under `columns`: launch period and
+                the int8 / HBM roofline fractions (TOP/s = int8_frac x 5000, GB/s = hbm_frac x 8000).
 `mfma_pipe` (and `--probe mfma`) is a yardstick: a loop of nothing but the int8 MFMA instruction on random and on zero operands.
 --probe runs a few untimed launches of one workload (or, for `copy`, of a plain device-to-device copy
 of COPY_BYTES bytes, the reference a counter reading is scaled by) so that a profiler sees nothing else.
@@ -553,12 +554,13 @@ def main():
             p2 = DeviceProblem(w2, layout, copies)
             _, sec, _ = p2.time(max(20, min(200, args.steps)), args.warmup)
             wk, tops, gbs = rates(w2, sec)
-            sweep.append({"workload": name, "layout": layout, "launch_us": sec * 1e6, "tops": tops,
-                          "int8_frac": tops / PEAK_INT8_TOPS, "gbs": gbs, "hbm_frac": gbs / PEAK_HBM_GBS,
-                          "weight_copies_rotated": copies, "prepack_ms": p2.prepack_ms, "kernel": p2.op.plan_info().split("kernel=")[1].split(" m=")[0]})
+            sweep.append([name, layout, sec * 1e6, tops / PEAK_INT8_TOPS, gbs / PEAK_HBM_GBS, copies,
+                          p2.op.plan_info().split("kernel=")[1].split(" ")[0]])
             del p2
             torch.cuda.empty_cache()
-        result["sweep"] = sweep
+        # (one row per case, columnar: the whole line has to survive a log tail; TOP/s = int8_frac x 5000, GB/s = hbm_frac x 8000)
+        result["sweep"] = {"columns": ["workload", "layout", "launch_us", "int8_frac", "hbm_frac", "weight_copies_rotated", "kernel"],
+                           "rows": sweep}
         result["moe_neighbours"] = moe_neighbours(max(20, min(100, args.steps)), 10)
         result["mfma_pipe"] = mfma_pipe_probe()
         result["read_floor"] = read_floor()

@@ -18,7 +18,9 @@ OBJ_DIR = os.path.join(PKG_DIR, "lib", "obj")
 INCLUDE = os.path.join(REPO_DIR, "include")
 
 BACKEND_LIB = os.path.join(LIB_DIR, "libmsco_gmm.so")
-HIP_SOURCES = ["gmm_tile_w8a8.hip", "gmm_tile4_w8a8.hip", "gmm_skinny_w8a8.hip", "gmm_skinny_a16w8.hip", "gmm_generic.hip", "gmm_stream.hip", "msco_gmm.hip", "moe_routing.hip", "gmm_w4.hip", "probes.hip"]
+PROBES_LIB = os.path.join(LIB_DIR, "libmsco_probes.so")   # measurement aids: not part of the operator library
+HIP_SOURCES = ["gmm_tile_w8a8.hip", "gmm_tile4_w8a8.hip", "gmm_skinny_w8a8.hip", "gmm_skinny_a16w8.hip", "gmm_generic.hip", "gmm_stream.hip", "msco_gmm.hip", "moe_routing.hip", "gmm_w4.hip"]
+PROBE_SOURCES = ["probes.hip"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -37,8 +39,9 @@ def _run(cmd):
     return proc.stdout
 
 
-def build_backend(verbose: bool = False) -> str:
-    """Compile every HIP source for gfx950 and link libmsco_gmm.so."""
+def build_backend(verbose: bool = False, tuning: bool = False) -> str:
+    """Compile every HIP source for gfx950 and link libmsco_gmm.so (the operators) and libmsco_probes.so (the
+    benchmark's two yardstick kernels)."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     hipcc = _hipcc()
     hip_dir = os.path.join(CSRC, "hip")
@@ -47,14 +50,17 @@ def build_backend(verbose: bool = False) -> str:
         obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
         cmd = [hipcc] + HIP_FLAGS + ["-DMSCO_BUILDING_LIB", "-I", INCLUDE, "-I", hip_dir, "-c",
                                      os.path.join(hip_dir, src), "-o", obj]
+        if tuning:   # development build: the planner's constants can be overridden from the environment (MSCO_TILE_CFG, ...)
+            cmd.insert(1, "-DMSCO_TUNING_SWITCHES")
         out = _run(cmd)
         if verbose and out.strip():
             print(out)
         return obj
 
     with cf.ThreadPoolExecutor(max_workers=8) as pool:
-        objs = list(pool.map(compile_one, HIP_SOURCES))
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", BACKEND_LIB] + objs)
+        objs = list(pool.map(compile_one, HIP_SOURCES + PROBE_SOURCES))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", BACKEND_LIB] + objs[:len(HIP_SOURCES)])
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", PROBES_LIB] + objs[len(HIP_SOURCES):])
     return BACKEND_LIB
 
 
@@ -120,11 +126,11 @@ def build_pybind(verbose: bool = False) -> str:
     return target
 
 
-def build_all(verbose: bool = False):
-    return build_backend(verbose), build_pybind(verbose)
+def build_all(verbose: bool = False, tuning: bool = False):
+    return build_backend(verbose, tuning), build_pybind(verbose)
 
 
 if __name__ == "__main__":
-    paths = build_attribution("-v" in sys.argv) if "--attribution" in sys.argv else build_all(verbose="-v" in sys.argv)
+    paths = build_attribution("-v" in sys.argv) if "--attribution" in sys.argv else build_all(verbose="-v" in sys.argv, tuning="--tuning" in sys.argv)
     for path in paths:
         print("built", path)

@@ -36,7 +36,8 @@ EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco
                     "msco_status_string", "msco_gmm_abi_version", "msco_transpose_2d",
                     "msco_packed_weight_bytes", "msco_pack_weight", "msco_gmm_a8w4", "msco_unpack_int4",
                     "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_init_routing_v2_quant",
-                    "msco_moe_token_unpermute", "msco_probe_mfma", "msco_probe_read", "msco_gmm_launch_static")
+                    "msco_moe_token_unpermute", "msco_gmm_launch_static")
+PROBE_SYMBOLS = ("msco_probe_mfma", "msco_probe_read")   # libmsco_probes.so, include/msco_probes.h
 STATIC_WORKSPACE_BYTES = 32 << 20
 PROBE_MFMA_WORKGROUPS, PROBE_MFMA_OPERAND_BYTES = 256, 8 * 256 * 16
 
@@ -55,6 +56,25 @@ class BackendError(RuntimeError):
 
 
 _lib = None
+
+
+_probes = None
+PROBES_LIB_PATH = os.path.join(_HERE, "lib", "libmsco_probes.so")
+
+
+def load_probes():
+    """Load the library of measurement aids (the benchmark's yardstick kernels; the operators never need it)."""
+    global _probes
+    if _probes is None:
+        if not os.path.exists(PROBES_LIB_PATH):
+            raise ImportError(f"probe library missing: {PROBES_LIB_PATH}; build it with `python ms_custom_ops_amd/build.py`")
+        lib = ctypes.CDLL(PROBES_LIB_PATH)
+        lib.msco_probe_read.restype = ctypes.c_int
+        lib.msco_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_probe_mfma.restype = ctypes.c_int
+        lib.msco_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
+        _probes = lib
+    return _probes
 
 
 def load():
@@ -105,10 +125,6 @@ def load():
         lib.msco_moe_token_unpermute.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int64] * 3 + [ctypes.c_int32, ctypes.c_void_p]
         lib.msco_gmm_launch_static.restype = ctypes.c_int
         lib.msco_gmm_launch_static.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_void_p]
-        lib.msco_probe_read.restype = ctypes.c_int
-        lib.msco_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
-        lib.msco_probe_mfma.restype = ctypes.c_int
-        lib.msco_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
         _lib = lib
     return _lib
 
@@ -155,16 +171,16 @@ def unpack_int4(src: int, dst: int, src_bytes: int, stream: Optional[int] = None
 
 
 def probe_mfma(operands: int, sink: int, iters: int, stream: Optional[int] = None):
-    """Raw-pointer call of msco_probe_mfma (see include/msco_gmm.h); PROBE_MFMA_WORKGROUPS * 4 * iters * 16 * 65536 int8
+    """Raw-pointer call of msco_probe_mfma (see include/msco_probes.h); PROBE_MFMA_WORKGROUPS * 4 * iters * 16 * 65536 int8
     operations per launch."""
     vp = lambda v: ctypes.c_void_p(v if v else None)
-    _check("msco_probe_mfma", load().msco_probe_mfma(vp(operands), vp(sink), iters, vp(stream)))
+    _check("msco_probe_mfma", load_probes().msco_probe_mfma(vp(operands), vp(sink), iters, vp(stream)))
 
 
 def probe_read(src: int, nbytes: int, sink: int, workgroups: int, stream: Optional[int] = None):
-    """Raw-pointer call of msco_probe_read (see include/msco_gmm.h)."""
+    """Raw-pointer call of msco_probe_read (see include/msco_probes.h)."""
     vp = lambda v: ctypes.c_void_p(v if v else None)
-    _check("msco_probe_read", load().msco_probe_read(vp(src), nbytes, vp(sink), workgroups, vp(stream)))
+    _check("msco_probe_read", load_probes().msco_probe_read(vp(src), nbytes, vp(sink), workgroups, vp(stream)))
 
 
 def moe_init_routing_v2_workspace_bytes(num_rows: int, k: int, expert_num: int) -> int:

@@ -41,12 +41,16 @@ int env_int(const char *name, int fallback) {
   return (v && *v) ? std::atoi(v) : fallback;
 }
 
-// Debug switches, read from the environment once per process (the first plan); planning itself reads no environment.
+// MSCO_PRINT_PLAN (the counterpart of the reference's INTERNAL_PRINT_TILING) is read from the environment once per
+// process, at the first plan; planning itself reads no environment.  The other fields override plan constants for
+// tuning sweeps and exist only in a library built with -DMSCO_TUNING_SWITCHES (build.py --tuning): the shipped
+// library has no such switches.
 struct Tuning {
   int print_plan, tile_cfg, tile_target_wgs, tile_split_k, stream_max_slots, skinny_wide16, stream_min_wgs, stream_groups,
       skinny_target_wgs, skinny_split_k, tile_wide_k, stream_tch, two_level;
 };
 const Tuning &tuning() {
+#ifdef MSCO_TUNING_SWITCHES
   static const Tuning t = {env_int("MSCO_PRINT_PLAN", 0),        env_int("MSCO_TILE_CFG", -1),
                            env_int("MSCO_TILE_TARGET_WGS", 0),   env_int("MSCO_TILE_SPLIT_K", 0),
                            env_int("MSCO_STREAM_MAX_SLOTS", 0),  env_int("MSCO_SKINNY_WIDE16", -1),
@@ -54,6 +58,9 @@ const Tuning &tuning() {
                            env_int("MSCO_SKINNY_TARGET_WGS", 0), env_int("MSCO_SKINNY_SPLIT_K", 0),
                            env_int("MSCO_TILE_WIDE_K", -1),      env_int("MSCO_STREAM_TCH", 0),
                            env_int("MSCO_TWO_LEVEL", 1)};
+#else
+  static const Tuning t = {env_int("MSCO_PRINT_PLAN", 0), -1, 0, 0, 0, -1, 0, 0, 0, 0, -1, 0, 1};
+#endif
   return t;
 }
 int or_default(int v, int fallback) { return v > 0 ? v : fallback; }

@@ -1,4 +1,4 @@
-// Measurement aids (nothing here enters the operators).
+// Measurement aids, built into a library of their own (nothing here enters the operators).
 //
 // 1. What the matrix pipe of this chip sustains on a given operand distribution with no memory traffic.
 // 256 workgroups (one per compute unit) of four wavefronts (one per SIMD) each run `iters` rounds of the 16
@@ -13,7 +13,7 @@
 // neighbouring 1 KiB pieces (16 bytes per lane), eight loads in flight per wavefront, non-temporal loads: the access
 // pattern of the packed-layout decode kernels.
 #include "gmm_common.h"
-#include "msco_gmm.h"
+#include "msco_probes.h"
 
 namespace msco {
 namespace {

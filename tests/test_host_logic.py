@@ -32,14 +32,21 @@ I8, I32, I64, U64, F16, F32, BF16 = 32, 34, 35, 40, 42, 43, 45
 
 # ------------------------------------------------------------------------------------- C ABI surface
 def test_header_symbols_are_exported():
-    declared = set()
-    for name in sorted(os.listdir(os.path.join(REPO, "include"))):   # every header: msco_gmm.h, msco_moe.h
+    declared, probes = set(), set()
+    for name in sorted(os.listdir(os.path.join(REPO, "include"))):   # every header: msco_gmm.h, msco_moe.h, msco_probes.h
         header = open(os.path.join(REPO, "include", name)).read()
-        declared |= set(re.findall(r"MSCO_API\s+[\w\s\*]+?\b(msco_\w+)\s*\(", header))
-    assert declared == set(cabi.EXPORTED_SYMBOLS)
+        found = set(re.findall(r"MSCO_API\s+[\w\s\*]+?\b(msco_\w+)\s*\(", header))
+        if name == "msco_probes.h":
+            probes |= found
+        else:
+            declared |= found
+    assert declared == set(cabi.EXPORTED_SYMBOLS) and probes == set(cabi.PROBE_SYMBOLS)
     lib = cabi.load()
     for name in declared:
         assert hasattr(lib, name), name
+    for name in probes:   # the measurement aids live in a library of their own; the operator library does not export them
+        assert hasattr(cabi.load_probes(), name), name
+        assert not hasattr(lib, name), name
     assert lib.msco_gmm_abi_version() == cabi.ABI_VERSION == _C._backend_abi_version()
 
 
