@@ -2,7 +2,8 @@
 """Benchmark of the grouped W8A8 matmul path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout packed|nk|kn] [--no-sweep] [--no-cpu]
-    python bench.py --probe c3|c2_m16|...|copy|moe|mfma|read [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs)
+    python bench.py --probe c3|c2_m16|...|copy|moe|mfma|read|plan [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs;
+                                                            `plan`: the planner's picks against forced kernel families)
 
 A step is one pass of the hot path over one batch of synthetic input (inputs resident in HBM before
 the timed region).  The headline workload is the Mixtral-shaped MoE configuration (E=8, top-2 over
@@ -437,9 +438,68 @@ def measured_traffic(workload, layout, kernel):
     return entry["hbm_bytes_per_launch"]
 
 
+def plan_regret(steps=30):
+    """What the planner's pick costs against the kernel families it could have picked: neighbouring shapes of the dense
+    linear (K=4096, N=11008) and of the MoE layer (8 experts, top-2, K=4096, N=14336) on packed and on [E,K,N] weights,
+    each timed with the plan's own choice and with every family forced through msco_gmm_desc.kernel_override.
+    A row reads [workload, layout, picked kernel, us, best forced family, us, pick / best]; a ratio well above 1 is a
+    planner rule that is wrong for that shape."""
+    import torch
+    from ms_custom_ops_amd import cabi, workloads
+    forced = (("tile_256", cabi.OV_TILE_256), ("tile_256_w4", cabi.OV_TILE_256_W4), ("tile_128x256", cabi.OV_TILE_128x256),
+              ("tile_128", cabi.OV_TILE_128), ("tile_64", cabi.OV_TILE_64), ("decode", cabi.OV_SKINNY))
+    names = ["c2_m%d" % m for m in (1, 16, 17, 32, 64, 65, 128, 192, 256, 320, 384, 448, 512, 640, 704, 768, 1024, 1280, 1536, 2048, 3072)]
+    names += ["c3_t%d" % t for t in (8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 2048)]
+    rows = []
+    for name in names:
+        wl = workloads.make(name)
+        per_group = wl.m / wl.e
+        for layout in ("packed", "kn"):
+            copies = max(1, int(np.ceil(ROTATE_BYTES / (wl.e * wl.k * wl.n))))
+            prob = DeviceProblem(wl, layout, copies)
+
+            def period():   # (the warm-up of the headline measurement: until the launch period has settled)
+                return prob.time(steps, 10)[1] * 1e6
+
+            picked = prob.op.plan_info().split("kernel=")[1].split(" ")[0]
+            picked_op, picked_ws, picked_bytes = prob.op, prob.ws, prob.ws_bytes
+            period()        # (the first kernel after the set-up meets a cold chip: its figure is taken again at the end)
+            best = (None, float("inf"))
+            for fam, ov in forced:
+                # (families that would stream the weights dozens of times, or multiply mostly padding, are not candidates)
+                if (fam == "decode" and per_group > 64) or (fam == "tile_64" and per_group > 512) or \
+                        (fam in ("tile_256", "tile_256_w4") and wl.m < 64) or (fam in ("tile_128", "tile_128x256") and wl.m < 32):
+                    continue
+                try:
+                    op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,
+                                    scale_dtype=cabi.DT_F32, per_token_dtype=cabi.DT_F32,
+                                    bias_dtype=cabi.DT_I32 if prob.bias is not None else cabi.DT_NONE, kernel_override=ov,
+                                    weight_layout=cabi.WL_PACKED if layout == "packed" else cabi.WL_ROW_MAJOR)
+                    ws_bytes = op.plan(wl.m, wl.k, wl.n, wl.e)
+                except cabi.BackendError:
+                    continue
+                prob.op, prob.ws_bytes = op, ws_bytes
+                prob.ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device="cuda:0")
+                us = period()
+                if us < best[1]:
+                    best = (fam, us)
+            prob.op, prob.ws, prob.ws_bytes = picked_op, picked_ws, picked_bytes
+            us_pick = period()
+            rows.append([name, layout, picked, us_pick, best[0], best[1], us_pick / best[1] if best[0] else None])
+            del prob
+            torch.cuda.empty_cache()
+            print("plan_regret", rows[-1], file=sys.stderr, flush=True)
+    worst = max((r for r in rows if r[6] is not None), key=lambda r: r[6])
+    return {"columns": ["workload", "layout", "picked", "us", "best_forced_family", "us_forced", "pick_over_best"], "rows": rows,
+            "worst": worst}
+
+
 def probe(args):
     import torch
     from ms_custom_ops_amd import workloads
+    if args.probe == "plan":
+        print(json.dumps(compact({"probe": "plan", "plan_regret": plan_regret()})))
+        return
     if args.probe == "copy":
         src = torch.randint(-127, 128, (COPY_BYTES,), dtype=torch.int8, device="cuda:0")
         dst = torch.empty_like(src)

@@ -131,7 +131,9 @@ typedef struct msco_gmm_desc {
   int32_t transpose_b;       /* 0: weight [E,K,N]; 1: weight [E,N,K] */
   int32_t scale_per_group;   /* 1: scale/bias are [E,N]; 0: one [N] (or [1]) row shared by all groups */
   int32_t scale_is_scalar;   /* 1: scale holds a single element broadcast over N */
-  int32_t kernel_override;   /* 0 auto; else force a kernel family (see msco_gmm_plan_info), for tests */
+  int32_t kernel_override;   /* 0 auto; else force a kernel family, for tests and planner checks: 1 eight-wave 256 x 256 tile,
+                              * 2 128 x 128, 3 64 x 128, 4 decode (streaming) kernels, 5 generic, 6 persistent four-wave
+                              * 256 x 256, 7 128 x 256 (msco_gmm_plan_info names what was planned) */
   int32_t weight_layout;     /* MSCO_WL_ROW_MAJOR: as transpose_b says; MSCO_WL_PACKED: written by msco_pack_weight */
   int32_t act_type;          /* msco_act: activation applied to the dequantised float32 value before the output cast */
   int32_t force_split_k;     /* 0 auto; else the K split across workgroups of the kernels that have one, for tests */

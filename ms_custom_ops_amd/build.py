@@ -64,7 +64,10 @@ def build_backend(verbose: bool = False, tuning: bool = False) -> str:
     return BACKEND_LIB
 
 
-ATTRIBUTION_BUILDS = {"noepi": 1, "nomfma": 2, "nomfma_noepi": 3, "nostore": 4}
+ATTRIBUTION_BUILDS = {"noepi": 1, "nomfma": 2, "nomfma_noepi": 3, "nostore": 4,
+                      # the K loop alone (no epilogue) without its memory requests, its LDS writes, its barriers, and with
+                      # nothing but MFMAs and fragment reads
+                      "kloop_noload": 1 | 8, "kloop_nowrite": 1 | 16, "kloop_nobarrier": 1 | 32, "kloop_mfma_lds": 1 | 8 | 16}
 
 
 def build_attribution(verbose: bool = False):
@@ -89,7 +92,8 @@ def build_attribution(verbose: bool = False):
         return lib
 
     with cf.ThreadPoolExecutor(max_workers=4) as pool:
-        return list(pool.map(build_one, ATTRIBUTION_BUILDS.items()))
+        only = [a for a in sys.argv if a in ATTRIBUTION_BUILDS]
+        return list(pool.map(build_one, [(k, v) for k, v in ATTRIBUTION_BUILDS.items() if not only or k in only]))
 
 
 def pybind_module_path() -> str:

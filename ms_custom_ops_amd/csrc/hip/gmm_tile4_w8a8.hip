@@ -59,7 +59,9 @@ constexpr int T4_LD = T4_BM / 8 / T4_NW;         // staging quads (8 rows x 128 
 // so that timing the rest says what that part costs (results are then wrong on purpose).  1: the epilogue sits behind
 // a branch that no launch takes (its code and registers stay); 2: every MFMA becomes an empty statement that keeps
 // both operand fragments alive (loads, LDS traffic and barriers unchanged); 4: the epilogue computes everything and
-// its output stores become empty statements.
+// its output stores become empty statements; 8: the K loop requests no operands from memory (the staging registers keep
+// what the prologue brought); 16: staging registers are not written to LDS (loads are still waited for); 32: the K
+// loop's workgroup barriers are left out.
 #ifndef MSCO_TILE4_ATTR
 #define MSCO_TILE4_ATTR 0
 #endif
@@ -326,6 +328,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   // slab s of the current tile, or slab s - k_slabs of the next one
   auto load_one = [&](int s, auto par_c, auto op_c, auto u_c) {
     constexpr int P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
+#if MSCO_TILE4_ATTR & 8
+    if (s >= 2) return;   // (the prologue's slabs 0 and 1 only)
+#endif
     const bool ahead = s >= k_slabs;
     const unsigned kbase = (unsigned)(ahead ? s - k_slabs : s) * T4_BK;
     const bool dead = (ahead && !nxt.valid) || kbase + d_chunk * 16 >= (unsigned)p.k;   // K tail, slabs past K, no next tile
@@ -353,7 +358,11 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
       v.y = y;
       v.z = z;
     }
+#if MSCO_TILE4_ATTR & 16
+    asm volatile("" ::"v"(v), "v"(addr));
+#else
     *reinterpret_cast<v4i *>(smem + addr) = v;
+#endif
   };
   // write quad (op, u) of slab s to its LDS stage and refill it with slab s + 2
   auto cycle_one = [&](int s, auto par_c, auto op_c, auto u_c) {
@@ -367,8 +376,12 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   auto cycle_clean = [&](auto ws_c, unsigned soff, __amdgpu_buffer_rsrc_t rw_s, unsigned soff_w, auto par_c, auto op_c, auto u_c) {
     constexpr int WS = decltype(ws_c)::value, P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
     put_quad((OP == 0 ? st_x : st_w) + WS * T4_OP_STAGE + U * 4096, stg[P][OP][U], op_c);
+#if MSCO_TILE4_ATTR & 8
+    asm volatile("" : "+v"(stg[P][OP][U]));
+#else
     if constexpr (OP == 0) stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rx_c, a_voff0 + U * rows32, soff, 0);
     else stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rw_s, b_voff0 + U * b_step, soff_w, 0);
+#endif
   };
   // [E,K,N] weight fragment: two transpose reads, K rows 0 .. 7 and 8 .. 15 of the lane's column
   auto read_tr = [&](unsigned addr) -> v4i {
@@ -548,7 +561,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         // slab kt+1 is in LDS (this wave's part) and the quarter-3 fragments are in registers: after the
         // barrier every wave's part is visible and nobody reads this stage any more
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#if !(MSCO_TILE4_ATTR & 32)
         t4_barrier();
+#endif
         quarter(c1, c0, stage ^ 1, 0, kt + 2, other, c0);
       };
       // The same with stage, quarter and parity known at compile time, for slabs whose look-ahead stays inside the
@@ -579,7 +594,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
         quarter_clean(c1, c0, stage_c, c2, other_stage, soff3, rw3, par_c, c2);
         quarter_clean(c0, c1, stage_c, c3, other_stage, soff3, rw3, par_c, c3);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#if !(MSCO_TILE4_ATTR & 32)
         t4_barrier();
+#endif
         quarter_clean(c1, c0, other_stage, c0, stage_c, soff4, rw4, other, c0);
       };
       // iterations whose furthest request (group 0 of slab kt + 5) ends inside K

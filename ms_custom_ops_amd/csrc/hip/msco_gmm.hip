@@ -23,7 +23,8 @@ enum Family : int { FAM_NONE = 0, FAM_TILE = 1, FAM_SKINNY = 2, FAM_GENERIC = 3 
 // values of msco_gmm_desc::kernel_override
 enum Override : int {
   OV_AUTO = 0, OV_TILE_256 = 1, OV_TILE_128 = 2, OV_TILE_64 = 3, OV_SKINNY = 4, OV_GENERIC = 5,
-  OV_TILE_256_W4 = 6   // persistent four-wave 256 x 256 kernel ([E,N,K] weights; other layouts fall back to OV_TILE_256)
+  OV_TILE_256_W4 = 6,  // persistent four-wave 256 x 256 kernel
+  OV_TILE_128x256 = 7  // four waves side by side, 128 x 256
 };
 
 constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned
@@ -105,7 +106,7 @@ int check_desc(const msco_gmm_desc &d) {
   if (d.group_list_dtype != MSCO_DT_NONE && d.group_list_dtype != MSCO_DT_I32 && d.group_list_dtype != MSCO_DT_I64)
     return MSCO_ERR_UNSUPPORTED;
   if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
-  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_256_W4) return MSCO_ERR_INVALID_ARG;
+  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_128x256) return MSCO_ERR_INVALID_ARG;
   if (d.weight_layout != MSCO_WL_ROW_MAJOR && d.weight_layout != MSCO_WL_PACKED) return MSCO_ERR_INVALID_ARG;
   if (d.force_split_k < 0) return MSCO_ERR_INVALID_ARG;
   if (d.act_type < MSCO_ACT_NONE || d.act_type > MSCO_ACT_SILU) return MSCO_ERR_INVALID_ARG;
@@ -197,7 +198,11 @@ void choose_plan(msco_gmm_op *op) {
     const int64_t busy = (num_cus > 0 ? num_cus : kTileTargetWorkgroups) * 3 / 4;
     // (the persistent four-wave kernel: at least four 128-byte K slabs per tile, a group table that fits in LDS)
     const bool w4_ok = k >= 512 && e <= 1024;
-    if (e > 1 && w4_ok && cover > 128 && cover <= 384 && group_tiles(256, 256) >= busy) {
+    // (128-row m-tiles while every group fits one: 8 experts, 72 .. 112 rows per group on average, the largest group 80 ..
+    // 126 rows: 84 - 92 us with 128 x 256 tiles against 100 - 109 us with 256 x 256; at 120 rows on average the largest
+    // group has 131, streams its weights twice and the launch takes 126 against 113 us -- so the 256-row tile takes
+    // over at 1.5 x the average = 160 rows, not at 128)
+    if (e > 1 && w4_ok && cover > 160 && cover <= 384 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
     } else if (e > 1 && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
       // (128 x 256 tiles re-read x half as often: 64 / 96 rows per group 93 / 99 us against 100 / 111 us)
@@ -229,6 +234,7 @@ void choose_plan(msco_gmm_op *op) {
     case OV_TILE_256: family = FAM_TILE; op->tile_cfg = TILE_256x256; break;
     case OV_TILE_256_W4: family = FAM_TILE; op->tile_cfg = TILE_256x256_W4; break;
     case OV_TILE_128: family = FAM_TILE; op->tile_cfg = TILE_128x128; break;
+    case OV_TILE_128x256: family = FAM_TILE; op->tile_cfg = TILE_128x256; break;
     case OV_TILE_64: family = FAM_TILE; op->tile_cfg = TILE_64x128; break;
     case OV_SKINNY: family = FAM_SKINNY; break;
     case OV_GENERIC: family = FAM_GENERIC; break;
