@@ -67,7 +67,8 @@ def build_backend(verbose: bool = False, tuning: bool = False) -> str:
 ATTRIBUTION_BUILDS = {"noepi": 1, "nomfma": 2, "nomfma_noepi": 3, "nostore": 4,
                       # the K loop alone (no epilogue) without its memory requests, its LDS writes, its barriers, and with
                       # nothing but MFMAs and fragment reads
-                      "kloop_noload": 1 | 8, "kloop_nowrite": 1 | 16, "kloop_nobarrier": 1 | 32, "kloop_mfma_lds": 1 | 8 | 16}
+                      "kloop_noload": 1 | 8, "kloop_nowrite": 1 | 16, "kloop_nobarrier": 1 | 32, "kloop_mfma_lds": 1 | 8 | 16,
+                      "kloop_mfma": 1 | 8 | 16 | 64, "kloop_noread": 1 | 64}
 
 
 def build_attribution(verbose: bool = False):

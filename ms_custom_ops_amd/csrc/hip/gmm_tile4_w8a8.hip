@@ -61,7 +61,8 @@ constexpr int T4_LD = T4_BM / 8 / T4_NW;         // staging quads (8 rows x 128 
 // both operand fragments alive (loads, LDS traffic and barriers unchanged); 4: the epilogue computes everything and
 // its output stores become empty statements; 8: the K loop requests no operands from memory (the staging registers keep
 // what the prologue brought); 16: staging registers are not written to LDS (loads are still waited for); 32: the K
-// loop's workgroup barriers are left out.
+// loop's workgroup barriers are left out; 64: the K loop reads no operand fragments from LDS (the MFMAs multiply what
+// the registers hold).
 #ifndef MSCO_TILE4_ATTR
 #define MSCO_TILE4_ATTR 0
 #endif
@@ -395,6 +396,10 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   // loop would park eight more addresses in registers that the loop does not have)
   auto read_w = [&](int stage, unsigned qx, auto set_c, auto f_c) {
     constexpr int S = decltype(set_c)::value, F = decltype(f_c)::value;
+#if MSCO_TILE4_ATTR & 64
+    asm volatile("" : "+v"(wf[S][F]));
+    return;
+#endif
     if constexpr (PK) {
       // qx = q << 5: K block q / 2 is 1024 bytes on, chunk pair q % 2 another 512
       wf[S][F] = *reinterpret_cast<const v4i *>(smem + stage * T4_OP_STAGE + (w_lane + (qx >> 6) * 1024 + ((qx >> 5) & 1) * 512) + F * 4096);
@@ -406,17 +411,29 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
   };
   auto read_x = [&](int stage, unsigned qx, auto set_c, auto i_c) {
     constexpr int S = decltype(set_c)::value, I = decltype(i_c)::value;
+#if MSCO_TILE4_ATTR & 64
+    asm volatile("" : "+v"(xf[S][I]));
+    return;
+#endif
     xf[S][I] = *reinterpret_cast<const v4i *>(smem + stage * T4_OP_STAGE + (x_lane ^ qx) + I * 32 * T4_BK);
   };
   // fragment reads with everything but the registers above known at compile time
   auto read_w_clean = [&](auto stage_c, auto q_c, auto set_c, auto f_c) {
     constexpr int ST = decltype(stage_c)::value, Q = decltype(q_c)::value, S = decltype(set_c)::value, F = decltype(f_c)::value;
+#if MSCO_TILE4_ATTR & 64
+    asm volatile("" : "+v"(wf[S][F]));
+    return;
+#endif
     if constexpr (PK) wf[S][F] = *reinterpret_cast<const v4i *>(smem + (w_lane + ST * T4_OP_STAGE + (Q >> 1) * 1024 + (Q & 1) * 512 + F * 4096));
     else if constexpr (KN) wf[S][F] = read_tr((w_lane ^ (unsigned)(F << 5)) + ST * T4_OP_STAGE + Q * 8192);
     else wf[S][F] = *reinterpret_cast<const v4i *>(smem + ((w_lane ^ (unsigned)(Q << 5)) + ST * T4_OP_STAGE + F * 4096));
   };
   auto read_x_clean = [&](auto stage_c, auto q_c, auto set_c, auto i_c) {
     constexpr int ST = decltype(stage_c)::value, Q = decltype(q_c)::value, S = decltype(set_c)::value, I = decltype(i_c)::value;
+#if MSCO_TILE4_ATTR & 64
+    asm volatile("" : "+v"(xf[S][I]));
+    return;
+#endif
     xf[S][I] = *reinterpret_cast<const v4i *>(smem + ((x_lane ^ (unsigned)(Q << 5)) + ST * T4_OP_STAGE + I * 4096));
   };
   auto opaque_q = [](int q) {
@@ -488,16 +505,25 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4_nk_kernel(const 
     const int rows_wave = rows_here - wave_m * T4_WT;
     const int fm_active = max(0, min(T4_F, (rows_wave + 31) / 32));
 
-    // (a zero the compiler cannot see through: a constant vector of zeros gets hoisted out of the tile loop into
-    // registers the K loops do not have)
-    int zero = 0;
-    asm volatile("" : "+v"(zero));
+    // The accumulators start at zero.  The matrix pipe clears them itself, a block of sixteen registers per instruction
+    // (zero operand, C = 0): 256 single register writes cost a wave that is alone on its SIMD three times as long.
+    // (the zero operand is made here, behind an empty asm: a constant vector of zeros would be hoisted out of the tile
+    // loop into registers the K loops do not have)
+    {
+      int zero = 0;
+      asm volatile("" : "+v"(zero));
+      const v4i z4 = {zero, zero, zero, zero};
+      // (the compiler does not know what the statements are, so the wait states between the zero's last write and the
+      // first read of it as a matrix operand, and between the last read and the register's next write, are written out;
+      // an accumulator block is first added to sixteen MFMAs after it was cleared)
+      asm volatile("s_nop 4" ::"v"(z4));
 #pragma unroll
-    for (int f = 0; f < T4_F; ++f)
+      for (int f = 0; f < T4_F; ++f)
 #pragma unroll
-      for (int i = 0; i < T4_F; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[f][i][r] = zero;
+        for (int i = 0; i < T4_F; ++i)
+          asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %1, 0" : "=a"(acc[f][i]) : "v"(z4));
+      asm volatile("s_nop 4" ::"v"(z4));
+    }
     // quarter-0 fragments of slab 0 (read here rather than behind the previous tile's last slab, so that
     // the epilogue does not have to keep them alive)
     read_w(0, 0, c0, c0); read_w(0, 0, c0, c1); read_w(0, 0, c0, c2); read_w(0, 0, c0, c3);
