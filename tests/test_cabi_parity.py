@@ -289,3 +289,24 @@ def test_hundreds_of_experts_few_rows_decode_kernels_enumerate_only_chunks_with_
         acc, info = run_w8a8(x, w, gl, bias, out="i32", transpose_b=layout == "nk", packed=layout == "packed",
                              group_list_type=gl_type)
         assert np.array_equal(acc[:last], ref_acc[:last]), info
+
+
+@pytest.mark.parametrize("layout", ["kn", "nk", "packed"])
+def test_groups_of_about_a_hundred_rows_take_128_row_tiles_and_the_forced_128x256_family_agrees(device, layout):
+    """Eight groups of 70 .. 126 rows (the MoE layer at a few hundred tokens): the plan gives them 128-row m-tiles while
+    1.5 x the average group stays within 160 rows, and 256-row tiles beyond; both are bit-exact, and so is the 128 x 256
+    family when it is forced (kernel_override 7) on groups that spill into a second m-tile."""
+    from gpu_utils import run_w8a8
+    e, k, n = 8, 512, 6144
+    for counts, want in (([96, 70, 126, 101, 88, 113, 90, 84], "128x256"), ([120, 131, 96, 150, 118, 109, 140, 96], "256x256")):
+        m = sum(counts) + 3                       # (three rows stay behind the last boundary)
+        rng, x, w, bias, scale, pt = _inputs(m, m, k, n, e)
+        ends = np.cumsum(counts)
+        last = int(ends[-1])
+        ref = O.grouped_matmul_w8a8(x, w, ends, bias, scale, pt)
+        for override in (0, cabi.OV_TILE_128x256):
+            bits, info = run_w8a8(x, w, ends, bias, scale, pt, out="bf16", transpose_b=layout == "nk", packed=layout == "packed",
+                                  override=override, launches=2)
+            assert ("128x256" if override else want) in info, info
+            assert np.array_equal(bits[:last], ref[:last]), info
+            assert (bits[last:] == 0x7FC0).all(), info
