@@ -10,8 +10,9 @@
 //   * group_type 0 (one x [M,K], one weight [E,K,N], one output [M,N]) is one grouped launch of the
 //     HIP backend: W8A8 with per-channel scale / per-token scale / int32 bias, or weight-only
 //     (bf16/f16 x, int8 weight, antiquant scale and offset [E,N]); with a qint4x2 weight [E,K,N/2] (A8W4,
-//     tests/st/test_grouped_matmul_v4_cops.py:429-485) the nibble pairs are widened to int8 on the device first
-//     (msco_unpack_int4) and the W8A8 launch multiplies them: exact, at the price of one more pass over the weights;
+//     tests/st/test_grouped_matmul_v4_cops.py:429-485, and A16W4, :197-262) the nibble pairs are widened to int8 on the
+//     device first (msco_unpack_int4) and the W8A8 or the weight-only launch multiplies them: exact, at the price of
+//     one more pass over the weights;
 //   * group_type -1 (independent x[i] @ weight[i]) is one dense launch per pair.
 // Not implemented on this backend and refused with a message: float x float matmuls,
 // uint64 scales with int8 output, `offset`, the activation inputs, group_type 1.  act_type selects an activation
@@ -65,11 +66,13 @@ void CheckV4Support(const V4Args &a) {
   }
   const TypeId xt = a.x[0].data_type(), wt = a.weight[0].data_type();
   if (wt == kNumberTypeInt4) {
-    // A8W4 (tests/st/test_grouped_matmul_v4_cops.py:429-485): int8 x, qint4x2 weight [E, K, N / 2], one output
-    if (xt != kNumberTypeInt8 || a.group_type != kGroupTypeSingleOutput || a.weight_format != kNdFormat) {
-      MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", int4 weights are implemented for Int8 'x', group_type 0 "
-                       << "and weight_format 'ND' only, but got x dtype " << xt << ", group_type " << a.group_type
-                       << ", weight_format '" << a.weight_format << "'.";
+    // qint4x2 weight [E, K, N / 2], one output: A8W4 with int8 x (tests/st/test_grouped_matmul_v4_cops.py:429-485) and
+    // A16W4 with float16 / bfloat16 x and the antiquant inputs (:197-262)
+    if ((xt != kNumberTypeInt8 && xt != kNumberTypeFloat16 && xt != kNumberTypeBFloat16) ||
+        a.group_type != kGroupTypeSingleOutput || a.weight_format != kNdFormat) {
+      MS_LOG_EXCEPTION << "For " << kGroupedMatmulV4CopsName << ", int4 weights are implemented for Int8, Float16 or "
+                       << "BFloat16 'x', group_type 0 and weight_format 'ND' only, but got x dtype " << xt
+                       << ", group_type " << a.group_type << ", weight_format '" << a.weight_format << "'.";
     }
     return;
   }

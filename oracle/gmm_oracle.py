@@ -42,6 +42,9 @@ How each function is pinned (tests/test_oracle_pins.py):
                            reference's own tolerances.
 * ``a16w8_*``              float64 evaluation of x @ ((w + o) * s) on the exact
                            bf16 operand values; closed forms with constant scale.
+* ``golden_v4_a16w4``      the reference's own packing loop written out per byte, the a16w8 formula on the unpacked
+                           values in float64, and the closed form of its test data (weights in {0, 1}, scale 0.01,
+                           offset 1: row sums of x times 0.01 plus 0.01 times the sum over the ones).
 * ``decode_scale_int64``   round trip against the two wire formats above.
 * ``activation``           what the mathematics fixes: torch's relu / silu / gelu(approximate="tanh") in float64,
                            the tanh form of the gelu against the sigmoid form used here, CANN's published fast-gelu
@@ -59,7 +62,7 @@ __all__ = [
     "pack_int4", "unpack_int4", "quant_int4_groups", "golden_grouped_a8w4", "grouped_a8w4_f64",
     "f32_to_bf16_bits", "bf16_bits_to_f32", "f32_to_f16", "int32_matmul_exact", "int32_matmul_bruteforce",
     "group_bounds", "grouped_int32_acc", "dequant_epilogue", "grouped_matmul_w8a8", "golden_np_qbmm",
-    "golden_grouped_w8a8", "golden_v4_pertoken", "golden_v4_perchannel_bias", "golden_v4_a16w8",
+    "golden_grouped_w8a8", "golden_v4_pertoken", "golden_v4_perchannel_bias", "golden_v4_a16w8", "golden_v4_a16w4",
     "quant_batch_matmul_oracle", "a16w8_grouped_f64", "encode_scale_int64", "encode_scale_int64_qbmm", "pack_weights",
     "decode_scale_int64", "random_group_list", "count_compare", "bf16_ulp_check", "activation",
     "ACT_NONE", "ACT_RELU", "ACT_GELU_TANH", "ACT_GELU_ERF", "ACT_FAST_GELU", "ACT_SILU",
@@ -344,6 +347,14 @@ def golden_v4_a16w8(x, w, antiquant_scale, antiquant_offset, ends):
     parts = [np.matmul(x[int(s):int(t)], (w[g] + antiquant_offset[g]) * antiquant_scale[g])
              for g, (s, t) in enumerate(zip(starts, ends_))]
     return np.concatenate(parts, axis=0)
+
+
+def golden_v4_a16w4(x, w, antiquant_scale, antiquant_offset, ends):
+    """The reference's expected value for grouped_matmul_v4_cops with float16 / bfloat16 x and 4-bit weights
+    (tests/st/test_grouped_matmul_v4_cops.py:223-241): w holds the int8 VALUES [e, k, n] (the op itself receives
+    pack_int4(w): value 2 i in the low nibble and 2 i + 1 in the high nibble of byte i along the flattened tensor, i.e.
+    pairs along n, :229-233); the expected value is the a16w8 formula on those values, matmul(x_g, (w_g + o_g) * s_g)."""
+    return golden_v4_a16w8(x, w, antiquant_scale, antiquant_offset, ends)
 
 
 # --------------------------------------------------------------------------

@@ -322,6 +322,68 @@ def test_v4_a8w4_full_nibble_range_ragged_groups_and_rules(device):
         ms_custom_ops.as_qint4x2(_t(x).int())
 
 
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_v4_a16w4_reference_case(device, mode, dtype):
+    """The reference's A16W4 case (tests/st/test_grouped_matmul_v4_cops.py:197-262): float16 x in [-128, 127), qint4x2
+    weight [e, k, n / 2] holding values 0 / 1 (two nibbles per byte along n, low nibble first), antiquant scale 0.01 and
+    offset 1 in x's dtype, cumulative group_list whose last boundary (30) lies below the 32 rows; same shapes, data
+    distribution and tolerance (rtol = atol = 1e-3 against the numpy golden on its float16 case).  This build's bar on
+    top, for both 16-bit types: one output ulp of the float64 value plus float32 accumulation noise."""
+    np.random.seed(3)
+    m, k, n, e = 32, 256, 128, 8
+    ends = np.array([1, 3, 10, 14, 18, 22, 24, 30], dtype=np.int64)
+    x_np = np.random.uniform(-128, 127, size=[m, k]).astype(np.float16)
+    w_np = (np.random.uniform(0, 2, size=[e, k, n]).astype(np.int8)) & 0xF
+    s_np = np.full([e, n], 0.01).astype(np.float16)
+    o_np = np.full([e, n], 1).astype(np.float16)
+    w_int4 = O.pack_int4(w_np)
+    assert w_int4.shape == (e, k, n // 2)
+    x, s, o = _t(x_np.astype(np.float32), dtype), _t(s_np.astype(np.float32), dtype), _t(o_np.astype(np.float32), dtype)
+    with ms_custom_ops.exec_mode(mode):
+        for _ in range(2):   # the second call reuses the graph-mode module and its staging slice
+            res = ms_custom_ops.grouped_matmul_v4_cops([x], [ms_custom_ops.as_qint4x2(_t(w_int4))], None, None, None, [s], [o],
+                                                       None, _t(ends), None, None, None, 3, 0, 0)
+            assert res[0].dtype == dtype and res[0].shape == (m, n)
+            got = res[0][:30].float().cpu().numpy().astype(np.float64)
+            if dtype == torch.float16:   # the reference's comparison, on its own golden
+                expect = O.golden_v4_a16w4(x_np, w_np, s_np, o_np, ends)
+                np.testing.assert_allclose(expect.astype(np.float64), got, rtol=1e-3, atol=1e-3)
+            xf, sf, of = x.float().cpu().numpy(), s.float().cpu().numpy(), o.float().cpu().numpy()
+            exact = O.a16w8_grouped_f64(xf, w_np, sf, of, ends)[:30]
+            mag = np.zeros_like(exact)
+            starts = np.concatenate([[0], ends[:-1]])
+            for g in range(e):
+                a, b = int(starts[g]), int(ends[g])
+                mag[a:b] = np.abs(xf[a:b].astype(np.float64)) @ (np.abs(w_np[g].astype(np.float64) + of[g]) * np.abs(sf[g]))
+            ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+            assert (np.abs(got - exact) <= ulp * np.abs(exact) + 1e-5 * mag).all()
+
+
+def test_v4_a16w4_signed_nibbles_ragged_groups_equal_the_a16w8_path(device):
+    """Every 4-bit value (-8 .. 7), empty groups, rows behind the last boundary: the A16W4 result is bit for bit the a16w8
+    result on the same values given as int8 (the nibbles are widened, then the same kernels run), in both modes."""
+    rng = np.random.default_rng(12)
+    e, m, k, n = 8, 70, 192, 96
+    w = rng.integers(-8, 8, (e, k, n), dtype=np.int8)
+    assert w.min() == -8 and w.max() == 7
+    counts = np.array([0, 9, 0, 27, 1, 0, 20, 6], dtype=np.int64)
+    for dtype in (torch.bfloat16, torch.float16):
+        x = _t(rng.uniform(-2, 2, (m, k)).astype(np.float32), dtype)
+        s = _t(rng.uniform(0.005, 0.02, (e, n)).astype(np.float32), dtype)
+        o = _t(rng.integers(-3, 4, (e, n)).astype(np.float32), dtype)
+        f = ms_custom_ops.grouped_matmul_v4_cops
+        ref = f([x], [_t(w)], None, None, None, [s], [o], None, _t(counts), None, None, None, 3, 0, 1)[0]
+        for mode in MODES:
+            with ms_custom_ops.exec_mode(mode):
+                out = f([x], [ms_custom_ops.as_qint4x2(_t(O.pack_int4(w)))], None, None, None, [s], [o], None, _t(counts), None,
+                        None, None, 3, 0, 1)[0]
+            last = int(counts.sum())
+            assert torch.equal(out[:last].view(torch.int16), ref[:last].view(torch.int16))
+    with pytest.raises(ValueError, match="needs 'antiquant_scale'"):
+        f([x], [ms_custom_ops.as_qint4x2(_t(O.pack_int4(w)))], group_list=_t(counts), split_item=3, group_type=0, group_list_type=1)
+
+
 def test_unpack_int4_through_the_c_abi(device):
     """msco_unpack_int4 against the oracle's unpack, sizes that end inside a 16-byte piece included."""
     from ms_custom_ops_amd import cabi

@@ -460,3 +460,41 @@ def test_v4_a8w4_golden_against_exact_integers_a_scalar_loop_and_the_wire_format
     literal = (flat[0::2] | (flat[1::2] << 4)).reshape(1, 1, 2)
     assert np.array_equal(literal.astype(np.uint8), np.array([[[0xF1, 0x87]]], dtype=np.uint8))
     assert np.array_equal(O.pack_int4(wn), literal.astype(np.uint8)) and np.array_equal(O.unpack_int4(O.pack_int4(w)), w)
+
+
+def test_v4_a16w4_golden_against_the_reference_packing_loop_float64_and_the_closed_form_of_its_data():
+    """golden_v4_a16w4 (tests/st/test_grouped_matmul_v4_cops.py:197-262): the nibble packing the reference's test writes
+    out as a loop (:229-233) is what pack_int4 produces; the expected value is the a16w8 formula on the unpacked values,
+    checked in float64 and, on the test's own data (weights in {0, 1}, scale 0.01, offset 1), against a closed form."""
+    rng = np.random.default_rng(21)
+    e, k, n, m = 3, 8, 6, 7
+    w = rng.integers(-8, 8, (e, k, n)).astype(np.int8)
+    flat = w.reshape(-1)
+    by_loop = np.zeros(flat.size // 2, dtype=np.int8)
+    for i in range(flat.size // 2):   # the reference's loop, values masked to their nibbles
+        by_loop[i] = np.int8(np.uint8((int(flat[2 * i]) & 15) | ((int(flat[2 * i + 1]) & 15) << 4)))
+    packed = O.pack_int4(w)
+    assert packed.shape == (e, k, n // 2) and np.array_equal(packed.reshape(-1).view(np.int8), by_loop)
+    assert np.array_equal(O.unpack_int4(packed), w)
+    # the formula in float64 on the unpacked values
+    ends = np.array([2, 2, 6], dtype=np.int64)          # an empty group, one row behind the last boundary
+    x = rng.uniform(-4, 4, (m, k)).astype(np.float16)
+    s = rng.uniform(0.01, 0.02, (e, n)).astype(np.float16)
+    o = rng.integers(-2, 3, (e, n)).astype(np.float16)
+    got = O.golden_v4_a16w4(x, O.unpack_int4(packed), s, o, ends)
+    assert got.shape == (6, n) and got.dtype == np.float16
+    starts = [0, 2, 2]
+    for g in range(e):
+        a, b = starts[g], int(ends[g])
+        want = x[a:b].astype(np.float64) @ ((w[g].astype(np.float64) + o[g].astype(np.float64)) * s[g].astype(np.float64))
+        np.testing.assert_allclose(got[a:b].astype(np.float64), want, rtol=2e-3, atol=2e-3)
+    # the test's data: weights 0 / 1, scale 0.01, offset 1  ->  0.01 * (rowsum(x) + x @ w), exactly in float64
+    w01 = rng.integers(0, 2, (e, k, n)).astype(np.int8)
+    s01, o01 = np.full((e, n), 0.01, np.float16), np.full((e, n), 1, np.float16)
+    got01 = O.a16w8_grouped_f64(x.astype(np.float32), O.unpack_int4(O.pack_int4(w01)), s01.astype(np.float32),
+                                o01.astype(np.float32), ends)
+    for g in range(e):
+        a, b = starts[g], int(ends[g])
+        xs = x[a:b].astype(np.float64)
+        want = np.float64(np.float16(0.01)) * (xs.sum(1, keepdims=True) + xs @ w01[g].astype(np.float64))
+        np.testing.assert_allclose(got01[a:b], want, rtol=1e-12, atol=1e-12)
