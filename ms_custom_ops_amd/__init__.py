@@ -51,7 +51,7 @@ except ImportError as exc:  # pragma: no cover - exercised only on a broken inst
 __all__ = ["grouped_matmul", "grouped_matmul_v4_cops", "grouped_matmul_w4", "quant_batch_matmul", "moe_init_routing_v2", "moe_init_routing_quant",
            "moe_token_unpermute", "set_context", "get_context", "exec_mode",
            "GRAPH_MODE", "PYNATIVE_MODE", "dtype_to_type_id", "type_id_to_dtype", "plan_cache_stats", "trans_data",
-           "qint4x2", "QInt4x2", "as_qint4x2"]
+           "qint4x2", "QInt4x2", "as_qint4x2", "widen_qint4x2"]
 
 GRAPH_MODE = 0
 PYNATIVE_MODE = 1
@@ -120,6 +120,23 @@ class QInt4x2:
 
 def as_qint4x2(tensor: torch.Tensor) -> QInt4x2:
     return QInt4x2(tensor)
+
+
+def widen_qint4x2(weight) -> torch.Tensor:
+    """4-bit weights widened to int8 once, at load time: [..., N / 2] nibble pairs (a QInt4x2 or the int8 / uint8 bytes
+    themselves; low nibble first, signed) become an int8 tensor [..., N] that grouped_matmul_v4_cops takes like any int8
+    weight.  The op widens a qint4x2 weight on every call (one more pass over the weights); a caller whose weights do
+    not change does it here and keeps the result.  No counterpart in the reference, whose kernels read 4-bit weights
+    directly (ops/c_api/grouped_matmul_v4_cops/grouped_matmul_v4_cops.cc:56-66)."""
+    t = weight.tensor if isinstance(weight, QInt4x2) else QInt4x2(weight).tensor
+    if not t.is_cuda:
+        raise RuntimeError("widen_qint4x2 takes a GPU tensor (the operators have no CPU path)")
+    from . import cabi
+    src = t.contiguous()
+    out = torch.empty(tuple(src.shape[:-1]) + (2 * src.shape[-1],), dtype=torch.int8, device=src.device)
+    with torch.cuda.device(src.device):
+        cabi.unpack_int4(src.data_ptr(), out.data_ptr(), src.numel(), torch.cuda.current_stream().cuda_stream)
+    return out
 
 
 # ---- framework hooks: PyTorch owns device memory and streams -------------------------------------

@@ -384,6 +384,35 @@ def test_v4_a16w4_signed_nibbles_ragged_groups_equal_the_a16w8_path(device):
         f([x], [ms_custom_ops.as_qint4x2(_t(O.pack_int4(w)))], group_list=_t(counts), split_item=3, group_type=0, group_list_type=1)
 
 
+def test_widen_qint4x2_once_then_the_int8_paths(device):
+    """Weights widened at load time give the same bits as the op's per-call widening, for A8W4 and for A16W4."""
+    rng = np.random.default_rng(13)
+    e, m, k, n = 4, 40, 128, 64
+    w = rng.integers(-8, 8, (e, k, n), dtype=np.int8)
+    packed = _t(O.pack_int4(w))
+    wide = ms_custom_ops.widen_qint4x2(ms_custom_ops.as_qint4x2(packed))
+    assert wide.dtype == torch.int8 and tuple(wide.shape) == (e, k, n) and np.array_equal(wide.cpu().numpy(), w)
+    assert torch.equal(ms_custom_ops.widen_qint4x2(packed.view(torch.uint8)), wide)
+    counts = _t(np.array([7, 0, 20, 13], dtype=np.int64))
+    f = ms_custom_ops.grouped_matmul_v4_cops
+    x8 = _t(rng.integers(-128, 128, (m, k), dtype=np.int8))
+    scale = rng.uniform(1e-3, 1e-2, (e, 1, n)).astype(np.float32)
+    pt = _t(rng.uniform(1e-3, 1e-2, (m, 1)).astype(np.float32))
+    su = torch.from_numpy(O.encode_scale_uint64(scale).view(np.int64)).cuda().view(torch.uint64)
+    a = f([x8], [ms_custom_ops.as_qint4x2(packed)], scale=[su], per_token_scale=[pt], group_list=counts, split_item=3, group_type=0,
+          group_list_type=1, output_dtype=torch.bfloat16)[0]
+    b = f([x8], [wide], scale=[_t(scale.reshape(e, n))], per_token_scale=[pt.reshape(m)], group_list=counts, split_item=3,
+          group_type=0, group_list_type=1, output_dtype=torch.bfloat16)[0]
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    x16 = _t(rng.uniform(-2, 2, (m, k)).astype(np.float32), torch.float16)
+    s16, o16 = _t(np.full((e, n), 0.01, np.float32), torch.float16), _t(np.full((e, n), 1, np.float32), torch.float16)
+    a = f([x16], [ms_custom_ops.as_qint4x2(packed)], None, None, None, [s16], [o16], None, counts, None, None, None, 3, 0, 1)[0]
+    b = f([x16], [wide], None, None, None, [s16], [o16], None, counts, None, None, None, 3, 0, 1)[0]
+    assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    with pytest.raises(RuntimeError, match="GPU tensor"):
+        ms_custom_ops.widen_qint4x2(packed.cpu())
+
+
 def test_unpack_int4_through_the_c_abi(device):
     """msco_unpack_int4 against the oracle's unpack, sizes that end inside a 16-byte piece included."""
     from ms_custom_ops_amd import cabi
