@@ -2,7 +2,7 @@
 """Benchmark of the grouped W8A8 matmul path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3] [--layout packed|nk|kn] [--no-sweep] [--no-cpu]
-    python bench.py --probe c3|c2_m16|...|copy|moe|mfma|read|plan [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs;
+    python bench.py --probe c3|c2_m16|...|copy|moe|mfma|issue|read|plan [--layout packed|nk|kn] [--steps K]     (for rocprofv3 counter runs;
                                                             `plan`: the planner's picks against forced kernel families)
 
 A step is one pass of the hot path over one batch of synthetic input (inputs resident in HBM before
@@ -19,7 +19,8 @@ Prints ONE JSON line.  Besides the contract keys it carries
   sweep         the other configurations (dense decode / prefill sweep, skewed MoE, weight-only decode, serving sizes,
                 the reference's own timing shapes) per weight layout, one row each under `columns`: launch period and
                 the int8 / HBM roofline fractions (TOP/s = int8_frac x 5000, GB/s = hbm_frac x 8000).
-`mfma_pipe` (and `--probe mfma`) is a yardstick: a loop of nothing but the int8 MFMA instruction on random and on zero operands.
+`mfma_pipe` (and `--probe mfma`) is a yardstick: loops of nothing but int8 MFMAs, either instruction shape, on random and on zero operands;
+`--probe issue` times the same loops with the K loop's memory operations woven in at different places.
 --probe runs a few untimed launches of one workload (or, for `copy`, of a plain device-to-device copy
 of COPY_BYTES bytes, the reference a counter reading is scaled by) so that a profiler sees nothing else.
 """
@@ -329,10 +330,11 @@ def moe_neighbours(steps, warmup):
 
 
 def mfma_pipe_probe(iters=20000, launches=12):
-    """Rate of a loop of nothing but v_mfma_i32_32x32x32_i8 (msco_probe_mfma: 256 workgroups, one wavefront per SIMD, no
-    memory traffic) on uniformly random int8 operands, the distribution of the workloads, and on zeros: what the matrix
-    pipe sustains at the clock the chip holds under each.  Every figure is the mean over the last half of the launches
-    (one pair of events around them), after the first half has let the clock settle."""
+    """Rate of a loop of nothing but int8 MFMAs (msco_probe_mfma_issue, patterns 0 and 12: 256 workgroups, one wavefront per
+    SIMD, no memory traffic) for both instruction shapes the tile kernels use, on uniformly random int8 operands, the
+    distribution of the workloads, and on zeros: what the matrix pipe sustains at the clock the chip holds under each.
+    Every figure is the mean over the last half of the launches (one pair of events around them), after the first half
+    has let the clock settle."""
     import torch
     from ms_custom_ops_amd import cabi
     dev = torch.device("cuda:0")
@@ -340,21 +342,59 @@ def mfma_pipe_probe(iters=20000, launches=12):
     g = torch.Generator(device=dev)
     g.manual_seed(0)
     sink = torch.empty(cabi.PROBE_MFMA_WORKGROUPS * 256, dtype=torch.int32, device=dev)
-    ops = cabi.PROBE_MFMA_WORKGROUPS * 4 * iters * 16 * 65536.0
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    ops = cabi.PROBE_MFMA_WORKGROUPS * 4 * iters * 2.0 ** 21
     out = {"ops_per_launch": ops, "iters": iters}
-    for name, operands in (("random_int8", torch.randint(-127, 128, (cabi.PROBE_MFMA_OPERAND_BYTES,), dtype=torch.int8, device=dev, generator=g)),
-                           ("zeros", torch.zeros(cabi.PROBE_MFMA_OPERAND_BYTES, dtype=torch.int8, device=dev))):
-        for _ in range(launches // 2):
-            cabi.probe_mfma(operands.data_ptr(), sink.data_ptr(), iters, st)
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(launches - launches // 2):
-            cabi.probe_mfma(operands.data_ptr(), sink.data_ptr(), iters, st)
-        b.record()
-        torch.cuda.synchronize()
-        sec = a.elapsed_time(b) * 1e-3 / (launches - launches // 2)
-        out[name] = {"launch_us": sec * 1e6, "tops": ops / sec / 1e12, "int8_frac": ops / sec / 1e12 / PEAK_INT8_TOPS}
+    for shape, pattern in (("16x16x64", 0), ("32x32x32", 12)):
+        for name, operands in (("random_int8", torch.randint(-127, 128, (cabi.PROBE_MFMA_OPERAND_BYTES,), dtype=torch.int8, device=dev, generator=g)),
+                               ("zeros", torch.zeros(cabi.PROBE_MFMA_OPERAND_BYTES, dtype=torch.int8, device=dev))):
+            run = lambda: cabi.probe_mfma_issue(operands.data_ptr(), sink.data_ptr(), clocks.data_ptr(), pattern, iters, st)
+            for _ in range(launches // 2):
+                run()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(launches - launches // 2):
+                run()
+            b.record()
+            torch.cuda.synchronize()
+            sec = a.elapsed_time(b) * 1e-3 / (launches - launches // 2)
+            c = clocks.cpu().numpy()
+            out[f"{shape}/{name}"] = {"launch_us": sec * 1e6, "tops": ops / sec / 1e12, "int8_frac": ops / sec / 1e12 / PEAK_INT8_TOPS,
+                                      "ghz": float(c[0]) / (float(c[1]) * 10.0)}
     return out
+
+
+ISSUE_PATTERNS = (
+    (0, "16x16x64 MFMAs only"), (1, "+ 16 ds_read_b128"), (2, "+ 16 reads + 8 buffer loads"),
+    (3, "+ 8 ds_write_b128 alone"), (4, "+ 16 ds_write_b64 alone"), (5, "+ 32 ds_write_b32 alone"),
+    (6, "reads + loads + 8 ds_write_b128, a read one MFMA later"), (7, "reads + loads + 8 ds_write_b128, the next read three MFMAs later"),
+    (8, "reads + loads + 16 ds_write_b64 in slots of their own"), (9, "reads + loads + 16 ds_write_b64 sharing the reads' slots"),
+    (10, "as 8, loads sharing a write's slot"), (11, "reads + loads + 32 ds_write_b32"),
+    (12, "32x32x32 MFMAs only"), (13, "32x32x32: reads + loads + 8 ds_write_b128"), (14, "32x32x32: reads + loads + 16 ds_write_b64"))
+
+
+def mfma_issue_probe(iters=20000):
+    """What a wavefront that is alone on its SIMD can issue between MFMAs (msco_probe_mfma_issue): core clocks per round of
+    64 v_mfma_i32_16x16x64_i8 (32 v_mfma_i32_32x32x32_i8) with the K loop's memory operations woven in at different
+    places, on zero operands (the nominal clock).  A row reads [pattern, what it adds, clocks per round, clocks beyond
+    the bare loop of its instruction shape]."""
+    import torch
+    from ms_custom_ops_amd import cabi
+    dev = torch.device("cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    sink = torch.empty(cabi.PROBE_MFMA_WORKGROUPS * 256, dtype=torch.int32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    operands = torch.zeros(cabi.PROBE_MFMA_OPERAND_BYTES, dtype=torch.int8, device=dev)
+    rows, bare = [], {}
+    for pattern, what in ISSUE_PATTERNS:
+        for _ in range(3):
+            cabi.probe_mfma_issue(operands.data_ptr(), sink.data_ptr(), clocks.data_ptr(), pattern, iters, st)
+        torch.cuda.synchronize()
+        per_round = float(clocks.cpu().numpy()[0]) / iters
+        shape = "32" if pattern >= 12 else "16"
+        bare.setdefault(shape, per_round)
+        rows.append([pattern, what, round(per_round, 1), round(per_round - bare[shape], 1)])
+    return {"iters": iters, "columns": ["pattern", "adds", "clocks_per_round", "beyond_bare_loop"], "rows": rows}
 
 
 def read_floor(sizes=(45.09e6, 469.8e6), steps=60):
@@ -446,7 +486,8 @@ def plan_regret(steps=30):
     planner rule that is wrong for that shape."""
     import torch
     from ms_custom_ops_amd import cabi, workloads
-    forced = (("tile_256", cabi.OV_TILE_256), ("tile_256_w4", cabi.OV_TILE_256_W4), ("tile_128x256", cabi.OV_TILE_128x256),
+    forced = (("tile_256", cabi.OV_TILE_256), ("tile_256_w4", cabi.OV_TILE_256_W4), ("tile_256_w4_mfma32", cabi.OV_TILE_256_W4_MFMA32),
+              ("tile_128x256", cabi.OV_TILE_128x256),
               ("tile_128", cabi.OV_TILE_128), ("tile_64", cabi.OV_TILE_64), ("decode", cabi.OV_SKINNY))
     names = ["c2_m%d" % m for m in (1, 16, 17, 32, 64, 65, 128, 192, 256, 320, 384, 448, 512, 640, 704, 768, 1024, 1280, 1536, 2048, 3072)]
     names += ["c3_t%d" % t for t in (8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512, 768, 1024, 2048)]
@@ -513,6 +554,9 @@ def probe(args):
         return
     if args.probe == "mfma":
         print(json.dumps({"probe": "mfma", "mfma_pipe": mfma_pipe_probe()}))
+        return
+    if args.probe == "issue":
+        print(json.dumps({"probe": "issue", "mfma_issue": mfma_issue_probe()}))
         return
     if args.probe == "moe":
         print(json.dumps({"probe": "moe", "moe_neighbours": moe_neighbours(args.steps, 5)}))

@@ -19,7 +19,7 @@ INCLUDE = os.path.join(REPO_DIR, "include")
 
 BACKEND_LIB = os.path.join(LIB_DIR, "libmsco_gmm.so")
 PROBES_LIB = os.path.join(LIB_DIR, "libmsco_probes.so")   # measurement aids: not part of the operator library
-HIP_SOURCES = ["gmm_tile_w8a8.hip", "gmm_tile4_w8a8.hip", "gmm_skinny_w8a8.hip", "gmm_skinny_a16w8.hip", "gmm_generic.hip", "gmm_stream.hip", "msco_gmm.hip", "moe_routing.hip", "gmm_w4.hip"]
+HIP_SOURCES = ["gmm_tile_w8a8.hip", "gmm_tile4_w8a8.hip", "gmm_tile4m_w8a8.hip", "gmm_skinny_w8a8.hip", "gmm_skinny_a16w8.hip", "gmm_generic.hip", "gmm_stream.hip", "msco_gmm.hip", "moe_routing.hip", "gmm_w4.hip"]
 PROBE_SOURCES = ["probes.hip"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -80,16 +80,20 @@ def build_attribution(verbose: bool = False):
     hip_dir = os.path.join(CSRC, "hip")
     out_dir = os.path.join(LIB_DIR, "attr")
     os.makedirs(out_dir, exist_ok=True)
-    others = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in HIP_SOURCES if s != "gmm_tile4_w8a8.hip"]
+    tile4 = ("gmm_tile4_w8a8.hip", "gmm_tile4m_w8a8.hip")
+    others = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in HIP_SOURCES if s not in tile4]
 
     def build_one(item):
         name, mask = item
-        obj = os.path.join(out_dir, "gmm_tile4_w8a8_%s.o" % name)
-        _run([hipcc] + HIP_FLAGS + ["-DMSCO_BUILDING_LIB", "-DMSCO_TILE4_ATTR=%d" % mask, "-I", INCLUDE, "-I", hip_dir, "-c",
-                                    os.path.join(hip_dir, "gmm_tile4_w8a8.hip"), "-o", obj])
+        objs = []
+        for src in tile4:
+            objs.append(os.path.join(out_dir, "%s_%s.o" % (src[:-4], name)))
+            _run([hipcc] + HIP_FLAGS + ["-DMSCO_BUILDING_LIB", "-DMSCO_TILE4_ATTR=%d" % mask, "-I", INCLUDE, "-I", hip_dir, "-c",
+                                        os.path.join(hip_dir, src), "-o", objs[-1]])
         lib = os.path.join(out_dir, "libmsco_gmm_%s.so" % name)
-        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + others + [obj])
-        os.remove(obj)
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib] + others + objs)
+        for obj in objs:
+            os.remove(obj)
         return lib
 
     with cf.ThreadPoolExecutor(max_workers=4) as pool:

@@ -24,7 +24,7 @@ IN_X, IN_WEIGHT, IN_BIAS, IN_SCALE, IN_GROUP_LIST, IN_PER_TOKEN_SCALE, IN_ANTIQU
 IN_COUNT = 8
 
 # msco_gmm_desc.kernel_override
-OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC, OV_TILE_256_W4, OV_TILE_128x256 = range(8)
+OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC, OV_TILE_256_W4, OV_TILE_128x256, OV_TILE_256_W4_MFMA32 = range(9)
 
 # msco_gmm_desc.act_type
 ACT_NONE, ACT_RELU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_FAST_GELU, ACT_SILU = range(6)
@@ -37,7 +37,7 @@ EXPORTED_SYMBOLS = ("msco_gmm_create", "msco_gmm_plan", "msco_gmm_launch", "msco
                     "msco_packed_weight_bytes", "msco_pack_weight", "msco_gmm_a8w4", "msco_unpack_int4",
                     "msco_moe_init_routing_v2_workspace_bytes", "msco_moe_init_routing_v2", "msco_moe_init_routing_v2_quant",
                     "msco_moe_token_unpermute", "msco_gmm_launch_static")
-PROBE_SYMBOLS = ("msco_probe_mfma", "msco_probe_read")   # libmsco_probes.so, include/msco_probes.h
+PROBE_SYMBOLS = ("msco_probe_mfma_issue", "msco_probe_read")   # libmsco_probes.so, include/msco_probes.h
 STATIC_WORKSPACE_BYTES = 32 << 20
 PROBE_MFMA_WORKGROUPS, PROBE_MFMA_OPERAND_BYTES = 256, 8 * 256 * 16
 
@@ -71,8 +71,8 @@ def load_probes():
         lib = ctypes.CDLL(PROBES_LIB_PATH)
         lib.msco_probe_read.restype = ctypes.c_int
         lib.msco_probe_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
-        lib.msco_probe_mfma.restype = ctypes.c_int
-        lib.msco_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_void_p]
+        lib.msco_probe_mfma_issue.restype = ctypes.c_int
+        lib.msco_probe_mfma_issue.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
         _probes = lib
     return _probes
 
@@ -170,11 +170,12 @@ def unpack_int4(src: int, dst: int, src_bytes: int, stream: Optional[int] = None
     _check("msco_unpack_int4", load().msco_unpack_int4(vp(src), vp(dst), src_bytes, vp(stream)))
 
 
-def probe_mfma(operands: int, sink: int, iters: int, stream: Optional[int] = None):
-    """Raw-pointer call of msco_probe_mfma (see include/msco_probes.h); PROBE_MFMA_WORKGROUPS * 4 * iters * 16 * 65536 int8
-    operations per launch."""
+def probe_mfma_issue(operands: int, sink: int, clocks: int, pattern: int, iters: int, stream: Optional[int] = None):
+    """Raw-pointer call of msco_probe_mfma_issue (see include/msco_probes.h): `pattern` names the memory operations woven
+    into rounds of 64 (32) MFMAs, PROBE_MFMA_WORKGROUPS * 4 * iters * 2 ** 21 int8 operations per launch; `clocks` receives
+    two int64 (core clocks, 100 MHz ticks of the loop)."""
     vp = lambda v: ctypes.c_void_p(v if v else None)
-    _check("msco_probe_mfma", load_probes().msco_probe_mfma(vp(operands), vp(sink), iters, vp(stream)))
+    _check("msco_probe_mfma_issue", load_probes().msco_probe_mfma_issue(vp(operands), vp(sink), vp(clocks), pattern, iters, vp(stream)))
 
 
 def probe_read(src: int, nbytes: int, sink: int, workgroups: int, stream: Optional[int] = None):

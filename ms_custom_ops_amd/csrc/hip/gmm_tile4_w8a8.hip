@@ -1,5 +1,8 @@
-// Grouped W8A8 GEMM, persistent register-heavy MFMA tile kernel for gfx950: 256 x 256 output tiles,
-// four wavefronts (one per SIMD), 128 x 128 accumulators per wavefront, weights stored [E,N,K].
+// Grouped W8A8 GEMM, persistent register-heavy MFMA tile kernel for gfx950 on v_mfma_i32_32x32x32_i8: 256 x 256
+// output tiles, four wavefronts (one per SIMD), 128 x 128 accumulators per wavefront; every weight layout.  The plan
+// takes it for [E,K,N] weights; K-major weights ([E,N,K], packed) run the 16 x 16 x 64 form of the same design
+// (gmm_tile4m_w8a8.hip), which draws less power per multiply-add, and reach this one only when it is forced, to be
+// measured against.
 //
 // Why this shape.  A wavefront that owns 128 x 128 outputs reads 8 operand fragments from LDS for every
 // 16 MFMAs (a 128 x 64 wave tile reads 12), so LDS traffic per multiply-add drops by a third.  The
@@ -39,22 +42,14 @@
 //     only touches the blocks that hold rows.
 #include "gmm_common.h"
 #include "gmm_kernels.h"
+#include "gmm_tile4_common.h"
 
 #include <type_traits>
 
 namespace msco {
 namespace {
 
-constexpr int T4_BM = 256, T4_BN = 256;
-constexpr int T4_BK = 128;                       // bytes of K per slab and LDS row
-constexpr int T4_NW = 4;                         // wavefronts: 2 (m) x 2 (n)
-constexpr int T4_WT = 128;                       // wave tile edge
 constexpr int T4_F = 4;                          // 32 x 32 MFMA blocks per wave tile edge
-constexpr int T4_OP_STAGE = T4_BM * T4_BK;       // one operand's share of a stage (32 KiB)
-constexpr int T4_W_BASE = 2 * T4_OP_STAGE;       // x stages 0 and 1, then weight stages 0 and 1: a stage and a block offset
-                                                 // together fit the 16-bit offset field of an LDS instruction
-constexpr int T4_RING = 2 * T4_W_BASE;           // 128 KiB
-constexpr int T4_LD = T4_BM / 8 / T4_NW;         // staging quads (8 rows x 128 B per wave) per operand and slab
 // Attribution builds, never the shipped library: MSCO_TILE4_ATTR is a bit mask that takes one part of the kernel out
 // so that timing the rest says what that part costs (results are then wrong on purpose).  1: the epilogue sits behind
 // a branch that no launch takes (its code and registers stay); 2: every MFMA becomes an empty statement that keeps
@@ -63,104 +58,18 @@ constexpr int T4_LD = T4_BM / 8 / T4_NW;         // staging quads (8 rows x 128 
 // what the prologue brought); 16: staging registers are not written to LDS (loads are still waited for); 32: the K
 // loop's workgroup barriers are left out; 64: the K loop reads no operand fragments from LDS (the MFMAs multiply what
 // the registers hold).
-#ifndef MSCO_TILE4_ATTR
-#define MSCO_TILE4_ATTR 0
-#endif
 constexpr int T4_EP_PITCH = 144;                 // epilogue staging: 128 payload bytes per row
-constexpr int T4_PARAM_OFF = T4_RING;            // epilogue operand tables (scale, bias, per-token; two tiles) behind the ring
-constexpr int T4_PARAM_BYTES = 3 * 1024;
 constexpr int T4_EP_OFF = T4_PARAM_OFF + 2 * T4_PARAM_BYTES;
 constexpr int T4_EP_WAVE = 32 * T4_EP_PITCH;     // one wave stages 32 rows at a time
 constexpr int T4_META_OFF = T4_EP_OFF + T4_NW * T4_EP_WAVE;   // per group: row end, tiles up to and including it
-constexpr int T4_MAX_E = 1024;
 constexpr int T4_LDS_BYTES = T4_META_OFF + 2 * T4_MAX_E * 4;
 static_assert(T4_LDS_BYTES <= 160 * 1024, "LDS of one CU");
-constexpr int T4_MAX_WGS = 256;                  // one persistent workgroup per CU
-constexpr unsigned T4_OOB = 0x80000000u;
 
 __device__ __forceinline__ int t4_col_of_q(int q) {
   const int g = q >> 3, hh = (q >> 2) & 1, t = q & 3;
   return 16 * (g >> 1) + 8 * hh + 4 * (g & 1) + t;
 }
 
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t t4_rsrc(const void *base, long long bytes) {
-  const unsigned n = bytes > 0x7FFFFFFFll ? 0x7FFFFFFFu : (unsigned)(bytes < 0 ? 0 : bytes);
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)n, 0x00020000);
-}
-
-// Publishes LDS data and retires a stage: the caller has waited for its own LDS traffic.
-__device__ __forceinline__ void t4_barrier() {
-  __builtin_amdgcn_sched_barrier(0);
-  asm volatile("s_barrier" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
-}
-
-// Raw buffer descriptor as four scalars (for hand-written buffer instructions).
-__device__ __forceinline__ v4i t4_raw_rsrc(const void *base, long long bytes) {
-  const unsigned long long a = (unsigned long long)base;
-  const unsigned n = bytes > 0x7FFFFFFFll ? 0x7FFFFFFFu : (unsigned)(bytes < 0 ? 0 : bytes);
-  v4i r;
-  r.x = __builtin_amdgcn_readfirstlane((int)(unsigned)a);
-  r.y = __builtin_amdgcn_readfirstlane((int)((unsigned)(a >> 32) & 0xFFFFu));
-  r.z = __builtin_amdgcn_readfirstlane((int)n);
-  r.w = 0x00020000;
-  return r;
-}
-
-// One dword (or zero-extended 16 bits) per lane from a buffer straight into LDS: lane L writes
-// lds_addr + 4 L.  Hand-written so that the compiler's wait-count bookkeeping never sees an LDS
-// write in flight (it would make every later LDS read wait for all outstanding loads); the
-// counter it does not know about can only make its own waits longer, never shorter, because
-// vector memory operations complete in order.
-__device__ __forceinline__ void t4_dma_b32(v4i rsrc, unsigned lds_addr, unsigned voffset) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory");
-}
-__device__ __forceinline__ void t4_dma_b16(v4i rsrc, unsigned lds_addr, unsigned voffset) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ushort %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory");
-}
-
-// A tile as the whole workgroup sees it (all fields wave-uniform).
-struct T4Tile {
-  int valid;
-  int grp, m0, n0, g_end;
-};
-
-// Tile lid -> (group, m-tile, n-tile).  The group walk was done once at kernel start and left in LDS
-// (row end and inclusive tile count per group): reading group_list from memory again for every tile
-// would put loads into the middle of the operand stream, and vector loads complete in order.
-// Order inside a group: panels of 8 m-tiles; inside a panel n-tile major, m-tile minor, so that
-// workgroups that run side by side share one streamed weight panel.
-__device__ __forceinline__ T4Tile t4_locate(const int *meta_end, const int *meta_upto, int e, int lid, int total,
-                                            int n_tiles, int lane) {
-  T4Tile t{0, 0, 0, 0, 0};
-  if (lid < 0 || lid >= total) return t;
-  int g_start = 0, t_in_group = 0;
-  for (int g0 = 0; g0 < e; g0 += 64) {
-    const int g = g0 + lane;
-    const int upto = g < e ? meta_upto[g] : 0x7FFFFFFF;
-    const int first = __popcll(__ballot(upto <= lid));              // `upto` is non-decreasing: first group beyond lid
-    if (first < 64) {
-      const int grp = g0 + first;
-      t.grp = grp;
-      t.g_end = __builtin_amdgcn_readfirstlane(meta_end[grp]);
-      g_start = grp > 0 ? __builtin_amdgcn_readfirstlane(meta_end[grp - 1]) : 0;
-      t_in_group = lid - (grp > 0 ? __builtin_amdgcn_readfirstlane(meta_upto[grp - 1]) : 0);
-      t.valid = 1;
-      break;
-    }
-  }
-  constexpr int PANEL = 8;
-  const int m_tiles = (t.g_end - g_start + T4_BM - 1) / T4_BM;
-  const int panel_tiles = PANEL * n_tiles;
-  const int panel = t_in_group / panel_tiles;
-  const int in_panel = t_in_group - panel * panel_tiles;
-  const int panel_m = max(1, min(PANEL, m_tiles - panel * PANEL));
-  const int nt = in_panel / panel_m;
-  const int mt = panel * PANEL + in_panel % panel_m;
-  t.m0 = g_start + mt * T4_BM;
-  t.n0 = nt * T4_BN;
-  return t;
-}
 
 }  // namespace
 

@@ -639,8 +639,9 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
   if (layout == 2 && p.n % 16 != 0) return hipErrorInvalidValue;
   // the persistent kernel needs at least four 128-byte K slabs per tile and a group table that fits in LDS; what it
   // cannot take runs the eight-wave kernel of the same tile shape
-  if (tile_cfg == TILE_256x256_W4) {
-    if (p.k >= 512 && p.e <= 1024) return launch_tile4_w8a8(p, layout, stream);
+  if (tile_cfg == TILE_256x256_W4 || tile_cfg == TILE_256x256_W4_MFMA32) {
+    if (p.k >= 512 && p.e <= 1024)
+      return layout != 2 && tile_cfg == TILE_256x256_W4 ? launch_tile4m_w8a8(p, layout, stream) : launch_tile4_w8a8(p, layout, stream);
     tile_cfg = TILE_256x256;
   }
   switch (tile_cfg) {
@@ -669,6 +670,7 @@ const char *tile_cfg_name(int tile_cfg) {
     case TILE_64x128: return "64x128";
     case TILE_128x256: return "128x256x64";
     case TILE_256x256_W4: return "256x256x128_w4";
+    case TILE_256x256_W4_MFMA32: return "256x256x128_w4_mfma32";
     default: return "?";
   }
 }
@@ -690,7 +692,7 @@ size_t tile_workspace_bytes(int tile_cfg, int64_t m, int64_t n, int64_t e, int s
 
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn) {
   switch (tile_cfg) {
-    case TILE_256x256: case TILE_256x256_W4: *bm = 256; *bn = 256; break;
+    case TILE_256x256: case TILE_256x256_W4: case TILE_256x256_W4_MFMA32: *bm = 256; *bn = 256; break;
     case TILE_128x128: *bm = 128; *bn = 128; break;
     case TILE_128x256: *bm = 128; *bn = 256; break;
     default: *bm = 64; *bn = 128; break;

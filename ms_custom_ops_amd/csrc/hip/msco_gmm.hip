@@ -24,7 +24,8 @@ enum Family : int { FAM_NONE = 0, FAM_TILE = 1, FAM_SKINNY = 2, FAM_GENERIC = 3 
 enum Override : int {
   OV_AUTO = 0, OV_TILE_256 = 1, OV_TILE_128 = 2, OV_TILE_64 = 3, OV_SKINNY = 4, OV_GENERIC = 5,
   OV_TILE_256_W4 = 6,  // persistent four-wave 256 x 256 kernel
-  OV_TILE_128x256 = 7  // four waves side by side, 128 x 256
+  OV_TILE_128x256 = 7,  // four waves side by side, 128 x 256
+  OV_TILE_256_W4_MFMA32 = 8  // the persistent kernel's 32 x 32 x 32 form on every layout (the plan takes it for [E,K,N] only)
 };
 
 constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned
@@ -106,7 +107,7 @@ int check_desc(const msco_gmm_desc &d) {
   if (d.group_list_dtype != MSCO_DT_NONE && d.group_list_dtype != MSCO_DT_I32 && d.group_list_dtype != MSCO_DT_I64)
     return MSCO_ERR_UNSUPPORTED;
   if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
-  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_128x256) return MSCO_ERR_INVALID_ARG;
+  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_256_W4_MFMA32) return MSCO_ERR_INVALID_ARG;
   if (d.weight_layout != MSCO_WL_ROW_MAJOR && d.weight_layout != MSCO_WL_PACKED) return MSCO_ERR_INVALID_ARG;
   if (d.force_split_k < 0) return MSCO_ERR_INVALID_ARG;
   if (d.act_type < MSCO_ACT_NONE || d.act_type > MSCO_ACT_SILU) return MSCO_ERR_INVALID_ARG;
@@ -233,6 +234,7 @@ void choose_plan(msco_gmm_op *op) {
   switch (d.kernel_override) {
     case OV_TILE_256: family = FAM_TILE; op->tile_cfg = TILE_256x256; break;
     case OV_TILE_256_W4: family = FAM_TILE; op->tile_cfg = TILE_256x256_W4; break;
+    case OV_TILE_256_W4_MFMA32: family = FAM_TILE; op->tile_cfg = TILE_256x256_W4_MFMA32; break;
     case OV_TILE_128: family = FAM_TILE; op->tile_cfg = TILE_128x128; break;
     case OV_TILE_128x256: family = FAM_TILE; op->tile_cfg = TILE_128x256; break;
     case OV_TILE_64: family = FAM_TILE; op->tile_cfg = TILE_64x128; break;
@@ -241,7 +243,7 @@ void choose_plan(msco_gmm_op *op) {
     default: break;
   }
   // (what the persistent kernel cannot take runs the eight-wave kernel of the same tile shape; the plan says so)
-  if (family == FAM_TILE && op->tile_cfg == TILE_256x256_W4 && !(k >= 512 && e <= 1024))
+  if (family == FAM_TILE && (op->tile_cfg == TILE_256x256_W4 || op->tile_cfg == TILE_256x256_W4_MFMA32) && !(k >= 512 && e <= 1024))
     op->tile_cfg = TILE_256x256;
   // the MFMA kernels address x and one group's weights through 32-bit buffer offsets
   const bool fits32 = (is_packed(d) ? (int64_t)packed_weight_bytes(k, n) : k * n) < ((int64_t)1 << 31) &&

@@ -15,7 +15,8 @@ from oracle import gmm_oracle as O
 pytestmark = pytest.mark.gpu
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 FAMILIES = [("generic", cabi.OV_GENERIC), ("skinny", cabi.OV_SKINNY), ("tile64", cabi.OV_TILE_64),
-            ("tile128", cabi.OV_TILE_128), ("tile256", cabi.OV_TILE_256), ("tile256_w4", cabi.OV_TILE_256_W4)]
+            ("tile128", cabi.OV_TILE_128), ("tile256", cabi.OV_TILE_256), ("tile256_w4", cabi.OV_TILE_256_W4),
+            ("tile256_w4_mfma32", cabi.OV_TILE_256_W4_MFMA32)]
 
 
 def _inputs(seed, m, k, n, e):
@@ -171,9 +172,12 @@ def test_few_tiles_split_k_across_workgroups(device, transpose_b):
 
 # ------------------------------------------------------------- persistent four-wave tile kernel
 W4 = cabi.OV_TILE_256_W4
+# both forms of the persistent kernel on [E,N,K] weights: 16 x 16 x 64 MFMAs (what the plan takes) and 32 x 32 x 32
+W4_FORMS = pytest.mark.parametrize("W4", [cabi.OV_TILE_256_W4, cabi.OV_TILE_256_W4_MFMA32], ids=["mfma16", "mfma32"])
 
 
-def test_w4_ragged_groups_k_tail_and_odd_slab_count(device):
+@W4_FORMS
+def test_w4_ragged_groups_k_tail_and_odd_slab_count(device, W4):
     # K = 1296: ten full 128-byte slabs and a 16-byte tail, an odd slab count (padded with a slab of
     # zeros); N = 400 leaves a partial n-tile; groups: empty, 1 row, exactly 256, 257, a few hundred
     rng, x, w, bias, scale, pt = _inputs(20, 1100, 1296, 400, 8)
@@ -182,7 +186,8 @@ def test_w4_ragged_groups_k_tail_and_odd_slab_count(device):
     assert "256x256x128_w4" in info
 
 
-def test_w4_workgroups_walk_several_tiles(device):
+@W4_FORMS
+def test_w4_workgroups_walk_several_tiles(device, W4):
     # 18 m-tiles x 16 n-tiles = 288 tiles for at most 256 persistent workgroups: some walk two tiles,
     # so the operand stream crosses a tile boundary, also into a tile of another group
     rng, x, w, bias, scale, pt = _inputs(21, 4200, 640, 4096, 3)
@@ -190,7 +195,8 @@ def test_w4_workgroups_walk_several_tiles(device):
     assert "256x256x128_w4" in info
 
 
-def test_w4_scale_wire_formats_f16_out_and_absent_operands(device):
+@W4_FORMS
+def test_w4_scale_wire_formats_f16_out_and_absent_operands(device, W4):
     from gpu_utils import run_w8a8
     rng, x, w, bias, scale, pt = _inputs(22, 700, 512, 528, 4)
     gl = [100, 300, 300, 700]

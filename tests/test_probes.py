@@ -1,4 +1,4 @@
-"""The two measurement aids of the C ABI (msco_probe_mfma, msco_probe_read) do what their headers say: the benchmark's
+"""The two measurement aids of the C ABI (msco_probe_mfma_issue, msco_probe_read) do what their headers say: the benchmark's
 yardsticks rest on them, so their arithmetic and their coverage of the buffer are checked, not only their timing."""
 import numpy as np
 import pytest
@@ -9,21 +9,31 @@ from ms_custom_ops_amd import cabi
 pytestmark = pytest.mark.gpu
 
 
-def test_mfma_probe_multiplies_what_it_is_given():
+@pytest.mark.parametrize("pattern", [0, 8, 12, 13])
+def test_mfma_probe_multiplies_what_it_is_given(pattern):
     st = torch.cuda.current_stream().cuda_stream
     sink = torch.full((cabi.PROBE_MFMA_WORKGROUPS * 256,), -1, dtype=torch.int32, device="cuda:0")
+    clocks = torch.zeros(2, dtype=torch.int64, device="cuda:0")
     iters = 37
-    # all ones: every round adds K = 32 to each of a lane's 256 accumulators; the sink holds their sum
+    # all ones: a round adds 64 blocks x 4 accumulators x K = 64 (16 blocks x 16 x K = 32, twice) to a lane's sum; the sink
+    # holds that sum plus the first word of four registers: fragments of ones, or what the woven-in operations last
+    # brought (LDS reads: zeros; buffer loads: operands again)
     ones = torch.ones(cabi.PROBE_MFMA_OPERAND_BYTES, dtype=torch.int8, device="cuda:0")
-    cabi.probe_mfma(ones.data_ptr(), sink.data_ptr(), iters, st)
+    cabi.probe_mfma_issue(ones.data_ptr(), sink.data_ptr(), clocks.data_ptr(), pattern, iters, st)
     torch.cuda.synchronize()
-    assert (sink.cpu().numpy() == 256 * 32 * iters).all()
+    word = 0x01010101
+    extra = 4 * word if pattern in (0, 12) else 2 * word
+    assert (sink.cpu().numpy() == 16384 * iters + extra).all()
+    c = clocks.cpu().numpy()
+    assert c[0] >= iters * 1000 and c[1] > 0   # 64 MFMAs of 16 cycles (32 of 32) per round at least
     zeros = torch.zeros(cabi.PROBE_MFMA_OPERAND_BYTES, dtype=torch.int8, device="cuda:0")
-    cabi.probe_mfma(zeros.data_ptr(), sink.data_ptr(), iters, st)
+    cabi.probe_mfma_issue(zeros.data_ptr(), sink.data_ptr(), clocks.data_ptr(), pattern, iters, st)
     torch.cuda.synchronize()
     assert (sink.cpu().numpy() == 0).all()
     with pytest.raises(cabi.BackendError):
-        cabi.probe_mfma(0, sink.data_ptr(), iters, st)
+        cabi.probe_mfma_issue(0, sink.data_ptr(), clocks.data_ptr(), pattern, iters, st)
+    with pytest.raises(cabi.BackendError):
+        cabi.probe_mfma_issue(ones.data_ptr(), sink.data_ptr(), clocks.data_ptr(), 99, iters, st)
 
 
 @pytest.mark.parametrize("nbytes,wgs", [(4096 * 64, 8), (4096 * 1000 + 123, 7), (4096 * 3, 16)])
