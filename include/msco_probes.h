@@ -15,7 +15,7 @@ extern "C" {
 
 /* Measurement aid with no counterpart in the reference: the rate the matrix pipe sustains on a given operand
  * distribution, the yardstick the benchmark quotes next to the grouped matmul's rate, and what a wavefront that is alone
- * on its SIMD can issue between MFMAs.  MSCO_PROBE_MFMA_WORKGROUPS workgroups of 256 threads run `iters` rounds of 64
+ * on its SIMD can issue between MFMAs.  MSCO_PROBE_MFMA_WORKGROUPS workgroups of 256 threads run `iters` (a multiple of 8) rounds of 64
  * v_mfma_i32_16x16x64_i8 (patterns 0 - 11) or 32 v_mfma_i32_32x32x32_i8 (12 - 14) -- 2^21 int8 operations per wavefront
  * and round either way, MSCO_PROBE_MFMA_WORKGROUPS * 4 * iters * 2^21 per launch -- on operand fragments read once from
  * `operands` (MSCO_PROBE_MFMA_OPERAND_BYTES bytes of int8; every workgroup reads the same), with memory operations woven
@@ -32,7 +32,8 @@ extern "C" {
  *   11  pattern 2 + 32 ds_write_b32 (n % 2 == 0)
  * Patterns 6 - 11, 13, 14 carry the traffic of the persistent tile kernels' K loop.  LDS reads find zeros, buffer loads
  * re-read `operands`.  `clocks` receives two int64: core clocks and 100 MHz ticks that workgroup 0 spent in the loop.  `sink` receives
- * MSCO_PROBE_MFMA_WORKGROUPS * 256 int32 values of no meaning.  Enqueues on the stream, allocates nothing. */
+ * MSCO_PROBE_MFMA_WORKGROUPS * 256 int32 values: each thread's sum over its accumulators.  Enqueues on the stream,
+ * allocates nothing. */
 #define MSCO_PROBE_MFMA_WORKGROUPS 256
 #define MSCO_PROBE_MFMA_OPERAND_BYTES (8 * 256 * 16)
 MSCO_API int msco_probe_mfma_issue(const void *operands, void *sink, void *clocks, int32_t pattern, int32_t iters, void *stream);

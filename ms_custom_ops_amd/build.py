@@ -73,7 +73,7 @@ ATTRIBUTION_BUILDS = {"noepi": 1, "nomfma": 2, "nomfma_noepi": 3, "nostore": 4,
 
 def build_attribution(verbose: bool = False):
     """Measurement builds of the backend, never the shipped one: lib/attr/libmsco_gmm_<name>.so is libmsco_gmm.so with
-    one part of the persistent tile kernel taken out (MSCO_TILE4_ATTR in gmm_tile4_w8a8.hip), so that timing the rest
+    one part of the persistent tile kernels taken out (MSCO_TILE4_ATTR in gmm_tile4_w8a8.hip and gmm_tile4m_w8a8.hip), so that timing the rest
     says what that part costs.  Select one with MSCO_GMM_LIB=<path>; their results are wrong on purpose."""
     build_backend(verbose)
     hipcc = _hipcc()

@@ -184,11 +184,10 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
   // one 8-byte half of a staging quad to LDS
   auto put_half = [&](unsigned addr, const v4i &v, auto h_c) __attribute__((always_inline)) {
     constexpr int H = decltype(h_c)::value;
-    const v2i half = H == 0 ? v2i{v.x, v.y} : v2i{v.z, v.w};
 #if MSCO_TILE4_ATTR & 16
-    asm volatile("" ::"v"(half), "v"(addr));
+    asm volatile("" ::"v"(v), "v"(addr));
 #else
-    *reinterpret_cast<v2i *>(smem + addr) = half;
+    *reinterpret_cast<v2i *>(smem + addr) = H == 0 ? v2i{v.x, v.y} : v2i{v.z, v.w};
 #endif
   };
   // write quad (op, u) of slab s to its LDS stage and refill it with slab s + 2

@@ -51,6 +51,7 @@ __global__ void __launch_bounds__(256) probe_read_kernel(const unsigned char *sr
 // MF: 0 16 x 16 x 64 (64 per round), 1 32 x 32 x 32 (32 per round, behind every second slot).  Per round of 64 slots: RD
 // ds_read_b128 in the slots n % (64 / RD) == 1; WR LDS writes of WB bytes per lane in the slots n % (64 / WR) == WP; LD
 // buffer loads in the slots n % (64 / LD) == LP.
+constexpr int kIssueRoundsPerPass = 8;
 template <int MF, int RD, int WB, int WR, int WP, int LD, int LP>
 __global__ void __launch_bounds__(256, 1) probe_issue_kernel(const v4i *operands, int *sink, int iters, long long *clocks) {
   __shared__ __align__(16) unsigned char lds[65536];
@@ -86,10 +87,14 @@ __global__ void __launch_bounds__(256, 1) probe_issue_kernel(const v4i *operands
   typedef int v2i_t __attribute__((ext_vector_type(2)));
   const v2i_t w8 = v2i_t{wf[3].x, wf[3].y};
   const int w4 = wf[3].z;
+  const int passes = iters / kIssueRoundsPerPass;
+  int last = passes - 1;   // (laundered: known to be the last pass, it would be peeled off and the copies move with it)
+  asm volatile("" : "+s"(last));
   const long long c0 = __builtin_readcyclecounter(), t0 = wall_clock64();
-  for (int it = 0; it < iters; ++it) {
+  for (int it = 0; it < passes; ++it) {
 #pragma unroll
-    for (int n = 0; n < 64; ++n) {
+    for (int slot = 0; slot < 64 * kIssueRoundsPerPass; ++slot) {
+      const int n = slot % 64;
       if constexpr (MF == 1) {
         if (n % 2 == 0)
           asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+a"(acc[(n / 8) % 4][(n / 2) % 4]) : "v"(wf[(n / 8) % 4]), "v"(xf[(n / 2) % 4]));
@@ -110,10 +115,15 @@ __global__ void __launch_bounds__(256, 1) probe_issue_kernel(const v4i *operands
         else asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(r3) : "v"(goff), "s"(rsrc));
       }
     }
+    // (the compiler does not know that the statements above are MFMAs and copies accumulators right behind the loop: the
+    // wait states between the last MFMA and the first read of its result stand here, inside the last pass; the test
+    // costs 48 clocks of issue, hence several rounds per pass)
+    if (it == last) asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15");
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   const long long c1 = __builtin_readcyclecounter(), t1 = wall_clock64();
-  int s = r0.x + r1.x + r2.x + r3.x;
+  asm volatile("" ::"v"(r0), "v"(r1), "v"(r2), "v"(r3));   // (what the woven-in loads brought is of no interest)
+  int s = 0;
 #pragma unroll
   for (int f = 0; f < NB; ++f)
 #pragma unroll
@@ -131,7 +141,7 @@ __global__ void __launch_bounds__(256, 1) probe_issue_kernel(const v4i *operands
 }  // namespace msco
 
 extern "C" int msco_probe_mfma_issue(const void *operands, void *sink, void *clocks, int32_t pattern, int32_t iters, void *stream) {
-  if (operands == nullptr || sink == nullptr || clocks == nullptr || iters < 0) return MSCO_ERR_INVALID_ARG;
+  if (operands == nullptr || sink == nullptr || clocks == nullptr || iters < 0 || iters % msco::kIssueRoundsPerPass != 0) return MSCO_ERR_INVALID_ARG;
   const auto st = static_cast<hipStream_t>(stream);
   const auto *ops = static_cast<const msco::v4i *>(operands);
   int *snk = static_cast<int *>(sink);
