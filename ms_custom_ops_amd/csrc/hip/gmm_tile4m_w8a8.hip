@@ -328,9 +328,9 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
       // Eight steps: K half 0 then K half 1, each over the quadrants (F0,I0) (F0,I1) (F1,I1) (F1,I0), so that a step needs
       // four new fragments.  A step also moves two staging quads to LDS and requests their successors.  What a lone wave
       // can issue next to 16-cycle MFMAs was measured on a loop of MFMAs with memory operations woven in: fragment reads
-      // and memory requests cost nothing; a 16-byte LDS write costs 12 cycles of MFMA issue by itself and 30 when a read
-      // follows within two MFMAs, an 8-byte write 4 cycles wherever it stands, two memory operations behind the same MFMA
-      // cost as much again.  So quads go to LDS in halves and no two operations share a slot:
+      // and memory requests cost nothing; a 16-byte LDS write costs 12 cycles of MFMA issue by itself and 35 when a read
+      // follows one MFMA later, an 8-byte write 4 cycles wherever it stands, two memory operations behind the same MFMA
+      // cost as much again (bench.py --probe issue).  So quads go to LDS in halves and no two operations share a slot:
       //   write a.lo, read 0, -, -, write a.hi, read 1, -, request a, write b.lo, read 2, -, -, write b.hi, read 3, -, request b
       // The step before the barrier has its LDS traffic in its first half, so that the wait before the barrier is short.
       // Behind the barrier every wave's part of the next slab is visible and nobody reads this stage any more: group 0 of
