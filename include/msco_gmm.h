@@ -133,8 +133,8 @@ typedef struct msco_gmm_desc {
   int32_t scale_is_scalar;   /* 1: scale holds a single element broadcast over N */
   int32_t kernel_override;   /* 0 auto; else force a kernel family, for tests and planner checks: 1 eight-wave 256 x 256 tile,
                               * 2 128 x 128, 3 64 x 128, 4 decode (streaming) kernels, 5 generic, 6 persistent four-wave
-                              * 256 x 256, 7 128 x 256, 8 the persistent kernel's 32 x 32 x 32 MFMA form on every layout (6 takes
-                              * the 16 x 16 x 64 form for packed and [E,N,K] weights) (msco_gmm_plan_info names what was planned) */
+                              * 256 x 256 (16 x 16 x 64 MFMAs), 7 128 x 256, 8 the persistent kernel's 32 x 32 x 32 MFMA form
+                              * (msco_gmm_plan_info names what was planned) */
   int32_t weight_layout;     /* MSCO_WL_ROW_MAJOR: as transpose_b says; MSCO_WL_PACKED: written by msco_pack_weight */
   int32_t act_type;          /* msco_act: activation applied to the dequantised float32 value before the output cast */
   int32_t force_split_k;     /* 0 auto; else the K split across workgroups of the kernels that have one, for tests */

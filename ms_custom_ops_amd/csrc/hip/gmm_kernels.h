@@ -10,15 +10,14 @@ namespace msco {
 enum TileCfg : int {
   TILE_256x256 = 0, TILE_128x128 = 1, TILE_64x128 = 2, TILE_128x256 = 3,
   TILE_256x256_W4 = 4,   // persistent, four wavefronts with 128 x 128 accumulators each: gmm_tile4m_w8a8.hip (16 x 16 x 64 MFMAs)
-                         // for K-major weights, gmm_tile4_w8a8.hip (32 x 32 x 32) for [E,K,N]
-  TILE_256x256_W4_MFMA32 = 5,   // gmm_tile4_w8a8.hip on every layout (never planned; kept to be measured against)
+  TILE_256x256_W4_MFMA32 = 5,   // the same on 32 x 32 x 32 MFMAs: gmm_tile4_w8a8.hip (never planned; kept to be measured against)
   TILE_CFG_COUNT = 6
 };
 
 // MFMA tile kernel for W8A8 (prefill shapes).  nk: weights stored [E,N,K]; packed: the packed layout (nk is ignored).
 hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool packed, hipStream_t stream);
 const char *tile_cfg_name(int tile_cfg);
-hipError_t launch_tile4m_w8a8(const GmmParams &p, int layout, hipStream_t stream);  // layout 0 [E,N,K], 1 packed
+hipError_t launch_tile4m_w8a8(const GmmParams &p, int layout, hipStream_t stream);  // layout 0 [E,N,K], 1 packed, 2 [E,K,N] (N % 16 == 0)
 hipError_t launch_tile4_w8a8(const GmmParams &p, int layout, hipStream_t stream);   // layout 0 [E,N,K], 1 packed, 2 [E,K,N] (N % 16 == 0)
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn);
 // K split across workgroups (p.split_k > 1; four-wave tile shapes only): partial tiles and arrival counters

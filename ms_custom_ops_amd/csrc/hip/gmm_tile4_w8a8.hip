@@ -1,8 +1,7 @@
 // Grouped W8A8 GEMM, persistent register-heavy MFMA tile kernel for gfx950 on v_mfma_i32_32x32x32_i8: 256 x 256
 // output tiles, four wavefronts (one per SIMD), 128 x 128 accumulators per wavefront; every weight layout.  The plan
-// takes it for [E,K,N] weights; K-major weights ([E,N,K], packed) run the 16 x 16 x 64 form of the same design
-// (gmm_tile4m_w8a8.hip), which draws less power per multiply-add, and reach this one only when it is forced, to be
-// measured against.
+// takes the 16 x 16 x 64 form of the same design (gmm_tile4m_w8a8.hip), which draws less power per multiply-add; this
+// one runs only when it is forced (kernel_override 8), to be measured against.
 //
 // Why this shape.  A wavefront that owns 128 x 128 outputs reads 8 operand fragments from LDS for every
 // 16 MFMAs (a 128 x 64 wave tile reads 12), so LDS traffic per multiply-add drops by a third.  The

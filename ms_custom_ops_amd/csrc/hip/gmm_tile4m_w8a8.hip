@@ -1,12 +1,12 @@
 // Grouped W8A8 GEMM, persistent four-wave tile kernel for gfx950 on v_mfma_i32_16x16x64_i8: 256 x 256 output tiles,
 // four wavefronts (one per SIMD), 128 x 128 accumulators per wavefront as 8 x 8 blocks of 16 x 16; weights stored
-// [E,N,K] or packed.
+// [E,N,K], packed or [E,K,N].
 //
 // Why this instruction.  On random int8 operands the chip runs against its power limit and the clock follows what the
 // matrix pipe draws; the 16 x 16 x 64 shape draws less for the same multiply-adds than 32 x 32 x 32 (64 products are added
 // up inside the array before an accumulator register is touched, instead of 32): a loop of nothing but MFMAs sustains
 // 4.1 - 4.3 POP/s with it against 3.5 POP/s.  The design around the MFMAs is that of the 32 x 32 x 32 kernel
-// (gmm_tile4_w8a8.hip, which keeps the [E,K,N] layout): 128-byte K slabs in two LDS stages, two further slabs in flight
+// (gmm_tile4_w8a8.hip, kept to be measured against): 128-byte K slabs in two LDS stages, two further slabs in flight
 // through staging registers, one barrier per slab, a compile-time K-loop body for the slabs inside a tile and a general
 // one for its last slabs, persistent workgroups with the operand stream carried across tiles, epilogue operands brought
 // into an LDS table by LDS-direct loads.
@@ -23,7 +23,7 @@
 //     [E,N,K] weights: LDS row rho is column rho, chunk c at position c ^ (bit 1 | bits 3..4 << 1 of rho) -- the rows a
 //     quarter wave reads differ in bits 0, 1, 3, 4.  Packed weights: a block (16 columns x 64 K bytes) goes to LDS as it
 //     is, odd column groups with bit 2 of the column index flipped; a fragment gathers from two column groups.  Both
-//     conflict free.
+//     conflict free.  [E,K,N] weights go through LDS transpose reads (at the kernel's head).
 //   * A K half of a slab is multiplied in four steps of 4 x 4 blocks, visited in the order (F0,I0) (F0,I1) (F1,I1) (F1,I0)
 //     (F: weight blocks 0..3 / 4..7, I: x blocks 0..3 / 4..7), so that every step needs only four new fragments and two
 //     sets of four weight and four x fragments (64 registers) are enough.  A step is 16 MFMAs (256 cycles), four
@@ -42,19 +42,38 @@ namespace {
 
 typedef int v2i __attribute__((ext_vector_type(2)));
 constexpr int T4M_B = 8;                                         // 16 x 16 blocks per wave tile edge
-constexpr int T4M_META_OFF = T4_PARAM_OFF + 2 * T4_PARAM_BYTES;  // per group: row end, tiles up to and including it
-constexpr int T4M_LDS_BYTES = T4M_META_OFF + 2 * T4_MAX_E * 4;
-static_assert(T4M_LDS_BYTES <= 160 * 1024, "LDS of one CU");
+// LDS: x stages 0 and 1 (32 KiB each), weight stages 0 and 1, two epilogue operand tables, the group table.  [E,K,N]
+// weights (WL == 2) lie in LDS as K rows of 256 column bytes at a pitch of 288 bytes (see the kernel's head).
+constexpr int T4M_KN_PITCH = 288;
+constexpr int t4m_w_stage(int wl) { return wl == 2 ? T4_BK * T4M_KN_PITCH : T4_OP_STAGE; }
+constexpr int t4m_param_off(int wl) { return T4_W_BASE + 2 * t4m_w_stage(wl); }
+constexpr int t4m_meta_off(int wl) { return t4m_param_off(wl) + 2 * T4_PARAM_BYTES; }   // per group: row end, tiles up to and including it
+constexpr int t4m_lds_bytes(int wl) { return t4m_meta_off(wl) + 2 * T4_MAX_E * 4; }
+static_assert(t4m_lds_bytes(2) <= 160 * 1024, "LDS of one CU");
 
 }  // namespace
 
-// MODE: output type, 0 bf16, 1 f16, 2 int32 (raw accumulators plus bias).  PK: weights in the packed layout (1 KiB blocks
+// MODE: output type, 0 bf16, 1 f16, 2 int32 (raw accumulators plus bias).  WL: weight layout, 0 [E,N,K], 1 packed, 2 [E,K,N]
+// (N a multiple of 16).  Packed (1 KiB blocks
 // of 16 columns x 64 K bytes; a slab of a tile is 16 column groups x 2 blocks, staging quad (u, wave) is block 4 u + wave =
 // (column group 2 u + wave / 2, K block wave % 2) and goes to LDS as it is) instead of [E,N,K].  ACT: 0 none, 1 gelu
 // (tanh form), 2 v * sigmoid(c v) (silu, fast gelu), 3 relu.
-template <int MODE, bool PK, int ACT>
+//
+// [E,K,N]: rows are N-contiguous and an MFMA operand wants 16 K-contiguous bytes per lane; the LDS transpose read of gfx950
+// (ds_read_b64_tr_b8) does that turn on the way out of LDS.  Of a block of 16 lanes, lane i names 8 bytes M[i][0..7];
+// lane j receives byte b = M[2 b + j / 8][j % 8].  A slab goes to LDS as it lies in memory -- K rows of 256 columns, one
+// staging quad = 4 K rows, lane L row L / 16, 16-column chunk L % 16 -- at a row pitch of 288 bytes, so that the eight K
+// rows and two chunks that one block of 16 lanes names fall into sixteen different 16-byte bank groups and every part of
+// a fragment address is additive.  The middle dwords of every chunk are swapped on the way in: the first 8 bytes of a
+// chunk then are columns 0..3 and 8..11, the second 8 bytes columns 4..7 and 12..15 -- fragment rows 0..7 of an even and of
+// an odd weight block (see the head of the file).  K rows 16..31 (mod 32) store the two halves the other way round: the
+// two blocks of 16 lanes that read together (K rows 16 apart) then use different banks.  A fragment is two transpose
+// reads, 8 K rows apart.
+template <int MODE, int WL, int ACT>
 __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const GmmParams p) {
   extern __shared__ __align__(16) unsigned char smem[];
+  constexpr bool PK = WL == 1, KN = WL == 2;
+  constexpr int W_STAGE = t4m_w_stage(WL), PARAM_OFF = t4m_param_off(WL), META_OFF = t4m_meta_off(WL);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -63,7 +82,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
 
   // ---- this workgroup's share of the tiles (as in gmm_tile4_w8a8.hip) ----------------------------------
   const int n_tiles = (p.n + T4_BN - 1) / T4_BN;
-  int *meta_end = reinterpret_cast<int *>(smem + T4M_META_OFF);
+  int *meta_end = reinterpret_cast<int *>(smem + META_OFF);
   int *meta_upto = meta_end + T4_MAX_E;
   int total = 0;
   for (int g0 = 0, carry = 0; g0 < p.e; g0 += 64) {
@@ -103,14 +122,30 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
     if constexpr (PK) {
       const long long cg_bytes = (long long)k_blocks * 1024;
       return t4_rsrc(p.w + ((long long)t.grp * col_groups + t.n0 / 16) * cg_bytes, (long long)(col_groups - t.n0 / 16) * cg_bytes);
+    } else if constexpr (KN) {
+      return t4_rsrc(p.w + (long long)t.grp * w_elems + t.n0, w_elems - t.n0);   // (loads use w_rsrc_at: a window per slab)
     } else {
       return t4_rsrc(p.w + (long long)t.grp * w_elems + (long long)t.n0 * p.k, (long long)(p.n - t.n0) * p.k);
     }
   };
+  // [E,K,N]: the window of a tile's weights from K row `krow0` on.  A slab's first row cannot go into the scalar offset
+  // of the load (the buffer unit range-checks the per-lane offset only, against the whole window): it goes into the
+  // base, and the window ends with the expert's matrix, so K rows past K and anything past the tensor read as zeros by
+  // the range check alone.  A chunk past N inside the matrix reads the next K row's bytes: columns that are never stored.
+  // (base and size of the tile's window are kept as scalars: K N < 2^31, so the size fits 32 bits)
+  struct T4Window {
+    const int8_t *base;
+    int bytes;
+  };
+  auto w_window = [&](const T4Tile &t) { return T4Window{p.w + (long long)t.grp * w_elems + t.n0, (int)w_elems - t.n0}; };
+  auto w_rsrc_at = [&](const T4Window &w, unsigned krow0) {
+    const unsigned off = krow0 * (unsigned)p.n;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(w.base + off), 0, max(w.bytes - (int)off, 0), 0x00020000);
+  };
 
   // ---- global -> staging registers: one quad = 1 KiB per wave = 8 rows x 128 B (packed weights: one block) ------------
   const unsigned rows32 = 32u * (unsigned)p.k;
-  const unsigned b_step = PK ? 2u * (unsigned)k_blocks * 1024u : rows32;   // staging quad u -> u + 1: two column groups / 32 rows
+  const unsigned b_step = PK ? 2u * (unsigned)k_blocks * 1024u : KN ? 16u * (unsigned)p.n : rows32;   // staging quad u -> u + 1: two column groups / 16 K rows / 32 rows
   int d_chunk, d_chunk_w;
   unsigned a_voff0, b_voff0;
   // ---- fragment addressing: see the head of the file ------------------------------------------------------
@@ -124,19 +159,26 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
     a_voff0 = (unsigned)d_row0 * (unsigned)p.k + d_chunk * 16;
     // weights [E,N,K]: LDS row rho is column rho of the tile, chunk c at position c ^ sw(rho) with sw(rho) = bit 1 and bits
     // 3..4 of rho (the rows a quarter wave reads differ in bits 0, 1, 3 and 4: see the head of the file)
-    d_chunk_w = PK ? d_chunk : ((ln & 7) ^ (((ln >> 4) & 1) | (wave << 1)));
-    b_voff0 = PK ? (unsigned)(((wave >> 1) * k_blocks + (wave & 1)) * 1024 + ln * 16) : (unsigned)d_row0 * (unsigned)p.k + d_chunk_w * 16;
+    d_chunk_w = WL != 0 ? d_chunk : ((ln & 7) ^ (((ln >> 4) & 1) | (wave << 1)));
+    b_voff0 = PK   ? (unsigned)(((wave >> 1) * k_blocks + (wave & 1)) * 1024 + ln * 16)
+              : KN ? (unsigned)(4 * wave + (ln >> 4)) * (unsigned)p.n + (unsigned)((ln & 15) * 16)   // K row 4 wave + lane / 16 of quad 0, chunk lane % 16
+                   : (unsigned)d_row0 * (unsigned)p.k + d_chunk_w * 16;
     const int swz = (m16 >> 1) & 7;
     x_lane = (unsigned)((wave_m * T4_WT + m16) * T4_BK + ((g4 ^ swz) << 4));
     const int w_row = 8 * (m16 >> 2) + (m16 & 3);   // fragment row m16 of blocks 0 and 1 is column w_row, w_row + 4 of the first 32
     if constexpr (PK) {
       // column group w_row / 16 (odd groups lie in LDS with bit 2 of the column swapped), column w_row % 16, chunk g4
       w_lane = (unsigned)(T4_W_BASE + wave_n * 16384 + (m16 >> 3) * 2048 + g4 * 256 + (((w_row & 15) ^ ((m16 >> 3) << 2)) << 4));
+    } else if constexpr (KN) {
+      // address lane m16 of its block of 16 names K row m16 / 2 of the 16 that lane group g4 multiplies, chunk m16 % 2 of
+      // the pair that holds the 32 columns of blocks 0 and 1, the half that holds an even block's columns
+      w_lane = (unsigned)(T4_W_BASE + (16 * g4 + (m16 >> 1)) * T4M_KN_PITCH + (wave_n * 8 + (m16 & 1)) * 16 + (g4 & 1) * 8);
     } else {
       w_lane = (unsigned)(T4_W_BASE + (wave_n * T4_WT + w_row) * T4_BK + ((g4 ^ (((m16 >> 1) & 1) | ((m16 >> 2) << 1))) << 4));
     }
     st_x = (unsigned)(wave * 1024 + ln * 16);
-    st_w = T4_W_BASE + (unsigned)(wave * 1024 + ((PK ? (ln ^ (((wave >> 1) & 1) << 2)) : ln) << 4));
+    st_w = KN ? T4_W_BASE + (unsigned)((4 * wave + (ln >> 4)) * T4M_KN_PITCH + (ln & 15) * 16)
+              : T4_W_BASE + (unsigned)(wave * 1024 + ((PK ? (ln ^ (((wave >> 1) & 1) << 2)) : ln) << 4));
     asm volatile("" : "+v"(st_w));
   };
   lane_constants();
@@ -152,6 +194,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
 
   T4Tile nxt = cur;        // tile that follows `cur` in this workgroup's walk (loads run ahead into it)
   __amdgpu_buffer_rsrc_t rx_c = x_rsrc(cur), rw_c = w_rsrc(cur), rx_n = rx_c, rw_n = rw_c;
+  T4Window ww_c = w_window(cur), ww_n = ww_c;   // ([E,K,N] only)
 
   // slab s of the current tile, or slab s - k_slabs of the next one
   auto load_one = [&](int s, auto par_c, auto op_c, auto u_c) __attribute__((always_inline)) {
@@ -165,6 +208,10 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
     const unsigned kill = dead ? T4_OOB : 0u;
     if constexpr (OP == 0) {
       stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rx_n : rx_c, (a_voff0 + U * rows32) | kill, kbase, 0);
+    } else if constexpr (KN) {
+      // K rows 16 U + 4 wave + lane / 16 of the slab, in the window that starts with the slab (rows past K fall outside it)
+      const unsigned kill_w = (ahead && !nxt.valid) ? T4_OOB : 0u;
+      stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc_at(ahead ? ww_n : ww_c, kbase), (b_voff0 + U * b_step) | kill_w, 0, 0);
     } else if constexpr (PK) {
       const unsigned kb = 2u * (unsigned)(ahead ? s - k_slabs : s) + (unsigned)(wave & 1);
       const unsigned kill_w = ((ahead && !nxt.valid) || kb >= (unsigned)k_blocks) ? T4_OOB : 0u;
@@ -174,26 +221,34 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
       stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(ahead ? rw_n : rw_c, (b_voff0 + U * b_step) | kill_n, kbase, 0);
     }
   };
-  auto put_quad = [&](unsigned addr, v4i v) __attribute__((always_inline)) {
-#if MSCO_TILE4_ATTR & 16
-    asm volatile("" ::"v"(v), "v"(addr));
-#else
-    *reinterpret_cast<v4i *>(smem + addr) = v;
-#endif
+  // LDS address of staging quad (op, u) in stage st (an int or a compile-time constant)
+  auto quad_addr = [&](auto st, auto op_c, auto u_c) __attribute__((always_inline)) -> unsigned {
+    constexpr int OP = decltype(op_c)::value, U = decltype(u_c)::value;
+    if constexpr (OP == 0) return st_x + (unsigned)st * T4_OP_STAGE + U * 4096;
+    else return st_w + (unsigned)st * W_STAGE + U * (KN ? 16 * T4M_KN_PITCH : 4096);
   };
-  // one 8-byte half of a staging quad to LDS
-  auto put_half = [&](unsigned addr, const v4i &v, auto h_c) __attribute__((always_inline)) {
-    constexpr int H = decltype(h_c)::value;
+  // one 8-byte half (H = 0 first) of staging quad (op, u) to LDS.  [E,K,N] weights: the middle dwords of the chunk
+  // change places before the first half leaves, and the K rows of odd quads store their halves the other way round.
+  auto put_half = [&](auto st, auto p_c, auto op_c, auto u_c, auto h_c) __attribute__((always_inline)) {
+    constexpr int P = decltype(p_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value, H = decltype(h_c)::value;
+    v4i &v = stg[P][OP][U];
+    if constexpr (KN && OP == 1 && H == 0) {
+      int y = v.y, z = v.z;
+      asm volatile("v_swap_b32 %0, %1" : "+v"(y), "+v"(z));
+      v.y = y;
+      v.z = z;
+    }
+    const unsigned addr = quad_addr(st, op_c, u_c) + 8 * ((KN && OP == 1) ? (H ^ (U & 1)) : H);
 #if MSCO_TILE4_ATTR & 16
     asm volatile("" ::"v"(v), "v"(addr));
 #else
     *reinterpret_cast<v2i *>(smem + addr) = H == 0 ? v2i{v.x, v.y} : v2i{v.z, v.w};
 #endif
   };
-  // write quad (op, u) of slab s to its LDS stage and refill it with slab s + 2
+  // write quad (op, u) of slab s to its LDS stage and refill it with slab s + 2 (the prologue's form: both halves at once)
   auto cycle_one = [&](int s, auto par_c, auto op_c, auto u_c) {
-    constexpr int P = decltype(par_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
-    put_quad((OP == 0 ? st_x : st_w) + (s & 1) * T4_OP_STAGE + U * 4096, stg[P][OP][U]);
+    put_half(s & 1, par_c, op_c, u_c, c0);
+    put_half(s & 1, par_c, op_c, u_c, c1);
     load_one(s + 2, par_c, op_c, u_c);
   };
   // fragment B (0..3) of block half BH (blocks 4 BH + B) of K half `half` in LDS stage `stage` (each an int or a
@@ -206,17 +261,27 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
 #endif
     xf[S][B] = *reinterpret_cast<const v4i *>(smem + ((x_lane ^ ((unsigned)half << 6)) + (unsigned)stage * T4_OP_STAGE + (4 * BH + B) * 2048));
   };
-  auto read_w = [&](auto stage, auto half, auto set_c, auto bh_c, auto b_c) __attribute__((always_inline)) {
-    constexpr int S = decltype(set_c)::value, BH = decltype(bh_c)::value, B = decltype(b_c)::value;
+  // (PART: [E,K,N] fragments are two transpose reads, 0 and 1, each in a slot of its own; the other layouts read in part 0)
+  auto read_w = [&](auto stage, auto half, auto set_c, auto bh_c, auto b_c, auto part_c) __attribute__((always_inline)) {
+    constexpr int S = decltype(set_c)::value, BH = decltype(bh_c)::value, B = decltype(b_c)::value, PART = decltype(part_c)::value;
 #if MSCO_TILE4_ATTR & 64
-    asm volatile("" : "+v"(wf[S][B]));
+    if constexpr (PART == 0) asm volatile("" : "+v"(wf[S][B]));
     return;
 #endif
     constexpr int F = 4 * BH + B;   // block f lies at 32 (f / 2) + 4 (f % 2) columns
-    if constexpr (PK)
-      wf[S][B] = *reinterpret_cast<const v4i *>(smem + ((w_lane ^ ((F & 1) << 6)) + (unsigned)stage * T4_OP_STAGE + (unsigned)half * 1024 + (F >> 1) * 4096));
-    else
-      wf[S][B] = *reinterpret_cast<const v4i *>(smem + ((w_lane ^ ((unsigned)half << 6)) + (unsigned)stage * T4_OP_STAGE + (F >> 1) * 4096 + (F & 1) * 512));
+    if constexpr (KN) {
+      typedef __attribute__((address_space(3))) v2i *lds_v2i;
+      const unsigned addr = (w_lane ^ ((F & 1) << 3)) + (unsigned)stage * W_STAGE + (unsigned)half * (64 * T4M_KN_PITCH) + (F >> 1) * 32 +
+                            PART * (8 * T4M_KN_PITCH);
+      const v2i got = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_v2i)(smem + addr));
+      if constexpr (PART == 0) { wf[S][B].x = got.x; wf[S][B].y = got.y; }
+      else { wf[S][B].z = got.x; wf[S][B].w = got.y; }
+    } else if constexpr (PART == 0) {
+      if constexpr (PK)
+        wf[S][B] = *reinterpret_cast<const v4i *>(smem + ((w_lane ^ ((F & 1) << 6)) + (unsigned)stage * W_STAGE + (unsigned)half * 1024 + (F >> 1) * 4096));
+      else
+        wf[S][B] = *reinterpret_cast<const v4i *>(smem + ((w_lane ^ ((unsigned)half << 6)) + (unsigned)stage * W_STAGE + (F >> 1) * 4096 + (F & 1) * 512));
+    }
   };
 
   // ---- stream prologue (once per workgroup): slabs 0 and 1 requested; slab 0 and group 0 of slab 1
@@ -241,12 +306,12 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
   for (int ti = 0;; ++ti) {
     // the tile after this one: the operand stream crosses into it during the last slabs
     nxt = tile_at(ti + 1);
-    if (nxt.valid) { rx_n = x_rsrc(nxt); rw_n = w_rsrc(nxt); }
+    if (nxt.valid) { rx_n = x_rsrc(nxt); rw_n = w_rsrc(nxt); ww_n = w_window(nxt); }
     if (ti > 0) lane_constants();
 
     // Epilogue operands of this tile (scale and bias of its 256 columns, per-token scale of its 256 rows) go straight
     // from memory into this tile's LDS table (two tables, alternating per tile); the K-loop barriers publish them.
-    unsigned char *table = smem + T4_PARAM_OFF + (ti & 1) * T4_PARAM_BYTES;
+    unsigned char *table = smem + PARAM_OFF + (ti & 1) * T4_PARAM_BYTES;
     {
       const unsigned lds = (unsigned)(unsigned long)(__attribute__((address_space(3))) unsigned char *)table + wave * 256;
       const int col = cur.n0 + tid, row = cur.m0 + tid;
@@ -280,7 +345,8 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
     const int bm_active = max(0, min(T4M_B, (rows_wave + 15) / 16));
 
     // the fragments of the first step of slab 0: weight blocks 0..3 into set 0, x blocks 0..3 into set 0, K half 0
-    read_w(c0, c0, c0, c0, c0); read_w(c0, c0, c0, c0, c1); read_w(c0, c0, c0, c0, c2); read_w(c0, c0, c0, c0, c3);
+    read_w(c0, c0, c0, c0, c0, c0); read_w(c0, c0, c0, c0, c1, c0); read_w(c0, c0, c0, c0, c2, c0); read_w(c0, c0, c0, c0, c3, c0);
+    read_w(c0, c0, c0, c0, c0, c1); read_w(c0, c0, c0, c0, c1, c1); read_w(c0, c0, c0, c0, c2, c1); read_w(c0, c0, c0, c0, c3, c1);
     read_x(c0, c0, c0, c0, c0); read_x(c0, c0, c0, c0, c1); read_x(c0, c0, c0, c0, c2); read_x(c0, c0, c0, c0, c3);
 
     {
@@ -345,8 +411,7 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
           constexpr int P = decltype(p_c)::value, OP = decltype(op_c)::value, G = decltype(g_c)::value;
           constexpr bool EARLY = decltype(early_c)::value != 0;
           auto wr = [&](auto q_c, auto h_c) __attribute__((always_inline)) {
-            constexpr int U = 2 * G + decltype(q_c)::value, H = decltype(h_c)::value;
-            put_half((OP == 0 ? st_x : st_w) + (unsigned)st * T4_OP_STAGE + U * 4096 + H * 8, stg[P][OP][U], h_c);
+            put_half(st, p_c, op_c, std::integral_constant<int, 2 * G + decltype(q_c)::value>{}, h_c);
           };
           auto rq = [&](auto q_c) __attribute__((always_inline)) {
             fill(p_c, op_c, std::integral_constant<int, 2 * G + decltype(q_c)::value>{});
@@ -355,49 +420,54 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
             constexpr int S = decltype(s_c)::value;
             if constexpr (!EARLY) {
               if constexpr (S == 0) wr(c0, c0);
-              else if constexpr (S == 1) rd(c0);
+              else if constexpr (S == 1) rd(c0, c0);
+              else if constexpr (S == 2) rd(c0, c1);
               else if constexpr (S == 4) wr(c0, c1);
-              else if constexpr (S == 5) rd(c1);
+              else if constexpr (S == 5) rd(c1, c0);
+              else if constexpr (S == 6) rd(c1, c1);
               else if constexpr (S == 7) rq(c0);
               else if constexpr (S == 8) wr(c1, c0);
-              else if constexpr (S == 9) rd(c2);
+              else if constexpr (S == 9) rd(c2, c0);
+              else if constexpr (S == 10) rd(c2, c1);
               else if constexpr (S == 12) wr(c1, c1);
-              else if constexpr (S == 13) rd(c3);
+              else if constexpr (S == 13) rd(c3, c0);
+              else if constexpr (S == 14) rd(c3, c1);
               else if constexpr (S == 15) rq(c1);
             } else {
               if constexpr (S == 0) wr(c0, c0);
-              else if constexpr (S == 1) rd(c0);
+              else if constexpr (S == 1) rd(c0, c0);
               else if constexpr (S == 2) wr(c0, c1);
-              else if constexpr (S == 3) rd(c1);
+              else if constexpr (S == 3) rd(c1, c0);
               else if constexpr (S == 4) wr(c1, c0);
-              else if constexpr (S == 5) rd(c2);
+              else if constexpr (S == 5) rd(c2, c0);
               else if constexpr (S == 6) wr(c1, c1);
-              else if constexpr (S == 7) rd(c3);
+              else if constexpr (S == 7) rd(c3, c0);
               else if constexpr (S == 9) rq(c0);
               else if constexpr (S == 11) rq(c1);
             }
           });
         };
         // 1: (F0,I0) of K half 0 from sets (0,0); x blocks 4..7 of K half 0 into set 1
-        step(c1, c0, c0, c0, c0, [&](auto b_c) __attribute__((always_inline)) { read_x(stage, c0, c1, c1, b_c); }, os, par_c, c0, c1, fill_a, c0);
+        step(c1, c0, c0, c0, c0, [&](auto b_c, auto part_c) __attribute__((always_inline)) { if constexpr (decltype(part_c)::value == 0) read_x(stage, c0, c1, c1, b_c); }, os, par_c, c0, c1, fill_a, c0);
         // 2: (F0,I1) from (0,1); weight blocks 4..7 of K half 0 into set 1
-        step(c1, c0, c1, c0, c1, [&](auto b_c) __attribute__((always_inline)) { read_w(stage, c0, c1, c1, b_c); }, os, par_c, c1, c1, fill_a, c0);
+        step(c1, c0, c1, c0, c1, [&](auto b_c, auto part_c) __attribute__((always_inline)) { read_w(stage, c0, c1, c1, b_c, part_c); }, os, par_c, c1, c1, fill_a, c0);
         // 3: (F1,I1) from (1,1); weight blocks 0..3 of K half 1 into set 0
-        step(c0, c1, c1, c1, c1, [&](auto b_c) __attribute__((always_inline)) { read_w(stage, c1, c0, c0, b_c); }, os, par_c, c0, c2, fill_a, c0);
+        step(c0, c1, c1, c1, c1, [&](auto b_c, auto part_c) __attribute__((always_inline)) { read_w(stage, c1, c0, c0, b_c, part_c); }, os, par_c, c0, c2, fill_a, c0);
         // 4: (F1,I0) from (1,0); x blocks 0..3 of K half 1 into set 1
-        step(c0, c1, c0, c1, c0, [&](auto b_c) __attribute__((always_inline)) { read_x(stage, c1, c1, c0, b_c); }, os, par_c, c1, c2, fill_a, c0);
+        step(c0, c1, c0, c1, c0, [&](auto b_c, auto part_c) __attribute__((always_inline)) { if constexpr (decltype(part_c)::value == 0) read_x(stage, c1, c1, c0, b_c); }, os, par_c, c1, c2, fill_a, c0);
         // 5: (F0,I0) of K half 1 from (0,1); x blocks 4..7 of K half 1 into set 0
-        step(c1, c0, c1, c0, c0, [&](auto b_c) __attribute__((always_inline)) { read_x(stage, c1, c0, c1, b_c); }, os, par_c, c0, c3, fill_a, c0);
+        step(c1, c0, c1, c0, c0, [&](auto b_c, auto part_c) __attribute__((always_inline)) { if constexpr (decltype(part_c)::value == 0) read_x(stage, c1, c0, c1, b_c); }, os, par_c, c0, c3, fill_a, c0);
         // 6: (F0,I1) from (0,0); weight blocks 4..7 of K half 1 into set 1
-        step(c1, c0, c0, c0, c1, [&](auto b_c) __attribute__((always_inline)) { read_w(stage, c1, c1, c1, b_c); }, os, par_c, c1, c3, fill_a, c1);
+        step(c1, c0, c0, c0, c1, [&](auto b_c, auto part_c) __attribute__((always_inline)) { read_w(stage, c1, c1, c1, b_c, part_c); }, os, par_c, c1, c3, fill_a,
+             std::integral_constant<int, KN ? 0 : 1>{});   // ([E,K,N]: eight reads do not fit the first half)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #if !(MSCO_TILE4_ATTR & 32)
         t4_barrier();
 #endif
         // 7: (F1,I1) from (1,0); next slab: weight blocks 0..3 of K half 0 into set 0; x group 0 of the slab after next
-        step(c0, c1, c0, c1, c1, [&](auto b_c) __attribute__((always_inline)) { read_w(os, c0, c0, c0, b_c); }, stage, oth, c0, c0, fill_b, c0);
+        step(c0, c1, c0, c1, c1, [&](auto b_c, auto part_c) __attribute__((always_inline)) { read_w(os, c0, c0, c0, b_c, part_c); }, stage, oth, c0, c0, fill_b, c0);
         // 8: (F1,I0) from (1,1); next slab: x blocks 0..3 of K half 0 into set 0; weight group 0 of the slab after next
-        step(c0, c1, c1, c1, c0, [&](auto b_c) __attribute__((always_inline)) { read_x(os, c0, c0, c0, b_c); }, stage, oth, c1, c0, fill_b, c0);
+        step(c0, c1, c1, c1, c0, [&](auto b_c, auto part_c) __attribute__((always_inline)) { if constexpr (decltype(part_c)::value == 0) read_x(os, c0, c0, c0, b_c); }, stage, oth, c1, c0, fill_b, c0);
       };
       // slab kt, its look-ahead anywhere (next tile, past K)
       auto slab_any = [&](int kt, auto par_c) __attribute__((always_inline)) {
@@ -410,18 +480,20 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
       auto slab_inside = [&](auto stage_c, auto par_c, unsigned soff3, unsigned soff4) __attribute__((always_inline)) {
         constexpr int ST = decltype(stage_c)::value;
         const std::integral_constant<int, ST ^ 1> os;
-        auto refill = [&](unsigned soff, auto p_c, auto op_c, auto u_c) __attribute__((always_inline)) {
+        // ([E,K,N]: one window per slab, made once per slab, and no offset)
+        const __amdgpu_buffer_rsrc_t rw3 = KN ? w_rsrc_at(ww_c, soff3) : rw_c, rw4 = KN ? w_rsrc_at(ww_c, soff4) : rw_c;
+        auto refill = [&](unsigned soff, __amdgpu_buffer_rsrc_t rw_s, auto p_c, auto op_c, auto u_c) __attribute__((always_inline)) {
           constexpr int P = decltype(p_c)::value, OP = decltype(op_c)::value, U = decltype(u_c)::value;
 #if MSCO_TILE4_ATTR & 8
           v4i &q = stg[P][OP][U];   // (named first: operands of an asm statement do not capture)
           asm volatile("" : "+v"(q));
 #else
           if constexpr (OP == 0) stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rx_c, a_voff0 + U * rows32, soff, 0);
-          else stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rw_c, b_voff0 + U * b_step, PK ? soff * 16 : soff, 0);
+          else stg[P][OP][U] = __builtin_amdgcn_raw_buffer_load_b128(rw_s, b_voff0 + U * b_step, PK ? soff * 16 : KN ? 0u : soff, 0);
 #endif
         };
-        slab(stage_c, os, par_c, [&](auto p_c, auto op_c, auto u_c) __attribute__((always_inline)) { refill(soff3, p_c, op_c, u_c); },
-             [&](auto p_c, auto op_c, auto u_c) __attribute__((always_inline)) { refill(soff4, p_c, op_c, u_c); });
+        slab(stage_c, os, par_c, [&](auto p_c, auto op_c, auto u_c) __attribute__((always_inline)) { refill(soff3, rw3, p_c, op_c, u_c); },
+             [&](auto p_c, auto op_c, auto u_c) __attribute__((always_inline)) { refill(soff4, rw4, p_c, op_c, u_c); });
       };
       // slabs whose furthest request (group 0 of the slab five on) ends inside K run the compile-time body, two per round
       const int k_clean = max(0, ((p.k / T4_BK - 4) / 2) * 2);
@@ -589,25 +661,27 @@ __global__ void __launch_bounds__(T4_NW * 64, 1) gmm_w8a8_tile4m_kernel(const Gm
     cur = nxt;
     rx_c = rx_n;
     rw_c = rw_n;
+    ww_c = ww_n;
   }
 }
 
-template <int MODE, bool PK, int ACT>
+template <int MODE, int WL, int ACT>
 static hipError_t t4m_launch(const GmmParams &p, unsigned grid, hipStream_t stream) {
-  auto kern = gmm_w8a8_tile4m_kernel<MODE, PK, ACT>;
+  auto kern = gmm_w8a8_tile4m_kernel<MODE, WL, ACT>;
   static std::atomic<bool> attr_set{false};   // the attribute call is idempotent: a race between first launches repeats it at worst
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, T4M_LDS_BYTES);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, t4m_lds_bytes(WL));
     if (e != hipSuccess) return e;
     attr_set = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(T4_NW * 64), T4M_LDS_BYTES, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(T4_NW * 64), t4m_lds_bytes(WL), stream, p);
   return hipGetLastError();
 }
 
 hipError_t launch_tile4m_w8a8(const GmmParams &p, int layout, hipStream_t stream) {
-  // layout 0 [E,N,K], 1 packed; the operand stream runs up to four slabs ahead inside one tile; the group table lives in LDS
-  if (p.k < 4 * T4_BK || p.e > T4_MAX_E || layout < 0 || layout > 1) return hipErrorInvalidValue;
+  // layout 0 [E,N,K], 1 packed, 2 [E,K,N] (read in 16-column chunks); the operand stream runs up to four slabs ahead inside
+  // one tile; the group table lives in LDS
+  if (p.k < 4 * T4_BK || p.e > T4_MAX_E || layout < 0 || layout > 2 || (layout == 2 && p.n % 16 != 0)) return hipErrorInvalidValue;
   const long long n_tiles = (p.n + T4_BN - 1) / T4_BN;
   const long long m_tiles_ub = (p.m + T4_BM - 1) / T4_BM + p.e;   // every non-empty group adds at most one partial tile
   const long long total_ub = m_tiles_ub * n_tiles;
@@ -616,16 +690,16 @@ hipError_t launch_tile4m_w8a8(const GmmParams &p, int layout, hipStream_t stream
   if (grid <= 0) return hipSuccess;
   const int act = p.act_type == ACT_NONE ? 0 : p.act_type == ACT_RELU ? 3 : (p.act_type == ACT_SILU || p.act_type == ACT_FAST_GELU) ? 2 : 1;
   const unsigned g = (unsigned)grid;
-#define MSCO_T4M_BY_ACT(MODE, PK)                                   \
-  (act == 0   ? t4m_launch<MODE, PK, 0>(p, g, stream)               \
-   : act == 1 ? t4m_launch<MODE, PK, 1>(p, g, stream)               \
-   : act == 2 ? t4m_launch<MODE, PK, 2>(p, g, stream)               \
-              : t4m_launch<MODE, PK, 3>(p, g, stream))
-#define MSCO_T4M_BY_LAYOUT(MODE) (layout == 1 ? MSCO_T4M_BY_ACT(MODE, true) : MSCO_T4M_BY_ACT(MODE, false))
+#define MSCO_T4M_BY_ACT(MODE, WL)                                   \
+  (act == 0   ? t4m_launch<MODE, WL, 0>(p, g, stream)               \
+   : act == 1 ? t4m_launch<MODE, WL, 1>(p, g, stream)               \
+   : act == 2 ? t4m_launch<MODE, WL, 2>(p, g, stream)               \
+              : t4m_launch<MODE, WL, 3>(p, g, stream))
+#define MSCO_T4M_BY_LAYOUT(MODE) (layout == 1 ? MSCO_T4M_BY_ACT(MODE, 1) : layout == 2 ? MSCO_T4M_BY_ACT(MODE, 2) : MSCO_T4M_BY_ACT(MODE, 0))
   switch (p.out_dtype) {
     case DT_BF16: return MSCO_T4M_BY_LAYOUT(0);
     case DT_F16: return MSCO_T4M_BY_LAYOUT(1);
-    case DT_I32: return layout == 1 ? t4m_launch<2, true, 0>(p, g, stream) : t4m_launch<2, false, 0>(p, g, stream);
+    case DT_I32: return layout == 1 ? t4m_launch<2, 1, 0>(p, g, stream) : layout == 2 ? t4m_launch<2, 2, 0>(p, g, stream) : t4m_launch<2, 0, 0>(p, g, stream);
     default: return hipErrorInvalidValue;
   }
 #undef MSCO_T4M_BY_LAYOUT

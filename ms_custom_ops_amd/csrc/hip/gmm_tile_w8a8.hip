@@ -641,7 +641,7 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
   // cannot take runs the eight-wave kernel of the same tile shape
   if (tile_cfg == TILE_256x256_W4 || tile_cfg == TILE_256x256_W4_MFMA32) {
     if (p.k >= 512 && p.e <= 1024)
-      return layout != 2 && tile_cfg == TILE_256x256_W4 ? launch_tile4m_w8a8(p, layout, stream) : launch_tile4_w8a8(p, layout, stream);
+      return tile_cfg == TILE_256x256_W4 ? launch_tile4m_w8a8(p, layout, stream) : launch_tile4_w8a8(p, layout, stream);
     tile_cfg = TILE_256x256;
   }
   switch (tile_cfg) {

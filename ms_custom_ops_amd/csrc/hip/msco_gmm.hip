@@ -25,7 +25,7 @@ enum Override : int {
   OV_AUTO = 0, OV_TILE_256 = 1, OV_TILE_128 = 2, OV_TILE_64 = 3, OV_SKINNY = 4, OV_GENERIC = 5,
   OV_TILE_256_W4 = 6,  // persistent four-wave 256 x 256 kernel
   OV_TILE_128x256 = 7,  // four waves side by side, 128 x 256
-  OV_TILE_256_W4_MFMA32 = 8  // the persistent kernel's 32 x 32 x 32 form on every layout (the plan takes it for [E,K,N] only)
+  OV_TILE_256_W4_MFMA32 = 8  // the persistent kernel's 32 x 32 x 32 form (never planned)
 };
 
 constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned

@@ -34,6 +34,7 @@ CASES = [
     ("tile256_w4_packed", cabi.OV_TILE_256_W4, False, True, (700, 640, 512, 3, [300, 300, 700])),
     ("tile256_w4_mfma32", cabi.OV_TILE_256_W4_MFMA32, True, False, (700, 640, 512, 3, [300, 300, 700])),
     ("tile256_w4_mfma32_packed", cabi.OV_TILE_256_W4_MFMA32, False, True, (700, 640, 512, 3, [300, 300, 700])),
+    ("tile256_w4_mfma32_kn", cabi.OV_TILE_256_W4_MFMA32, False, False, (700, 640 + 48, 512 - 16, 3, [300, 300, 700])),
     ("tile256_w4_kn", cabi.OV_TILE_256_W4, False, False, (700, 640 + 48, 512 - 16, 3, [300, 300, 700])),   # [E,K,N] through transpose reads, K and N tails
     # 128 x 256 tiles (several groups of about a hundred rows, enough columns to fill the chip with them)
     ("tile128x256", cabi.OV_AUTO, True, False, (800, 256, 6144, 8, [90, 200, 310, 400, 400, 530, 700, 800])),

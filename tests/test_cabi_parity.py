@@ -172,7 +172,7 @@ def test_few_tiles_split_k_across_workgroups(device, transpose_b):
 
 # ------------------------------------------------------------- persistent four-wave tile kernel
 W4 = cabi.OV_TILE_256_W4
-# both forms of the persistent kernel on [E,N,K] weights: 16 x 16 x 64 MFMAs (what the plan takes) and 32 x 32 x 32
+# both forms of the persistent kernel: 16 x 16 x 64 MFMAs (what the plan takes) and 32 x 32 x 32
 W4_FORMS = pytest.mark.parametrize("W4", [cabi.OV_TILE_256_W4, cabi.OV_TILE_256_W4_MFMA32], ids=["mfma16", "mfma32"])
 
 
