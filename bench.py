@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 ROTATE_BYTES = 768e6      # HBM-bound cases rotate over weight copies totalling more than the 256 MB Infinity Cache
 LAYOUT_TEXT = {"nk": "prepacked once to [E,N,K]", "kn": "[E,K,N] as generated",
                "packed": "prepacked once to the blocked layout"}
-WARM_MIN_LAUNCHES, WARM_MIN_MS, WARM_MAX_MS, WARM_TOLERANCE = 40, 30.0, 1500.0, 0.01
+WARM_MIN_LAUNCHES, WARM_MIN_MS, WARM_MAX_MS, WARM_TOLERANCE = 60, 30.0, 1500.0, 0.01
 COPY_BYTES = 1 << 29      # --probe copy: one launch reads and writes this many bytes
 TRAFFIC_FILE = os.path.join(REPO, "ms_custom_ops_amd", "measured_traffic.json")
 
@@ -149,7 +149,7 @@ class DeviceProblem:
 
         `warmup` is a floor.  The shader clock takes tens of launches to settle under this load, so the untimed phase
         goes on (in batches of ten launches, each timed with events) until at least WARM_MIN_LAUNCHES launches and
-        WARM_MIN_MS of device time have passed and two batches in a row agree within WARM_TOLERANCE, or WARM_MAX_MS is
+        WARM_MIN_MS of device time have passed and three batches in a row agree within WARM_TOLERANCE, or WARM_MAX_MS is
         used up.  `details` records the warm-up launches actually made and the period of the first and the last
         quarter of the timed steps, so a figure taken while the clock still moved shows."""
         torch = self.torch
@@ -157,7 +157,7 @@ class DeviceProblem:
         for _ in range(warmup):
             self.step()
         torch.cuda.synchronize()
-        done, spent_ms, prev, stable = warmup, 0.0, None, False
+        done, spent_ms, recent, stable = warmup, 0.0, [], False
         while spent_ms < WARM_MAX_MS:
             a, b = ev(), ev()
             a.record()
@@ -168,8 +168,8 @@ class DeviceProblem:
             batch = a.elapsed_time(b)
             done += 10
             spent_ms += batch
-            stable = prev is not None and abs(batch - prev) <= WARM_TOLERANCE * prev
-            prev = batch
+            recent = (recent + [batch])[-3:]
+            stable = len(recent) == 3 and max(recent) - min(recent) <= WARM_TOLERANCE * min(recent)
             if stable and done >= WARM_MIN_LAUNCHES and spent_ms >= WARM_MIN_MS:
                 break
         marks = sorted({0, steps // 4, steps - steps // 4, steps})
