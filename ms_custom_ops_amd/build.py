@@ -19,7 +19,7 @@ INCLUDE = os.path.join(REPO_DIR, "include")
 
 BACKEND_LIB = os.path.join(LIB_DIR, "libmsco_gmm.so")
 PROBES_LIB = os.path.join(LIB_DIR, "libmsco_probes.so")   # measurement aids: not part of the operator library
-HIP_SOURCES = ["gmm_tile_w8a8.hip", "gmm_tile4_w8a8.hip", "gmm_tile4m_w8a8.hip", "gmm_skinny_w8a8.hip", "gmm_skinny_a16w8.hip", "gmm_generic.hip", "gmm_stream.hip", "msco_gmm.hip", "moe_routing.hip", "gmm_w4.hip"]
+HIP_SOURCES = ["gmm_tile_w8a8.hip", "gmm_tile4_w8a8.hip", "gmm_tile4m_w8a8.hip", "gmm_rows_w8a8.hip", "gmm_skinny_w8a8.hip", "gmm_skinny_a16w8.hip", "gmm_generic.hip", "gmm_stream.hip", "msco_gmm.hip", "moe_routing.hip", "gmm_w4.hip"]
 PROBE_SOURCES = ["probes.hip"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

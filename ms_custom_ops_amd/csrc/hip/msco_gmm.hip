@@ -25,7 +25,9 @@ enum Override : int {
   OV_AUTO = 0, OV_TILE_256 = 1, OV_TILE_128 = 2, OV_TILE_64 = 3, OV_SKINNY = 4, OV_GENERIC = 5,
   OV_TILE_256_W4 = 6,  // persistent four-wave 256 x 256 kernel
   OV_TILE_128x256 = 7,  // four waves side by side, 128 x 256
-  OV_TILE_256_W4_MFMA32 = 8  // the persistent kernel's 32 x 32 x 32 form (never planned)
+  OV_TILE_256_W4_MFMA32 = 8,  // the persistent kernel's 32 x 32 x 32 form (never planned)
+  OV_ROWS128 = 9,  // packed weights: chunks of up to 128 rows through LDS, weights straight into MFMA operands (other layouts: 128 x 256 tiles)
+  OV_ROWS256 = 10  // the same with chunks of up to 256 rows (other layouts: the persistent kernel)
 };
 
 constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned
@@ -107,7 +109,7 @@ int check_desc(const msco_gmm_desc &d) {
   if (d.group_list_dtype != MSCO_DT_NONE && d.group_list_dtype != MSCO_DT_I32 && d.group_list_dtype != MSCO_DT_I64)
     return MSCO_ERR_UNSUPPORTED;
   if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
-  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_TILE_256_W4_MFMA32) return MSCO_ERR_INVALID_ARG;
+  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_ROWS256) return MSCO_ERR_INVALID_ARG;
   if (d.weight_layout != MSCO_WL_ROW_MAJOR && d.weight_layout != MSCO_WL_PACKED) return MSCO_ERR_INVALID_ARG;
   if (d.force_split_k < 0) return MSCO_ERR_INVALID_ARG;
   if (d.act_type < MSCO_ACT_NONE || d.act_type > MSCO_ACT_SILU) return MSCO_ERR_INVALID_ARG;
@@ -203,7 +205,21 @@ void choose_plan(msco_gmm_op *op) {
     // 126 rows: 84 - 92 us with 128 x 256 tiles against 100 - 109 us with 256 x 256; at 120 rows on average the largest
     // group has 131, streams its weights twice and the launch takes 126 against 113 us -- so the 256-row tile takes
     // over at 1.5 x the average = 160 rows, not at 128)
-    if (e > 1 && w4_ok && cover > 160 && cover <= 384 && group_tiles(256, 256) >= busy) {
+    // Packed weights, several groups of up to about 130 rows each and enough columns that 256-column strips give every CU
+    // a workgroup: the row-chunk kernel streams a group's weights once, straight into MFMA operands, and multiplies only
+    // the 16-row blocks that hold rows.  Measured, 8 experts, K = 4096, N = 14336 (470 MB of weights; a launch that only
+    // reads them takes 72 us), rows per group 16 / 32 / 64 / 96 / 112 / 128: 72.8 / 75.8 / 79.2 / 83.8 / 85.9 / 107.6 us
+    // (the last with 256-row chunks, one workgroup per CU) against 76.5 / 79.6 / 82.4 / 89.1 / 111.0 / 112.4 us for the
+    // tiles picked below.  A group that overflows its 128-row chunk streams its weights a second time (128 rows on average,
+    // half of the groups above: 131 us), hence 256-row chunks from 116 rows on average; at 144 rows they tie with the
+    // persistent kernel (110.9 against 111.3 us) and lose beyond (160 rows: 118.1 against 113.8 us).  Few columns leave
+    // CUs idle: N = 1344, K = 5120: 41 against 24 us for 64 x 128 tiles with a K split.
+    const bool rows_kernel_ok = is_packed(d) && e > 1 && k >= 1024 && ((n + 255) / 256) * std::min<int64_t>(e, m) >= num_cus;
+    if (rows_kernel_ok && avg_rows <= 116) {
+      op->tile_cfg = TILE_ROWS128;
+    } else if (rows_kernel_ok && avg_rows <= 136) {
+      op->tile_cfg = TILE_ROWS256;
+    } else if (e > 1 && w4_ok && cover > 160 && cover <= 384 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
     } else if (e > 1 && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
       // (128 x 256 tiles re-read x half as often: 64 / 96 rows per group 93 / 99 us against 100 / 111 us)
@@ -238,6 +254,8 @@ void choose_plan(msco_gmm_op *op) {
     case OV_TILE_128: family = FAM_TILE; op->tile_cfg = TILE_128x128; break;
     case OV_TILE_128x256: family = FAM_TILE; op->tile_cfg = TILE_128x256; break;
     case OV_TILE_64: family = FAM_TILE; op->tile_cfg = TILE_64x128; break;
+    case OV_ROWS128: family = FAM_TILE; op->tile_cfg = is_packed(d) ? TILE_ROWS128 : TILE_128x256; break;
+    case OV_ROWS256: family = FAM_TILE; op->tile_cfg = is_packed(d) ? TILE_ROWS256 : TILE_256x256_W4; break;
     case OV_SKINNY: family = FAM_SKINNY; break;
     case OV_GENERIC: family = FAM_GENERIC; break;
     default: break;
@@ -253,6 +271,8 @@ void choose_plan(msco_gmm_op *op) {
   if (family == FAM_TILE) {
     const int forced = tuning().tile_cfg;
     if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO) op->tile_cfg = forced;
+    if (op->tile_cfg == TILE_ROWS256 && !is_packed(d)) op->tile_cfg = TILE_256x256_W4;
+    if (op->tile_cfg == TILE_ROWS128 && !is_packed(d)) op->tile_cfg = TILE_128x256;
     // Few tiles (M of a few hundred rows): split K across workgroups until about kTileTargetWorkgroups of them
     // stream operands; every slice keeps at least kTileMinSlabs 64-byte K slabs.  Small tile shapes only.
     if (op->tile_cfg == TILE_128x128 || op->tile_cfg == TILE_64x128) {
@@ -307,6 +327,24 @@ void choose_plan(msco_gmm_op *op) {
       op->w_nontemporal = (is_packed(d) || d.transpose_b == 0) && e * k * n >= nt_bytes && (group_rows + bm - 1) / bm <= 2;
     }
     if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
+  }
+  if (family == FAM_TILE && (op->tile_cfg == TILE_ROWS256 || op->tile_cfg == TILE_ROWS128)) {
+    // Row-chunk kernel: every workgroup streams a strip of up to 16 column groups over all of K, so a launch takes whole
+    // rounds of equally long workgroups (two per CU with 128-row chunks, one with 256-row chunks).  The strip is as wide
+    // as makes the rounds shortest: 8 experts x 14336 columns on 256 CUs give 448 workgroups = two rounds of 16 column
+    // groups, or 512 = two of 14.  One chunk per group is expected.
+    const int64_t slots = (int64_t)(num_cus > 0 ? num_cus : kDefaultCUs) * (op->tile_cfg == TILE_ROWS128 ? 2 : 1);
+    const int64_t col_groups = (n + 15) / 16, chunks = std::max<int64_t>(1, std::min<int64_t>(e, m));
+    int best = 16;
+    int64_t best_cost = INT64_MAX;
+    for (int sg = 16; sg >= 10; --sg) {
+      const int64_t rounds = (((col_groups + sg - 1) / sg) * chunks + slots - 1) / slots;
+      if (rounds * sg < best_cost) { best_cost = rounds * sg; best = sg; }
+    }
+    op->strip_groups = best;
+    const int forced_groups = tuning().stream_groups;
+    if (forced_groups >= 1 && forced_groups <= 16) op->strip_groups = forced_groups;
+    op->n_strips = (int)((col_groups + op->strip_groups - 1) / op->strip_groups);
   }
   // Many experts with uneven loads (a skewed routing): every group of a few rows costs the persistent kernel a whole
   // 256-row m-tile per n-tile.  The groups of at most 64 rows go to a second launch of 64 x 128 tiles instead, which
