@@ -43,6 +43,15 @@ struct XrShape {
 };
 }  // namespace
 
+// acc += a x b with the accumulator tied to one block of accumulation registers (256-row chunks: one wave per SIMD,
+// 256 accumulation registers).  Left to the register allocator, the accumulator blocks of that form change places
+// between the unrolled slabs of the K loop -- two to three register copies per MFMA, 44 % of the MFMA rate where this
+// form reaches 80 %.  Declared to touch memory, the statement also keeps the LDS reads and memory requests around it
+// in the order they are written in.
+__device__ __forceinline__ void mfma_pinned(v4i &acc, const v4i &a, const v4i &b) {
+  asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b) : "memory");
+}
+
 template <int RBMAX, int RB>
 __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem, int grp, int m0, int chunk_rows, int strip) {
   using S = XrShape<RBMAX>;
@@ -166,8 +175,10 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
       constexpr int I = decltype(i_c)::value, KBS = I / RB, R = I % RB;
       if constexpr (I + XR_AHEAD < 2 * RB) fq[(I + XR_AHEAD) % (XR_AHEAD + 1)] = frag(I + XR_AHEAD);
 #pragma unroll
-      for (int cg = 0; cg < XR_CG; ++cg)
-        acc[cg][R] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fq[I % (XR_AHEAD + 1)], ring[2 * J + KBS][cg], acc[cg][R], 0, 0, 0);
+      for (int cg = 0; cg < XR_CG; ++cg) {
+        if constexpr (RBMAX == 16) mfma_pinned(acc[cg][R], fq[I % (XR_AHEAD + 1)], ring[2 * J + KBS][cg]);
+        else acc[cg][R] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fq[I % (XR_AHEAD + 1)], ring[2 * J + KBS][cg], acc[cg][R], 0, 0, 0);
+      }
       if constexpr (R == RB - 1) {
 #pragma unroll
         for (int cg = 0; cg < XR_CG; ++cg) ring[2 * J + KBS][cg] = wload(2 * s + KBS + DEPTH, cg);
@@ -176,7 +187,8 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
     xstore(ST ^ 1, std::integral_constant<int, XD == 2 ? (ST ^ 1) : 0>{});   // slab s + 1 to its stage
     // the order the instructions of this slab are issued in: x requests, fragment reads XR_AHEAD ahead of their four
     // MFMAs, a K block's four weight requests behind its last MFMA, staging writes at the end (0x008 MFMA, 0x020 memory
-    // read, 0x100 LDS read, 0x200 LDS write)
+    // read, 0x100 LDS read, 0x200 LDS write).  (The pinned MFMAs of the 256-row form keep the written order by themselves.)
+    if constexpr (RBMAX != 16) {
     __builtin_amdgcn_sched_group_barrier(0x020, XP, 0);
     __builtin_amdgcn_sched_group_barrier(0x100, XR_AHEAD < 2 * RB ? XR_AHEAD : 2 * RB, 0);
     static_for<2 * RB>([&](auto i_c) {
@@ -186,6 +198,7 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
       if constexpr (I % RB == RB - 1) __builtin_amdgcn_sched_group_barrier(0x020, XR_CG, 0);
     });
     __builtin_amdgcn_sched_group_barrier(0x200, XP, 0);
+    }
   };
   const int slabs = (k_blocks + 1) / 2;
   for (int s = 0; s < slabs; s += DEPTH / 2) {

@@ -205,19 +205,19 @@ void choose_plan(msco_gmm_op *op) {
     // 126 rows: 84 - 92 us with 128 x 256 tiles against 100 - 109 us with 256 x 256; at 120 rows on average the largest
     // group has 131, streams its weights twice and the launch takes 126 against 113 us -- so the 256-row tile takes
     // over at 1.5 x the average = 160 rows, not at 128)
-    // Packed weights, several groups of up to about 130 rows each and enough columns that 256-column strips give every CU
-    // a workgroup: the row-chunk kernel streams a group's weights once, straight into MFMA operands, and multiplies only
+    // Packed weights, several groups of up to about 150 rows each and enough columns that 256-column strips give every CU
+    // a workgroup: the row-chunk kernels stream a group's weights once, straight into MFMA operands, and multiply only
     // the 16-row blocks that hold rows.  Measured, 8 experts, K = 4096, N = 14336 (470 MB of weights; a launch that only
-    // reads them takes 72 us), rows per group 16 / 32 / 64 / 96 / 112 / 128: 72.8 / 75.8 / 79.2 / 83.8 / 85.9 / 107.6 us
-    // (the last with 256-row chunks, one workgroup per CU) against 76.5 / 79.6 / 82.4 / 89.1 / 111.0 / 112.4 us for the
-    // tiles picked below.  A group that overflows its 128-row chunk streams its weights a second time (128 rows on average,
-    // half of the groups above: 131 us), hence 256-row chunks from 116 rows on average; at 144 rows they tie with the
-    // persistent kernel (110.9 against 111.3 us) and lose beyond (160 rows: 118.1 against 113.8 us).  Few columns leave
-    // CUs idle: N = 1344, K = 5120: 41 against 24 us for 64 x 128 tiles with a K split.
+    // reads them takes 72 us), rows per group 16 / 32 / 64 / 96 / 112: 72.8 / 75.8 / 79.2 / 83.8 / 85.9 us with 128-row
+    // chunks (two workgroups per CU) against 76.5 / 79.6 / 82.4 / 89.1 / 111.0 us for the tiles picked below.  A group
+    // that overflows its 128-row chunk takes a second workgroup that streams its weights again (128 rows on average, half
+    // of the groups above: 131 us), hence 256-row chunks (one workgroup per CU) from 116 rows on average: 128 / 144 / 160
+    // rows per group 104 / 102 / 110 us against 112 / 110 / 112 us for the persistent kernel, which wins beyond (192 rows:
+    // 125 against 115 us).  Few columns leave CUs idle: N = 1344, K = 5120: 41 against 24 us for 64 x 128 tiles with a K split.
     const bool rows_kernel_ok = is_packed(d) && e > 1 && k >= 1024 && ((n + 255) / 256) * std::min<int64_t>(e, m) >= num_cus;
     if (rows_kernel_ok && avg_rows <= 116) {
       op->tile_cfg = TILE_ROWS128;
-    } else if (rows_kernel_ok && avg_rows <= 136) {
+    } else if (rows_kernel_ok && avg_rows <= 150) {
       op->tile_cfg = TILE_ROWS256;
     } else if (e > 1 && w4_ok && cover > 160 && cover <= 384 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
