@@ -204,7 +204,8 @@ void choose_plan(msco_gmm_op *op) {
     // (128-row m-tiles while every group fits one: 8 experts, 72 .. 112 rows per group on average, the largest group 80 ..
     // 126 rows: 84 - 92 us with 128 x 256 tiles against 100 - 109 us with 256 x 256; at 120 rows on average the largest
     // group has 131, streams its weights twice and the launch takes 126 against 113 us -- so the 256-row tile takes
-    // over at 1.5 x the average = 160 rows, not at 128)
+    // over at 1.5 x the average = 174 rows, not at 128; at 112 rows on average, the largest group 126, [E,K,N] weights:
+    // 104 us with 128 x 256 tiles against 116 us)
     // Packed weights, several groups of up to about 150 rows each and enough columns that 256-column strips give every CU
     // a workgroup: the row-chunk kernels stream a group's weights once, straight into MFMA operands, and multiply only
     // the 16-row blocks that hold rows.  Measured, 8 experts, K = 4096, N = 14336 (470 MB of weights; a launch that only
@@ -214,12 +215,14 @@ void choose_plan(msco_gmm_op *op) {
     // of the groups above: 131 us), hence 256-row chunks (one workgroup per CU) from 116 rows on average: 128 / 144 / 160
     // rows per group 104 / 102 / 110 us against 112 / 110 / 112 us for the persistent kernel, which wins beyond (192 rows:
     // 125 against 115 us).  Few columns leave CUs idle: N = 1344, K = 5120: 41 against 24 us for 64 x 128 tiles with a K split.
+    // (narrower strips for fewer columns do not pay: with one or two column groups per wave, strips of 6 / 3 column groups,
+    // 8 experts, 1024 rows, K = 5120, N = 2688 / 1344: 55 / 40 us against 46 / 24 us for the 64 x 128 tiles)
     const bool rows_kernel_ok = is_packed(d) && e > 1 && k >= 1024 && ((n + 255) / 256) * std::min<int64_t>(e, m) >= num_cus;
     if (rows_kernel_ok && avg_rows <= 116) {
       op->tile_cfg = TILE_ROWS128;
     } else if (rows_kernel_ok && avg_rows <= 150) {
       op->tile_cfg = TILE_ROWS256;
-    } else if (e > 1 && w4_ok && cover > 160 && cover <= 384 && group_tiles(256, 256) >= busy) {
+    } else if (e > 1 && w4_ok && cover > 174 && cover <= 384 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
     } else if (e > 1 && cover > 64 && cover <= 192 && group_tiles(128, 128) >= busy) {
       // (128 x 256 tiles re-read x half as often: 64 / 96 rows per group 93 / 99 us against 100 / 111 us)
@@ -329,17 +332,20 @@ void choose_plan(msco_gmm_op *op) {
     if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
   }
   if (family == FAM_TILE && (op->tile_cfg == TILE_ROWS256 || op->tile_cfg == TILE_ROWS128)) {
-    // Row-chunk kernel: every workgroup streams a strip of up to 16 column groups over all of K, so a launch takes whole
-    // rounds of equally long workgroups (two per CU with 128-row chunks, one with 256-row chunks).  The strip is as wide
-    // as makes the rounds shortest: 8 experts x 14336 columns on 256 CUs give 448 workgroups = two rounds of 16 column
-    // groups, or 512 = two of 14.  One chunk per group is expected.
-    const int64_t slots = (int64_t)(num_cus > 0 ? num_cus : kDefaultCUs) * (op->tile_cfg == TILE_ROWS128 ? 2 : 1);
+    // Row-chunk kernel: every workgroup streams a strip of up to 16 column groups over all of K plus its chunk's x rows,
+    // and the workgroups that share a CU share its operand path.  The strip is as wide as makes the bytes a CU moves
+    // least: ceil(workgroups / CUs) x (strip bytes + x bytes of a chunk), one chunk per group expected.  8 experts x 14336
+    // columns on 256 CUs: 448 workgroups of 16 column groups cost two per CU as 512 of 14 do (c3_t64 82.2 -> 72.8 us).
+    const int64_t cus = num_cus > 0 ? num_cus : kDefaultCUs;
     const int64_t col_groups = (n + 15) / 16, chunks = std::max<int64_t>(1, std::min<int64_t>(e, m));
+    const int64_t chunk_rows = op->tile_cfg == TILE_ROWS128 ? 128 : 256;
+    const int64_t x_bytes = std::min<int64_t>(avg_rows, chunk_rows) * k;
     int best = 16;
     int64_t best_cost = INT64_MAX;
     for (int sg = 16; sg >= 10; --sg) {
-      const int64_t rounds = (((col_groups + sg - 1) / sg) * chunks + slots - 1) / slots;
-      if (rounds * sg < best_cost) { best_cost = rounds * sg; best = sg; }
+      const int64_t wgs = ((col_groups + sg - 1) / sg) * chunks;
+      const int64_t cost = ((wgs + cus - 1) / cus) * ((int64_t)sg * 16 * k + x_bytes);
+      if (cost < best_cost) { best_cost = cost; best = sg; }
     }
     op->strip_groups = best;
     const int forced_groups = tuning().stream_groups;

@@ -134,3 +134,4 @@ def test_the_plan_picks_the_rows_kernels_for_several_groups_of_up_to_about_130_r
     last = int(gl[-1])
     assert np.array_equal(bits[:last], ref[:last]), info
     assert (bits[last:] == 0x7FC0).all(), info
+
