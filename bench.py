@@ -637,7 +637,7 @@ def main():
                              ("c2_m16", "kn"), ("c2_m16", "packed"), ("c2_m1", "kn"), ("c2_m1", "packed"), ("c5", "kn"),
                              ("c5", "packed"), ("c3_decode", "kn"), ("c3_decode", "packed"),
                              # the headline MoE layer at serving batch sizes (T tokens, top-2 of 8): bound by the 470 MB of weights
-                             ("c3_t64", "packed"), ("c3_t128", "packed"), ("c3_t256", "packed"), ("c3_t512", "packed"),
+                             ("c3_t64", "packed"), ("c3_t128", "packed"), ("c3_t256", "packed"), ("c3_t448", "packed"), ("c3_t512", "packed"),
                              ("c3_t1024", "packed"),
                              # the weight-only layer beyond decode: chunks of 32 .. 128 rows share a pass over the weights
                              ("c5_t64", "packed"), ("c5_t256", "packed"), ("c5_t256", "kn"),
