@@ -98,6 +98,31 @@ def _gmm_args(x=(64, 64), w=(8, 64, 128), gl=(8,), xt=I8, wt=I8, glt=I32, bias=N
             None if aq is None else fake((e, w[-2], 1), aq), ta, tb, xf, od]
 
 
+def test_plan_of_the_serving_range_on_packed_weights_without_a_gpu():
+    # shapes only: eight experts, K = 4096, N = 14336 (no device: the plan assumes 256 CUs).  Packed weights take the row-chunk
+    # kernels up to about 150 rows per group, 128-row chunks up to 116, in strips of 14 column groups (512 workgroups);
+    # other layouts and few columns keep the tiles; the forced forms fall back to tiles on row-major weights.
+    def plan(m, n=14336, k=4096, e=8, packed=True, override=0):
+        op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64, scale_dtype=cabi.DT_F32,
+                        per_token_dtype=cabi.DT_F32, weight_layout=cabi.WL_PACKED if packed else cabi.WL_ROW_MAJOR,
+                        kernel_override=override)
+        ws = op.plan(m, k, n, e)
+        info = op.plan_info()
+        op.close()
+        return info, ws
+    for m, want in ((128, "tile_rows128"), (896, "tile_rows128"), (8 * 116, "tile_rows128"), (8 * 117, "tile_rows256"), (1024, "tile_rows256"),
+                    (8 * 150, "tile_rows256"), (8 * 151, "tile_256x256x128_w4"), (2048, "tile_256x256x128_w4"), (64, "w8a8_stream")):
+        info, ws = plan(m)
+        assert want in info and ws == 0, (m, info)
+    assert "strips=64 " in plan(896)[0] and "strips=64 " in plan(1024)[0]
+    assert "rows" not in plan(896, packed=False)[0]
+    assert "rows" not in plan(1024, n=1344, k=5120)[0]                 # few columns: CUs would idle
+    assert "rows" not in plan(896, k=512)[0]
+    assert "tile_128x256" in plan(896, packed=False, override=cabi.OV_ROWS128)[0]
+    assert "tile_256x256x128_w4" in plan(896, packed=False, override=cabi.OV_ROWS256)[0]
+    assert "tile_rows256" in plan(300, n=512, k=256, e=2, override=cabi.OV_ROWS256)[0]
+
+
 def test_grouped_matmul_infer_shape_and_type():
     shapes, types = _C._graph_infer("grouped_matmul", _gmm_args())
     assert shapes == [[64, 128]] and types == [F16]          # the reference's float16 output
