@@ -489,7 +489,7 @@ def plan_regret(steps=30):
     forced = (("tile_256", cabi.OV_TILE_256), ("tile_256_w4", cabi.OV_TILE_256_W4), ("tile_256_w4_mfma32", cabi.OV_TILE_256_W4_MFMA32),
               ("tile_128x256", cabi.OV_TILE_128x256),
               ("tile_128", cabi.OV_TILE_128), ("tile_64", cabi.OV_TILE_64), ("decode", cabi.OV_SKINNY),
-              ("rows_128", cabi.OV_ROWS128), ("rows_256", cabi.OV_ROWS256))
+              ("rows_128", cabi.OV_ROWS128), ("rows_160", cabi.OV_ROWS160), ("rows_256", cabi.OV_ROWS256))
     names = ["c2_m%d" % m for m in (1, 16, 17, 32, 64, 65, 128, 192, 256, 320, 384, 448, 512, 640, 704, 768, 1024, 1280, 1536, 2048, 3072)]
     names += ["c3_t%d" % t for t in (8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 448, 512, 576, 768, 1024, 2048)]
     rows = []
@@ -511,7 +511,7 @@ def plan_regret(steps=30):
                 # (families that would stream the weights dozens of times, or multiply mostly padding, are not candidates)
                 if (fam == "decode" and per_group > 64) or (fam == "tile_64" and per_group > 512) or \
                         (fam in ("tile_256", "tile_256_w4") and wl.m < 64) or (fam in ("tile_128", "tile_128x256") and wl.m < 32) or \
-                        (fam in ("rows_128", "rows_256") and (layout != "packed" or wl.e == 1 or wl.m < 32)):
+                        (fam in ("rows_128", "rows_160", "rows_256") and (layout != "packed" or wl.e == 1 or wl.m < 32)):
                     continue
                 try:
                     op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64,

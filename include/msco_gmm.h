@@ -134,8 +134,8 @@ typedef struct msco_gmm_desc {
   int32_t kernel_override;   /* 0 auto; else force a kernel family, for tests and planner checks: 1 eight-wave 256 x 256 tile,
                               * 2 128 x 128, 3 64 x 128, 4 decode (streaming) kernels, 5 generic, 6 persistent four-wave
                               * 256 x 256 (16 x 16 x 64 MFMAs), 7 128 x 256, 8 the persistent kernel's 32 x 32 x 32 MFMA form,
-                              * 9 / 10 packed weights: chunks of up to 128 / 256 rows through LDS and weights straight into
-                              * MFMA operands
+                              * 9 / 10 / 11 packed weights: chunks of up to 128 / 256 / 160 rows through LDS and weights
+                              * straight into MFMA operands
                               * (msco_gmm_plan_info names what was planned) */
   int32_t weight_layout;     /* MSCO_WL_ROW_MAJOR: as transpose_b says; MSCO_WL_PACKED: written by msco_pack_weight */
   int32_t act_type;          /* msco_act: activation applied to the dequantised float32 value before the output cast */

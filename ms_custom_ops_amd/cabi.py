@@ -24,7 +24,7 @@ IN_X, IN_WEIGHT, IN_BIAS, IN_SCALE, IN_GROUP_LIST, IN_PER_TOKEN_SCALE, IN_ANTIQU
 IN_COUNT = 8
 
 # msco_gmm_desc.kernel_override
-OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC, OV_TILE_256_W4, OV_TILE_128x256, OV_TILE_256_W4_MFMA32, OV_ROWS128, OV_ROWS256 = range(11)
+OV_AUTO, OV_TILE_256, OV_TILE_128, OV_TILE_64, OV_SKINNY, OV_GENERIC, OV_TILE_256_W4, OV_TILE_128x256, OV_TILE_256_W4_MFMA32, OV_ROWS128, OV_ROWS256, OV_ROWS160 = range(12)
 
 # msco_gmm_desc.act_type
 ACT_NONE, ACT_RELU, ACT_GELU_TANH, ACT_GELU_ERF, ACT_FAST_GELU, ACT_SILU = range(6)

@@ -13,7 +13,8 @@ enum TileCfg : int {
   TILE_256x256_W4_MFMA32 = 5,   // the same on 32 x 32 x 32 MFMAs: gmm_tile4_w8a8.hip (never planned; kept to be measured against)
   TILE_ROWS256 = 6,   // packed weights only: chunks of up to 256 rows x strips of 256 columns, x through LDS, weights straight into MFMA operands: gmm_rows_w8a8.hip
   TILE_ROWS128 = 7,   // the same with chunks of up to 128 rows and two workgroups per CU
-  TILE_CFG_COUNT = 8
+  TILE_ROWS160 = 8,   // ... of up to 160 rows, two workgroups per CU, two K blocks of weights in flight
+  TILE_CFG_COUNT = 9
 };
 
 // MFMA tile kernel for W8A8 (prefill shapes).  nk: weights stored [E,N,K]; packed: the packed layout (nk is ignored).
@@ -22,7 +23,7 @@ const char *tile_cfg_name(int tile_cfg);
 hipError_t launch_tile4m_w8a8(const GmmParams &p, int layout, hipStream_t stream);  // layout 0 [E,N,K], 1 packed, 2 [E,K,N] (N % 16 == 0)
 hipError_t launch_tile4_w8a8(const GmmParams &p, int layout, hipStream_t stream);   // layout 0 [E,N,K], 1 packed, 2 [E,K,N] (N % 16 == 0)
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn);
-// packed weights, several groups of a few dozen to a few hundred rows: chunks of 16 rbmax rows (rbmax = 8 or 16), see gmm_rows_w8a8.hip
+// packed weights, several groups of a few dozen to a few hundred rows: chunks of 16 rbmax rows (rbmax = 8, 10 or 16), see gmm_rows_w8a8.hip
 hipError_t launch_rows_w8a8(const GmmParams &p, int rbmax, hipStream_t stream);
 // K split across workgroups (p.split_k > 1; four-wave tile shapes only): partial tiles and arrival counters
 size_t tile_count_bound(int tile_cfg, int64_t m, int64_t n, int64_t e);

@@ -17,6 +17,9 @@
 //     the two rows of a staging write fall into 16 different bank groups.
 //   * the K loop exists once per number of live 16-row blocks RB (1 .. RBMAX): accumulators are registers and a group of
 //     130 rows costs the MFMAs of 144, not of 256.
+//   * three forms: chunks of up to 128 rows (accumulators in VGPRs, two workgroups per CU, 4 or 8 K blocks of weights
+//     in flight per wave), of up to 160 rows (160 accumulators in VGPRs leave room for two K blocks in flight; the second
+//     workgroup of the CU covers the wait) and of up to 256 rows (256 accumulation registers, one wave per SIMD);
 //   * epilogue as everywhere: float32(acc + bias) * scale[n] * per_token[m], activation, 16-bit output, staged through
 //     LDS 16 rows at a time for whole-row stores.
 #include "gmm_common.h"
@@ -58,7 +61,10 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
   // K blocks of weights in flight per wave (a multiple of 4: stages alternate inside a round of DEPTH / 2 slabs): eight
   // while few rows are multiplied and a slab passes in less than a memory round trip, four where the accumulators and
   // the x staging registers leave room for no more
-  constexpr int DEPTH = 2 * RB <= RBMAX ? 8 : 4;
+  // (the 160-row form keeps 160 accumulators in VGPRs beside a second workgroup on the CU: two K blocks is all the room
+  // left, and the other workgroup's MFMAs are what covers the wait for them)
+  constexpr int DEPTH = RBMAX == 10 ? 2 : 2 * RB <= RBMAX ? 8 : 4;
+  constexpr int ROUND = DEPTH >= 4 ? DEPTH / 2 : 2;   // steps per trip round the loop (an even number: stages alternate)
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c16 = lane & 15, h = lane >> 4;
@@ -93,7 +99,7 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
   unsigned char *xw = smem + xrow * XR_SLAB + ((xpiece ^ ((xrow >> 1) & 7)) << 4);
   // A slab's rows are requested XD slabs before they are written to their stage (register set slab % XD): one slab of
   // weights passes in less than the round trip of an x request while few rows are multiplied, two where registers allow
-  constexpr int XD = (2 * RB <= RBMAX || (RBMAX == 16 && RB <= 12)) ? 2 : 1;
+  constexpr int XD = (RBMAX != 10 && (2 * RB <= RBMAX || (RBMAX == 16 && RB <= 12))) ? 2 : 1;
   v4i xs[XD][XP];
   auto xload = [&](int slab, auto set_c) {
     constexpr int SET = decltype(set_c)::value;
@@ -144,18 +150,18 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
   v4i ring[DEPTH][XR_CG];
   __builtin_amdgcn_sched_barrier(0);
   static_for<DEPTH / 2>([&](auto j_c) {
-    constexpr int J = decltype(j_c)::value, ST = J & 1, SLAB = J - DEPTH / 2;
+    constexpr int SLAB = decltype(j_c)::value - DEPTH / 2, J = SLAB + ROUND, ST = J & 1;   // the last steps of a round
     xload(SLAB + XD > 0 ? SLAB + XD : 0, std::integral_constant<int, XD == 2 ? ST : 0>{});
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kbs = 0; kbs < 2; ++kbs)
 #pragma unroll
-      for (int cg = 0; cg < XR_CG; ++cg) ring[2 * J + kbs][cg] = wload(2 * J + kbs, cg);
+      for (int cg = 0; cg < XR_CG; ++cg) ring[(2 * J + kbs) % DEPTH][cg] = wload(2 * SLAB + kbs + DEPTH, cg);
     if constexpr (SLAB == -1) xstore(0, std::integral_constant<int, XD == 2 ? (ST ^ 1) : 0>{});
     __builtin_amdgcn_sched_barrier(0);
   });
 
-  // slab s = DEPTH / 2 * i + J: stage J % 2, K blocks 2 s and 2 s + 1 in ring slots 2 J and 2 J + 1.  The 2 RB fragment
+  // slab s = ROUND i + J: stage J % 2, K blocks 2 s and 2 s + 1 in ring slots (2 J) % DEPTH and (2 J + 1) % DEPTH.  The 2 RB fragment
   // reads of a slab run XR_AHEAD fragments ahead of the MFMAs that use them.
   auto step = [&](int s, auto j_c) {
     constexpr int J = decltype(j_c)::value, ST = J & 1;
@@ -176,12 +182,12 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
       if constexpr (I + XR_AHEAD < 2 * RB) fq[(I + XR_AHEAD) % (XR_AHEAD + 1)] = frag(I + XR_AHEAD);
 #pragma unroll
       for (int cg = 0; cg < XR_CG; ++cg) {
-        if constexpr (RBMAX == 16) mfma_pinned(acc[cg][R], fq[I % (XR_AHEAD + 1)], ring[2 * J + KBS][cg]);
-        else acc[cg][R] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fq[I % (XR_AHEAD + 1)], ring[2 * J + KBS][cg], acc[cg][R], 0, 0, 0);
+        if constexpr (RBMAX == 16) mfma_pinned(acc[cg][R], fq[I % (XR_AHEAD + 1)], ring[(2 * J + KBS) % DEPTH][cg]);
+        else acc[cg][R] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fq[I % (XR_AHEAD + 1)], ring[(2 * J + KBS) % DEPTH][cg], acc[cg][R], 0, 0, 0);
       }
       if constexpr (R == RB - 1) {
 #pragma unroll
-        for (int cg = 0; cg < XR_CG; ++cg) ring[2 * J + KBS][cg] = wload(2 * s + KBS + DEPTH, cg);
+        for (int cg = 0; cg < XR_CG; ++cg) ring[(2 * J + KBS) % DEPTH][cg] = wload(2 * s + KBS + DEPTH, cg);
       }
     });
     xstore(ST ^ 1, std::integral_constant<int, XD == 2 ? (ST ^ 1) : 0>{});   // slab s + 1 to its stage
@@ -201,10 +207,10 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
     }
   };
   const int slabs = (k_blocks + 1) / 2;
-  for (int s = 0; s < slabs; s += DEPTH / 2) {
+  for (int s = 0; s < slabs; s += ROUND) {
     // (whole rounds only, without a branch inside: slabs past K multiply masked weight blocks, zeros; a skipped step
     // would be one more way round the loop for the wait counts to allow for)
-    static_for<DEPTH / 2>([&](auto j_c) { step(s + decltype(j_c)::value, j_c); });
+    static_for<ROUND>([&](auto j_c) { step(s + decltype(j_c)::value, j_c); });
   }
 
   // ---- epilogue: acc[cg][rb][r] = row 16 rb + 4 h + r, column 16 (4 wave + cg) + c16 of the tile -------------------------
@@ -266,7 +272,7 @@ __device__ __forceinline__ void rows_run(const GmmParams &p, unsigned char *smem
 }
 
 template <int RBMAX>
-__global__ void __launch_bounds__(XR_THREADS, RBMAX <= 8 ? 2 : 1) gmm_w8a8_rows_kernel(const GmmParams p) {
+__global__ void __launch_bounds__(XR_THREADS, RBMAX <= 10 ? 2 : 1) gmm_w8a8_rows_kernel(const GmmParams p) {
   extern __shared__ __align__(16) unsigned char xr_smem[];
   const int lane = threadIdx.x & 63;
   // (grid.y enumerates the chunks that hold rows, group after group: a slot past the last one has nothing to do)
@@ -278,8 +284,9 @@ __global__ void __launch_bounds__(XR_THREADS, RBMAX <= 8 ? 2 : 1) gmm_w8a8_rows_
   const int strip = blockIdx.x;
   // one copy of the K loop per number of live 32-row block pairs
   bool done = false;
-  static_for<RBMAX / 2>([&](auto i_c) {
-    constexpr int RB = 2 * decltype(i_c)::value + 2;
+  // (the 160-row form is for groups that just miss 128 rows: it has copies for 6, 8 and 10 blocks only)
+  static_for<(RBMAX == 10 ? 3 : RBMAX / 2)>([&](auto i_c) {
+    constexpr int RB = RBMAX == 10 ? 2 * decltype(i_c)::value + 6 : 2 * decltype(i_c)::value + 2;
     if (!done && rb <= RB) {
       rows_run<RBMAX, RB>(p, xr_smem, grp, m0, chunk_rows, strip);
       done = true;
@@ -312,6 +319,7 @@ hipError_t launch_rows_w8a8(const GmmParams &p, int rbmax, hipStream_t stream) {
   if (p.m == 0) return hipSuccess;
   if (p.k % 16 != 0 || p.n % 16 != 0) return hipErrorInvalidValue;
   if (rbmax == 8) return rows_launch<8>(p, stream);
+  if (rbmax == 10) return rows_launch<10>(p, stream);
   if (rbmax == 16) return rows_launch<16>(p, stream);
   return hipErrorInvalidValue;
 }

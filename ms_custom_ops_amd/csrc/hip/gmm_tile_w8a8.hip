@@ -644,8 +644,8 @@ hipError_t launch_tile_w8a8(const GmmParams &p, int tile_cfg, bool nk, bool pack
       return tile_cfg == TILE_256x256_W4 ? launch_tile4m_w8a8(p, layout, stream) : launch_tile4_w8a8(p, layout, stream);
     tile_cfg = TILE_256x256;
   }
-  if (tile_cfg == TILE_ROWS256 || tile_cfg == TILE_ROWS128)
-    return packed ? launch_rows_w8a8(p, tile_cfg == TILE_ROWS256 ? 16 : 8, stream) : hipErrorInvalidValue;
+  if (tile_cfg == TILE_ROWS256 || tile_cfg == TILE_ROWS128 || tile_cfg == TILE_ROWS160)
+    return packed ? launch_rows_w8a8(p, tile_cfg == TILE_ROWS256 ? 16 : tile_cfg == TILE_ROWS160 ? 10 : 8, stream) : hipErrorInvalidValue;
   switch (tile_cfg) {
     case TILE_128x128: return launch_small<128, 128>(p, layout, stream);
     case TILE_64x128: return launch_small<64, 128>(p, layout, stream);
@@ -675,6 +675,7 @@ const char *tile_cfg_name(int tile_cfg) {
     case TILE_256x256_W4_MFMA32: return "256x256x128_w4_mfma32";
     case TILE_ROWS256: return "rows256";
     case TILE_ROWS128: return "rows128";
+    case TILE_ROWS160: return "rows160";
     default: return "?";
   }
 }
@@ -696,7 +697,7 @@ size_t tile_workspace_bytes(int tile_cfg, int64_t m, int64_t n, int64_t e, int s
 
 void tile_cfg_dims(int tile_cfg, int *bm, int *bn) {
   switch (tile_cfg) {
-    case TILE_256x256: case TILE_256x256_W4: case TILE_256x256_W4_MFMA32: case TILE_ROWS256: *bm = 256; *bn = 256; break;
+    case TILE_256x256: case TILE_256x256_W4: case TILE_256x256_W4_MFMA32: case TILE_ROWS256: case TILE_ROWS160: *bm = 256; *bn = 256; break;
     case TILE_128x128: *bm = 128; *bn = 128; break;
     case TILE_128x256: case TILE_ROWS128: *bm = 128; *bn = 256; break;
     default: *bm = 64; *bn = 128; break;

@@ -27,7 +27,8 @@ enum Override : int {
   OV_TILE_128x256 = 7,  // four waves side by side, 128 x 256
   OV_TILE_256_W4_MFMA32 = 8,  // the persistent kernel's 32 x 32 x 32 form (never planned)
   OV_ROWS128 = 9,  // packed weights: chunks of up to 128 rows through LDS, weights straight into MFMA operands (other layouts: 128 x 256 tiles)
-  OV_ROWS256 = 10  // the same with chunks of up to 256 rows (other layouts: the persistent kernel)
+  OV_ROWS256 = 10,  // the same with chunks of up to 256 rows (other layouts: the persistent kernel)
+  OV_ROWS160 = 11   // ... of up to 160 rows (other layouts: the persistent kernel)
 };
 
 constexpr int64_t kSkinnyMaxRows = 64;   // total rows up to which the weight-streaming kernel is planned
@@ -109,7 +110,7 @@ int check_desc(const msco_gmm_desc &d) {
   if (d.group_list_dtype != MSCO_DT_NONE && d.group_list_dtype != MSCO_DT_I32 && d.group_list_dtype != MSCO_DT_I64)
     return MSCO_ERR_UNSUPPORTED;
   if (d.group_list_type != 0 && d.group_list_type != 1) return MSCO_ERR_INVALID_ARG;
-  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_ROWS256) return MSCO_ERR_INVALID_ARG;
+  if (d.kernel_override < OV_AUTO || d.kernel_override > OV_ROWS160) return MSCO_ERR_INVALID_ARG;
   if (d.weight_layout != MSCO_WL_ROW_MAJOR && d.weight_layout != MSCO_WL_PACKED) return MSCO_ERR_INVALID_ARG;
   if (d.force_split_k < 0) return MSCO_ERR_INVALID_ARG;
   if (d.act_type < MSCO_ACT_NONE || d.act_type > MSCO_ACT_SILU) return MSCO_ERR_INVALID_ARG;
@@ -210,17 +211,22 @@ void choose_plan(msco_gmm_op *op) {
     // a workgroup: the row-chunk kernels stream a group's weights once, straight into MFMA operands, and multiply only
     // the 16-row blocks that hold rows.  Measured, 8 experts, K = 4096, N = 14336 (470 MB of weights; a launch that only
     // reads them takes 72 us), rows per group 16 / 32 / 64 / 96 / 112: 72.8 / 75.8 / 79.2 / 83.8 / 85.9 us with 128-row
-    // chunks (two workgroups per CU) against 76.5 / 79.6 / 82.4 / 89.1 / 111.0 us for the tiles picked below.  A group
-    // that overflows its 128-row chunk takes a second workgroup that streams its weights again (128 rows on average, half
-    // of the groups above: 131 us), hence 256-row chunks (one workgroup per CU) from 116 rows on average: 128 / 144 / 160
-    // rows per group 104 / 102 / 110 us against 112 / 110 / 112 us for the persistent kernel, which wins beyond (192 rows:
-    // 125 against 115 us).  Few columns leave CUs idle: N = 1344, K = 5120: 41 against 24 us for 64 x 128 tiles with a K split.
+    // chunks against 76.5 / 79.6 / 82.4 / 89.1 / 111.0 us for the tiles picked below.  A group that overflows its chunk
+    // takes a second workgroup that streams its weights again (128 rows on average, half of the groups above 128: 131 us),
+    // hence 160-row chunks from 116 rows on average (still two workgroups per CU, with room for two K blocks of weights
+    // in flight only): 120 / 128 / 136 / 144 rows per group 88.6 / 89.3 / 91.6 / 91.7 us against 100 / 103 / 103 / 105 us
+    // with 256-row chunks (one workgroup per CU) and 110 - 112 us for the persistent kernel.  256-row chunks are left with
+    // 147 .. 155 rows per group (152 rows, the largest group 164: 107.9 against 118 us); the persistent kernel wins beyond
+    // (160 rows: 115 us either way; 192 rows: 125 against 115 us).  Few columns leave CUs idle: N = 1344, K = 5120: 41
+    // against 24 us for 64 x 128 tiles with a K split.
     // (narrower strips for fewer columns do not pay: with one or two column groups per wave, strips of 6 / 3 column groups,
     // 8 experts, 1024 rows, K = 5120, N = 2688 / 1344: 55 / 40 us against 46 / 24 us for the 64 x 128 tiles)
     const bool rows_kernel_ok = is_packed(d) && e > 1 && k >= 1024 && ((n + 255) / 256) * std::min<int64_t>(e, m) >= num_cus;
     if (rows_kernel_ok && avg_rows <= 116) {
       op->tile_cfg = TILE_ROWS128;
-    } else if (rows_kernel_ok && avg_rows <= 150) {
+    } else if (rows_kernel_ok && avg_rows <= 146) {
+      op->tile_cfg = TILE_ROWS160;
+    } else if (rows_kernel_ok && avg_rows <= 155) {
       op->tile_cfg = TILE_ROWS256;
     } else if (e > 1 && w4_ok && cover > 174 && cover <= 384 && group_tiles(256, 256) >= busy) {
       op->tile_cfg = TILE_256x256_W4;
@@ -259,6 +265,7 @@ void choose_plan(msco_gmm_op *op) {
     case OV_TILE_64: family = FAM_TILE; op->tile_cfg = TILE_64x128; break;
     case OV_ROWS128: family = FAM_TILE; op->tile_cfg = is_packed(d) ? TILE_ROWS128 : TILE_128x256; break;
     case OV_ROWS256: family = FAM_TILE; op->tile_cfg = is_packed(d) ? TILE_ROWS256 : TILE_256x256_W4; break;
+    case OV_ROWS160: family = FAM_TILE; op->tile_cfg = is_packed(d) ? TILE_ROWS160 : TILE_256x256_W4; break;
     case OV_SKINNY: family = FAM_SKINNY; break;
     case OV_GENERIC: family = FAM_GENERIC; break;
     default: break;
@@ -274,7 +281,7 @@ void choose_plan(msco_gmm_op *op) {
   if (family == FAM_TILE) {
     const int forced = tuning().tile_cfg;
     if (forced >= 0 && forced < TILE_CFG_COUNT && d.kernel_override == OV_AUTO) op->tile_cfg = forced;
-    if (op->tile_cfg == TILE_ROWS256 && !is_packed(d)) op->tile_cfg = TILE_256x256_W4;
+    if ((op->tile_cfg == TILE_ROWS256 || op->tile_cfg == TILE_ROWS160) && !is_packed(d)) op->tile_cfg = TILE_256x256_W4;
     if (op->tile_cfg == TILE_ROWS128 && !is_packed(d)) op->tile_cfg = TILE_128x256;
     // Few tiles (M of a few hundred rows): split K across workgroups until about kTileTargetWorkgroups of them
     // stream operands; every slice keeps at least kTileMinSlabs 64-byte K slabs.  Small tile shapes only.
@@ -331,14 +338,14 @@ void choose_plan(msco_gmm_op *op) {
     }
     if (op->tile_cfg == TILE_128x256 && tuning().tile_wide_k >= 0) op->wide_k_slabs = tuning().tile_wide_k != 0;   // (measured slower with 128-byte slabs: 99 against 93 us)
   }
-  if (family == FAM_TILE && (op->tile_cfg == TILE_ROWS256 || op->tile_cfg == TILE_ROWS128)) {
+  if (family == FAM_TILE && (op->tile_cfg == TILE_ROWS256 || op->tile_cfg == TILE_ROWS128 || op->tile_cfg == TILE_ROWS160)) {
     // Row-chunk kernel: every workgroup streams a strip of up to 16 column groups over all of K plus its chunk's x rows,
     // and the workgroups that share a CU share its operand path.  The strip is as wide as makes the bytes a CU moves
     // least: ceil(workgroups / CUs) x (strip bytes + x bytes of a chunk), one chunk per group expected.  8 experts x 14336
     // columns on 256 CUs: 448 workgroups of 16 column groups cost two per CU as 512 of 14 do (c3_t64 82.2 -> 72.8 us).
     const int64_t cus = num_cus > 0 ? num_cus : kDefaultCUs;
     const int64_t col_groups = (n + 15) / 16, chunks = std::max<int64_t>(1, std::min<int64_t>(e, m));
-    const int64_t chunk_rows = op->tile_cfg == TILE_ROWS128 ? 128 : 256;
+    const int64_t chunk_rows = op->tile_cfg == TILE_ROWS128 ? 128 : op->tile_cfg == TILE_ROWS160 ? 160 : 256;
     const int64_t x_bytes = std::min<int64_t>(avg_rows, chunk_rows) * k;
     int best = 16;
     int64_t best_cost = INT64_MAX;

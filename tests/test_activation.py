@@ -42,6 +42,7 @@ CASES = [
     # row chunks through LDS, weights straight into MFMA operands (packed weights): 128- and 256-row chunks
     ("rows128_packed", cabi.OV_ROWS128, False, True, RAGGED),
     ("rows256_packed", cabi.OV_ROWS256, False, True, RAGGED),
+    ("rows160_packed", cabi.OV_ROWS160, False, True, RAGGED),
     # sixteen uneven groups: the persistent kernel takes the large ones, a second launch of 64 x 128 tiles the small ones
     ("two_launches_packed", cabi.OV_TILE_256_W4, False, True,
      (1200, 512, 512, 16, [300, 303, 303, 373, 437, 502, 503, 783, 783, 800, 830, 900, 964, 1100, 1101, 1200])),
@@ -50,7 +51,7 @@ CASES = [
 ]
 # what the plan of a case has to name, so that the case keeps reaching the code it is there for
 PLAN_MUST_NAME = {"tile128x256": "128x256", "tile128x256_packed": "128x256", "two_launches_packed": "small_groups=64",
-                  "two_launches_kn": "small_groups=64", "stream_rows": "stream_rows", "rows128_packed": "rows128", "rows256_packed": "rows256"}
+                  "two_launches_kn": "small_groups=64", "stream_rows": "stream_rows", "rows128_packed": "rows128", "rows256_packed": "rows256", "rows160_packed": "rows160"}
 
 
 def _reference(x, w, gl, bias, scale, pt, act):

@@ -100,7 +100,8 @@ def _gmm_args(x=(64, 64), w=(8, 64, 128), gl=(8,), xt=I8, wt=I8, glt=I32, bias=N
 
 def test_plan_of_the_serving_range_on_packed_weights_without_a_gpu():
     # shapes only: eight experts, K = 4096, N = 14336 (no device: the plan assumes 256 CUs).  Packed weights take the row-chunk
-    # kernels up to about 150 rows per group, 128-row chunks up to 116, in strips of 14 column groups (512 workgroups);
+    # kernels up to about 155 rows per group (chunks of 128 rows up to 116 per group, of 160 up to 146), in strips of 14 column
+    # groups (512 workgroups);
     # other layouts and few columns keep the tiles; the forced forms fall back to tiles on row-major weights.
     def plan(m, n=14336, k=4096, e=8, packed=True, override=0):
         op = cabi.GmmOp(x_dtype=cabi.DT_I8, out_dtype=cabi.DT_BF16, group_list_dtype=cabi.DT_I64, scale_dtype=cabi.DT_F32,
@@ -110,8 +111,9 @@ def test_plan_of_the_serving_range_on_packed_weights_without_a_gpu():
         info = op.plan_info()
         op.close()
         return info, ws
-    for m, want in ((128, "tile_rows128"), (896, "tile_rows128"), (8 * 116, "tile_rows128"), (8 * 117, "tile_rows256"), (1024, "tile_rows256"),
-                    (8 * 150, "tile_rows256"), (8 * 151, "tile_256x256x128_w4"), (2048, "tile_256x256x128_w4"), (64, "w8a8_stream")):
+    for m, want in ((128, "tile_rows128"), (896, "tile_rows128"), (8 * 116, "tile_rows128"), (8 * 117, "tile_rows160"), (1024, "tile_rows160"),
+                    (8 * 146, "tile_rows160"), (8 * 147, "tile_rows256"), (8 * 155, "tile_rows256"), (8 * 156, "tile_256x256x128_w4"),
+                    (2048, "tile_256x256x128_w4"), (64, "w8a8_stream")):
         info, ws = plan(m)
         assert want in info and ws == 0, (m, info)
     assert "strips=64 " in plan(896)[0] and "strips=64 " in plan(1024)[0]
@@ -121,6 +123,7 @@ def test_plan_of_the_serving_range_on_packed_weights_without_a_gpu():
     assert "tile_128x256" in plan(896, packed=False, override=cabi.OV_ROWS128)[0]
     assert "tile_256x256x128_w4" in plan(896, packed=False, override=cabi.OV_ROWS256)[0]
     assert "tile_rows256" in plan(300, n=512, k=256, e=2, override=cabi.OV_ROWS256)[0]
+    assert "tile_rows160" in plan(300, n=512, k=256, e=2, override=cabi.OV_ROWS160)[0]
 
 
 def test_grouped_matmul_infer_shape_and_type():

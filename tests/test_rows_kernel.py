@@ -1,4 +1,4 @@
-"""The row-chunk kernels for packed weights (kernel_override 9: chunks of up to 128 rows, 10: of up to 256 rows; several groups of a few dozen to a few hundred rows): the
+"""The row-chunk kernels for packed weights (kernel_override 9: chunks of up to 128 rows, 10: of up to 256 rows, 11: of up to 160 rows; several groups of a few dozen to a few hundred rows): the
 group's x rows pass through LDS, the weights go from memory straight into MFMA operands.  GPU parity against the CPU
 oracle through the C ABI; bar: int32 accumulators and 16-bit outputs bit-exact."""
 import numpy as np
@@ -20,7 +20,8 @@ def _inputs(seed, m, k, n, e):
     return x, w, bias, scale, pt
 
 
-BOTH = [cabi.OV_ROWS128, cabi.OV_ROWS256]
+BOTH = [cabi.OV_ROWS128, cabi.OV_ROWS256, cabi.OV_ROWS160]
+NAME = {cabi.OV_ROWS128: "_rows128", cabi.OV_ROWS256: "_rows256", cabi.OV_ROWS160: "_rows160"}
 
 
 def _check(x, w, gl, bias, scale, pt, *, override, group_list_type=0, src_transposed=False):
@@ -31,7 +32,7 @@ def _check(x, w, gl, bias, scale, pt, *, override, group_list_type=0, src_transp
     ref_bits = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt, group_list_type=group_list_type)
     acc, info = run_w8a8(x, w, gl, bias, out="i32", override=override, packed=True, transpose_b=src_transposed,
                          group_list_type=group_list_type, launches=2)
-    assert ("_rows128" if override == cabi.OV_ROWS128 else "_rows256") in info and "layout=packed" in info, info
+    assert NAME[override] in info and "layout=packed" in info, info
     assert np.array_equal(acc[:last], ref_acc[:last]), info
     assert (acc[last:] == -7777).all(), info                       # rows past the last boundary stay untouched
     bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", override=override, packed=True,
@@ -116,10 +117,10 @@ def test_rows_kernel_without_bias_scale_or_per_token(device):
     assert np.array_equal(got, O.grouped_matmul_w8a8(x, w, gl, None, np.broadcast_to(scale[0], scale.shape), pt))
 
 
-@pytest.mark.parametrize("seed,per_group,want", [(0, 40, "rows128"), (1, 100, "rows128"), (2, 112, "rows128"), (3, 126, "rows256"), (4, 146, "rows256")])
+@pytest.mark.parametrize("seed,per_group,want", [(0, 40, "rows128"), (1, 100, "rows128"), (2, 112, "rows128"), (3, 126, "rows160"), (4, 144, "rows160"), (5, 152, "rows256")])
 def test_the_plan_picks_the_rows_kernels_for_several_groups_of_up_to_about_130_rows(device, seed, per_group, want):
     # eight groups, enough columns that 256-column strips give every CU a workgroup: 128-row chunks up to 116 rows per group
-    # on average, 256-row chunks up to 150; uneven groups (some spill into a second chunk), three rows behind the last boundary
+    # on average, 160-row chunks up to 146, 256-row chunks up to 155; uneven groups (some spill into a second chunk), three rows behind the last boundary
     from gpu_utils import run_w8a8
     rng = np.random.default_rng(7000 + seed)
     e, k, n = 8, 1024, 8192
