@@ -48,9 +48,9 @@ struct XrShape {
 
 // acc += a x b with the accumulator tied to one block of accumulation registers (256-row chunks: one wave per SIMD,
 // 256 accumulation registers).  Left to the register allocator, the accumulator blocks of that form change places
-// between the unrolled slabs of the K loop -- two to three register copies per MFMA, 44 % of the MFMA rate where this
-// form reaches 80 %.  Declared to touch memory, the statement also keeps the LDS reads and memory requests around it
-// in the order they are written in.
+// between the unrolled slabs of the K loop: two to three v_accvgpr_mov / read / write per MFMA (8 experts x 128 / 192 / 256
+// rows, K = 4096, N = 14336: 107.6 / 132 / 222 us against 104.2 / 125 / 195 us pinned).  Declared to touch memory, the
+// statement also keeps the LDS reads and memory requests around it in the order they are written in.
 __device__ __forceinline__ void mfma_pinned(v4i &acc, const v4i &a, const v4i &b) {
   asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b) : "memory");
 }
@@ -293,8 +293,6 @@ __global__ void __launch_bounds__(XR_THREADS, RBMAX <= 10 ? 2 : 1) gmm_w8a8_rows
     }
   });
 }
-
-int rows_w8a8_chunk_rows(int rbmax) { return 16 * rbmax; }
 
 template <int RBMAX>
 static hipError_t rows_launch(const GmmParams &p, hipStream_t stream) {
