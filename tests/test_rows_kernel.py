@@ -50,6 +50,7 @@ def _check(x, w, gl, bias, scale, pt, *, override, group_list_type=0, src_transp
     (1500, 720, 1040, 8, [0, 40, 300, 300, 900, 1210, 1480, 1490]),   # K not a multiple of 64, ragged and empty groups
     (530, 4096, 512, 5, [1, 18, 19, 275, 530]),                 # 1, 17, 1, 256 and 255 rows: every block count edge
     (257, 192, 256, 1, [257]),                                  # a second chunk of one row
+    (20, 80, 48, 2, [7, 20]),                                   # K of one and a quarter blocks, three column groups
 ])
 def test_rows_kernel_is_bit_exact(device, m, k, n, e, gl, override):
     x, w, bias, scale, pt = _inputs(41, m, k, n, e)
