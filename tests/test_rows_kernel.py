@@ -137,3 +137,26 @@ def test_the_plan_picks_the_rows_kernels_for_several_groups_of_up_to_about_130_r
     assert np.array_equal(bits[:last], ref[:last]), info
     assert (bits[last:] == 0x7FC0).all(), info
 
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_rows_kernels_random_shapes(device, seed):
+    # a seeded sweep: one to seventeen groups, a handful to three hundred rows per group (several chunks per group for the
+    # smaller forms), K with and without 64-byte tails, N from one column group to 225; every form against the oracle
+    from gpu_utils import run_w8a8
+    rng = np.random.default_rng(9000 + seed)
+    e = int(rng.choice([1, 2, 3, 5, 8, 17]))
+    per = int(rng.choice([3, 20, 60, 100, 128, 140, 170, 260, 300]))
+    m = max(1, int(per * e * rng.uniform(0.6, 1.3)))
+    k = int(rng.integers(1, 20)) * 64 + int(rng.choice([0, 0, 16, 32, 48]))
+    n = int(rng.choice([16, 48, 224, 256, 272, 1008, 2240, 3600]))
+    cuts = np.sort(rng.integers(0, m + 1, e - 1)) if e > 1 else np.array([], dtype=np.int64)
+    gl = np.maximum.accumulate(np.concatenate([cuts, [m - int(rng.choice([0, 0, 5]))]]).astype(np.int64).clip(0))
+    x, w, bias, scale, pt = _inputs(9000 + seed, m, k, n, e)
+    ref = O.grouped_matmul_w8a8(x, w, gl, bias, scale, pt)
+    last = int(gl[-1])
+    for override in BOTH:
+        bits, info = run_w8a8(x, w, gl, bias, scale, pt, out="bf16", packed=True, override=override, launches=2)
+        assert NAME[override] in info, info
+        assert np.array_equal(bits[:last], ref[:last]), (m, k, n, e, gl.tolist(), info)
+        assert (bits[last:] == 0x7FC0).all(), info
